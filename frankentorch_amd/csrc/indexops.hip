@@ -1,0 +1,325 @@
+// Integer-exact kernels: index_select / embedding gather, argmax, head split/merge permute.
+// Pure copies and comparisons; results are bit-for-bit those of the CPU reference.
+
+#include <type_traits>
+
+#include "common.hpp"
+
+namespace {
+
+constexpr int kWave = 64;
+constexpr int kBlock = 256;
+constexpr int64_t kMaxGrid = 2147483647LL;
+
+// normalize_strict_index_value (crates/ft-kernel-cpu/src/lib.rs:20058-20090): finite, no
+// fractional part beyond f64::EPSILON, non-negative, < dim_size. Returns -1 when invalid.
+__device__ __forceinline__ int64_t strict_index(double v, int64_t dim_size) {
+    if (!isfinite(v)) return -1;
+    double t = trunc(v);
+    if (fabs(v - t) > 2.220446049250313e-16) return -1;
+    if (v < 0.0 || v >= 9.2233720368547758e18) return -1;
+    int64_t i = (int64_t)v;
+    if (i < 0 || i >= dim_size) return -1;
+    return i;
+}
+
+// 64-bit minimum over all launches' invalid positions. An integer min does not depend on the
+// order in which the updates land, so the reported position is the same on every run.
+__device__ __forceinline__ void report_bad(int64_t *bad, int64_t pos) {
+    if (bad) atomicMin(reinterpret_cast<unsigned long long *>(bad), (unsigned long long)pos);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void index_select_kernel(const T *__restrict__ input, int64_t outer,
+                                                              int64_t dim_size, int64_t inner,
+                                                              const double *__restrict__ indices, int64_t num_indices,
+                                                              T *__restrict__ out, int64_t *bad) {
+    // One wavefront per gathered run of `inner` elements.
+    const int64_t run = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+    if (run >= outer * num_indices) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t o = run / num_indices, ii = run % num_indices;
+    const int64_t idx = strict_index(indices[ii], dim_size);
+    if (idx < 0) {
+        if (lane == 0 && o == 0) report_bad(bad, ii);
+        return;
+    }
+    const T *src = input + (o * dim_size + idx) * inner;
+    T *dst = out + run * inner;
+    constexpr int EPV = 16 / sizeof(T);
+    using V = typename std::conditional<sizeof(T) == 4, float4, double2>::type;
+    if (inner % EPV == 0 && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0) {
+        const int64_t nvec = inner / EPV;
+        for (int64_t v = lane; v < nvec; v += kWave) reinterpret_cast<V *>(dst)[v] = reinterpret_cast<const V *>(src)[v];
+    } else {
+        for (int64_t j = lane; j < inner; j += kWave) dst[j] = src[j];
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void embedding_add_kernel(const float *__restrict__ wte, int64_t vocab,
+                                                               const float *__restrict__ wpe,
+                                                               const double *__restrict__ ids, int64_t tokens,
+                                                               int64_t seq, int64_t width, float *__restrict__ out,
+                                                               int64_t *bad) {
+    const int64_t t = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+    if (t >= tokens) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t idx = strict_index(ids[t], vocab);
+    if (idx < 0) {
+        if (lane == 0) report_bad(bad, t);
+        return;
+    }
+    const float *a = wte + idx * width;
+    const float *b = wpe + (t % seq) * width;
+    float *dst = out + t * width;
+    if (width % 4 == 0 &&
+        ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0) {
+        for (int64_t v = lane; v < width / 4; v += kWave) {
+            float4 x = reinterpret_cast<const float4 *>(a)[v];
+            float4 y = reinterpret_cast<const float4 *>(b)[v];
+            reinterpret_cast<float4 *>(dst)[v] = make_float4(x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w);
+        }
+    } else {
+        for (int64_t j = lane; j < width; j += kWave) dst[j] = a[j] + b[j];
+    }
+}
+
+__global__ void set_i64_kernel(int64_t *p, int64_t v) { *p = v; }
+// An index that failed validation was recorded as an unsigned minimum; "none" is all ones == -1.
+
+// ---- argmax ----------------------------------------------------------------------------------
+// Candidate = (value, first index reaching it) plus the first NaN position. Combining two
+// candidates keeps the larger value, the smaller index on equal values, and the smaller NaN
+// position: associative and commutative, so the tree shape cannot change the answer, and the
+// answer equals the sequential scan of crates/ft-kernel-cpu/src/lib.rs:39518-39535
+// (first strict maximum wins; the first NaN wins and ends the scan; all -inf gives index 0).
+template <typename T> struct Cand {
+    T val;
+    int64_t idx;
+    int64_t nan_idx;
+};
+constexpr int64_t kNoNan = 0x7fffffffffffffffLL;
+
+template <typename T> __device__ __forceinline__ Cand<T> cand_init() {
+    return Cand<T>{sizeof(T) == 4 ? (T)-__builtin_inff() : (T)-__builtin_inf(), 0, kNoNan};
+}
+template <typename T> __device__ __forceinline__ void cand_feed(Cand<T> &c, T v, int64_t i) {
+    if (v != v) {
+        if (i < c.nan_idx) c.nan_idx = i;
+    } else if (v > c.val) {
+        c.val = v;
+        c.idx = i;
+    }
+}
+template <typename T> __device__ __forceinline__ Cand<T> cand_merge(const Cand<T> &a, const Cand<T> &b) {
+    Cand<T> r;
+    if (b.val > a.val || (b.val == a.val && b.idx < a.idx)) {
+        r.val = b.val;
+        r.idx = b.idx;
+    } else {
+        r.val = a.val;
+        r.idx = a.idx;
+    }
+    r.nan_idx = a.nan_idx < b.nan_idx ? a.nan_idx : b.nan_idx;
+    return r;
+}
+template <typename T> __device__ __forceinline__ Cand<T> cand_shfl_xor(const Cand<T> &c, int off) {
+    Cand<T> r;
+    r.val = __shfl_xor(c.val, off, kWave);
+    r.idx = __shfl_xor(c.idx, off, kWave);
+    r.nan_idx = __shfl_xor(c.nan_idx, off, kWave);
+    return r;
+}
+
+// Last-dim argmax: one block per row, lanes stride the row (coalesced dword loads; rows such as
+// 50 257 floats are only 4-byte aligned, so no wider load is assumed).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void argmax_lastdim_kernel(const T *__restrict__ x, int64_t rows, int64_t cols,
+                                                                T *__restrict__ out) {
+    __shared__ Cand<T> smem[kBlock / kWave];
+    const T *xr = x + (int64_t)blockIdx.x * cols;
+    Cand<T> c = cand_init<T>();
+    int64_t j = threadIdx.x;
+    // Four independent loads in flight per lane.
+    for (; j + 3 * kBlock < cols; j += 4 * kBlock) {
+        T v0 = xr[j], v1 = xr[j + kBlock], v2 = xr[j + 2 * kBlock], v3 = xr[j + 3 * kBlock];
+        cand_feed(c, v0, j);
+        cand_feed(c, v1, j + kBlock);
+        cand_feed(c, v2, j + 2 * kBlock);
+        cand_feed(c, v3, j + 3 * kBlock);
+    }
+    for (; j < cols; j += kBlock) cand_feed(c, xr[j], j);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) c = cand_merge(c, cand_shfl_xor(c, off));
+    if ((threadIdx.x & (kWave - 1)) == 0) smem[threadIdx.x / kWave] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        Cand<T> r = smem[0];
+#pragma unroll
+        for (int w = 1; w < kBlock / kWave; ++w) r = cand_merge(r, smem[w]);
+        out[blockIdx.x] = (T)(r.nan_idx != kNoNan ? r.nan_idx : r.idx);
+    }
+}
+
+// Strided argmax over [outer, reduce, inner], inner > 1: one thread per output, coalesced on inner.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void argmax_strided_kernel(const T *__restrict__ x, int64_t outer, int64_t reduce,
+                                                                int64_t inner, T *__restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= outer * inner) return;
+    const int64_t o = i / inner, in = i % inner;
+    const T *xb = x + o * reduce * inner + in;
+    Cand<T> c = cand_init<T>();
+    for (int64_t r = 0; r < reduce; ++r) {
+        T v = xb[r * inner];
+        if (v != v) {
+            c.nan_idx = r;
+            break;
+        }
+        if (v > c.val) {
+            c.val = v;
+            c.idx = r;
+        }
+    }
+    out[i] = (T)(c.nan_idx != kNoNan ? c.nan_idx : c.idx);
+}
+
+// ---- permute [d0, d1, d2, d3] -> [d0, d2, d1, d3] ------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(kBlock) void permute_0213_kernel(const T *__restrict__ src, T *__restrict__ dst,
+                                                              int64_t d0, int64_t d1, int64_t d2, int64_t d3,
+                                                              int vec) {
+    // One thread per `vec`-element chunk of the destination.
+    const int64_t chunks_per_run = d3 / vec;
+    const int64_t total = d0 * d1 * d2 * chunks_per_run;
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int64_t c = i % chunks_per_run;
+    int64_t t = i / chunks_per_run;
+    const int64_t i1 = t % d1;  // destination order: [d0][d2][d1][d3]
+    t /= d1;
+    const int64_t i2 = t % d2;
+    const int64_t i0 = t / d2;
+    const T *s = src + (((i0 * d1 + i1) * d2 + i2) * d3) + c * vec;
+    T *d = dst + (((i0 * d2 + i2) * d1 + i1) * d3) + c * vec;
+    if (vec == 1) {
+        *d = *s;
+    } else {
+        using V = typename std::conditional<sizeof(T) == 4, float4, double2>::type;
+        *reinterpret_cast<V *>(d) = *reinterpret_cast<const V *>(s);
+    }
+}
+
+template <typename T>
+int32_t launch_index_select(const T *input, int64_t outer, int64_t dim_size, int64_t inner, const double *indices,
+                            int64_t num_indices, T *out, int64_t *bad, fth_stream s) {
+    FTH_REQUIRE_DEVICE();
+    FTH_ARG(outer >= 0 && dim_size >= 0 && inner >= 0 && num_indices >= 0, "index_select: negative extent");
+    hipStream_t st = fth::resolve_stream(s);
+    if (bad) {
+        set_i64_kernel<<<1, 1, 0, st>>>(bad, -1);
+        FTH_CHECK_LAUNCH("index_select(bad_index reset)");
+    }
+    if (outer == 0 || inner == 0 || num_indices == 0) return FTH_OK;
+    FTH_ARG(input && indices && out, "index_select: NULL operand");
+    int64_t grid = fth::ceil_div(outer * num_indices, kBlock / kWave);
+    FTH_ARG(grid <= kMaxGrid, "index_select: too many rows for one launch");
+    index_select_kernel<T><<<dim3((unsigned)grid), dim3(kBlock), 0, st>>>(input, outer, dim_size, inner, indices,
+                                                                           num_indices, out, bad);
+    FTH_CHECK_LAUNCH("index_select");
+    return FTH_OK;
+}
+
+template <typename T>
+int32_t launch_argmax(const T *x, int64_t outer, int64_t reduce, int64_t inner, T *out, fth_stream s) {
+    FTH_REQUIRE_DEVICE();
+    FTH_ARG(outer >= 0 && reduce >= 0 && inner >= 0, "argmax: negative extent");
+    if (outer == 0 || inner == 0) return FTH_OK;
+    if (reduce == 0) {
+        fth::set_error(FTH_ERR_EMPTY_REDUCTION_DIM, "argmax over an empty dimension");
+        fth::last_error().a = 0;
+        return FTH_ERR_EMPTY_REDUCTION_DIM;
+    }
+    FTH_ARG(x && out, "argmax: NULL operand");
+    hipStream_t st = fth::resolve_stream(s);
+    if (inner == 1) {
+        FTH_ARG(outer <= kMaxGrid, "argmax: too many rows for one launch");
+        argmax_lastdim_kernel<T><<<dim3((unsigned)outer), dim3(kBlock), 0, st>>>(x, outer, reduce, out);
+    } else {
+        int64_t grid = fth::ceil_div(outer * inner, kBlock);
+        FTH_ARG(grid <= kMaxGrid, "argmax: too many lanes for one launch");
+        argmax_strided_kernel<T><<<dim3((unsigned)grid), dim3(kBlock), 0, st>>>(x, outer, reduce, inner, out);
+    }
+    FTH_CHECK_LAUNCH("argmax");
+    return FTH_OK;
+}
+
+template <typename T>
+int32_t launch_permute(const T *src, T *dst, int64_t d0, int64_t d1, int64_t d2, int64_t d3, fth_stream s) {
+    FTH_REQUIRE_DEVICE();
+    FTH_ARG(d0 >= 0 && d1 >= 0 && d2 >= 0 && d3 >= 0, "permute: negative extent");
+    if (d0 == 0 || d1 == 0 || d2 == 0 || d3 == 0) return FTH_OK;
+    FTH_ARG(src && dst, "permute: NULL operand");
+    constexpr int EPV = 16 / sizeof(T);
+    int vec = (d3 % EPV == 0 && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0) ? EPV : 1;
+    int64_t total = d0 * d1 * d2 * (d3 / vec);
+    int64_t grid = fth::ceil_div(total, kBlock);
+    FTH_ARG(grid <= kMaxGrid, "permute: too long for one launch");
+    permute_0213_kernel<T><<<dim3((unsigned)grid), dim3(kBlock), 0, fth::resolve_stream(s)>>>(src, dst, d0, d1, d2, d3, vec);
+    FTH_CHECK_LAUNCH("permute_0213");
+    return FTH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t fth_dev_index_select_f32(const float *input, int64_t outer, int64_t dim_size, int64_t inner,
+                                 const double *indices, int64_t num_indices, float *out, int64_t *bad_index,
+                                 fth_stream s) {
+    return launch_index_select<float>(input, outer, dim_size, inner, indices, num_indices, out, bad_index, s);
+}
+int32_t fth_dev_index_select_f64(const double *input, int64_t outer, int64_t dim_size, int64_t inner,
+                                 const double *indices, int64_t num_indices, double *out, int64_t *bad_index,
+                                 fth_stream s) {
+    return launch_index_select<double>(input, outer, dim_size, inner, indices, num_indices, out, bad_index, s);
+}
+
+int32_t fth_dev_embedding_add_f32(const float *wte, int64_t vocab, const float *wpe, int64_t max_pos,
+                                  const double *ids, int64_t tokens, int64_t seq, int64_t width, float *out,
+                                  int64_t *bad_index, fth_stream s) {
+    FTH_REQUIRE_DEVICE();
+    FTH_ARG(vocab >= 0 && max_pos >= 0 && tokens >= 0 && seq >= 0 && width >= 0, "embedding: negative extent");
+    hipStream_t st = fth::resolve_stream(s);
+    if (bad_index) {
+        set_i64_kernel<<<1, 1, 0, st>>>(bad_index, -1);
+        FTH_CHECK_LAUNCH("embedding(bad_index reset)");
+    }
+    if (tokens == 0 || width == 0) return FTH_OK;
+    FTH_ARG(seq > 0 && seq <= max_pos, "embedding: seq %lld exceeds the %lld learned positions", (long long)seq,
+            (long long)max_pos);
+    FTH_ARG(wte && wpe && ids && out, "embedding: NULL operand");
+    int64_t grid = fth::ceil_div(tokens, kBlock / kWave);
+    FTH_ARG(grid <= kMaxGrid, "embedding: too many tokens for one launch");
+    embedding_add_kernel<<<dim3((unsigned)grid), dim3(kBlock), 0, st>>>(wte, vocab, wpe, ids, tokens, seq, width, out,
+                                                                        bad_index);
+    FTH_CHECK_LAUNCH("embedding_add");
+    return FTH_OK;
+}
+
+int32_t fth_dev_argmax_f32(const float *x, int64_t outer, int64_t reduce, int64_t inner, float *out, fth_stream s) {
+    return launch_argmax<float>(x, outer, reduce, inner, out, s);
+}
+int32_t fth_dev_argmax_f64(const double *x, int64_t outer, int64_t reduce, int64_t inner, double *out, fth_stream s) {
+    return launch_argmax<double>(x, outer, reduce, inner, out, s);
+}
+int32_t fth_dev_permute_0213_f32(const float *src, float *dst, int64_t d0, int64_t d1, int64_t d2, int64_t d3,
+                                 fth_stream s) {
+    return launch_permute<float>(src, dst, d0, d1, d2, d3, s);
+}
+int32_t fth_dev_permute_0213_f64(const double *src, double *dst, int64_t d0, int64_t d1, int64_t d2, int64_t d3,
+                                 fth_stream s) {
+    return launch_permute<double>(src, dst, d0, d1, d2, d3, s);
+}
+
+}  // extern "C"

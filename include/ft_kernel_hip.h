@@ -1,0 +1,436 @@
+/*
+ * ft_kernel_hip.h -- C ABI of the MI355X (gfx950) kernel backend for the FrankenTorch
+ * transformer forward op set.
+ *
+ * Three tiers, all `extern "C"`, plain pointers and sizes only:
+ *
+ *   Tier D  (fth_dev_*)   device pointers in, device pointers out, launched on a caller stream.
+ *                         This is what a resident runtime (and the benchmark) calls.
+ *   Tier A  (fth_*_tensor_contiguous_* / fth_*_forward_* / fth_linear_tensor_*)
+ *                         host slices in, caller-provided host buffer out: the shape of the
+ *                         `ft_kernel_cpu::*` free functions that `ft-dispatch` routes to
+ *                         (crates/ft-dispatch/src/lib.rs:14-250). Each call validates exactly as
+ *                         the reference does, uploads, launches Tier D, downloads, synchronises.
+ *   Tier B  (fth_tensor_*, fth_batch_*, fth_encoder_*, fth_gpt2_*)
+ *                         resident tensors and a stream-ordered batch, the shape of
+ *                         `ft_kernel_metal::fused::{GpuTensor, Batch, EncoderGpu}`
+ *                         (crates/ft-kernel-metal/src/fused.rs:540-933, 986-1190).
+ *
+ * Every function returns an `int32_t` status (FTH_OK == 0). Nothing aborts; nothing falls back to
+ * a CPU implementation: without a usable HIP device every compute entry point returns
+ * FTH_ERR_UNAVAILABLE (the contract of ft_kernel_metal::Error::Unavailable,
+ * crates/ft-kernel-metal/src/lib.rs:60-77, 255-272).
+ *
+ * All tensors are row-major contiguous. Reductions use fixed-order trees (no atomics), so two
+ * calls with the same arguments return bitwise identical results.
+ */
+#ifndef FT_KERNEL_HIP_H
+#define FT_KERNEL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------------------------ */
+/* Status codes                                                                               */
+/* ------------------------------------------------------------------------------------------ */
+
+/* 1..9 mirror `KernelError` (crates/ft-kernel-cpu/src/lib.rs:1697-1733) variant for variant;
+ * 100.. mirror `ft_kernel_metal::Error` (crates/ft-kernel-metal/src/lib.rs:60-77);
+ * FTH_ERR_INVALID_ARGUMENT stands where the reference's infallible fused entry points would
+ * panic on a short slice (plain indexing, e.g. crates/ft-kernel-cpu/src/lib.rs:5888). */
+enum {
+    FTH_OK = 0,
+    FTH_ERR_DTYPE_MISMATCH = 1,        /* Incompatible(DTypeMismatch)   */
+    FTH_ERR_DEVICE_MISMATCH = 2,       /* Incompatible(DeviceMismatch)  */
+    FTH_ERR_SHAPE_MISMATCH = 3,        /* ShapeMismatch{lhs,rhs}        */
+    FTH_ERR_UNSUPPORTED_LAYOUT = 4,    /* UnsupportedLayout{side}       */
+    FTH_ERR_STORAGE_SPAN_OVERFLOW = 5, /* StorageSpanOverflow{...}      */
+    FTH_ERR_INSUFFICIENT_STORAGE = 6,  /* InsufficientStorage{...}      */
+    FTH_ERR_INVALID_DIMENSION = 7,     /* InvalidDimension{dim,ndim}    */
+    FTH_ERR_SHAPE_OVERFLOW = 8,        /* ShapeOverflow{context}        */
+    FTH_ERR_EMPTY_REDUCTION_DIM = 9,   /* EmptyReductionDim{dim}        */
+    FTH_ERR_UNAVAILABLE = 100,         /* Error::Unavailable            */
+    FTH_ERR_KERNEL = 101,              /* Error::Kernel(String)         */
+    FTH_ERR_SIZE_OVERFLOW = 102,       /* Error::SizeOverflow           */
+    FTH_ERR_BUFFER_TOO_LARGE = 103,    /* Error::BufferTooLarge         */
+    FTH_ERR_STREAM = 104,              /* Error::CommandBuffer(state)   */
+    FTH_ERR_INVALID_ARGUMENT = 105,    /* reference would panic         */
+    FTH_ERR_OUTPUT_TOO_SMALL = 106     /* caller's out buffer < result  */
+};
+
+/* DType / Device tags: crates/ft-core/src/lib.rs:23-35 and :176-179, plus the HIP device id the
+ * backend adds to `Device`. Only F64 and F32 are computed here (crates/ft-dispatch/src/lib.rs:
+ * 4123-4308 narrows F16/BF16 above the kernels). */
+enum { FTH_DTYPE_F64 = 0, FTH_DTYPE_F32 = 1 };
+enum { FTH_DEVICE_CPU = 0, FTH_DEVICE_CUDA = 1, FTH_DEVICE_HIP = 2 };
+
+#define FTH_MAX_DIMS 8
+
+/* Flattened `TensorMeta` (crates/ft-core/src/lib.rs:340-348). Strides are in elements. */
+typedef struct fth_meta {
+    int32_t ndim;
+    int32_t dtype;  /* FTH_DTYPE_*  */
+    int32_t device; /* FTH_DEVICE_* */
+    int32_t reserved;
+    uint64_t shape[FTH_MAX_DIMS];
+    uint64_t strides[FTH_MAX_DIMS];
+    uint64_t storage_offset;
+} fth_meta;
+
+/* Payload of the last failing call on this thread (the fields of the KernelError variant). */
+typedef struct fth_error_info {
+    int32_t code;
+    int32_t lhs_ndim;
+    int32_t rhs_ndim;
+    int32_t reserved;
+    uint64_t lhs_shape[FTH_MAX_DIMS]; /* ShapeMismatch.lhs */
+    uint64_t rhs_shape[FTH_MAX_DIMS]; /* ShapeMismatch.rhs */
+    uint64_t a; /* dim | needed | storage_offset | lhs dtype/device tag */
+    uint64_t b; /* ndim | available | numel | rhs dtype/device tag      */
+    char side[16];     /* "lhs", "rhs", "mat1", "mat2", "input" */
+    char message[200]; /* Display-style text, or the HIP error string */
+} fth_error_info;
+
+/* Copies the calling thread's last error payload. Returns its code. */
+int32_t fth_last_error(fth_error_info *out);
+/* Static name for a status code ("ShapeMismatch", "Unavailable", ...). Never NULL. */
+const char *fth_status_name(int32_t code);
+
+/* ------------------------------------------------------------------------------------------ */
+/* Runtime: availability, memory, streams, timing                                             */
+/* ------------------------------------------------------------------------------------------ */
+
+/* ft_kernel_metal::fused::is_available (crates/ft-kernel-metal/src/fused.rs:631-633):
+ * 1 when a gfx950 device is present and the kernels in this library can run on it. */
+int32_t fth_is_available(void);
+/* Fills name (e.g. "gfx950:sramecc+:xnack-"), CU count, HBM bytes, clocks in kHz. */
+int32_t fth_device_info(char *arch, size_t arch_cap, int32_t *compute_units, uint64_t *hbm_bytes,
+                        int32_t *engine_clock_khz, int32_t *memory_clock_khz);
+
+/* hipMalloc-backed buffers with explicit copies (the `ft-core` storage the backend adds).
+ * fth_malloc never zero-fills (crates/ft-kernel-cpu/src/lib.rs:2611-2639 `build_uninit`). */
+int32_t fth_malloc(void **dptr, size_t bytes);
+int32_t fth_free(void *dptr);
+int32_t fth_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes);
+int32_t fth_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes);
+int32_t fth_memcpy_d2d(void *dst_dev, const void *src_dev, size_t bytes);
+int32_t fth_memset_zero(void *dst_dev, size_t bytes);
+
+typedef void *fth_stream; /* a hipStream_t; NULL selects the library's own ordered stream */
+typedef void *fth_event;  /* a hipEvent_t */
+int32_t fth_stream_create(fth_stream *s);
+int32_t fth_stream_destroy(fth_stream s);
+int32_t fth_stream_synchronize(fth_stream s);
+int32_t fth_device_synchronize(void);
+int32_t fth_event_create(fth_event *e);
+int32_t fth_event_destroy(fth_event e);
+int32_t fth_event_record(fth_event e, fth_stream s);
+int32_t fth_event_synchronize(fth_event e);
+int32_t fth_event_elapsed_ms(fth_event start, fth_event stop, float *ms);
+
+/* ------------------------------------------------------------------------------------------ */
+/* Tier D: device-pointer kernels                                                             */
+/* ------------------------------------------------------------------------------------------ */
+
+/* Last-dim softmax over `rows` rows of `cols` elements.
+ * replaces the inner_size==1 branch of softmax_dim_tensor_contiguous_f32
+ * (crates/ft-kernel-cpu/src/lib.rs:39219-39242) / _f64 (:18350-18399). */
+int32_t fth_dev_softmax_lastdim_f32(const float *x, float *y, int64_t rows, int64_t cols, fth_stream s);
+int32_t fth_dev_softmax_lastdim_f64(const double *x, double *y, int64_t rows, int64_t cols, fth_stream s);
+/* Softmax over a middle dim of a contiguous [outer, reduce, inner] view
+ * (crates/ft-kernel-cpu/src/lib.rs:39244-39293). */
+int32_t fth_dev_softmax_strided_f32(const float *x, float *y, int64_t outer, int64_t reduce, int64_t inner, fth_stream s);
+int32_t fth_dev_softmax_strided_f64(const double *x, double *y, int64_t outer, int64_t reduce, int64_t inner, fth_stream s);
+
+/* layer_norm_forward_f32 (crates/ft-kernel-cpu/src/lib.rs:5877-5923), _f64 (:5824-5870).
+ * weight / bias may be NULL (the reference's Option::None). */
+int32_t fth_dev_layer_norm_f32(const float *x, const float *weight, const float *bias, float *y,
+                               int64_t batch, int64_t norm_size, float eps, fth_stream s);
+int32_t fth_dev_layer_norm_f64(const double *x, const double *weight, const double *bias, double *y,
+                               int64_t batch, int64_t norm_size, double eps, fth_stream s);
+/* add_layer_norm_forward_f32 (crates/ft-kernel-cpu/src/lib.rs:5932-5984): y = LN(a + b). */
+int32_t fth_dev_add_layer_norm_f32(const float *a, const float *b, const float *weight, const float *bias,
+                                   float *y, int64_t batch, int64_t norm_size, float eps, fth_stream s);
+/* rms_norm_forward_f32 (crates/ft-kernel-cpu/src/lib.rs:6459-6494), _f64 (:6418-6453). */
+int32_t fth_dev_rms_norm_f32(const float *x, const float *weight, float *y, int64_t batch,
+                             int64_t norm_size, float eps, fth_stream s);
+int32_t fth_dev_rms_norm_f64(const double *x, const double *weight, double *y, int64_t batch,
+                             int64_t norm_size, double eps, fth_stream s);
+
+/* gelu_tensor_contiguous_f32 (crates/ft-kernel-cpu/src/lib.rs:37123-37127, 36966-36969): erf form. */
+int32_t fth_dev_gelu_f32(const float *x, float *y, int64_t n, fth_stream s);
+int32_t fth_dev_gelu_f64(const double *x, double *y, int64_t n, fth_stream s);
+/* add_tensor_contiguous_f32 (crates/ft-kernel-cpu/src/lib.rs:36870-36877): exact IEEE l + r. */
+int32_t fth_dev_add_f32(const float *a, const float *b, float *y, int64_t n, fth_stream s);
+int32_t fth_dev_add_f64(const double *a, const double *b, double *y, int64_t n, fth_stream s);
+/* The bias pass of linear_tensor_f32 (crates/ft-kernel-cpu/src/lib.rs:17336-17351):
+ * y[r, j] = x[r, j] + bias[j]. x == y is allowed. */
+int32_t fth_dev_bias_add_f32(const float *x, const float *bias, float *y, int64_t rows, int64_t cols, fth_stream s);
+int32_t fth_dev_bias_add_f64(const double *x, const double *bias, double *y, int64_t rows, int64_t cols, fth_stream s);
+/* Bias pass followed by the residual add, in one sweep with the same two roundings:
+ * y[r, j] = (x[r, j] + bias[j]) + residual[r, j]
+ * (crates/ft-kernel-cpu/src/lib.rs:17336-17351 then :36870-36877). */
+int32_t fth_dev_bias_residual_add_f32(const float *x, const float *bias, const float *residual, float *y,
+                                      int64_t rows, int64_t cols, fth_stream s);
+
+/* index_select along dim 0 of a [table_rows, width] table: the embedding gather of
+ * index_select_tensor_contiguous_f32 (crates/ft-kernel-cpu/src/lib.rs:40216-40253). Indices are
+ * f64 VALUES on the device, validated by normalize_strict_index_value's rules
+ * (crates/ft-kernel-cpu/src/lib.rs:20058-20090). `bad_index` (device, one int64, may be NULL)
+ * receives the smallest position of an invalid index, or -1; rows with an invalid index are
+ * left untouched. General [outer, dim, inner] form: fth_dev_index_select_f32. */
+int32_t fth_dev_index_select_f32(const float *input, int64_t outer, int64_t dim_size, int64_t inner,
+                                 const double *indices, int64_t num_indices, float *out,
+                                 int64_t *bad_index, fth_stream s);
+int32_t fth_dev_index_select_f64(const double *input, int64_t outer, int64_t dim_size, int64_t inner,
+                                 const double *indices, int64_t num_indices, double *out,
+                                 int64_t *bad_index, fth_stream s);
+/* Fused token + position embedding: out[t, :] = wte[ids[t], :] + wpe[t % seq, :]
+ * (Embedding::forward crates/ft-nn/src/lib.rs:3080-3135 twice, then add_tensor_contiguous_f32). */
+int32_t fth_dev_embedding_add_f32(const float *wte, int64_t vocab, const float *wpe, int64_t max_pos,
+                                  const double *ids, int64_t tokens, int64_t seq, int64_t width,
+                                  float *out, int64_t *bad_index, fth_stream s);
+
+/* argmax over the reduce dim of a contiguous [outer, reduce, inner] view; indices are written as
+ * floating-point values; first strict maximum wins, the first NaN wins and ends the scan
+ * (crates/ft-kernel-cpu/src/lib.rs:39443-39550; f64 :18653). */
+int32_t fth_dev_argmax_f32(const float *x, int64_t outer, int64_t reduce, int64_t inner, float *out, fth_stream s);
+int32_t fth_dev_argmax_f64(const double *x, int64_t outer, int64_t reduce, int64_t inner, double *out, fth_stream s);
+
+/* Head split / merge: dst[((b*H+h)*S+s)*hd+c] = src[((b*S+s)*H+h)*hd+c] and its inverse
+ * (TensorTape::permute_slice, perm [0,2,1,3], crates/ft-autograd/src/lib.rs:10733-10882). */
+int32_t fth_dev_permute_0213_f32(const float *src, float *dst, int64_t d0, int64_t d1, int64_t d2, int64_t d3, fth_stream s);
+int32_t fth_dev_permute_0213_f64(const double *src, double *dst, int64_t d0, int64_t d1, int64_t d2, int64_t d3, fth_stream s);
+
+/* Dense contraction on MFMA. C[b] = alpha * A[b] * op(B[b]) (+ epilogue), beta = 0 (C is fully
+ * overwritten, crates/ft-kernel-cpu/src/lib.rs:1310-1338).
+ *   trans_b == 0: B is [k, n] row-major         -> gemm::sgemm / dgemm   (:1310, :107)
+ *   trans_b == 1: B is [n, k] row-major (W)     -> gemm::sgemm_bt / dgemm_bt (:1430, :201)
+ * lda/ldb/ldc are row pitches in elements; batch strides in elements (0 = shared operand).
+ * Epilogue, applied to the rounded product in this order (each its own rounding):
+ *   FTH_EPI_BIAS      + bias[n]             (linear_tensor_f32, :17336-17351)
+ *   FTH_EPI_GELU      gelu_erf(.)           (:36966-36969)
+ *   FTH_EPI_RESIDUAL  + residual[m, n]      (row pitch ldc; add_tensor_contiguous_f32)
+ * k == 0 writes zeros (or the epilogue of zero); m == 0 or n == 0 returns at once. */
+enum { FTH_EPI_NONE = 0, FTH_EPI_BIAS = 1, FTH_EPI_GELU = 2, FTH_EPI_RESIDUAL = 4 };
+typedef struct fth_gemm_desc {
+    int64_t m, n, k;
+    int64_t lda, ldb, ldc;
+    int64_t batch;
+    int64_t stride_a, stride_b, stride_c;
+    int32_t trans_b;
+    int32_t epilogue; /* bit set of FTH_EPI_* */
+} fth_gemm_desc;
+int32_t fth_dev_gemm_f32(const fth_gemm_desc *d, float alpha, const float *a, const float *b, float *c,
+                         const float *bias, const float *residual, fth_stream s);
+int32_t fth_dev_gemm_f64(const fth_gemm_desc *d, double alpha, const double *a, const double *b, double *c,
+                         const double *bias, const double *residual, fth_stream s);
+
+/* Fused scaled-dot-product attention forward, q [num_bh, seq_q, d_k], k [num_bh, seq_k, d_k],
+ * v [num_bh, seq_k, d_v] -> out [num_bh, seq_q, d_v]; causal limit = min(qi + 1, seq_k)
+ * (sdpa_forward_f32, crates/ft-kernel-cpu/src/lib.rs:5200-5284; _f64 :4572-4651).
+ * Row pitches let the kernel read a packed [tokens, 3*d_model] QKV projection and write a
+ * [tokens, d_model] context directly (the head split/merge of MultiheadAttention::
+ * forward_qkv_masked, crates/ft-nn/src/lib.rs:5088-5198, without the permuted copies):
+ * element (bh, s, c) of q lives at q[(bh / heads) * q_batch_stride + (bh % heads) * q_head_stride
+ * + s * q_row_stride + c]; likewise k, v, out. */
+typedef struct fth_sdpa_desc {
+    int64_t num_bh, heads; /* heads divides num_bh; heads == 1 for plain [num_bh, seq, d] */
+    int64_t seq_q, seq_k, d_k, d_v;
+    int64_t q_batch_stride, q_head_stride, q_row_stride;
+    int64_t k_batch_stride, k_head_stride, k_row_stride;
+    int64_t v_batch_stride, v_head_stride, v_row_stride;
+    int64_t o_batch_stride, o_head_stride, o_row_stride;
+    int32_t causal;
+    int32_t reserved;
+} fth_sdpa_desc;
+/* Fills the strides for contiguous [num_bh, seq, d] operands. */
+void fth_sdpa_desc_contiguous(fth_sdpa_desc *d, int64_t num_bh, int64_t seq_q, int64_t seq_k,
+                              int64_t d_k, int64_t d_v, int32_t causal);
+int32_t fth_dev_sdpa_forward_f32(const fth_sdpa_desc *d, float scale, const float *q, const float *k,
+                                 const float *v, float *out, fth_stream s);
+int32_t fth_dev_sdpa_forward_f64(const fth_sdpa_desc *d, double scale, const double *q, const double *k,
+                                 const double *v, double *out, fth_stream s);
+
+/* ------------------------------------------------------------------------------------------ */
+/* Tier A: host slices in, host buffer out (the ft_kernel_cpu surface)                        */
+/* ------------------------------------------------------------------------------------------ */
+/* `*_len` are slice lengths in elements. `out` must hold `out_cap` elements; `*out_len` receives
+ * the result length (the length of the Vec the reference returns). A NULL `out` with out_cap 0
+ * only validates and reports `*out_len`. Validation order follows the reference
+ * (crates/ft-kernel-cpu/src/lib.rs:36935-36962, 37787-37793). */
+
+/* matmul_tensor_contiguous_f32 (:37752) / _f64 (:17355) */
+int32_t fth_matmul_tensor_contiguous_f32(const float *lhs, size_t lhs_len, const float *rhs, size_t rhs_len,
+                                         const fth_meta *lhs_meta, const fth_meta *rhs_meta,
+                                         float *out, size_t out_cap, size_t *out_len);
+int32_t fth_matmul_tensor_contiguous_f64(const double *lhs, size_t lhs_len, const double *rhs, size_t rhs_len,
+                                         const fth_meta *lhs_meta, const fth_meta *rhs_meta,
+                                         double *out, size_t out_cap, size_t *out_len);
+/* bmm_tensor_contiguous_f32 (:38496) / _f64 (:17785) */
+int32_t fth_bmm_tensor_contiguous_f32(const float *lhs, size_t lhs_len, const float *rhs, size_t rhs_len,
+                                      const fth_meta *lhs_meta, const fth_meta *rhs_meta,
+                                      float *out, size_t out_cap, size_t *out_len);
+int32_t fth_bmm_tensor_contiguous_f64(const double *lhs, size_t lhs_len, const double *rhs, size_t rhs_len,
+                                      const fth_meta *lhs_meta, const fth_meta *rhs_meta,
+                                      double *out, size_t out_cap, size_t *out_len);
+/* addmm_tensor_contiguous_f32 (:41562) / _f64 (:17514) */
+int32_t fth_addmm_tensor_contiguous_f32(const float *input, size_t input_len, const float *mat1, size_t mat1_len,
+                                        const float *mat2, size_t mat2_len, const fth_meta *input_meta,
+                                        const fth_meta *mat1_meta, const fth_meta *mat2_meta, float beta,
+                                        float alpha, float *out, size_t out_cap, size_t *out_len);
+int32_t fth_addmm_tensor_contiguous_f64(const double *input, size_t input_len, const double *mat1, size_t mat1_len,
+                                        const double *mat2, size_t mat2_len, const fth_meta *input_meta,
+                                        const fth_meta *mat1_meta, const fth_meta *mat2_meta, double beta,
+                                        double alpha, double *out, size_t out_cap, size_t *out_len);
+/* linear_tensor_f32 (:17306) / _f64 (:17162); bias may be NULL */
+int32_t fth_linear_tensor_f32(const float *x, size_t x_len, const float *weight, size_t weight_len,
+                              const float *bias, size_t bias_len, size_t batch, size_t in_features,
+                              size_t out_features, float *out, size_t out_cap, size_t *out_len);
+int32_t fth_linear_tensor_f64(const double *x, size_t x_len, const double *weight, size_t weight_len,
+                              const double *bias, size_t bias_len, size_t batch, size_t in_features,
+                              size_t out_features, double *out, size_t out_cap, size_t *out_len);
+/* matmul_rhs_transposed_contiguous_f32 (:17408) / _f64 (:17381) */
+int32_t fth_matmul_rhs_transposed_contiguous_f32(size_t m, size_t k, size_t n, const float *lhs, size_t lhs_len,
+                                                 const float *rhs_nk, size_t rhs_len, float *out,
+                                                 size_t out_cap, size_t *out_len);
+int32_t fth_matmul_rhs_transposed_contiguous_f64(size_t m, size_t k, size_t n, const double *lhs, size_t lhs_len,
+                                                 const double *rhs_nk, size_t rhs_len, double *out,
+                                                 size_t out_cap, size_t *out_len);
+/* softmax_dim_tensor_contiguous_f32 (:39193) / _f64 (:18350) */
+int32_t fth_softmax_dim_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta,
+                                              size_t dim, float *out, size_t out_cap, size_t *out_len);
+int32_t fth_softmax_dim_tensor_contiguous_f64(const double *input, size_t input_len, const fth_meta *meta,
+                                              size_t dim, double *out, size_t out_cap, size_t *out_len);
+/* layer_norm_forward_f32 (:5877) / _f64 (:5824); add_layer_norm_forward_f32 (:5932);
+ * rms_norm_forward_f32 (:6459) / _f64 (:6418). weight/bias may be NULL. */
+int32_t fth_layer_norm_forward_f32(const float *x, size_t x_len, const float *weight, const float *bias,
+                                   size_t batch, size_t norm_size, float eps, float *out, size_t out_cap);
+int32_t fth_layer_norm_forward_f64(const double *x, size_t x_len, const double *weight, const double *bias,
+                                   size_t batch, size_t norm_size, double eps, double *out, size_t out_cap);
+int32_t fth_add_layer_norm_forward_f32(const float *a, const float *b, size_t ab_len, const float *weight,
+                                       const float *bias, size_t batch, size_t norm_size, float eps,
+                                       float *out, size_t out_cap);
+int32_t fth_rms_norm_forward_f32(const float *x, size_t x_len, const float *weight, size_t batch,
+                                 size_t norm_size, float eps, float *out, size_t out_cap);
+int32_t fth_rms_norm_forward_f64(const double *x, size_t x_len, const double *weight, size_t batch,
+                                 size_t norm_size, double eps, double *out, size_t out_cap);
+/* gelu_tensor_contiguous_f32 (:37123) / _f64 (:3657); add_tensor_contiguous_f32 (:36870) / _f64 */
+int32_t fth_gelu_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta,
+                                       float *out, size_t out_cap, size_t *out_len);
+int32_t fth_gelu_tensor_contiguous_f64(const double *input, size_t input_len, const fth_meta *meta,
+                                       double *out, size_t out_cap, size_t *out_len);
+int32_t fth_add_tensor_contiguous_f32(const float *lhs, size_t lhs_len, const float *rhs, size_t rhs_len,
+                                      const fth_meta *lhs_meta, const fth_meta *rhs_meta,
+                                      float *out, size_t out_cap, size_t *out_len);
+int32_t fth_add_tensor_contiguous_f64(const double *lhs, size_t lhs_len, const double *rhs, size_t rhs_len,
+                                      const fth_meta *lhs_meta, const fth_meta *rhs_meta,
+                                      double *out, size_t out_cap, size_t *out_len);
+/* sdpa_forward_f32 (:5200) / _f64 (:4572) */
+int32_t fth_sdpa_forward_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v,
+                             size_t v_len, size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v,
+                             float scale, int32_t causal, float *out, size_t out_cap);
+int32_t fth_sdpa_forward_f64(const double *q, size_t q_len, const double *k, size_t k_len, const double *v,
+                             size_t v_len, size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v,
+                             double scale, int32_t causal, double *out, size_t out_cap);
+/* index_select_tensor_contiguous_f32 (:40216) / _f64; indices are f64 values */
+int32_t fth_index_select_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta,
+                                               size_t dim, const double *indices, size_t num_indices,
+                                               float *out, size_t out_cap, size_t *out_len);
+int32_t fth_index_select_tensor_contiguous_f64(const double *input, size_t input_len, const fth_meta *meta,
+                                               size_t dim, const double *indices, size_t num_indices,
+                                               double *out, size_t out_cap, size_t *out_len);
+/* argmax_dim_tensor_contiguous_f32 (:39443) / _f64 (:18653); indices returned as float values */
+int32_t fth_argmax_dim_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta,
+                                             size_t dim, float *out, size_t out_cap, size_t *out_len);
+int32_t fth_argmax_dim_tensor_contiguous_f64(const double *input, size_t input_len, const fth_meta *meta,
+                                             size_t dim, double *out, size_t out_cap, size_t *out_len);
+
+/* ------------------------------------------------------------------------------------------ */
+/* Tier B: resident tensors, stream-ordered batch, block and GPT-2-shaped runners             */
+/* ------------------------------------------------------------------------------------------ */
+
+/* GpuTensor (crates/ft-kernel-metal/src/fused.rs:540-580): a resident f32 [rows, cols] matrix. */
+typedef struct fth_tensor fth_tensor;
+int32_t fth_tensor_upload(const float *host, int64_t rows, int64_t cols, fth_tensor **out);
+int32_t fth_tensor_alloc(int64_t rows, int64_t cols, fth_tensor **out);
+int32_t fth_tensor_download(const fth_tensor *t, float *host, size_t host_cap);
+int32_t fth_tensor_shape(const fth_tensor *t, int64_t *rows, int64_t *cols);
+void *fth_tensor_data(const fth_tensor *t); /* device pointer */
+int32_t fth_tensor_free(fth_tensor *t);
+/* Bytes currently held by, and cached inside, the library's buffer pool
+ * (crates/ft-core/src/buffer_pool.rs:206-329 recycles host Vecs the same way). */
+int32_t fth_pool_stats(uint64_t *bytes_in_use, uint64_t *bytes_cached);
+int32_t fth_pool_trim(void);
+
+/* Batch (crates/ft-kernel-metal/src/fused.rs:676-932): every op enqueues on the batch's stream
+ * and returns a fresh resident tensor; fth_batch_finish is the only synchronisation. */
+typedef struct fth_batch fth_batch;
+int32_t fth_batch_new(fth_batch **out);
+int32_t fth_batch_free(fth_batch *b);
+int32_t fth_batch_finish(fth_batch *b);
+/* y = a[m,k] * w[n,k]^T (+ bias[n])  -- Batch::matmul_bias, :676-762, with the weight in the
+ * [out, in] layout of ft-nn Linear (crates/ft-nn/src/lib.rs:902-1118). */
+int32_t fth_batch_linear(fth_batch *b, const fth_tensor *a, const fth_tensor *w, const fth_tensor *bias, fth_tensor **out);
+/* y = a[m,k] * rhs[k,n]  -- tensor_matmul layout */
+int32_t fth_batch_matmul(fth_batch *b, const fth_tensor *a, const fth_tensor *rhs, fth_tensor **out);
+int32_t fth_batch_layernorm(fth_batch *b, const fth_tensor *x, const fth_tensor *gamma, const fth_tensor *beta, float eps, fth_tensor **out);
+int32_t fth_batch_rmsnorm(fth_batch *b, const fth_tensor *x, const fth_tensor *gamma, float eps, fth_tensor **out);
+int32_t fth_batch_gelu(fth_batch *b, const fth_tensor *x, fth_tensor **out);
+int32_t fth_batch_add(fth_batch *b, const fth_tensor *x, const fth_tensor *y, fth_tensor **out);
+int32_t fth_batch_softmax(fth_batch *b, const fth_tensor *x, fth_tensor **out);
+/* Multi-head attention over [seq, d_model] q/k/v with n_heads heads (Batch::mha, :861-925);
+ * `batch` sequences are stacked along rows (rows = batch * seq). */
+int32_t fth_batch_mha(fth_batch *b, const fth_tensor *q, const fth_tensor *k, const fth_tensor *v,
+                      int64_t n_heads, int64_t batch, int32_t causal, fth_tensor **out);
+
+/* One layer's weights, host pointers, nn.Linear layout [out, in]
+ * (LayerWeightsRef, crates/ft-kernel-metal/src/fused.rs:986-1016; topology of
+ * TransformerEncoderLayer::forward_layer_masked with norm_first, crates/ft-nn/src/lib.rs:14709-14744). */
+typedef struct fth_layer_weights {
+    const float *ln1_w, *ln1_b;     /* [d_model] */
+    const float *wq, *bq;           /* [d_model, d_model], [d_model] */
+    const float *wk, *bk;
+    const float *wv, *bv;
+    const float *wo, *bo;
+    const float *ln2_w, *ln2_b;
+    const float *w1, *b1;           /* [d_ff, d_model], [d_ff] */
+    const float *w2, *b2;           /* [d_model, d_ff], [d_model] */
+} fth_layer_weights;
+
+/* EncoderGpu (crates/ft-kernel-metal/src/fused.rs:1024-1190): weights uploaded once; forward
+ * runs `n_layers` pre-LN blocks on a resident [batch*seq, d_model] activation. */
+typedef struct fth_encoder fth_encoder;
+int32_t fth_encoder_new(int64_t d_model, int64_t n_heads, int64_t d_ff, float ln_eps, int32_t causal,
+                        const fth_layer_weights *layers, int64_t n_layers, fth_encoder **out);
+int32_t fth_encoder_free(fth_encoder *e);
+/* Host in / host out (EncoderGpu::forward, :1136-1146). */
+int32_t fth_encoder_forward(fth_encoder *e, const float *input, int64_t batch, int64_t seq, float *out, size_t out_cap);
+/* Resident in / resident out on stream `s`; no synchronisation. `x` [batch*seq, d_model]. */
+int32_t fth_encoder_forward_dev(fth_encoder *e, const float *x_dev, int64_t batch, int64_t seq, float *out_dev, fth_stream s);
+/* Captures forward_dev for (batch, seq) into a HIP graph and replays it: one launch per forward. */
+int32_t fth_encoder_forward_graph(fth_encoder *e, const float *x_dev, int64_t batch, int64_t seq, float *out_dev, fth_stream s);
+
+/* GPT-2-shaped decoder: learned positions, pre-LN blocks, final LN, LM head tied to wte. */
+typedef struct fth_gpt2 fth_gpt2;
+int32_t fth_gpt2_new(int64_t vocab, int64_t max_pos, int64_t d_model, int64_t n_heads, int64_t d_ff, float ln_eps,
+                     const float *wte, const float *wpe, const fth_layer_weights *layers, int64_t n_layers,
+                     const float *lnf_w, const float *lnf_b, fth_gpt2 **out);
+int32_t fth_gpt2_free(fth_gpt2 *g);
+/* ids: device f64 token-id values [batch*seq] (indices are float-valued tensors in the reference,
+ * crates/ft-nn/examples/bert_rerank_spike.rs:61-63). logits_dev [batch*seq, vocab] and
+ * argmax_dev [batch*seq] (f32 index values) may each be NULL to skip that output; when logits_dev
+ * is NULL and argmax_dev is not, logits go to an internal buffer. */
+int32_t fth_gpt2_forward_dev(fth_gpt2 *g, const double *ids_dev, int64_t batch, int64_t seq,
+                             float *logits_dev, float *argmax_dev, fth_stream s);
+/* Final hidden state [batch*seq, d_model] of the last forward (device pointer, valid until the next). */
+const float *fth_gpt2_hidden_dev(const fth_gpt2 *g);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FT_KERNEL_HIP_H */

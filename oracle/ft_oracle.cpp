@@ -1,0 +1,672 @@
+// TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+//
+// CPU restatement of the transformer forward ops of the reference's `ft-kernel-cpu` crate, used
+// only as the checker in tests/, in __graft_entry__.smoke() and as the `cpu_baseline` leg of
+// bench.py. Nothing under frankentorch_amd/ links, loads or calls this file.
+//
+// Build: g++ -O2 -ffp-contract=off -fno-fast-math -fopenmp (see oracle/build_oracle.py). The
+// reference is Rust, which never contracts a*b+c into an FMA, hence -ffp-contract=off.
+//
+// Each function cites the reference lines it follows (paths relative to the reference root;
+// KC = crates/ft-kernel-cpu/src/lib.rs). Parity status per function:
+//   pinned by the reference's own fixtures / closed forms (tests/test_oracle_golden.py):
+//     softmax, gelu, add, matmul (small exact + stored f64 checksums), bmm, addmm, linear,
+//     index_select, argmax, layer_norm / rms_norm (closed form + textbook), sdpa (textbook
+//     attention + brute force), permute.
+//   third-party arithmetic that is NOT in the reference tree:
+//     * GEMM: `matrixmultiply 0.3.11` (Cargo.lock:1420-1423; call sites KC:1645, KC:1673). Its
+//       f32 accumulation order is unspecified and the reference's own test shows it is not the
+//       sequential-k sum (KC:50617-50689). fto_gemm_f32 therefore accumulates in f64 and rounds
+//       once: the exact product to within 2^-24 relative, which every order matrixmultiply
+//       could use must also approach. Tolerance parity only; bit parity with matrixmultiply is
+//       unreachable and not claimed.
+//     * erff / erf: `libm 0.2.16` (Cargo.lock:1366-1369; KC:36968, KC:1928), a port of
+//       FreeBSD msun. This file calls the platform libm (glibc) instead; both are documented
+//       <= 1 ULP, and the reference's gelu fixture (5 points, 1e-10) pins the f64 form.
+//     * expf / exp: Rust std calls the platform libm, as this file does.
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+#include <limits>
+#include <vector>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#if defined(__x86_64__)
+#include <immintrin.h>
+#endif
+
+extern "C" {
+
+// ------------------------------------------------------------------------------------------
+// Threads (the reference's rayon pool defaults to one worker per logical core,
+// crates/ft-kernel-cpu/src/pool.rs:5-8; size gates never change results, KC:2576, 3053, 5773)
+// ------------------------------------------------------------------------------------------
+int fto_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+void fto_set_threads(int n) {
+#ifdef _OPENMP
+    if (n > 0) omp_set_num_threads(n);
+#else
+    (void)n;
+#endif
+}
+
+}  // extern "C"
+
+namespace {
+
+// pairwise_sum_f32 / _f64 (KC:37521-37528): <= 128 elements sequentially, else split at len / 2.
+template <typename T> T pairwise_sum(const T *v, size_t n) {
+    if (n <= 128) {
+        T s = 0;
+        for (size_t i = 0; i < n; ++i) s += v[i];
+        return s;
+    }
+    size_t mid = n / 2;
+    return pairwise_sum(v, mid) + pairwise_sum(v + mid, n - mid);
+}
+
+// f32::max / f64::max (IEEE maxNum: a NaN operand is ignored), as used in the fold at KC:39221.
+template <typename T> T max_num(T a, T b) {
+    if (a != a) return b;
+    if (b != b) return a;
+    return a > b ? a : b;
+}
+
+inline float t_exp(float x) { return expf(x); }
+inline double t_exp(double x) { return exp(x); }
+inline float t_erf(float x) { return erff(x); }
+inline double t_erf(double x) { return erf(x); }
+inline float t_sqrt(float x) { return sqrtf(x); }
+inline double t_sqrt(double x) { return sqrt(x); }
+
+// softmax_dim_tensor_contiguous_f32 (KC:39193-39296), _f64 (KC:18350-18461): per lane,
+// max = fold(-inf, max); out = exp(x - max); sum = pairwise_sum(out); out /= sum.
+template <typename T> void softmax_impl(const T *x, T *y, int64_t outer, int64_t reduce, int64_t inner) {
+    if (outer <= 0 || reduce <= 0 || inner <= 0) return;
+    if (inner == 1) {
+#pragma omp parallel for schedule(static)
+        for (int64_t o = 0; o < outer; ++o) {
+            const T *in = x + o * reduce;
+            T *out = y + o * reduce;
+            T m = -std::numeric_limits<T>::infinity();
+            for (int64_t j = 0; j < reduce; ++j) m = max_num(m, in[j]);
+            for (int64_t j = 0; j < reduce; ++j) out[j] = t_exp(in[j] - m);
+            T s = pairwise_sum(out, (size_t)reduce);
+            for (int64_t j = 0; j < reduce; ++j) out[j] /= s;
+        }
+        return;
+    }
+#pragma omp parallel
+    {
+        std::vector<T> scratch((size_t)reduce);
+#pragma omp for schedule(static)
+        for (int64_t o = 0; o < outer; ++o) {
+            const T *in = x + o * reduce * inner;
+            T *out = y + o * reduce * inner;
+            for (int64_t c = 0; c < inner; ++c) {
+                for (int64_t r = 0; r < reduce; ++r) scratch[r] = in[r * inner + c];
+                T m = -std::numeric_limits<T>::infinity();
+                for (int64_t r = 0; r < reduce; ++r) m = max_num(m, scratch[r]);
+                for (int64_t r = 0; r < reduce; ++r) scratch[r] = t_exp(scratch[r] - m);
+                T s = pairwise_sum(scratch.data(), (size_t)reduce);
+                for (int64_t r = 0; r < reduce; ++r) out[r * inner + c] = scratch[r] / s;
+            }
+        }
+    }
+}
+
+// layer_norm_forward_f32 (KC:5877-5923), _f64 (KC:5824-5870); with `b2` non-null it is
+// add_layer_norm_forward_f32 (KC:5932-5984): a + b materialised once, then the same passes.
+template <typename T>
+void layer_norm_impl(const T *x, const T *x2, const T *w, const T *b, T *y, int64_t batch, int64_t n, T eps) {
+    if (batch <= 0 || n <= 0) return;
+    const T inv_n = T(1) / (T)n;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < batch; ++r) {
+        const T *xr = x + r * n;
+        T *o = y + r * n;
+        T sum = 0;
+        if (x2) {
+            const T *x2r = x2 + r * n;
+            for (int64_t j = 0; j < n; ++j) {
+                T s = xr[j] + x2r[j];
+                o[j] = s;
+                sum += s;
+            }
+            xr = o;
+        } else {
+            for (int64_t j = 0; j < n; ++j) sum += xr[j];
+        }
+        const T mean = sum * inv_n;
+        T vsum = 0;
+        for (int64_t j = 0; j < n; ++j) {
+            T d = xr[j] - mean;
+            vsum += d * d;
+        }
+        const T rstd = T(1) / t_sqrt(vsum * inv_n + eps);
+        for (int64_t j = 0; j < n; ++j) {
+            T v = (xr[j] - mean) * rstd;
+            if (w) v *= w[j];
+            if (b) v += b[j];
+            o[j] = v;
+        }
+    }
+}
+
+// rms_norm_forward_f32 (KC:6459-6494), _f64 (KC:6418-6453).
+template <typename T> void rms_norm_impl(const T *x, const T *w, T *y, int64_t batch, int64_t n, T eps) {
+    if (batch <= 0 || n <= 0) return;
+    const T inv_n = T(1) / (T)n;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < batch; ++r) {
+        const T *xr = x + r * n;
+        T *o = y + r * n;
+        T ss = 0;
+        for (int64_t j = 0; j < n; ++j) ss += xr[j] * xr[j];
+        const T rstd = T(1) / t_sqrt(ss * inv_n + eps);
+        for (int64_t j = 0; j < n; ++j) {
+            T v = xr[j] * rstd;
+            if (w) v *= w[j];
+            o[j] = v;
+        }
+    }
+}
+
+// gelu_value_f32 (KC:36966-36969); f64 form KC:1924-1929.
+inline float gelu_value(float x) { return 0.5f * x * (1.0f + t_erf(x * 0.70710678118654752440f)); }
+inline double gelu_value(double x) { return 0.5 * x * (1.0 + t_erf(x * 0.70710678118654752440)); }
+
+// GEMM truth for f32: accumulate in f64 (each product of two f32 is exact in f64), round once.
+// b_kn is [k, n] row-major with pitch ldb.
+void gemm_f32_kn(int64_t m, int64_t n, int64_t k, const float *a, int64_t lda, const float *b, int64_t ldb,
+                 float *c, int64_t ldc) {
+#pragma omp parallel
+    {
+        std::vector<double> acc((size_t)n);
+#pragma omp for schedule(dynamic, 4)
+        for (int64_t i = 0; i < m; ++i) {
+            std::fill(acc.begin(), acc.end(), 0.0);
+            const float *ar = a + i * lda;
+            for (int64_t p = 0; p < k; ++p) {
+                const double av = (double)ar[p];
+                const float *br = b + p * ldb;
+                double *ac = acc.data();
+                for (int64_t j = 0; j < n; ++j) ac[j] += av * (double)br[j];
+            }
+            float *cr = c + i * ldc;
+            for (int64_t j = 0; j < n; ++j) cr[j] = (float)acc[j];
+        }
+    }
+}
+
+// GEMM truth for f64: accumulate in long double (x87 80-bit), round once.
+void gemm_f64_kn(int64_t m, int64_t n, int64_t k, const double *a, int64_t lda, const double *b, int64_t ldb,
+                 double *c, int64_t ldc) {
+#pragma omp parallel
+    {
+        std::vector<long double> acc((size_t)n);
+#pragma omp for schedule(dynamic, 4)
+        for (int64_t i = 0; i < m; ++i) {
+            std::fill(acc.begin(), acc.end(), 0.0L);
+            const double *ar = a + i * lda;
+            for (int64_t p = 0; p < k; ++p) {
+                const long double av = (long double)ar[p];
+                const double *br = b + p * ldb;
+                for (int64_t j = 0; j < n; ++j) acc[j] += av * (long double)br[j];
+            }
+            double *cr = c + i * ldc;
+            for (int64_t j = 0; j < n; ++j) cr[j] = (double)acc[j];
+        }
+    }
+}
+
+template <typename T> void transpose_nk_to_kn(const T *w, int64_t n, int64_t k, int64_t ldw, std::vector<T> &out) {
+    out.resize((size_t)n * (size_t)k);
+#pragma omp parallel for schedule(static)
+    for (int64_t j = 0; j < n; ++j)
+        for (int64_t p = 0; p < k; ++p) out[(size_t)p * n + j] = w[j * ldw + p];
+}
+
+void gemm_any(int trans_b, int64_t m, int64_t n, int64_t k, const float *a, int64_t lda, const float *b, int64_t ldb,
+              float *c, int64_t ldc) {
+    if (m <= 0 || n <= 0) return;
+    if (!trans_b) return gemm_f32_kn(m, n, k, a, lda, b, ldb, c, ldc);
+    std::vector<float> t;
+    transpose_nk_to_kn(b, n, k, ldb, t);
+    gemm_f32_kn(m, n, k, a, lda, t.data(), n, c, ldc);
+}
+void gemm_any(int trans_b, int64_t m, int64_t n, int64_t k, const double *a, int64_t lda, const double *b,
+              int64_t ldb, double *c, int64_t ldc) {
+    if (m <= 0 || n <= 0) return;
+    if (!trans_b) return gemm_f64_kn(m, n, k, a, lda, b, ldb, c, ldc);
+    std::vector<double> t;
+    transpose_nk_to_kn(b, n, k, ldb, t);
+    gemm_f64_kn(m, n, k, a, lda, t.data(), n, c, ldc);
+}
+
+// linear_tensor_f32 (KC:17306-17353): y = x . W^T, then the bias pass on the rounded result.
+template <typename T>
+void linear_impl(const T *x, const T *w, const T *bias, int64_t batch, int64_t in_f, int64_t out_f, T *y) {
+    if (batch <= 0 || out_f <= 0) return;
+    gemm_any(1, batch, out_f, in_f, x, in_f, w, in_f, y, out_f);
+    if (bias) {
+#pragma omp parallel for schedule(static)
+        for (int64_t r = 0; r < batch; ++r)
+            for (int64_t j = 0; j < out_f; ++j) y[r * out_f + j] += bias[j];
+    }
+}
+
+// sdpa_forward_f32 (KC:5200-5284), _f64 (KC:4572-4651). The block height cannot change results
+// (KC:4982-4984), so rows are processed one at a time. The two GEMMs are the f64-accumulated
+// truth; the row softmax between them is the reference's scalar loop verbatim (KC:5238-5256):
+// scale after the product, strict `>` max scan over the first `limit` entries, exp, sequential
+// sum, divide, zero the tail.
+template <typename T>
+void sdpa_impl(const T *q, const T *k, const T *v, int64_t num_bh, int64_t seq_q, int64_t seq_k, int64_t d_k,
+               int64_t d_v, T scale, int causal, T *out) {
+    if (num_bh <= 0 || seq_q <= 0 || d_v <= 0) return;
+    using Wide = typename std::conditional<sizeof(T) == 4, double, long double>::type;
+#pragma omp parallel
+    {
+        std::vector<T> sc((size_t)std::max<int64_t>(seq_k, 1));
+        std::vector<Wide> acc((size_t)d_v);
+#pragma omp for schedule(dynamic, 8) collapse(2)
+        for (int64_t bh = 0; bh < num_bh; ++bh) {
+            for (int64_t qi = 0; qi < seq_q; ++qi) {
+                const T *qr = q + (bh * seq_q + qi) * d_k;
+                const T *kh = k + bh * seq_k * d_k;
+                const T *vh = v + bh * seq_k * d_v;
+                // gemm::sgemm_bt(br, d_k, seq_k, q_block, kh, sc): the FULL row of scores, KC:5229
+                for (int64_t j = 0; j < seq_k; ++j) {
+                    Wide dot = 0;
+                    const T *kr = kh + j * d_k;
+                    for (int64_t c = 0; c < d_k; ++c) dot += (Wide)qr[c] * (Wide)kr[c];
+                    sc[j] = (T)dot;
+                }
+                const int64_t limit = causal ? std::min<int64_t>(qi + 1, seq_k) : seq_k;
+                T m = -std::numeric_limits<T>::infinity();
+                for (int64_t j = 0; j < limit; ++j) {
+                    sc[j] *= scale;
+                    if (sc[j] > m) m = sc[j];
+                }
+                T sum = 0;
+                for (int64_t j = 0; j < limit; ++j) {
+                    T e = t_exp(sc[j] - m);
+                    sc[j] = e;
+                    sum += e;
+                }
+                for (int64_t j = 0; j < limit; ++j) sc[j] /= sum;
+                for (int64_t j = limit; j < seq_k; ++j) sc[j] = 0;
+                // gemm::sgemm(br, seq_k, d_v, sc, vh, o_block), KC:5258
+                std::fill(acc.begin(), acc.end(), (Wide)0);
+                for (int64_t j = 0; j < seq_k; ++j) {
+                    const Wide pj = (Wide)sc[j];
+                    const T *vr = vh + j * d_v;
+                    for (int64_t c = 0; c < d_v; ++c) acc[c] += pj * (Wide)vr[c];
+                }
+                T *o = out + (bh * seq_q + qi) * d_v;
+                for (int64_t c = 0; c < d_v; ++c) o[c] = (T)acc[c];
+            }
+        }
+    }
+}
+
+// normalize_strict_index_value (KC:20058-20090).
+inline int64_t strict_index(double v, int64_t dim_size) {
+    if (!std::isfinite(v)) return -1;
+    if (std::fabs(v - std::trunc(v)) > std::numeric_limits<double>::epsilon()) return -1;
+    if (v < 0.0 || v >= 9.2233720368547758e18) return -1;
+    int64_t i = (int64_t)v;
+    if (i < 0 || i >= dim_size) return -1;
+    return i;
+}
+
+// index_select_tensor_contiguous_f32 (KC:40216-40253). Returns the position of the first
+// invalid index (the reference returns Err there), or -1.
+template <typename T>
+int64_t index_select_impl(const T *input, int64_t outer, int64_t dim_size, int64_t inner, const double *indices,
+                          int64_t n_idx, T *out) {
+    for (int64_t i = 0; i < n_idx; ++i)
+        if (strict_index(indices[i], dim_size) < 0) return i;
+    for (int64_t o = 0; o < outer; ++o)
+        for (int64_t i = 0; i < n_idx; ++i) {
+            const int64_t idx = strict_index(indices[i], dim_size);
+            const T *src = input + (o * dim_size + idx) * inner;
+            T *dst = out + (o * n_idx + i) * inner;
+            for (int64_t c = 0; c < inner; ++c) dst[c] = src[c];
+        }
+    return -1;
+}
+
+// argmax_dim_tensor_contiguous_f32 (KC:39443-39550), the serial lane loop KC:39518-39535:
+// first strict maximum wins; the first NaN wins and ends the scan.
+template <typename T> void argmax_impl(const T *x, int64_t outer, int64_t reduce, int64_t inner, T *out) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < outer * inner; ++i) {
+        const int64_t o = i / inner, c = i % inner;
+        const T *base = x + o * reduce * inner + c;
+        int64_t best = 0;
+        T best_val = -std::numeric_limits<T>::infinity();
+        for (int64_t r = 0; r < reduce; ++r) {
+            T val = base[r * inner];
+            if (val != val) {
+                best = r;
+                break;
+            } else if (val > best_val) {
+                best_val = val;
+                best = r;
+            }
+        }
+        out[i] = (T)best;
+    }
+}
+
+// permute [d0,d1,d2,d3] -> [d0,d2,d1,d3] (crates/ft-autograd/src/lib.rs:10733-10882).
+template <typename T> void permute_0213_impl(const T *src, T *dst, int64_t d0, int64_t d1, int64_t d2, int64_t d3) {
+#pragma omp parallel for schedule(static) collapse(2)
+    for (int64_t i0 = 0; i0 < d0; ++i0)
+        for (int64_t i2 = 0; i2 < d2; ++i2)
+            for (int64_t i1 = 0; i1 < d1; ++i1)
+                std::memcpy(dst + (((i0 * d2 + i2) * d1 + i1) * d3), src + (((i0 * d1 + i1) * d2 + i2) * d3),
+                            sizeof(T) * (size_t)d3);
+}
+
+struct LayerW {
+    const float *ln1_w, *ln1_b, *wq, *bq, *wk, *bk, *wv, *bv, *wo, *bo, *ln2_w, *ln2_b, *w1, *b1, *w2, *b2;
+};
+
+// TransformerEncoderLayer::forward_layer_masked with norm_first (crates/ft-nn/src/lib.rs:
+// 14709-14744): x = x + MHA(LN1(x)); x = x + W2.gelu(W1.LN2(x)); MHA as
+// MultiheadAttention::forward_qkv_masked (crates/ft-nn/src/lib.rs:5088-5198), scale 1/sqrt(hd).
+void encoder_layer_impl(const LayerW &w, float *x, int64_t batch, int64_t seq, int64_t d_model, int64_t heads,
+                        int64_t d_ff, float eps, int causal) {
+    const int64_t tokens = batch * seq, hd = d_model / heads;
+    std::vector<float> h((size_t)tokens * d_model), qv(h.size()), kv(h.size()), vv(h.size());
+    std::vector<float> qh(h.size()), kh(h.size()), vh(h.size()), ctx(h.size()), merged(h.size()), proj(h.size());
+    layer_norm_impl<float>(x, nullptr, w.ln1_w, w.ln1_b, h.data(), tokens, d_model, eps);
+    linear_impl<float>(h.data(), w.wq, w.bq, tokens, d_model, d_model, qv.data());
+    linear_impl<float>(h.data(), w.wk, w.bk, tokens, d_model, d_model, kv.data());
+    linear_impl<float>(h.data(), w.wv, w.bv, tokens, d_model, d_model, vv.data());
+    permute_0213_impl<float>(qv.data(), qh.data(), batch, seq, heads, hd);
+    permute_0213_impl<float>(kv.data(), kh.data(), batch, seq, heads, hd);
+    permute_0213_impl<float>(vv.data(), vh.data(), batch, seq, heads, hd);
+    const float scale = (float)(1.0 / std::sqrt((double)hd));
+    sdpa_impl<float>(qh.data(), kh.data(), vh.data(), batch * heads, seq, seq, hd, hd, scale, causal, ctx.data());
+    permute_0213_impl<float>(ctx.data(), merged.data(), batch, heads, seq, hd);
+    linear_impl<float>(merged.data(), w.wo, w.bo, tokens, d_model, d_model, proj.data());
+    for (size_t i = 0; i < proj.size(); ++i) x[i] = x[i] + proj[i];
+    layer_norm_impl<float>(x, nullptr, w.ln2_w, w.ln2_b, h.data(), tokens, d_model, eps);
+    std::vector<float> f1((size_t)tokens * d_ff);
+    linear_impl<float>(h.data(), w.w1, w.b1, tokens, d_model, d_ff, f1.data());
+    for (size_t i = 0; i < f1.size(); ++i) f1[i] = gelu_value(f1[i]);
+    linear_impl<float>(f1.data(), w.w2, w.b2, tokens, d_ff, d_model, proj.data());
+    for (size_t i = 0; i < proj.size(); ++i) x[i] = x[i] + proj[i];
+}
+
+#if defined(__x86_64__)
+// Blocked f32 GEMM with an AVX2/FMA 6x16 register tile, standing in for matrixmultiply's packed
+// micro-kernel when the CPU path is TIMED (never used as the truth). b is [k, n].
+__attribute__((target("avx2,fma"))) void sgemm_blocked_avx2(int64_t m, int64_t n, int64_t k, const float *a,
+                                                            int64_t lda, const float *b, int64_t ldb, float *c,
+                                                            int64_t ldc) {
+    constexpr int64_t MR = 6, NR = 16, KC = 256, NC = 1024;
+#pragma omp parallel
+    {
+        std::vector<float> bp((size_t)KC * NC);
+        for (int64_t jc = 0; jc < n; jc += NC) {
+            const int64_t nc = std::min(NC, n - jc);
+            for (int64_t pc = 0; pc < k; pc += KC) {
+                const int64_t kc = std::min(KC, k - pc);
+                // every thread packs its own copy of the B panel, NR-wide column strips
+                for (int64_t j0 = 0; j0 < nc; j0 += NR)
+                    for (int64_t p = 0; p < kc; ++p)
+                        for (int64_t j = 0; j < NR; ++j)
+                            bp[(size_t)(j0 * kc + p * NR + j)] =
+                                (j0 + j < nc) ? b[(pc + p) * ldb + jc + j0 + j] : 0.0f;
+#pragma omp for schedule(static)
+                for (int64_t i0 = 0; i0 < m; i0 += MR) {
+                    const int64_t mr = std::min(MR, m - i0);
+                    for (int64_t j0 = 0; j0 < nc; j0 += NR) {
+                        __m256 acc[MR][2];
+                        for (int r = 0; r < MR; ++r) acc[r][0] = acc[r][1] = _mm256_setzero_ps();
+                        const float *bs = bp.data() + j0 * kc;
+                        for (int64_t p = 0; p < kc; ++p) {
+                            const __m256 b0 = _mm256_loadu_ps(bs + p * NR), b1 = _mm256_loadu_ps(bs + p * NR + 8);
+                            for (int r = 0; r < MR; ++r) {
+                                const float av = (r < mr) ? a[(i0 + r) * lda + pc + p] : 0.0f;
+                                const __m256 ab = _mm256_set1_ps(av);
+                                acc[r][0] = _mm256_fmadd_ps(ab, b0, acc[r][0]);
+                                acc[r][1] = _mm256_fmadd_ps(ab, b1, acc[r][1]);
+                            }
+                        }
+                        float tmp[NR];
+                        for (int r = 0; r < mr; ++r) {
+                            _mm256_storeu_ps(tmp, acc[r][0]);
+                            _mm256_storeu_ps(tmp + 8, acc[r][1]);
+                            float *cr = c + (i0 + r) * ldc + jc + j0;
+                            const int64_t w = std::min<int64_t>(NR, nc - j0);
+                            if (pc == 0) for (int64_t j = 0; j < w; ++j) cr[j] = tmp[j];
+                            else for (int64_t j = 0; j < w; ++j) cr[j] += tmp[j];
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+#endif
+
+}  // namespace
+
+extern "C" {
+
+void fto_softmax_f32(const float *x, float *y, int64_t outer, int64_t reduce, int64_t inner) {
+    softmax_impl<float>(x, y, outer, reduce, inner);
+}
+void fto_softmax_f64(const double *x, double *y, int64_t outer, int64_t reduce, int64_t inner) {
+    softmax_impl<double>(x, y, outer, reduce, inner);
+}
+void fto_layer_norm_f32(const float *x, const float *w, const float *b, float *y, int64_t batch, int64_t n, float eps) {
+    layer_norm_impl<float>(x, nullptr, w, b, y, batch, n, eps);
+}
+void fto_layer_norm_f64(const double *x, const double *w, const double *b, double *y, int64_t batch, int64_t n,
+                        double eps) {
+    layer_norm_impl<double>(x, nullptr, w, b, y, batch, n, eps);
+}
+void fto_add_layer_norm_f32(const float *a, const float *b2, const float *w, const float *b, float *y, int64_t batch,
+                            int64_t n, float eps) {
+    layer_norm_impl<float>(a, b2, w, b, y, batch, n, eps);
+}
+void fto_rms_norm_f32(const float *x, const float *w, float *y, int64_t batch, int64_t n, float eps) {
+    rms_norm_impl<float>(x, w, y, batch, n, eps);
+}
+void fto_rms_norm_f64(const double *x, const double *w, double *y, int64_t batch, int64_t n, double eps) {
+    rms_norm_impl<double>(x, w, y, batch, n, eps);
+}
+// gelu_tensor_contiguous_f32 (KC:37123-37127)
+void fto_gelu_f32(const float *x, float *y, int64_t n) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i) y[i] = gelu_value(x[i]);
+}
+void fto_gelu_f64(const double *x, double *y, int64_t n) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i) y[i] = gelu_value(x[i]);
+}
+// add_tensor_contiguous_f32 (KC:36870-36877)
+void fto_add_f32(const float *a, const float *b, float *y, int64_t n) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i) y[i] = a[i] + b[i];
+}
+void fto_add_f64(const double *a, const double *b, double *y, int64_t n) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i) y[i] = a[i] + b[i];
+}
+// bias pass of linear_tensor_f32 (KC:17336-17351), optionally followed by the residual add
+void fto_bias_add_f32(const float *x, const float *bias, const float *residual, float *y, int64_t rows, int64_t cols) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t j = 0; j < cols; ++j) {
+            float v = x[r * cols + j] + bias[j];
+            if (residual) v = v + residual[r * cols + j];
+            y[r * cols + j] = v;
+        }
+}
+void fto_bias_add_f64(const double *x, const double *bias, const double *residual, double *y, int64_t rows,
+                      int64_t cols) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t j = 0; j < cols; ++j) {
+            double v = x[r * cols + j] + bias[j];
+            if (residual) v = v + residual[r * cols + j];
+            y[r * cols + j] = v;
+        }
+}
+
+// gemm::sgemm / sgemm_bt (KC:1310-1338, 1430-1481) and dgemm / dgemm_bt (KC:107-138, 201-255)
+void fto_gemm_f32(int trans_b, int64_t m, int64_t n, int64_t k, const float *a, int64_t lda, const float *b,
+                  int64_t ldb, float *c, int64_t ldc) {
+    gemm_any(trans_b, m, n, k, a, lda, b, ldb, c, ldc);
+}
+void fto_gemm_f64(int trans_b, int64_t m, int64_t n, int64_t k, const double *a, int64_t lda, const double *b,
+                  int64_t ldb, double *c, int64_t ldc) {
+    gemm_any(trans_b, m, n, k, a, lda, b, ldb, c, ldc);
+}
+// Timed stand-in for matrixmultiply (not a truth): returns 0 when AVX2/FMA is unavailable.
+int fto_sgemm_blocked(int64_t m, int64_t n, int64_t k, const float *a, int64_t lda, const float *b, int64_t ldb,
+                      float *c, int64_t ldc) {
+#if defined(__x86_64__)
+    if (__builtin_cpu_supports("avx2") && __builtin_cpu_supports("fma")) {
+        sgemm_blocked_avx2(m, n, k, a, lda, b, ldb, c, ldc);
+        return 1;
+    }
+#endif
+    return 0;
+}
+// bmm_tensor_contiguous_f32 (KC:38496-38606): per-batch sgemm
+void fto_bmm_f32(int64_t batch, int64_t m, int64_t n, int64_t k, const float *a, const float *b, float *c) {
+    for (int64_t i = 0; i < batch; ++i) gemm_any(0, m, n, k, a + i * m * k, k, b + i * k * n, n, c + i * m * n, n);
+}
+void fto_bmm_f64(int64_t batch, int64_t m, int64_t n, int64_t k, const double *a, const double *b, double *c) {
+    for (int64_t i = 0; i < batch; ++i) gemm_any(0, m, n, k, a + i * m * k, k, b + i * k * n, n, c + i * m * n, n);
+}
+// addmm_tensor_contiguous_f32 (KC:41562-41648): beta * input_at(i) + alpha * g, input [n] or [m,n]
+void fto_addmm_f32(const float *input, int input_is_1d, const float *mat1, const float *mat2, int64_t m, int64_t n,
+                   int64_t k, float beta, float alpha, float *out) {
+    uint32_t abits;
+    std::memcpy(&abits, &alpha, 4);
+    if (abits == 0) {
+        for (int64_t i = 0; i < m * n; ++i) out[i] = beta * (input_is_1d ? input[i % n] : input[i]);
+        return;
+    }
+    std::vector<float> g((size_t)(m * n));
+    gemm_any(0, m, n, k, mat1, k, mat2, n, g.data(), n);
+    for (int64_t i = 0; i < m * n; ++i) out[i] = beta * (input_is_1d ? input[i % n] : input[i]) + alpha * g[i];
+}
+void fto_addmm_f64(const double *input, int input_is_1d, const double *mat1, const double *mat2, int64_t m,
+                   int64_t n, int64_t k, double beta, double alpha, double *out) {
+    uint64_t abits;
+    std::memcpy(&abits, &alpha, 8);
+    if (abits == 0) {
+        for (int64_t i = 0; i < m * n; ++i) out[i] = beta * (input_is_1d ? input[i % n] : input[i]);
+        return;
+    }
+    std::vector<double> g((size_t)(m * n));
+    gemm_any(0, m, n, k, mat1, k, mat2, n, g.data(), n);
+    for (int64_t i = 0; i < m * n; ++i) out[i] = beta * (input_is_1d ? input[i % n] : input[i]) + alpha * g[i];
+}
+void fto_linear_f32(const float *x, const float *w, const float *bias, int64_t batch, int64_t in_f, int64_t out_f,
+                    float *y) {
+    linear_impl<float>(x, w, bias, batch, in_f, out_f, y);
+}
+void fto_linear_f64(const double *x, const double *w, const double *bias, int64_t batch, int64_t in_f, int64_t out_f,
+                    double *y) {
+    linear_impl<double>(x, w, bias, batch, in_f, out_f, y);
+}
+void fto_sdpa_forward_f32(const float *q, const float *k, const float *v, int64_t num_bh, int64_t seq_q,
+                          int64_t seq_k, int64_t d_k, int64_t d_v, float scale, int causal, float *out) {
+    sdpa_impl<float>(q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, out);
+}
+void fto_sdpa_forward_f64(const double *q, const double *k, const double *v, int64_t num_bh, int64_t seq_q,
+                          int64_t seq_k, int64_t d_k, int64_t d_v, double scale, int causal, double *out) {
+    sdpa_impl<double>(q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, out);
+}
+int64_t fto_index_select_f32(const float *input, int64_t outer, int64_t dim_size, int64_t inner,
+                             const double *indices, int64_t n_idx, float *out) {
+    return index_select_impl<float>(input, outer, dim_size, inner, indices, n_idx, out);
+}
+int64_t fto_index_select_f64(const double *input, int64_t outer, int64_t dim_size, int64_t inner,
+                             const double *indices, int64_t n_idx, double *out) {
+    return index_select_impl<double>(input, outer, dim_size, inner, indices, n_idx, out);
+}
+void fto_argmax_f32(const float *x, int64_t outer, int64_t reduce, int64_t inner, float *out) {
+    argmax_impl<float>(x, outer, reduce, inner, out);
+}
+void fto_argmax_f64(const double *x, int64_t outer, int64_t reduce, int64_t inner, double *out) {
+    argmax_impl<double>(x, outer, reduce, inner, out);
+}
+void fto_permute_0213_f32(const float *src, float *dst, int64_t d0, int64_t d1, int64_t d2, int64_t d3) {
+    permute_0213_impl<float>(src, dst, d0, d1, d2, d3);
+}
+void fto_permute_0213_f64(const double *src, double *dst, int64_t d0, int64_t d1, int64_t d2, int64_t d3) {
+    permute_0213_impl<double>(src, dst, d0, d1, d2, d3);
+}
+
+// One pre-LN block, in place on x [batch*seq, d_model]. `w` is 16 pointers in the order of LayerW.
+void fto_encoder_layer_f32(const float *const *w, float *x, int64_t batch, int64_t seq, int64_t d_model,
+                           int64_t heads, int64_t d_ff, float eps, int causal) {
+    LayerW lw = {w[0], w[1], w[2], w[3], w[4], w[5], w[6], w[7], w[8], w[9], w[10], w[11], w[12], w[13], w[14], w[15]};
+    encoder_layer_impl(lw, x, batch, seq, d_model, heads, d_ff, eps, causal);
+}
+
+// GPT-2-shaped forward: x = wte[ids] + wpe[pos] (Embedding::forward, crates/ft-nn/src/lib.rs:
+// 3080-3135, twice, then add); n_layers pre-LN causal blocks; final LayerNorm; logits = x . wte^T
+// (tied head); argmax over the vocabulary. `layers` is n_layers * 16 pointers. `hidden`
+// (tokens * d_model), `logits` (tokens * vocab) and `argmax` (tokens) may each be NULL.
+// Returns the position of the first invalid token id, or -1.
+int64_t fto_gpt2_forward_f32(int64_t vocab, int64_t max_pos, int64_t d_model, int64_t heads, int64_t d_ff, float eps,
+                             const float *wte, const float *wpe, const float *const *layers, int64_t n_layers,
+                             const float *lnf_w, const float *lnf_b, const double *ids, int64_t batch, int64_t seq,
+                             float *hidden, float *logits, float *argmax) {
+    const int64_t tokens = batch * seq;
+    if (seq > max_pos) return 0;
+    std::vector<float> x((size_t)tokens * d_model), tok((size_t)tokens * d_model), pos((size_t)tokens * d_model);
+    int64_t bad = index_select_impl<float>(wte, 1, vocab, d_model, ids, tokens, tok.data());
+    if (bad >= 0) return bad;
+    std::vector<double> pidx((size_t)tokens);
+    for (int64_t t = 0; t < tokens; ++t) pidx[t] = (double)(t % seq);
+    index_select_impl<float>(wpe, 1, max_pos, d_model, pidx.data(), tokens, pos.data());
+    for (size_t i = 0; i < x.size(); ++i) x[i] = tok[i] + pos[i];
+    for (int64_t l = 0; l < n_layers; ++l) {
+        const float *const *w = layers + l * 16;
+        LayerW lw = {w[0], w[1], w[2], w[3], w[4], w[5], w[6], w[7], w[8], w[9], w[10], w[11], w[12], w[13], w[14], w[15]};
+        encoder_layer_impl(lw, x.data(), batch, seq, d_model, heads, d_ff, eps, 1);
+    }
+    std::vector<float> hf(x.size());
+    layer_norm_impl<float>(x.data(), nullptr, lnf_w, lnf_b, hf.data(), tokens, d_model, eps);
+    if (hidden) std::memcpy(hidden, hf.data(), hf.size() * sizeof(float));
+    if (logits || argmax) {
+        std::vector<float> own;
+        float *lg = logits;
+        if (!lg) {
+            own.resize((size_t)tokens * vocab);
+            lg = own.data();
+        }
+        linear_impl<float>(hf.data(), wte, nullptr, tokens, d_model, vocab, lg);
+        if (argmax) argmax_impl<float>(lg, tokens, vocab, 1, argmax);
+    }
+    return -1;
+}
+
+}  // extern "C"

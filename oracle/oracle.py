@@ -1,0 +1,283 @@
+"""numpy front end of the CPU checker (oracle/ft_oracle.cpp). TEST INFRASTRUCTURE ONLY.
+
+Only tests/, __graft_entry__.smoke() and the cpu_baseline leg of bench.py import this module.
+Every function takes and returns C-contiguous numpy arrays and mirrors one `ft_kernel_cpu`
+entry point (names and argument meaning follow the reference; see ft_oracle.cpp for file:line).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "_build", "libft_oracle.so")
+_lib = None
+
+_i64 = C.c_int64
+_vp = C.c_void_p
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            import importlib.util
+
+            spec = importlib.util.spec_from_file_location("build_oracle", os.path.join(_HERE, "build_oracle.py"))
+            mod = importlib.util.module_from_spec(spec)
+            spec.loader.exec_module(mod)
+            mod.build_oracle()
+        _lib = C.CDLL(_LIB_PATH)
+        _lib.fto_threads.restype = C.c_int
+        _lib.fto_index_select_f32.restype = _i64
+        _lib.fto_index_select_f64.restype = _i64
+        _lib.fto_gpt2_forward_f32.restype = _i64
+        _lib.fto_sgemm_blocked.restype = C.c_int
+    return _lib
+
+
+def threads() -> int:
+    return lib().fto_threads()
+
+
+def set_threads(n: int) -> None:
+    lib().fto_set_threads(C.c_int(n))
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(_vp)
+
+
+def _c(a, dtype=None):
+    if a is None:
+        return None
+    return np.ascontiguousarray(a, dtype=dtype if dtype is not None else a.dtype)
+
+
+def _sfx(dtype):
+    dtype = np.dtype(dtype)
+    if dtype == np.float32:
+        return "f32", C.c_float
+    if dtype == np.float64:
+        return "f64", C.c_double
+    raise TypeError("oracle computes f32 and f64 only, got %s" % dtype)
+
+
+def softmax(x, dim: int = -1):
+    x = _c(x)
+    sfx, _ = _sfx(x.dtype)
+    dim = dim % x.ndim
+    outer = int(np.prod(x.shape[:dim], dtype=np.int64))
+    reduce = x.shape[dim]
+    inner = int(np.prod(x.shape[dim + 1:], dtype=np.int64))
+    y = np.empty_like(x)
+    getattr(lib(), "fto_softmax_" + sfx)(_p(x), _p(y), _i64(outer), _i64(reduce), _i64(inner))
+    return y
+
+
+def layer_norm(x, weight, bias, eps):
+    x = _c(x)
+    sfx, ct = _sfx(x.dtype)
+    batch, n = x.reshape(-1, x.shape[-1]).shape
+    y = np.empty_like(x)
+    getattr(lib(), "fto_layer_norm_" + sfx)(_p(x), _p(_c(weight)), _p(_c(bias)), _p(y), _i64(batch), _i64(n), ct(eps))
+    return y
+
+
+def add_layer_norm(a, b, weight, bias, eps):
+    a = _c(a, np.float32)
+    b = _c(b, np.float32)
+    batch, n = a.reshape(-1, a.shape[-1]).shape
+    y = np.empty_like(a)
+    lib().fto_add_layer_norm_f32(_p(a), _p(b), _p(_c(weight)), _p(_c(bias)), _p(y), _i64(batch), _i64(n), C.c_float(eps))
+    return y
+
+
+def rms_norm(x, weight, eps):
+    x = _c(x)
+    sfx, ct = _sfx(x.dtype)
+    batch, n = x.reshape(-1, x.shape[-1]).shape
+    y = np.empty_like(x)
+    getattr(lib(), "fto_rms_norm_" + sfx)(_p(x), _p(_c(weight)), _p(y), _i64(batch), _i64(n), ct(eps))
+    return y
+
+
+def gelu(x):
+    x = _c(x)
+    sfx, _ = _sfx(x.dtype)
+    y = np.empty_like(x)
+    getattr(lib(), "fto_gelu_" + sfx)(_p(x), _p(y), _i64(x.size))
+    return y
+
+
+def add(a, b):
+    a = _c(a)
+    b = _c(b)
+    sfx, _ = _sfx(a.dtype)
+    y = np.empty_like(a)
+    getattr(lib(), "fto_add_" + sfx)(_p(a), _p(b), _p(y), _i64(a.size))
+    return y
+
+
+def bias_add(x, bias, residual=None):
+    x = _c(x)
+    sfx, _ = _sfx(x.dtype)
+    rows, cols = x.reshape(-1, x.shape[-1]).shape
+    y = np.empty_like(x)
+    getattr(lib(), "fto_bias_add_" + sfx)(_p(x), _p(_c(bias)), _p(_c(residual)), _p(y), _i64(rows), _i64(cols))
+    return y
+
+
+def gemm(a, b, trans_b: bool = False):
+    """a [m,k] . b ([k,n], or [n,k] when trans_b) -> [m,n]; wide accumulation, one rounding."""
+    a = _c(a)
+    b = _c(b)
+    sfx, _ = _sfx(a.dtype)
+    m, k = a.shape
+    n = b.shape[0] if trans_b else b.shape[1]
+    assert (b.shape[1] if trans_b else b.shape[0]) == k
+    c = np.empty((m, n), dtype=a.dtype)
+    getattr(lib(), "fto_gemm_" + sfx)(C.c_int(1 if trans_b else 0), _i64(m), _i64(n), _i64(k), _p(a), _i64(k), _p(b),
+                                      _i64(b.shape[1]), _p(c), _i64(n))
+    return c
+
+
+def sgemm_blocked(a, b):
+    """Timed stand-in for matrixmultiply's f32 kernel; returns None without AVX2/FMA."""
+    a = _c(a, np.float32)
+    b = _c(b, np.float32)
+    m, k = a.shape
+    n = b.shape[1]
+    c = np.empty((m, n), dtype=np.float32)
+    ok = lib().fto_sgemm_blocked(_i64(m), _i64(n), _i64(k), _p(a), _i64(k), _p(b), _i64(n), _p(c), _i64(n))
+    return c if ok else None
+
+
+def bmm(a, b):
+    a = _c(a)
+    b = _c(b)
+    sfx, _ = _sfx(a.dtype)
+    batch, m, k = a.shape
+    n = b.shape[2]
+    c = np.empty((batch, m, n), dtype=a.dtype)
+    getattr(lib(), "fto_bmm_" + sfx)(_i64(batch), _i64(m), _i64(n), _i64(k), _p(a), _p(b), _p(c))
+    return c
+
+
+def addmm(inp, mat1, mat2, beta, alpha):
+    mat1 = _c(mat1)
+    mat2 = _c(mat2)
+    inp = _c(inp)
+    sfx, ct = _sfx(mat1.dtype)
+    m, k = mat1.shape
+    n = mat2.shape[1]
+    out = np.empty((m, n), dtype=mat1.dtype)
+    getattr(lib(), "fto_addmm_" + sfx)(_p(inp), C.c_int(1 if inp.ndim == 1 else 0), _p(mat1), _p(mat2), _i64(m),
+                                       _i64(n), _i64(k), ct(beta), ct(alpha), _p(out))
+    return out
+
+
+def linear(x, weight, bias=None):
+    x = _c(x)
+    weight = _c(weight)
+    sfx, _ = _sfx(x.dtype)
+    batch, in_f = x.shape
+    out_f = weight.shape[0]
+    y = np.empty((batch, out_f), dtype=x.dtype)
+    getattr(lib(), "fto_linear_" + sfx)(_p(x), _p(weight), _p(_c(bias)), _i64(batch), _i64(in_f), _i64(out_f), _p(y))
+    return y
+
+
+def sdpa_forward(q, k, v, scale, causal):
+    q = _c(q)
+    k = _c(k)
+    v = _c(v)
+    sfx, ct = _sfx(q.dtype)
+    num_bh, seq_q, d_k = q.shape
+    seq_k = k.shape[1]
+    d_v = v.shape[2]
+    out = np.zeros((num_bh, seq_q, d_v), dtype=q.dtype)
+    getattr(lib(), "fto_sdpa_forward_" + sfx)(_p(q), _p(k), _p(v), _i64(num_bh), _i64(seq_q), _i64(seq_k), _i64(d_k),
+                                              _i64(d_v), ct(scale), C.c_int(1 if causal else 0), _p(out))
+    return out
+
+
+def index_select(x, dim, indices):
+    """Returns (out, bad): bad is the position of the first invalid index, or -1."""
+    x = _c(x)
+    sfx, _ = _sfx(x.dtype)
+    idx = _c(np.asarray(indices, dtype=np.float64))
+    outer = int(np.prod(x.shape[:dim], dtype=np.int64))
+    inner = int(np.prod(x.shape[dim + 1:], dtype=np.int64))
+    out = np.zeros(x.shape[:dim] + (idx.size,) + x.shape[dim + 1:], dtype=x.dtype)
+    bad = getattr(lib(), "fto_index_select_" + sfx)(_p(x), _i64(outer), _i64(x.shape[dim]), _i64(inner), _p(idx),
+                                                    _i64(idx.size), _p(out))
+    return out, int(bad)
+
+
+def argmax(x, dim):
+    x = _c(x)
+    sfx, _ = _sfx(x.dtype)
+    dim = dim % x.ndim
+    outer = int(np.prod(x.shape[:dim], dtype=np.int64))
+    inner = int(np.prod(x.shape[dim + 1:], dtype=np.int64))
+    out = np.empty(x.shape[:dim] + x.shape[dim + 1:], dtype=x.dtype)
+    getattr(lib(), "fto_argmax_" + sfx)(_p(x), _i64(outer), _i64(x.shape[dim]), _i64(inner), _p(out))
+    return out
+
+
+def permute_0213(x):
+    x = _c(x)
+    sfx, _ = _sfx(x.dtype)
+    d0, d1, d2, d3 = x.shape
+    out = np.empty((d0, d2, d1, d3), dtype=x.dtype)
+    getattr(lib(), "fto_permute_0213_" + sfx)(_p(x), _p(out), _i64(d0), _i64(d1), _i64(d2), _i64(d3))
+    return out
+
+
+LAYER_KEYS = ("ln1_w", "ln1_b", "wq", "bq", "wk", "bk", "wv", "bv", "wo", "bo", "ln2_w", "ln2_b", "w1", "b1", "w2", "b2")
+
+
+def _layer_ptrs(layers):
+    keep = []
+    arr = (_vp * (16 * len(layers)))()
+    for li, lw in enumerate(layers):
+        for ki, key in enumerate(LAYER_KEYS):
+            a = _c(lw[key], np.float32)
+            keep.append(a)
+            arr[li * 16 + ki] = a.ctypes.data
+    return arr, keep
+
+
+def encoder_layer(layer, x, batch, seq, heads, eps, causal):
+    """One pre-LN block on x [batch*seq, d_model]; returns a new array."""
+    x = np.array(x, dtype=np.float32, order="C", copy=True)
+    d_model = x.shape[-1]
+    d_ff = layer["w1"].shape[0]
+    arr, keep = _layer_ptrs([layer])
+    lib().fto_encoder_layer_f32(arr, _p(x), _i64(batch), _i64(seq), _i64(d_model), _i64(heads), _i64(d_ff),
+                                C.c_float(eps), C.c_int(1 if causal else 0))
+    del keep
+    return x
+
+
+def gpt2_forward(wte, wpe, layers, lnf_w, lnf_b, ids, batch, seq, heads, eps, want_logits=True):
+    """Returns dict(hidden, logits (or None), argmax, bad)."""
+    wte = _c(wte, np.float32)
+    wpe = _c(wpe, np.float32)
+    vocab, d_model = wte.shape
+    d_ff = layers[0]["w1"].shape[0]
+    arr, keep = _layer_ptrs(layers)
+    ids = _c(np.asarray(ids, dtype=np.float64).reshape(-1))
+    tokens = batch * seq
+    hidden = np.empty((tokens, d_model), dtype=np.float32)
+    logits = np.empty((tokens, vocab), dtype=np.float32) if want_logits else None
+    am = np.empty((tokens,), dtype=np.float32)
+    bad = lib().fto_gpt2_forward_f32(_i64(vocab), _i64(wpe.shape[0]), _i64(d_model), _i64(heads), _i64(d_ff),
+                                     C.c_float(eps), _p(wte), _p(wpe), arr, _i64(len(layers)), _p(_c(lnf_w, np.float32)),
+                                     _p(_c(lnf_b, np.float32)), _p(ids), _i64(batch), _i64(seq), _p(hidden), _p(logits),
+                                     _p(am))
+    del keep
+    return {"hidden": hidden, "logits": logits, "argmax": am, "bad": int(bad)}
