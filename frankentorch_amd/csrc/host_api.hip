@@ -1,0 +1,754 @@
+// Tier A of the C ABI: host slices in, caller-provided host buffer out -- the call shape of the
+// `ft_kernel_cpu::*` free functions that ft-dispatch routes to (crates/ft-dispatch/src/lib.rs:
+// 14-250). Every function validates exactly as its reference counterpart does (same checks, same
+// order, same error variant and payload), then uploads, launches the device-pointer kernels on
+// the library stream, downloads and synchronises. There is no CPU computation here.
+
+#include <cmath>
+#include <limits>
+#include <type_traits>
+
+#include "common.hpp"
+#include "pool.hpp"
+
+namespace {
+
+using fth::set_error;
+
+// ---- TensorMeta semantics (crates/ft-core/src/lib.rs:340-348, 575-607) ------------------------
+bool meta_ok(const fth_meta *m) { return m && m->ndim >= 0 && m->ndim <= FTH_MAX_DIMS; }
+
+// saturated_numel: product of the shape, saturating (the cached `numel` field).
+uint64_t meta_numel(const fth_meta *m) {
+    uint64_t n = 1;
+    for (int i = 0; i < m->ndim; ++i) {
+        if (__builtin_mul_overflow(n, m->shape[i], &n)) return std::numeric_limits<uint64_t>::max();
+    }
+    return n;
+}
+
+// TensorMeta::is_contiguous: size-1 dims are contiguous whatever their stride.
+bool meta_contiguous(const fth_meta *m) {
+    uint64_t expected = 1;
+    for (int i = m->ndim - 1; i >= 0; --i) {
+        if (m->shape[i] == 1) continue;
+        if (m->strides[i] != expected) return false;
+        if (__builtin_mul_overflow(expected, m->shape[i], &expected)) return false;
+    }
+    return true;
+}
+
+void fill_shapes(const uint64_t *l, int ln, const uint64_t *r, int rn) {
+    fth_error_info &e = fth::last_error();
+    e.lhs_ndim = ln;
+    e.rhs_ndim = rn;
+    for (int i = 0; i < ln && i < FTH_MAX_DIMS; ++i) e.lhs_shape[i] = l[i];
+    for (int i = 0; i < rn && i < FTH_MAX_DIMS; ++i) e.rhs_shape[i] = r[i];
+}
+
+int32_t err_shape_mismatch(const fth_meta *l, const fth_meta *r) {
+    set_error(FTH_ERR_SHAPE_MISMATCH, "shape mismatch: lhs rank %d, rhs rank %d", l->ndim, r->ndim);
+    fill_shapes(l->shape, l->ndim, r->shape, r->ndim);
+    return FTH_ERR_SHAPE_MISMATCH;
+}
+
+int32_t err_layout(const char *side) {
+    set_error(FTH_ERR_UNSUPPORTED_LAYOUT, "unsupported (non-contiguous) layout on %s", side);
+    std::snprintf(fth::last_error().side, sizeof(fth::last_error().side), "%s", side);
+    return FTH_ERR_UNSUPPORTED_LAYOUT;
+}
+
+int32_t err_overflow(const char *context) { return set_error(FTH_ERR_SHAPE_OVERFLOW, "%s", context); }
+
+int32_t err_invalid_dim(uint64_t dim, uint64_t ndim) {
+    set_error(FTH_ERR_INVALID_DIMENSION, "invalid dimension %llu for ndim %llu", (unsigned long long)dim,
+              (unsigned long long)ndim);
+    fth::last_error().a = dim;
+    fth::last_error().b = ndim;
+    return FTH_ERR_INVALID_DIMENSION;
+}
+
+// ensure_dtype_device_and_layout[_f32] (crates/ft-kernel-cpu/src/lib.rs:2256-2284, 36935-36962):
+// dtype, then device, then lhs layout, then rhs layout.
+int32_t ensure_dtype_device(const fth_meta *l, const fth_meta *r) {
+    if (l->dtype != r->dtype) {
+        set_error(FTH_ERR_DTYPE_MISMATCH, "dtype mismatch: lhs %d, rhs %d", l->dtype, r->dtype);
+        fth::last_error().a = (uint64_t)l->dtype;
+        fth::last_error().b = (uint64_t)r->dtype;
+        return FTH_ERR_DTYPE_MISMATCH;
+    }
+    if (l->device != r->device) {
+        set_error(FTH_ERR_DEVICE_MISMATCH, "device mismatch: lhs %d, rhs %d", l->device, r->device);
+        fth::last_error().a = (uint64_t)l->device;
+        fth::last_error().b = (uint64_t)r->device;
+        return FTH_ERR_DEVICE_MISMATCH;
+    }
+    return FTH_OK;
+}
+int32_t ensure_dtype_device_and_layout(const fth_meta *l, const fth_meta *r) {
+    if (int32_t rc = ensure_dtype_device(l, r)) return rc;
+    if (!meta_contiguous(l)) return err_layout("lhs");
+    if (!meta_contiguous(r)) return err_layout("rhs");
+    return FTH_OK;
+}
+
+// contiguous_required_len + ensure_storage_len (crates/ft-kernel-cpu/src/lib.rs:2340-2369).
+int32_t ensure_storage_len(size_t len, const fth_meta *m, const char *side) {
+    const uint64_t numel = meta_numel(m);
+    uint64_t needed = 0;
+    if (numel != 0 && __builtin_add_overflow(m->storage_offset, numel, &needed)) {
+        set_error(FTH_ERR_STORAGE_SPAN_OVERFLOW, "storage span overflow on %s", side);
+        fth_error_info &e = fth::last_error();
+        std::snprintf(e.side, sizeof(e.side), "%s", side);
+        e.a = m->storage_offset;
+        e.b = numel;
+        return FTH_ERR_STORAGE_SPAN_OVERFLOW;
+    }
+    if ((uint64_t)len < needed) {
+        set_error(FTH_ERR_INSUFFICIENT_STORAGE, "insufficient storage on %s: needed %llu, available %llu", side,
+                  (unsigned long long)needed, (unsigned long long)len);
+        fth_error_info &e = fth::last_error();
+        std::snprintf(e.side, sizeof(e.side), "%s", side);
+        e.a = needed;
+        e.b = len;
+        return FTH_ERR_INSUFFICIENT_STORAGE;
+    }
+    return FTH_OK;
+}
+
+bool checked_mul(uint64_t a, uint64_t b, uint64_t *out) { return !__builtin_mul_overflow(a, b, out); }
+
+// checked_dim_loop_sizes (crates/ft-kernel-cpu/src/lib.rs:2565-2574).
+int32_t dim_loop_sizes(const fth_meta *m, size_t dim, const char *context, uint64_t *outer, uint64_t *inner,
+                       uint64_t *total) {
+    uint64_t o = 1, in = 1;
+    for (size_t i = 0; i < dim; ++i)
+        if (!checked_mul(o, m->shape[i], &o)) return err_overflow(context);
+    for (int i = (int)dim + 1; i < m->ndim; ++i)
+        if (!checked_mul(in, m->shape[i], &in)) return err_overflow(context);
+    uint64_t t = 1;
+    for (int i = 0; i < m->ndim; ++i)
+        if (!checked_mul(t, m->shape[i], &t)) return err_overflow(context);
+    *outer = o;
+    *inner = in;
+    *total = t;
+    return FTH_OK;
+}
+
+int32_t check_out(const void *out, size_t out_cap, size_t need) {
+    if (out_cap < need || (need > 0 && out == nullptr))
+        return set_error(FTH_ERR_OUTPUT_TOO_SMALL, "output buffer holds %zu elements, result has %zu", out_cap, need);
+    return FTH_OK;
+}
+
+// ---- staging ---------------------------------------------------------------------------------
+template <typename T> int32_t stage_in(fth::Scratch &sc, const T *host, size_t n, T **dev) {
+    void *p = nullptr;
+    if (int32_t rc = sc.get(&p, n * sizeof(T))) return rc;
+    *dev = static_cast<T *>(p);
+    if (n) FTH_HIP(hipMemcpyAsync(p, host, n * sizeof(T), hipMemcpyHostToDevice, fth::resolve_stream(nullptr)));
+    return FTH_OK;
+}
+template <typename T> int32_t stage_out(fth::Scratch &sc, size_t n, T **dev) {
+    void *p = nullptr;
+    if (int32_t rc = sc.get(&p, n * sizeof(T))) return rc;
+    *dev = static_cast<T *>(p);
+    return FTH_OK;
+}
+template <typename T> int32_t fetch(T *host, const T *dev, size_t n) {
+    hipStream_t st = fth::resolve_stream(nullptr);
+    if (n) FTH_HIP(hipMemcpyAsync(host, dev, n * sizeof(T), hipMemcpyDeviceToHost, st));
+    hipError_t e = hipStreamSynchronize(st);
+    if (e != hipSuccess) {
+        fth::hip_fail(e, "hipStreamSynchronize");
+        fth::last_error().code = FTH_ERR_STREAM;
+        return FTH_ERR_STREAM;
+    }
+    return FTH_OK;
+}
+
+template <typename T> struct Dev;
+template <> struct Dev<float> {
+    static int32_t gemm(const fth_gemm_desc *d, float al, const float *a, const float *b, float *c, const float *bias) {
+        return fth_dev_gemm_f32(d, al, a, b, c, bias, nullptr, nullptr);
+    }
+    static int32_t softmax(const float *x, float *y, int64_t o, int64_t r, int64_t i) { return fth_dev_softmax_strided_f32(x, y, o, r, i, nullptr); }
+    static int32_t layer_norm(const float *x, const float *w, const float *b, float *y, int64_t n, int64_t c, float e) { return fth_dev_layer_norm_f32(x, w, b, y, n, c, e, nullptr); }
+    static int32_t rms_norm(const float *x, const float *w, float *y, int64_t n, int64_t c, float e) { return fth_dev_rms_norm_f32(x, w, y, n, c, e, nullptr); }
+    static int32_t gelu(const float *x, float *y, int64_t n) { return fth_dev_gelu_f32(x, y, n, nullptr); }
+    static int32_t add(const float *a, const float *b, float *y, int64_t n) { return fth_dev_add_f32(a, b, y, n, nullptr); }
+    static int32_t sdpa(const fth_sdpa_desc *d, float s, const float *q, const float *k, const float *v, float *o) { return fth_dev_sdpa_forward_f32(d, s, q, k, v, o, nullptr); }
+    static int32_t index_select(const float *x, int64_t o, int64_t ds, int64_t in, const double *idx, int64_t n, float *out) { return fth_dev_index_select_f32(x, o, ds, in, idx, n, out, nullptr, nullptr); }
+    static int32_t argmax(const float *x, int64_t o, int64_t r, int64_t in, float *out) { return fth_dev_argmax_f32(x, o, r, in, out, nullptr); }
+    static constexpr int32_t dtype = FTH_DTYPE_F32;
+};
+template <> struct Dev<double> {
+    static int32_t gemm(const fth_gemm_desc *d, double al, const double *a, const double *b, double *c, const double *bias) {
+        return fth_dev_gemm_f64(d, al, a, b, c, bias, nullptr, nullptr);
+    }
+    static int32_t softmax(const double *x, double *y, int64_t o, int64_t r, int64_t i) { return fth_dev_softmax_strided_f64(x, y, o, r, i, nullptr); }
+    static int32_t layer_norm(const double *x, const double *w, const double *b, double *y, int64_t n, int64_t c, double e) { return fth_dev_layer_norm_f64(x, w, b, y, n, c, e, nullptr); }
+    static int32_t rms_norm(const double *x, const double *w, double *y, int64_t n, int64_t c, double e) { return fth_dev_rms_norm_f64(x, w, y, n, c, e, nullptr); }
+    static int32_t gelu(const double *x, double *y, int64_t n) { return fth_dev_gelu_f64(x, y, n, nullptr); }
+    static int32_t add(const double *a, const double *b, double *y, int64_t n) { return fth_dev_add_f64(a, b, y, n, nullptr); }
+    static int32_t sdpa(const fth_sdpa_desc *d, double s, const double *q, const double *k, const double *v, double *o) { return fth_dev_sdpa_forward_f64(d, s, q, k, v, o, nullptr); }
+    static int32_t index_select(const double *x, int64_t o, int64_t ds, int64_t in, const double *idx, int64_t n, double *out) { return fth_dev_index_select_f64(x, o, ds, in, idx, n, out, nullptr, nullptr); }
+    static int32_t argmax(const double *x, int64_t o, int64_t r, int64_t in, double *out) { return fth_dev_argmax_f64(x, o, r, in, out, nullptr); }
+    static constexpr int32_t dtype = FTH_DTYPE_F64;
+};
+
+fth_gemm_desc gemm_desc(int64_t m, int64_t n, int64_t k, int trans_b, int64_t batch, int epi) {
+    fth_gemm_desc d;
+    d.m = m; d.n = n; d.k = k;
+    d.lda = k; d.ldb = trans_b ? k : n; d.ldc = n;
+    d.batch = batch;
+    d.stride_a = m * k; d.stride_b = k * n; d.stride_c = m * n;
+    d.trans_b = trans_b;
+    d.epilogue = epi;
+    return d;
+}
+
+// The addmm combine of crates/ft-kernel-cpu/src/lib.rs:41614-41645: two multiplies, one add.
+template <typename T>
+__global__ __launch_bounds__(256) void addmm_combine_kernel(const T *__restrict__ input, int input_1d,
+                                                            const T *__restrict__ g, T *__restrict__ out,
+                                                            int64_t total, int64_t n, T beta, T alpha, int alpha_zero) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const T in = input_1d ? input[i % n] : input[i];
+    out[i] = alpha_zero ? beta * in : beta * in + alpha * g[i];
+}
+
+// ---- matmul_tensor_contiguous (crates/ft-kernel-cpu/src/lib.rs:37780-37823 / 17355-17379) ------
+template <typename T>
+int32_t matmul_impl(const T *lhs, size_t lhs_len, const T *rhs, size_t rhs_len, const fth_meta *lm, const fth_meta *rm,
+                    T *out, size_t out_cap, size_t *out_len) {
+    FTH_ARG(meta_ok(lm) && meta_ok(rm), "matmul: bad meta");
+    if (out_len) *out_len = 0;
+    if (int32_t rc = ensure_dtype_device_and_layout(lm, rm)) return rc;
+    if (lm->ndim != 2 || rm->ndim != 2 || lm->shape[1] != rm->shape[0]) return err_shape_mismatch(lm, rm);
+    const uint64_t m = lm->shape[0], k = lm->shape[1], n = rm->shape[1];
+    uint64_t t, out_numel;
+    if (!checked_mul(m, k, &t)) return err_overflow("matmul lhs overflow");
+    if (!checked_mul(k, n, &t)) return err_overflow("matmul rhs overflow");
+    if (!checked_mul(m, n, &out_numel)) return err_overflow("matmul output overflow");
+    if (int32_t rc = ensure_storage_len(lhs_len, lm, "lhs")) return rc;
+    if (int32_t rc = ensure_storage_len(rhs_len, rm, "rhs")) return rc;
+    if (out_len) *out_len = (size_t)out_numel;
+    if (out == nullptr && out_cap == 0) return FTH_OK;  // validation only
+    if (int32_t rc = check_out(out, out_cap, (size_t)out_numel)) return rc;
+    if (out_numel == 0) return FTH_OK;
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *da, *db, *dc;
+    if (int32_t rc = stage_in(sc, lhs + lm->storage_offset, (size_t)(m * k), &da)) return rc;
+    if (int32_t rc = stage_in(sc, rhs + rm->storage_offset, (size_t)(k * n), &db)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)out_numel, &dc)) return rc;
+    fth_gemm_desc d = gemm_desc((int64_t)m, (int64_t)n, (int64_t)k, 0, 1, FTH_EPI_NONE);
+    if (int32_t rc = Dev<T>::gemm(&d, T(1), da, db, dc, nullptr)) return rc;
+    return fetch(out, dc, (size_t)out_numel);
+}
+
+// ---- bmm_tensor_contiguous (crates/ft-kernel-cpu/src/lib.rs:38496-38606 / 17785-17872) --------
+template <typename T>
+int32_t bmm_impl(const T *lhs, size_t lhs_len, const T *rhs, size_t rhs_len, const fth_meta *lm, const fth_meta *rm,
+                 T *out, size_t out_cap, size_t *out_len) {
+    FTH_ARG(meta_ok(lm) && meta_ok(rm), "bmm: bad meta");
+    if (out_len) *out_len = 0;
+    if (int32_t rc = ensure_dtype_device_and_layout(lm, rm)) return rc;
+    if (lm->ndim != 3 || rm->ndim != 3) return err_shape_mismatch(lm, rm);
+    const uint64_t batch = lm->shape[0], m = lm->shape[1], k = lm->shape[2], n = rm->shape[2];
+    if (batch != rm->shape[0] || k != rm->shape[1]) return err_shape_mismatch(lm, rm);
+    uint64_t ls, rs, os, t, out_numel;
+    if (!checked_mul(m, k, &ls)) return err_overflow("bmm lhs batch stride overflow");
+    if (!checked_mul(k, n, &rs)) return err_overflow("bmm rhs batch stride overflow");
+    if (!checked_mul(m, n, &os)) return err_overflow("bmm output batch stride overflow");
+    if (!checked_mul(batch, ls, &t)) return err_overflow("bmm lhs overflow");
+    if (!checked_mul(batch, rs, &t)) return err_overflow("bmm rhs overflow");
+    if (!checked_mul(batch, os, &out_numel)) return err_overflow("bmm output overflow");
+    if (int32_t rc = ensure_storage_len(lhs_len, lm, "lhs")) return rc;
+    if (int32_t rc = ensure_storage_len(rhs_len, rm, "rhs")) return rc;
+    if (out_len) *out_len = (size_t)out_numel;
+    if (out == nullptr && out_cap == 0) return FTH_OK;
+    if (int32_t rc = check_out(out, out_cap, (size_t)out_numel)) return rc;
+    if (out_numel == 0) return FTH_OK;
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *da, *db, *dc;
+    if (int32_t rc = stage_in(sc, lhs + lm->storage_offset, (size_t)(batch * ls), &da)) return rc;
+    if (int32_t rc = stage_in(sc, rhs + rm->storage_offset, (size_t)(batch * rs), &db)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)out_numel, &dc)) return rc;
+    // The grid's batch axis holds 65 535 entries; larger batches go in slices.
+    for (uint64_t b0 = 0; b0 < batch; b0 += 65535) {
+        const uint64_t nb = (batch - b0) < 65535 ? (batch - b0) : 65535;
+        fth_gemm_desc d = gemm_desc((int64_t)m, (int64_t)n, (int64_t)k, 0, (int64_t)nb, FTH_EPI_NONE);
+        if (int32_t rc = Dev<T>::gemm(&d, T(1), da + b0 * ls, db + b0 * rs, dc + b0 * os, nullptr)) return rc;
+    }
+    return fetch(out, dc, (size_t)out_numel);
+}
+
+// ---- addmm_tensor_contiguous (crates/ft-kernel-cpu/src/lib.rs:41562-41648 / 17514-17606) ------
+template <typename T>
+int32_t addmm_impl(const T *input, size_t input_len, const T *mat1, size_t mat1_len, const T *mat2, size_t mat2_len,
+                   const fth_meta *im, const fth_meta *m1, const fth_meta *m2, T beta, T alpha, T *out,
+                   size_t out_cap, size_t *out_len) {
+    FTH_ARG(meta_ok(im) && meta_ok(m1) && meta_ok(m2), "addmm: bad meta");
+    if (out_len) *out_len = 0;
+    if (m1->ndim != 2 || m2->ndim != 2 || m1->shape[1] != m2->shape[0]) return err_shape_mismatch(m1, m2);
+    const uint64_t m = m1->shape[0], k = m1->shape[1], n = m2->shape[1];
+    uint64_t out_numel;
+    if (!checked_mul(m, n, &out_numel)) return err_overflow("addmm output overflow");
+    if (int32_t rc = ensure_storage_len(mat1_len, m1, "mat1")) return rc;
+    if (int32_t rc = ensure_storage_len(mat2_len, m2, "mat2")) return rc;
+    const bool in1d = im->ndim == 1 && im->shape[0] == n;
+    const bool in2d = im->ndim == 2 && im->shape[0] == m && im->shape[1] == n;
+    if (!in1d && !in2d) {
+        set_error(FTH_ERR_SHAPE_MISMATCH, "addmm: input shape does not broadcast to [m, n]");
+        const uint64_t want[2] = {m, n};
+        fill_shapes(im->shape, im->ndim, want, 2);
+        return FTH_ERR_SHAPE_MISMATCH;
+    }
+    if (int32_t rc = ensure_storage_len(input_len, im, "input")) return rc;
+    if (!meta_contiguous(m1)) return err_layout("mat1");
+    if (!meta_contiguous(m2)) return err_layout("mat2");
+    if (!meta_contiguous(im)) return err_layout("input");
+    if (out_len) *out_len = (size_t)out_numel;
+    if (out == nullptr && out_cap == 0) return FTH_OK;
+    if (int32_t rc = check_out(out, out_cap, (size_t)out_numel)) return rc;
+    if (out_numel == 0) return FTH_OK;
+    FTH_REQUIRE_DEVICE();
+    // alpha.to_bits() == 0: only +0.0 takes the shortcut (crates/ft-kernel-cpu/src/lib.rs:41614).
+    bool alpha_zero;
+    if constexpr (sizeof(T) == 4) {
+        uint32_t bits;
+        std::memcpy(&bits, &alpha, 4);
+        alpha_zero = bits == 0;
+    } else {
+        uint64_t bits;
+        std::memcpy(&bits, &alpha, 8);
+        alpha_zero = bits == 0;
+    }
+    fth::Scratch sc;
+    T *di, *d1 = nullptr, *d2 = nullptr, *dg = nullptr, *dout;
+    if (int32_t rc = stage_in(sc, input + im->storage_offset, (size_t)(in1d ? n : out_numel), &di)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)out_numel, &dout)) return rc;
+    if (!alpha_zero) {
+        if (int32_t rc = stage_in(sc, mat1 + m1->storage_offset, (size_t)(m * k), &d1)) return rc;
+        if (int32_t rc = stage_in(sc, mat2 + m2->storage_offset, (size_t)(k * n), &d2)) return rc;
+        if (int32_t rc = stage_out(sc, (size_t)out_numel, &dg)) return rc;
+        fth_gemm_desc d = gemm_desc((int64_t)m, (int64_t)n, (int64_t)k, 0, 1, FTH_EPI_NONE);
+        if (int32_t rc = Dev<T>::gemm(&d, T(1), d1, d2, dg, nullptr)) return rc;
+    }
+    const int64_t grid = fth::ceil_div((int64_t)out_numel, 256);
+    FTH_ARG(grid <= 2147483647LL, "addmm: output too large for one launch");
+    addmm_combine_kernel<T><<<dim3((unsigned)grid), dim3(256), 0, fth::resolve_stream(nullptr)>>>(
+        di, in1d ? 1 : 0, dg, dout, (int64_t)out_numel, (int64_t)n, beta, alpha, alpha_zero ? 1 : 0);
+    FTH_CHECK_LAUNCH("addmm_combine");
+    return fetch(out, dout, (size_t)out_numel);
+}
+
+// ---- linear_tensor (crates/ft-kernel-cpu/src/lib.rs:17306-17353 / 17162-17211) ----------------
+// The reference is infallible and panics on short slices; here that is FTH_ERR_INVALID_ARGUMENT.
+template <typename T>
+int32_t linear_impl(const T *x, size_t x_len, const T *w, size_t w_len, const T *bias, size_t bias_len, size_t batch,
+                    size_t in_f, size_t out_f, T *out, size_t out_cap, size_t *out_len) {
+    uint64_t xn, wn, on;
+    FTH_ARG(checked_mul(batch, in_f, &xn) && checked_mul(out_f, in_f, &wn) && checked_mul(batch, out_f, &on),
+            "linear: shape product overflows");
+    if (out_len) *out_len = (size_t)on;
+    if (out == nullptr && out_cap == 0) return FTH_OK;
+    if (int32_t rc = check_out(out, out_cap, (size_t)on)) return rc;
+    if (on == 0) return FTH_OK;
+    FTH_ARG(x_len >= xn && w_len >= wn, "linear: slice shorter than batch*in (%zu < %llu) or out*in (%zu < %llu)", x_len,
+            (unsigned long long)xn, w_len, (unsigned long long)wn);
+    FTH_ARG(bias == nullptr || bias_len >= out_f, "linear: bias shorter than out_features");
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *dx, *dw, *db = nullptr, *dy;
+    if (int32_t rc = stage_in(sc, x, (size_t)xn, &dx)) return rc;
+    if (int32_t rc = stage_in(sc, w, (size_t)wn, &dw)) return rc;
+    if (bias)
+        if (int32_t rc = stage_in(sc, bias, out_f, &db)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)on, &dy)) return rc;
+    fth_gemm_desc d = gemm_desc((int64_t)batch, (int64_t)out_f, (int64_t)in_f, 1, 1, bias ? FTH_EPI_BIAS : FTH_EPI_NONE);
+    if (int32_t rc = Dev<T>::gemm(&d, T(1), dx, dw, dy, db)) return rc;
+    return fetch(out, dy, (size_t)on);
+}
+
+// ---- matmul_rhs_transposed_contiguous (crates/ft-kernel-cpu/src/lib.rs:17381-17436) -----------
+template <typename T>
+int32_t matmul_bt_impl(size_t m, size_t k, size_t n, const T *lhs, size_t lhs_len, const T *rhs, size_t rhs_len, T *out,
+                       size_t out_cap, size_t *out_len) {
+    if (out_len) *out_len = 0;
+    uint64_t ll, rl, ol;
+    if (!checked_mul(m, k, &ll)) return err_overflow("matmul_rhs_transposed lhs overflow");
+    if (!checked_mul(n, k, &rl)) return err_overflow("matmul_rhs_transposed rhs overflow");
+    if (!checked_mul(m, n, &ol)) return err_overflow("matmul_rhs_transposed output overflow");
+    if (lhs_len < ll) {
+        set_error(FTH_ERR_SHAPE_MISMATCH, "matmul_rhs_transposed: lhs slice shorter than m*k");
+        const uint64_t a[1] = {ll}, b[1] = {lhs_len};
+        fill_shapes(a, 1, b, 1);
+        return FTH_ERR_SHAPE_MISMATCH;
+    }
+    if (rhs_len < rl) {
+        set_error(FTH_ERR_SHAPE_MISMATCH, "matmul_rhs_transposed: rhs slice shorter than n*k");
+        const uint64_t a[1] = {rl}, b[1] = {rhs_len};
+        fill_shapes(a, 1, b, 1);
+        return FTH_ERR_SHAPE_MISMATCH;
+    }
+    if (out_len) *out_len = (size_t)ol;
+    if (out == nullptr && out_cap == 0) return FTH_OK;
+    if (int32_t rc = check_out(out, out_cap, (size_t)ol)) return rc;
+    if (ol == 0) return FTH_OK;
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *da, *db, *dc;
+    if (int32_t rc = stage_in(sc, lhs, (size_t)ll, &da)) return rc;
+    if (int32_t rc = stage_in(sc, rhs, (size_t)rl, &db)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)ol, &dc)) return rc;
+    fth_gemm_desc d = gemm_desc((int64_t)m, (int64_t)n, (int64_t)k, 1, 1, FTH_EPI_NONE);
+    if (int32_t rc = Dev<T>::gemm(&d, T(1), da, db, dc, nullptr)) return rc;
+    return fetch(out, dc, (size_t)ol);
+}
+
+// ---- unary / dim ops -----------------------------------------------------------------------
+int32_t ensure_unary(size_t len, const fth_meta *m) {
+    if (!meta_contiguous(m)) return err_layout("input");
+    return ensure_storage_len(len, m, "input");
+}
+
+// softmax_dim_tensor_contiguous (crates/ft-kernel-cpu/src/lib.rs:39193-39296 / 18350-18461)
+template <typename T>
+int32_t softmax_impl(const T *input, size_t input_len, const fth_meta *meta, size_t dim, T *out, size_t out_cap,
+                     size_t *out_len) {
+    FTH_ARG(meta_ok(meta), "softmax: bad meta");
+    if (out_len) *out_len = 0;
+    if (int32_t rc = ensure_unary(input_len, meta)) return rc;
+    if (dim >= (size_t)meta->ndim) return err_invalid_dim(dim, (uint64_t)meta->ndim);
+    uint64_t outer, inner, numel;
+    if (int32_t rc = dim_loop_sizes(meta, dim, "softmax overflow", &outer, &inner, &numel)) return rc;
+    if (out_len) *out_len = (size_t)numel;
+    if (out == nullptr && out_cap == 0) return FTH_OK;
+    if (int32_t rc = check_out(out, out_cap, (size_t)numel)) return rc;
+    if (numel == 0) return FTH_OK;
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *dx, *dy;
+    if (int32_t rc = stage_in(sc, input + meta->storage_offset, (size_t)numel, &dx)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)numel, &dy)) return rc;
+    if (int32_t rc = Dev<T>::softmax(dx, dy, (int64_t)outer, (int64_t)meta->shape[dim], (int64_t)inner)) return rc;
+    return fetch(out, dy, (size_t)numel);
+}
+
+// layer_norm_forward (crates/ft-kernel-cpu/src/lib.rs:5877-5923 / 5824-5870), optionally fused
+// with the residual add (add_layer_norm_forward_f32, :5932-5984).
+template <typename T>
+int32_t layer_norm_impl(const T *x, const T *x2, size_t x_len, const T *w, const T *b, size_t batch, size_t n, T eps,
+                        T *out, size_t out_cap) {
+    uint64_t total;
+    FTH_ARG(checked_mul(batch, n, &total), "layer_norm: batch * norm_size overflows");
+    if (int32_t rc = check_out(out, out_cap, (size_t)total)) return rc;
+    if (total == 0) return FTH_OK;
+    FTH_ARG(x_len >= total, "layer_norm: input slice shorter than batch * norm_size");
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *dx, *dx2 = nullptr, *dw = nullptr, *db = nullptr, *dy;
+    if (int32_t rc = stage_in(sc, x, (size_t)total, &dx)) return rc;
+    if (x2)
+        if (int32_t rc = stage_in(sc, x2, (size_t)total, &dx2)) return rc;
+    if (w)
+        if (int32_t rc = stage_in(sc, w, n, &dw)) return rc;
+    if (b)
+        if (int32_t rc = stage_in(sc, b, n, &db)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)total, &dy)) return rc;
+    int32_t rc;
+    if constexpr (std::is_same<T, float>::value) {
+        rc = x2 ? fth_dev_add_layer_norm_f32(dx, dx2, dw, db, dy, (int64_t)batch, (int64_t)n, eps, nullptr)
+                : fth_dev_layer_norm_f32(dx, dw, db, dy, (int64_t)batch, (int64_t)n, eps, nullptr);
+    } else {
+        rc = fth_dev_layer_norm_f64(dx, dw, db, dy, (int64_t)batch, (int64_t)n, eps, nullptr);
+    }
+    if (rc) return rc;
+    return fetch(out, dy, (size_t)total);
+}
+
+// rms_norm_forward (crates/ft-kernel-cpu/src/lib.rs:6459-6494 / 6418-6453)
+template <typename T>
+int32_t rms_norm_impl(const T *x, size_t x_len, const T *w, size_t batch, size_t n, T eps, T *out, size_t out_cap) {
+    uint64_t total;
+    FTH_ARG(checked_mul(batch, n, &total), "rms_norm: batch * norm_size overflows");
+    if (int32_t rc = check_out(out, out_cap, (size_t)total)) return rc;
+    if (total == 0) return FTH_OK;
+    FTH_ARG(x_len >= total, "rms_norm: input slice shorter than batch * norm_size");
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *dx, *dw = nullptr, *dy;
+    if (int32_t rc = stage_in(sc, x, (size_t)total, &dx)) return rc;
+    if (w)
+        if (int32_t rc = stage_in(sc, w, n, &dw)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)total, &dy)) return rc;
+    if (int32_t rc = Dev<T>::rms_norm(dx, dw, dy, (int64_t)batch, (int64_t)n, eps)) return rc;
+    return fetch(out, dy, (size_t)total);
+}
+
+// gelu_tensor_contiguous (unary_contiguous_f32 via define_unary_f32!, crates/ft-kernel-cpu/src/
+// lib.rs:37051-37064, 37123-37127)
+template <typename T>
+int32_t gelu_impl(const T *input, size_t input_len, const fth_meta *meta, T *out, size_t out_cap, size_t *out_len) {
+    FTH_ARG(meta_ok(meta), "gelu: bad meta");
+    if (out_len) *out_len = 0;
+    if (int32_t rc = ensure_unary(input_len, meta)) return rc;
+    const uint64_t numel = meta_numel(meta);
+    if (out_len) *out_len = (size_t)numel;
+    if (out == nullptr && out_cap == 0) return FTH_OK;
+    if (int32_t rc = check_out(out, out_cap, (size_t)numel)) return rc;
+    if (numel == 0) return FTH_OK;
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *dx, *dy;
+    if (int32_t rc = stage_in(sc, input + meta->storage_offset, (size_t)numel, &dx)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)numel, &dy)) return rc;
+    if (int32_t rc = Dev<T>::gelu(dx, dy, (int64_t)numel)) return rc;
+    return fetch(out, dy, (size_t)numel);
+}
+
+// add_tensor_contiguous (simd_elementwise_f32, crates/ft-kernel-cpu/src/lib.rs:36558-36593):
+// dtype, device, equal shapes, then storage lengths; no broadcast.
+template <typename T>
+int32_t add_impl(const T *lhs, size_t lhs_len, const T *rhs, size_t rhs_len, const fth_meta *lm, const fth_meta *rm,
+                 T *out, size_t out_cap, size_t *out_len) {
+    FTH_ARG(meta_ok(lm) && meta_ok(rm), "add: bad meta");
+    if (out_len) *out_len = 0;
+    if (int32_t rc = ensure_dtype_device(lm, rm)) return rc;
+    bool same = lm->ndim == rm->ndim;
+    for (int i = 0; same && i < lm->ndim; ++i) same = lm->shape[i] == rm->shape[i];
+    if (!same) return err_shape_mismatch(lm, rm);
+    if (int32_t rc = ensure_storage_len(lhs_len, lm, "lhs")) return rc;
+    if (int32_t rc = ensure_storage_len(rhs_len, rm, "rhs")) return rc;
+    const uint64_t numel = meta_numel(lm);
+    if (out_len) *out_len = (size_t)numel;
+    if (out == nullptr && out_cap == 0) return FTH_OK;
+    if (int32_t rc = check_out(out, out_cap, (size_t)numel)) return rc;
+    if (numel == 0) return FTH_OK;
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *da, *db, *dy;
+    if (int32_t rc = stage_in(sc, lhs + lm->storage_offset, (size_t)numel, &da)) return rc;
+    if (int32_t rc = stage_in(sc, rhs + rm->storage_offset, (size_t)numel, &db)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)numel, &dy)) return rc;
+    if (int32_t rc = Dev<T>::add(da, db, dy, (int64_t)numel)) return rc;
+    return fetch(out, dy, (size_t)numel);
+}
+
+// sdpa_forward (crates/ft-kernel-cpu/src/lib.rs:5200-5284 / 4572-4651)
+template <typename T>
+int32_t sdpa_impl(const T *q, size_t q_len, const T *k, size_t k_len, const T *v, size_t v_len, size_t num_bh,
+                  size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, T scale, int32_t causal, T *out, size_t out_cap) {
+    uint64_t qn, kn, vn, on, t;
+    FTH_ARG(checked_mul(num_bh, seq_q, &t) && checked_mul(t, d_k, &qn) && checked_mul(t, d_v, &on) &&
+                checked_mul(num_bh, seq_k, &t) && checked_mul(t, d_k, &kn) && checked_mul(t, d_v, &vn),
+            "sdpa: shape product overflows");
+    if (int32_t rc = check_out(out, out_cap, (size_t)on)) return rc;
+    if (on == 0) return FTH_OK;
+    FTH_ARG(q_len >= qn && k_len >= kn && v_len >= vn, "sdpa: q/k/v slice shorter than its shape");
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *dq, *dk, *dv, *dout;
+    if (int32_t rc = stage_in(sc, q, (size_t)qn, &dq)) return rc;
+    if (int32_t rc = stage_in(sc, k, (size_t)kn, &dk)) return rc;
+    if (int32_t rc = stage_in(sc, v, (size_t)vn, &dv)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)on, &dout)) return rc;
+    fth_sdpa_desc d;
+    fth_sdpa_desc_contiguous(&d, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k, (int64_t)d_v, causal ? 1 : 0);
+    if (int32_t rc = Dev<T>::sdpa(&d, scale, dq, dk, dv, dout)) return rc;
+    return fetch(out, dout, (size_t)on);
+}
+
+// normalize_strict_index_value (crates/ft-kernel-cpu/src/lib.rs:20058-20090), host side: the
+// reference returns Err at the first bad index before producing anything.
+bool strict_index_ok(double v, uint64_t dim_size) {
+    if (!std::isfinite(v)) return false;
+    if (std::fabs(v - std::trunc(v)) > std::numeric_limits<double>::epsilon()) return false;
+    if (v < 0.0 || v >= 9.2233720368547758e18) return false;
+    return (uint64_t)(int64_t)v < dim_size;
+}
+
+// index_select_tensor_contiguous (crates/ft-kernel-cpu/src/lib.rs:40216-40253)
+template <typename T>
+int32_t index_select_impl(const T *input, size_t input_len, const fth_meta *meta, size_t dim, const double *indices,
+                          size_t num_indices, T *out, size_t out_cap, size_t *out_len) {
+    FTH_ARG(meta_ok(meta), "index_select: bad meta");
+    if (out_len) *out_len = 0;
+    if (int32_t rc = ensure_unary(input_len, meta)) return rc;
+    if (dim >= (size_t)meta->ndim) return err_invalid_dim(dim, (uint64_t)meta->ndim);
+    const uint64_t dim_size = meta->shape[dim];
+    uint64_t outer, inner, total, t, out_numel;
+    if (int32_t rc = dim_loop_sizes(meta, dim, "index_select overflow", &outer, &inner, &total)) return rc;
+    if (!checked_mul(outer, num_indices, &t) || !checked_mul(t, inner, &out_numel)) return err_overflow("index_select overflow");
+    if (out_numel == 0) return FTH_OK;  // empty result before any index is looked at, as in the reference
+    FTH_ARG(indices != nullptr, "index_select: indices is NULL");
+    for (size_t i = 0; i < num_indices; ++i)
+        if (!strict_index_ok(indices[i], dim_size)) return err_invalid_dim(dim_size, dim_size);
+    if (out_len) *out_len = (size_t)out_numel;
+    if (out == nullptr && out_cap == 0) return FTH_OK;
+    if (int32_t rc = check_out(out, out_cap, (size_t)out_numel)) return rc;
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *dx, *dy;
+    double *di;
+    if (int32_t rc = stage_in(sc, input + meta->storage_offset, (size_t)total, &dx)) return rc;
+    if (int32_t rc = stage_in(sc, indices, num_indices, &di)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)out_numel, &dy)) return rc;
+    if (int32_t rc = Dev<T>::index_select(dx, (int64_t)outer, (int64_t)dim_size, (int64_t)inner, di, (int64_t)num_indices, dy)) return rc;
+    return fetch(out, dy, (size_t)out_numel);
+}
+
+// argmax_dim_tensor_contiguous (crates/ft-kernel-cpu/src/lib.rs:39443-39550 / 18653)
+template <typename T>
+int32_t argmax_impl(const T *input, size_t input_len, const fth_meta *meta, size_t dim, T *out, size_t out_cap,
+                    size_t *out_len) {
+    FTH_ARG(meta_ok(meta), "argmax: bad meta");
+    if (out_len) *out_len = 0;
+    if (int32_t rc = ensure_unary(input_len, meta)) return rc;
+    if (dim >= (size_t)meta->ndim) return err_invalid_dim(dim, (uint64_t)meta->ndim);
+    const uint64_t reduce = meta->shape[dim];
+    uint64_t outer, inner, total, out_numel;
+    if (int32_t rc = dim_loop_sizes(meta, dim, "argmax overflow", &outer, &inner, &total)) return rc;
+    if (!checked_mul(outer, inner, &out_numel)) return err_overflow("argmax overflow");
+    if (out_numel == 0) return FTH_OK;
+    if (reduce == 0) {
+        set_error(FTH_ERR_EMPTY_REDUCTION_DIM, "argmax over dimension %zu of size zero", dim);
+        fth::last_error().a = dim;
+        return FTH_ERR_EMPTY_REDUCTION_DIM;
+    }
+    if (out_len) *out_len = (size_t)out_numel;
+    if (out == nullptr && out_cap == 0) return FTH_OK;
+    if (int32_t rc = check_out(out, out_cap, (size_t)out_numel)) return rc;
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *dx, *dy;
+    if (int32_t rc = stage_in(sc, input + meta->storage_offset, (size_t)total, &dx)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)out_numel, &dy)) return rc;
+    if (int32_t rc = Dev<T>::argmax(dx, (int64_t)outer, (int64_t)reduce, (int64_t)inner, dy)) return rc;
+    return fetch(out, dy, (size_t)out_numel);
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t fth_matmul_tensor_contiguous_f32(const float *lhs, size_t lhs_len, const float *rhs, size_t rhs_len,
+                                         const fth_meta *lm, const fth_meta *rm, float *out, size_t out_cap, size_t *out_len) {
+    return matmul_impl<float>(lhs, lhs_len, rhs, rhs_len, lm, rm, out, out_cap, out_len);
+}
+int32_t fth_matmul_tensor_contiguous_f64(const double *lhs, size_t lhs_len, const double *rhs, size_t rhs_len,
+                                         const fth_meta *lm, const fth_meta *rm, double *out, size_t out_cap, size_t *out_len) {
+    return matmul_impl<double>(lhs, lhs_len, rhs, rhs_len, lm, rm, out, out_cap, out_len);
+}
+int32_t fth_bmm_tensor_contiguous_f32(const float *lhs, size_t lhs_len, const float *rhs, size_t rhs_len,
+                                      const fth_meta *lm, const fth_meta *rm, float *out, size_t out_cap, size_t *out_len) {
+    return bmm_impl<float>(lhs, lhs_len, rhs, rhs_len, lm, rm, out, out_cap, out_len);
+}
+int32_t fth_bmm_tensor_contiguous_f64(const double *lhs, size_t lhs_len, const double *rhs, size_t rhs_len,
+                                      const fth_meta *lm, const fth_meta *rm, double *out, size_t out_cap, size_t *out_len) {
+    return bmm_impl<double>(lhs, lhs_len, rhs, rhs_len, lm, rm, out, out_cap, out_len);
+}
+int32_t fth_addmm_tensor_contiguous_f32(const float *input, size_t input_len, const float *mat1, size_t mat1_len,
+                                        const float *mat2, size_t mat2_len, const fth_meta *im, const fth_meta *m1,
+                                        const fth_meta *m2, float beta, float alpha, float *out, size_t out_cap, size_t *out_len) {
+    return addmm_impl<float>(input, input_len, mat1, mat1_len, mat2, mat2_len, im, m1, m2, beta, alpha, out, out_cap, out_len);
+}
+int32_t fth_addmm_tensor_contiguous_f64(const double *input, size_t input_len, const double *mat1, size_t mat1_len,
+                                        const double *mat2, size_t mat2_len, const fth_meta *im, const fth_meta *m1,
+                                        const fth_meta *m2, double beta, double alpha, double *out, size_t out_cap, size_t *out_len) {
+    return addmm_impl<double>(input, input_len, mat1, mat1_len, mat2, mat2_len, im, m1, m2, beta, alpha, out, out_cap, out_len);
+}
+int32_t fth_linear_tensor_f32(const float *x, size_t x_len, const float *w, size_t w_len, const float *bias, size_t bias_len,
+                              size_t batch, size_t in_f, size_t out_f, float *out, size_t out_cap, size_t *out_len) {
+    return linear_impl<float>(x, x_len, w, w_len, bias, bias_len, batch, in_f, out_f, out, out_cap, out_len);
+}
+int32_t fth_linear_tensor_f64(const double *x, size_t x_len, const double *w, size_t w_len, const double *bias, size_t bias_len,
+                              size_t batch, size_t in_f, size_t out_f, double *out, size_t out_cap, size_t *out_len) {
+    return linear_impl<double>(x, x_len, w, w_len, bias, bias_len, batch, in_f, out_f, out, out_cap, out_len);
+}
+int32_t fth_matmul_rhs_transposed_contiguous_f32(size_t m, size_t k, size_t n, const float *lhs, size_t lhs_len,
+                                                 const float *rhs, size_t rhs_len, float *out, size_t out_cap, size_t *out_len) {
+    return matmul_bt_impl<float>(m, k, n, lhs, lhs_len, rhs, rhs_len, out, out_cap, out_len);
+}
+int32_t fth_matmul_rhs_transposed_contiguous_f64(size_t m, size_t k, size_t n, const double *lhs, size_t lhs_len,
+                                                 const double *rhs, size_t rhs_len, double *out, size_t out_cap, size_t *out_len) {
+    return matmul_bt_impl<double>(m, k, n, lhs, lhs_len, rhs, rhs_len, out, out_cap, out_len);
+}
+int32_t fth_softmax_dim_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta, size_t dim,
+                                              float *out, size_t out_cap, size_t *out_len) {
+    return softmax_impl<float>(input, input_len, meta, dim, out, out_cap, out_len);
+}
+int32_t fth_softmax_dim_tensor_contiguous_f64(const double *input, size_t input_len, const fth_meta *meta, size_t dim,
+                                              double *out, size_t out_cap, size_t *out_len) {
+    return softmax_impl<double>(input, input_len, meta, dim, out, out_cap, out_len);
+}
+int32_t fth_layer_norm_forward_f32(const float *x, size_t x_len, const float *w, const float *b, size_t batch, size_t n,
+                                   float eps, float *out, size_t out_cap) {
+    return layer_norm_impl<float>(x, nullptr, x_len, w, b, batch, n, eps, out, out_cap);
+}
+int32_t fth_layer_norm_forward_f64(const double *x, size_t x_len, const double *w, const double *b, size_t batch, size_t n,
+                                   double eps, double *out, size_t out_cap) {
+    return layer_norm_impl<double>(x, nullptr, x_len, w, b, batch, n, eps, out, out_cap);
+}
+int32_t fth_add_layer_norm_forward_f32(const float *a, const float *b2, size_t ab_len, const float *w, const float *b,
+                                       size_t batch, size_t n, float eps, float *out, size_t out_cap) {
+    FTH_ARG(a != nullptr && b2 != nullptr, "add_layer_norm: NULL operand");
+    return layer_norm_impl<float>(a, b2, ab_len, w, b, batch, n, eps, out, out_cap);
+}
+int32_t fth_rms_norm_forward_f32(const float *x, size_t x_len, const float *w, size_t batch, size_t n, float eps,
+                                 float *out, size_t out_cap) {
+    return rms_norm_impl<float>(x, x_len, w, batch, n, eps, out, out_cap);
+}
+int32_t fth_rms_norm_forward_f64(const double *x, size_t x_len, const double *w, size_t batch, size_t n, double eps,
+                                 double *out, size_t out_cap) {
+    return rms_norm_impl<double>(x, x_len, w, batch, n, eps, out, out_cap);
+}
+int32_t fth_gelu_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta, float *out,
+                                       size_t out_cap, size_t *out_len) {
+    return gelu_impl<float>(input, input_len, meta, out, out_cap, out_len);
+}
+int32_t fth_gelu_tensor_contiguous_f64(const double *input, size_t input_len, const fth_meta *meta, double *out,
+                                       size_t out_cap, size_t *out_len) {
+    return gelu_impl<double>(input, input_len, meta, out, out_cap, out_len);
+}
+int32_t fth_add_tensor_contiguous_f32(const float *lhs, size_t lhs_len, const float *rhs, size_t rhs_len,
+                                      const fth_meta *lm, const fth_meta *rm, float *out, size_t out_cap, size_t *out_len) {
+    return add_impl<float>(lhs, lhs_len, rhs, rhs_len, lm, rm, out, out_cap, out_len);
+}
+int32_t fth_add_tensor_contiguous_f64(const double *lhs, size_t lhs_len, const double *rhs, size_t rhs_len,
+                                      const fth_meta *lm, const fth_meta *rm, double *out, size_t out_cap, size_t *out_len) {
+    return add_impl<double>(lhs, lhs_len, rhs, rhs_len, lm, rm, out, out_cap, out_len);
+}
+int32_t fth_sdpa_forward_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len,
+                             size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, float scale,
+                             int32_t causal, float *out, size_t out_cap) {
+    return sdpa_impl<float>(q, q_len, k, k_len, v, v_len, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, out, out_cap);
+}
+int32_t fth_sdpa_forward_f64(const double *q, size_t q_len, const double *k, size_t k_len, const double *v, size_t v_len,
+                             size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, double scale,
+                             int32_t causal, double *out, size_t out_cap) {
+    return sdpa_impl<double>(q, q_len, k, k_len, v, v_len, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, out, out_cap);
+}
+int32_t fth_index_select_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta, size_t dim,
+                                               const double *indices, size_t num_indices, float *out, size_t out_cap, size_t *out_len) {
+    return index_select_impl<float>(input, input_len, meta, dim, indices, num_indices, out, out_cap, out_len);
+}
+int32_t fth_index_select_tensor_contiguous_f64(const double *input, size_t input_len, const fth_meta *meta, size_t dim,
+                                               const double *indices, size_t num_indices, double *out, size_t out_cap, size_t *out_len) {
+    return index_select_impl<double>(input, input_len, meta, dim, indices, num_indices, out, out_cap, out_len);
+}
+int32_t fth_argmax_dim_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta, size_t dim,
+                                             float *out, size_t out_cap, size_t *out_len) {
+    return argmax_impl<float>(input, input_len, meta, dim, out, out_cap, out_len);
+}
+int32_t fth_argmax_dim_tensor_contiguous_f64(const double *input, size_t input_len, const fth_meta *meta, size_t dim,
+                                             double *out, size_t out_cap, size_t *out_len) {
+    return argmax_impl<double>(input, input_len, meta, dim, out, out_cap, out_len);
+}
+
+}  // extern "C"

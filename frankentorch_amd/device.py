@@ -1,0 +1,210 @@
+"""Device-pointer tier (fth_dev_*): hipMalloc-backed buffers with explicit copies, streams,
+events, and one thin Python function per kernel. Inputs are already resident in HBM; nothing here
+copies implicitly, and nothing computes on the host.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+
+import numpy as np
+
+from . import _lib
+from .core import check
+
+EPI_NONE, EPI_BIAS, EPI_GELU, EPI_RESIDUAL = 0, 1, 2, 4
+
+
+def is_available() -> bool:
+    """ft_kernel_metal::fused::is_available: True when a gfx950 device can run the kernels."""
+    return bool(_lib.load().fth_is_available())
+
+
+def device_info() -> dict:
+    arch = C.create_string_buffer(64)
+    cus, eclk, mclk, hbm = C.c_int32(), C.c_int32(), C.c_int32(), C.c_uint64()
+    check(_lib.load().fth_device_info(arch, 64, C.byref(cus), C.byref(hbm), C.byref(eclk), C.byref(mclk)))
+    return {"arch": arch.value.decode(), "compute_units": cus.value, "hbm_bytes": hbm.value,
+            "engine_clock_khz": eclk.value, "memory_clock_khz": mclk.value}
+
+
+class DeviceBuffer:
+    """A typed, hipMalloc-backed array. Copies are explicit: `from_host`, `to_host`."""
+
+    def __init__(self, shape, dtype=np.float32):
+        self.shape = tuple(int(s) for s in (shape if hasattr(shape, "__len__") else (shape,)))
+        self.dtype = np.dtype(dtype)
+        self.size = int(np.prod(self.shape, dtype=np.int64))
+        self.nbytes = self.size * self.dtype.itemsize
+        p = C.c_void_p()
+        check(_lib.load().fth_malloc(C.byref(p), self.nbytes))
+        self.ptr = p.value or 0
+        self._owned = True
+
+    @classmethod
+    def from_host(cls, array) -> "DeviceBuffer":
+        array = np.ascontiguousarray(array)
+        buf = cls(array.shape, array.dtype)
+        if buf.nbytes:
+            check(_lib.load().fth_memcpy_h2d(buf.ptr, array.ctypes.data, buf.nbytes))
+        return buf
+
+    def to_host(self) -> np.ndarray:
+        out = np.empty(self.shape, dtype=self.dtype)
+        if self.nbytes:
+            check(_lib.load().fth_memcpy_d2h(out.ctypes.data, self.ptr, self.nbytes))
+        return out
+
+    def view(self, offset_elems: int) -> int:
+        """Device address of element `offset_elems`."""
+        return self.ptr + offset_elems * self.dtype.itemsize
+
+    def free(self) -> None:
+        if self._owned and self.ptr:
+            _lib.load().fth_free(self.ptr)
+        self.ptr = 0
+        self._owned = False
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def synchronize() -> None:
+    check(_lib.load().fth_device_synchronize())
+
+
+class Event:
+    def __init__(self):
+        e = C.c_void_p()
+        check(_lib.load().fth_event_create(C.byref(e)))
+        self.handle = e.value
+
+    def record(self, stream=None) -> None:
+        check(_lib.load().fth_event_record(self.handle, stream))
+
+    def synchronize(self) -> None:
+        check(_lib.load().fth_event_synchronize(self.handle))
+
+    def elapsed_ms(self, stop: "Event") -> float:
+        ms = C.c_float()
+        check(_lib.load().fth_event_elapsed_ms(self.handle, stop.handle, C.byref(ms)))
+        return ms.value
+
+    def __del__(self):
+        try:
+            _lib.load().fth_event_destroy(self.handle)
+        except Exception:
+            pass
+
+
+def _sfx(buf: DeviceBuffer) -> str:
+    if buf.dtype == np.float32:
+        return "f32"
+    if buf.dtype == np.float64:
+        return "f64"
+    raise TypeError("kernels compute f32 and f64 only, got %s" % buf.dtype)
+
+
+def _ptr(buf):
+    return None if buf is None else (buf.ptr if isinstance(buf, DeviceBuffer) else int(buf))
+
+
+def _real(buf, v):
+    return C.c_float(v) if buf.dtype == np.float32 else C.c_double(v)
+
+
+def softmax_lastdim(x, y, rows, cols, stream=None):
+    check(getattr(_lib.load(), "fth_dev_softmax_lastdim_" + _sfx(x))(_ptr(x), _ptr(y), rows, cols, stream))
+
+
+def softmax_strided(x, y, outer, reduce, inner, stream=None):
+    check(getattr(_lib.load(), "fth_dev_softmax_strided_" + _sfx(x))(_ptr(x), _ptr(y), outer, reduce, inner, stream))
+
+
+def layer_norm(x, weight, bias, y, batch, norm_size, eps, stream=None):
+    check(getattr(_lib.load(), "fth_dev_layer_norm_" + _sfx(x))(_ptr(x), _ptr(weight), _ptr(bias), _ptr(y), batch,
+                                                                norm_size, _real(x, eps), stream))
+
+
+def add_layer_norm(a, b, weight, bias, y, batch, norm_size, eps, stream=None):
+    check(_lib.load().fth_dev_add_layer_norm_f32(_ptr(a), _ptr(b), _ptr(weight), _ptr(bias), _ptr(y), batch, norm_size,
+                                                 C.c_float(eps), stream))
+
+
+def rms_norm(x, weight, y, batch, norm_size, eps, stream=None):
+    check(getattr(_lib.load(), "fth_dev_rms_norm_" + _sfx(x))(_ptr(x), _ptr(weight), _ptr(y), batch, norm_size,
+                                                              _real(x, eps), stream))
+
+
+def gelu(x, y, n, stream=None):
+    check(getattr(_lib.load(), "fth_dev_gelu_" + _sfx(x))(_ptr(x), _ptr(y), n, stream))
+
+
+def add(a, b, y, n, stream=None):
+    check(getattr(_lib.load(), "fth_dev_add_" + _sfx(a))(_ptr(a), _ptr(b), _ptr(y), n, stream))
+
+
+def bias_add(x, bias, y, rows, cols, stream=None):
+    check(getattr(_lib.load(), "fth_dev_bias_add_" + _sfx(x))(_ptr(x), _ptr(bias), _ptr(y), rows, cols, stream))
+
+
+def bias_residual_add(x, bias, residual, y, rows, cols, stream=None):
+    check(_lib.load().fth_dev_bias_residual_add_f32(_ptr(x), _ptr(bias), _ptr(residual), _ptr(y), rows, cols, stream))
+
+
+def index_select(inp, outer, dim_size, inner, indices, num_indices, out, bad_index=None, stream=None):
+    check(getattr(_lib.load(), "fth_dev_index_select_" + _sfx(inp))(_ptr(inp), outer, dim_size, inner, _ptr(indices),
+                                                                    num_indices, _ptr(out), _ptr(bad_index), stream))
+
+
+def embedding_add(wte, vocab, wpe, max_pos, ids, tokens, seq, width, out, bad_index=None, stream=None):
+    check(_lib.load().fth_dev_embedding_add_f32(_ptr(wte), vocab, _ptr(wpe), max_pos, _ptr(ids), tokens, seq, width,
+                                                _ptr(out), _ptr(bad_index), stream))
+
+
+def argmax(x, outer, reduce, inner, out, stream=None):
+    check(getattr(_lib.load(), "fth_dev_argmax_" + _sfx(x))(_ptr(x), outer, reduce, inner, _ptr(out), stream))
+
+
+def permute_0213(src, dst, d0, d1, d2, d3, stream=None):
+    check(getattr(_lib.load(), "fth_dev_permute_0213_" + _sfx(src))(_ptr(src), _ptr(dst), d0, d1, d2, d3, stream))
+
+
+def gemm_desc(m, n, k, trans_b=False, batch=1, epilogue=EPI_NONE, lda=None, ldb=None, ldc=None, stride_a=None,
+              stride_b=None, stride_c=None) -> _lib.GemmDesc:
+    d = _lib.GemmDesc()
+    d.m, d.n, d.k = m, n, k
+    d.lda = k if lda is None else lda
+    d.ldb = (k if trans_b else n) if ldb is None else ldb
+    d.ldc = n if ldc is None else ldc
+    d.batch = batch
+    d.stride_a = m * k if stride_a is None else stride_a
+    d.stride_b = k * n if stride_b is None else stride_b
+    d.stride_c = m * n if stride_c is None else stride_c
+    d.trans_b = 1 if trans_b else 0
+    d.epilogue = epilogue
+    return d
+
+
+def gemm(desc, a, b, c, bias=None, residual=None, alpha=1.0, stream=None):
+    """C = alpha * A . op(B) (+ bias, GELU, residual per desc.epilogue)."""
+    check(getattr(_lib.load(), "fth_dev_gemm_" + _sfx(a))(C.byref(desc), _real(a, alpha), _ptr(a), _ptr(b), _ptr(c),
+                                                          _ptr(bias), _ptr(residual), stream))
+
+
+def sdpa_desc_contiguous(num_bh, seq_q, seq_k, d_k, d_v, causal) -> _lib.SdpaDesc:
+    d = _lib.SdpaDesc()
+    _lib.load().fth_sdpa_desc_contiguous(C.byref(d), num_bh, seq_q, seq_k, d_k, d_v, 1 if causal else 0)
+    return d
+
+
+def sdpa_forward(desc, scale, q, k, v, out, stream=None):
+    check(getattr(_lib.load(), "fth_dev_sdpa_forward_" + _sfx(q))(C.byref(desc), _real(q, scale), _ptr(q), _ptr(k),
+                                                                  _ptr(v), _ptr(out), stream))
+
+
+def default_scale(head_dim: int) -> float:
+    return 1.0 / math.sqrt(head_dim)

@@ -1,0 +1,224 @@
+"""`ft_kernel_hip`: the operator entry points of `ft_kernel_cpu`, same names, same argument
+meaning, same errors -- host arrays in, a freshly allocated host array out -- computed on the
+MI355X through the host-slice tier of the C ABI.
+
+The reference's signatures take `&[T]` slices plus `&TensorMeta`; here a slice is a 1-D
+C-contiguous numpy array (f32 or f64) and the meta is `core.TensorMeta`. Fallible entry points
+raise `core.KernelError` with the reference's variant; the fused entry points that the reference
+leaves infallible (and that panic on short slices) raise `core.HipError(InvalidArgument)`.
+
+Reference lines (crates/ft-kernel-cpu/src/lib.rs): matmul :37752 / :17355, bmm :38496 / :17785,
+addmm :41562 / :17514, linear :17306 / :17162, matmul_rhs_transposed :17408 / :17381,
+softmax_dim :39193 / :18350, layer_norm_forward :5877 / :5824, add_layer_norm_forward :5932,
+rms_norm_forward :6459 / :6418, gelu :37123, add :36870, sdpa_forward :5200 / :4572,
+index_select :40216, argmax_dim :39443 / :18653.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from .core import TensorMeta, check
+
+
+def _slice(a, dtype):
+    a = np.ascontiguousarray(a, dtype=dtype)
+    return a.reshape(-1)
+
+
+def _opt(a, dtype):
+    return None if a is None else _slice(a, dtype)
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data
+
+
+def _call_sized(fn, dtype, *args_before_out):
+    """Two-step call: validate and size (out == NULL), then run into an exact-size array."""
+    out_len = C.c_size_t(0)
+    check(fn(*args_before_out, None, 0, C.byref(out_len)))
+    out = np.empty(out_len.value, dtype=dtype)
+    if out_len.value:
+        check(fn(*args_before_out, out.ctypes.data, out.size, C.byref(out_len)))
+    return out
+
+
+def _binary(name, dtype, lhs, rhs, lhs_meta: TensorMeta, rhs_meta: TensorMeta):
+    lhs, rhs = _slice(lhs, dtype), _slice(rhs, dtype)
+    lm, rm = lhs_meta.to_c(), rhs_meta.to_c()
+    return _call_sized(getattr(_lib.load(), name), dtype, _p(lhs), lhs.size, _p(rhs), rhs.size, C.byref(lm), C.byref(rm))
+
+
+def matmul_tensor_contiguous_f32(lhs, rhs, lhs_meta, rhs_meta):
+    return _binary("fth_matmul_tensor_contiguous_f32", np.float32, lhs, rhs, lhs_meta, rhs_meta)
+
+
+def matmul_tensor_contiguous_f64(lhs, rhs, lhs_meta, rhs_meta):
+    return _binary("fth_matmul_tensor_contiguous_f64", np.float64, lhs, rhs, lhs_meta, rhs_meta)
+
+
+def bmm_tensor_contiguous_f32(lhs, rhs, lhs_meta, rhs_meta):
+    return _binary("fth_bmm_tensor_contiguous_f32", np.float32, lhs, rhs, lhs_meta, rhs_meta)
+
+
+def bmm_tensor_contiguous_f64(lhs, rhs, lhs_meta, rhs_meta):
+    return _binary("fth_bmm_tensor_contiguous_f64", np.float64, lhs, rhs, lhs_meta, rhs_meta)
+
+
+def add_tensor_contiguous_f32(lhs, rhs, lhs_meta, rhs_meta):
+    return _binary("fth_add_tensor_contiguous_f32", np.float32, lhs, rhs, lhs_meta, rhs_meta)
+
+
+def add_tensor_contiguous_f64(lhs, rhs, lhs_meta, rhs_meta):
+    return _binary("fth_add_tensor_contiguous_f64", np.float64, lhs, rhs, lhs_meta, rhs_meta)
+
+
+def _addmm(name, dtype, ctype, inp, mat1, mat2, input_meta, mat1_meta, mat2_meta, beta, alpha):
+    inp, mat1, mat2 = _slice(inp, dtype), _slice(mat1, dtype), _slice(mat2, dtype)
+    im, m1, m2 = input_meta.to_c(), mat1_meta.to_c(), mat2_meta.to_c()
+    return _call_sized(getattr(_lib.load(), name), dtype, _p(inp), inp.size, _p(mat1), mat1.size, _p(mat2), mat2.size,
+                       C.byref(im), C.byref(m1), C.byref(m2), ctype(beta), ctype(alpha))
+
+
+def addmm_tensor_contiguous_f32(inp, mat1, mat2, input_meta, mat1_meta, mat2_meta, beta, alpha):
+    return _addmm("fth_addmm_tensor_contiguous_f32", np.float32, C.c_float, inp, mat1, mat2, input_meta, mat1_meta,
+                  mat2_meta, beta, alpha)
+
+
+def addmm_tensor_contiguous_f64(inp, mat1, mat2, input_meta, mat1_meta, mat2_meta, beta, alpha):
+    return _addmm("fth_addmm_tensor_contiguous_f64", np.float64, C.c_double, inp, mat1, mat2, input_meta, mat1_meta,
+                  mat2_meta, beta, alpha)
+
+
+def _linear(name, dtype, x, weight, bias, batch, in_features, out_features):
+    x, weight, bias = _slice(x, dtype), _slice(weight, dtype), _opt(bias, dtype)
+    return _call_sized(getattr(_lib.load(), name), dtype, _p(x), x.size, _p(weight), weight.size, _p(bias),
+                       0 if bias is None else bias.size, batch, in_features, out_features)
+
+
+def linear_tensor_f32(x, weight, bias, batch, in_features, out_features):
+    return _linear("fth_linear_tensor_f32", np.float32, x, weight, bias, batch, in_features, out_features)
+
+
+def linear_tensor_f64(x, weight, bias, batch, in_features, out_features):
+    return _linear("fth_linear_tensor_f64", np.float64, x, weight, bias, batch, in_features, out_features)
+
+
+def _matmul_bt(name, dtype, m, k, n, lhs, rhs_nk):
+    lhs, rhs_nk = _slice(lhs, dtype), _slice(rhs_nk, dtype)
+    return _call_sized(getattr(_lib.load(), name), dtype, m, k, n, _p(lhs), lhs.size, _p(rhs_nk), rhs_nk.size)
+
+
+def matmul_rhs_transposed_contiguous_f32(m, k, n, lhs, rhs_nk):
+    return _matmul_bt("fth_matmul_rhs_transposed_contiguous_f32", np.float32, m, k, n, lhs, rhs_nk)
+
+
+def matmul_rhs_transposed_contiguous_f64(m, k, n, lhs, rhs_nk):
+    return _matmul_bt("fth_matmul_rhs_transposed_contiguous_f64", np.float64, m, k, n, lhs, rhs_nk)
+
+
+def _unary_dim(name, dtype, inp, meta: TensorMeta, dim):
+    inp = _slice(inp, dtype)
+    m = meta.to_c()
+    return _call_sized(getattr(_lib.load(), name), dtype, _p(inp), inp.size, C.byref(m), dim)
+
+
+def softmax_dim_tensor_contiguous_f32(inp, meta, dim):
+    return _unary_dim("fth_softmax_dim_tensor_contiguous_f32", np.float32, inp, meta, dim)
+
+
+def softmax_dim_tensor_contiguous_f64(inp, meta, dim):
+    return _unary_dim("fth_softmax_dim_tensor_contiguous_f64", np.float64, inp, meta, dim)
+
+
+def argmax_dim_tensor_contiguous_f32(inp, meta, dim):
+    return _unary_dim("fth_argmax_dim_tensor_contiguous_f32", np.float32, inp, meta, dim)
+
+
+def argmax_dim_tensor_contiguous_f64(inp, meta, dim):
+    return _unary_dim("fth_argmax_dim_tensor_contiguous_f64", np.float64, inp, meta, dim)
+
+
+def _gelu(name, dtype, inp, meta: TensorMeta):
+    inp = _slice(inp, dtype)
+    m = meta.to_c()
+    return _call_sized(getattr(_lib.load(), name), dtype, _p(inp), inp.size, C.byref(m))
+
+
+def gelu_tensor_contiguous_f32(inp, meta):
+    return _gelu("fth_gelu_tensor_contiguous_f32", np.float32, inp, meta)
+
+
+def gelu_tensor_contiguous_f64(inp, meta):
+    return _gelu("fth_gelu_tensor_contiguous_f64", np.float64, inp, meta)
+
+
+def _index_select(name, dtype, inp, meta: TensorMeta, dim, indices):
+    inp = _slice(inp, dtype)
+    idx = _slice(indices, np.float64)
+    m = meta.to_c()
+    return _call_sized(getattr(_lib.load(), name), dtype, _p(inp), inp.size, C.byref(m), dim, _p(idx), idx.size)
+
+
+def index_select_tensor_contiguous_f32(inp, meta, dim, indices):
+    return _index_select("fth_index_select_tensor_contiguous_f32", np.float32, inp, meta, dim, indices)
+
+
+def index_select_tensor_contiguous_f64(inp, meta, dim, indices):
+    return _index_select("fth_index_select_tensor_contiguous_f64", np.float64, inp, meta, dim, indices)
+
+
+def layer_norm_forward_f32(x, weight, bias, batch, norm_size, eps):
+    x, weight, bias = _slice(x, np.float32), _opt(weight, np.float32), _opt(bias, np.float32)
+    out = np.empty(batch * norm_size, dtype=np.float32)
+    check(_lib.load().fth_layer_norm_forward_f32(_p(x), x.size, _p(weight), _p(bias), batch, norm_size, eps, _p(out), out.size))
+    return out
+
+
+def layer_norm_forward_f64(x, weight, bias, batch, norm_size, eps):
+    x, weight, bias = _slice(x, np.float64), _opt(weight, np.float64), _opt(bias, np.float64)
+    out = np.empty(batch * norm_size, dtype=np.float64)
+    check(_lib.load().fth_layer_norm_forward_f64(_p(x), x.size, _p(weight), _p(bias), batch, norm_size, eps, _p(out), out.size))
+    return out
+
+
+def add_layer_norm_forward_f32(a, b, weight, bias, batch, norm_size, eps):
+    a, b = _slice(a, np.float32), _slice(b, np.float32)
+    weight, bias = _opt(weight, np.float32), _opt(bias, np.float32)
+    out = np.empty(batch * norm_size, dtype=np.float32)
+    check(_lib.load().fth_add_layer_norm_forward_f32(_p(a), _p(b), min(a.size, b.size), _p(weight), _p(bias), batch,
+                                                     norm_size, eps, _p(out), out.size))
+    return out
+
+
+def rms_norm_forward_f32(x, weight, batch, norm_size, eps):
+    x, weight = _slice(x, np.float32), _opt(weight, np.float32)
+    out = np.empty(batch * norm_size, dtype=np.float32)
+    check(_lib.load().fth_rms_norm_forward_f32(_p(x), x.size, _p(weight), batch, norm_size, eps, _p(out), out.size))
+    return out
+
+
+def rms_norm_forward_f64(x, weight, batch, norm_size, eps):
+    x, weight = _slice(x, np.float64), _opt(weight, np.float64)
+    out = np.empty(batch * norm_size, dtype=np.float64)
+    check(_lib.load().fth_rms_norm_forward_f64(_p(x), x.size, _p(weight), batch, norm_size, eps, _p(out), out.size))
+    return out
+
+
+def _sdpa(name, dtype, q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal):
+    q, k, v = _slice(q, dtype), _slice(k, dtype), _slice(v, dtype)
+    out = np.empty(num_bh * seq_q * d_v, dtype=dtype)
+    check(getattr(_lib.load(), name)(_p(q), q.size, _p(k), k.size, _p(v), v.size, num_bh, seq_q, seq_k, d_k, d_v, scale,
+                                     1 if causal else 0, _p(out), out.size))
+    return out
+
+
+def sdpa_forward_f32(q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal):
+    return _sdpa("fth_sdpa_forward_f32", np.float32, q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal)
+
+
+def sdpa_forward_f64(q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal):
+    return _sdpa("fth_sdpa_forward_f64", np.float64, q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal)

@@ -429,6 +429,11 @@ int32_t fth_gpt2_forward_dev(fth_gpt2 *g, const double *ids_dev, int64_t batch, 
                              float *logits_dev, float *argmax_dev, fth_stream s);
 /* Final hidden state [batch*seq, d_model] of the last forward (device pointer, valid until the next). */
 const float *fth_gpt2_hidden_dev(const fth_gpt2 *g);
+/* Position of the first token id of the last forward that failed normalize_strict_index_value
+ * (crates/ft-kernel-cpu/src/lib.rs:20058-20090), or -1. Synchronises. The reference returns
+ * InvalidDimension for such an id; here the affected rows of the embedding are left unwritten and
+ * the caller checks this after the forward. */
+int32_t fth_gpt2_bad_index(const fth_gpt2 *g, int64_t *position);
 
 #ifdef __cplusplus
 }

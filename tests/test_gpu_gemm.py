@@ -1,0 +1,164 @@
+"""fp32 / fp64 MFMA GEMM against the wide-accumulation CPU checker.
+fp32: max|d| / max|ref| <= 2e-5; fp64: <= 1e-12."""
+import numpy as np
+import pytest
+
+from conftest import TOL_F64, TOL_GEMM_F32, rel_err
+from frankentorch_amd import synth
+from frankentorch_amd.device import EPI_BIAS, EPI_GELU, EPI_RESIDUAL, DeviceBuffer
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(hip, a, b, trans_b, bias=None, residual=None, epilogue=0, alpha=1.0):
+    m, k = a.shape
+    n = b.shape[0] if trans_b else b.shape[1]
+    da, db = DeviceBuffer.from_host(a), DeviceBuffer.from_host(b)
+    dc = DeviceBuffer((m, n), a.dtype)
+    dbias = None if bias is None else DeviceBuffer.from_host(bias)
+    dres = None if residual is None else DeviceBuffer.from_host(residual)
+    hip.gemm(hip.gemm_desc(m, n, k, trans_b=trans_b, epilogue=epilogue), da, db, dc, dbias, dres, alpha)
+    return dc.to_host()
+
+
+# full tiles, ragged edges in every dimension, k not a multiple of the vector width, tiny, skinny
+SHAPES = [(128, 128, 64), (256, 384, 128), (200, 300, 100), (77, 50, 33), (1, 1, 1), (5, 1000, 7), (1000, 5, 7), (130, 130, 513),
+          (64, 64, 4096), (512, 768, 256), (3, 129, 2)]
+
+
+@pytest.mark.parametrize("m,n,k", SHAPES)
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_gemm_matches_oracle(hip, oracle, m, n, k, trans_b, dtype):
+    tol = TOL_GEMM_F32 if dtype == np.float32 else TOL_F64
+    a = synth.uniform(2, "a", (m, k), -1, 1, dtype=dtype)
+    b = synth.uniform(2, "b", (n, k) if trans_b else (k, n), -1, 1, dtype=dtype)
+    got = _run(hip, a, b, trans_b)
+    assert rel_err(got, oracle.gemm(a, b, trans_b)) <= tol
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_epilogues_keep_their_own_roundings(hip, oracle, dtype):
+    """bias, GELU and residual applied in the epilogue equal the separate ops applied to the
+    GEMM's own rounded output, bit for bit."""
+    tol = TOL_GEMM_F32 if dtype == np.float32 else TOL_F64
+    m, n, k = 150, 200, 96
+    a = synth.uniform(2, "a", (m, k), -1, 1, dtype=dtype)
+    w = synth.uniform(2, "w", (n, k), -1, 1, dtype=dtype)
+    bias = synth.normal(2, "bias", (n,), dtype=dtype)
+    res = synth.normal(2, "res", (m, n), dtype=dtype)
+    plain = _run(hip, a, w, True)
+    got = _run(hip, a, w, True, bias, None, EPI_BIAS)
+    assert np.array_equal(got, plain + bias)
+    assert rel_err(got, oracle.linear(a, w, bias)) <= tol
+    got = _run(hip, a, w, True, bias, res, EPI_BIAS | EPI_RESIDUAL)
+    assert np.array_equal(got, (plain + bias) + res)
+    got = _run(hip, a, w, True, bias, None, EPI_BIAS | EPI_GELU)
+    assert rel_err(got, oracle.gelu(oracle.linear(a, w, bias))) <= tol
+    got = _run(hip, a, w, True, None, None, 0, alpha=0.5)
+    assert np.array_equal(got, dtype(0.5) * plain)
+
+
+def test_degenerate_extents(hip):
+    a = np.ones((4, 0), np.float32)
+    b = np.ones((0, 6), np.float32)
+    bias = np.arange(6, dtype=np.float32)
+    da, db, dbias = DeviceBuffer((1,)), DeviceBuffer((1,)), DeviceBuffer.from_host(bias)
+    dc = DeviceBuffer.from_host(np.full((4, 6), 7.0, np.float32))
+    hip.gemm(hip.gemm_desc(4, 6, 0), da, db, dc)           # k == 0: zeros (overwrite, beta = 0)
+    assert np.all(dc.to_host() == 0.0)
+    hip.gemm(hip.gemm_desc(4, 6, 0, epilogue=EPI_BIAS), da, db, dc, dbias)
+    assert np.array_equal(dc.to_host(), np.tile(bias, (4, 1)))
+    dc = DeviceBuffer.from_host(np.full((4, 6), 7.0, np.float32))
+    hip.gemm(hip.gemm_desc(0, 6, 3), da, db, dc)           # m == 0: returns at once, C untouched
+    hip.gemm(hip.gemm_desc(4, 0, 3), da, db, dc)
+    assert np.all(dc.to_host() == 7.0)
+
+
+def test_batched_and_strided(hip, oracle):
+    """Config 3 batched case [32,512,128] @ [32,128,512], plus a shared (stride 0) right operand."""
+    a = synth.uniform(2, "ba", (32, 512, 128), -1, 1)
+    b = synth.uniform(2, "bb", (32, 128, 512), -1, 1)
+    da, db = DeviceBuffer.from_host(a), DeviceBuffer.from_host(b)
+    dc = DeviceBuffer((32, 512, 512))
+    hip.gemm(hip.gemm_desc(512, 512, 128, batch=32), da, db, dc)
+    got = dc.to_host()
+    assert rel_err(got, oracle.bmm(a, b)) <= TOL_GEMM_F32
+    hip.gemm(hip.gemm_desc(512, 512, 128, batch=32, stride_b=0), da, db, dc)
+    assert rel_err(dc.to_host()[5], oracle.gemm(a[5], b[0])) <= TOL_GEMM_F32
+    # row pitches larger than the rows: operate on a sub-block of larger buffers
+    big_a = synth.uniform(2, "pa", (70, 200), -1, 1)
+    big_b = synth.uniform(2, "pb", (90, 150), -1, 1)
+    dA, dB = DeviceBuffer.from_host(big_a), DeviceBuffer.from_host(big_b)
+    dC = DeviceBuffer.from_host(np.zeros((70, 130), np.float32))
+    hip.gemm(hip.gemm_desc(60, 100, 80, lda=200, ldb=150, ldc=130), dA.view(3), dB.view(7), dC.view(5))
+    ref = oracle.gemm(np.ascontiguousarray(big_a.ravel()[3:].reshape(-1)[: 60 * 200].reshape(60, 200)[:, :80]),
+                      np.ascontiguousarray(big_b.ravel()[7:][: 80 * 150].reshape(80, 150)[:, :100]))
+    got = dC.to_host().ravel()[5:][: 60 * 130].reshape(60, 130)[:, :100]
+    assert rel_err(got, ref) <= TOL_GEMM_F32
+
+
+def test_reference_f64_checksums_on_the_gpu(hip, vectors):
+    """The reference's stored sums of its own dgemm outputs (sin/cos inputs), 12 decimals."""
+    for s in vectors["golden_text"]["gemm_f64_checksums"]["sums"]:
+        m, k, n = s["m"], s["k"], s["n"]
+        a = np.sin(np.arange(m * k, dtype=np.float64) * 0.001).reshape(m, k)
+        b = np.cos(np.arange(n * k, dtype=np.float64) * 0.0017).reshape((n, k) if s["bt"] else (k, n))
+        got = _run(hip, a, b, bool(s["bt"]))
+        total = float(np.sum(got.ravel().tolist()))
+        assert abs(total - s["sum"]) <= 5e-11 * max(1.0, abs(s["sum"])), (s, total)
+
+
+def test_known_answers_and_precision_contract(hip, vectors):
+    by = {c["name"]: c for c in vectors["in_source"]}
+    c = by["matmul_tensor_contiguous_returns_expected_values"]
+    for dt in (np.float32, np.float64):
+        a = np.array(c["lhs"], dt).reshape(c["lhs_shape"])
+        b = np.array(c["rhs"], dt).reshape(c["rhs_shape"])
+        assert _run(hip, a, b, False).ravel().tolist() == [float(v) for v in c["expected_output"]]
+    c = by["matmul_unit_vector_dot_k10001"]
+    r = 1.0 / np.sqrt(c["k"])
+    got = _run(hip, np.full((1, c["k"]), r), np.full((c["k"], 1), r), False)
+    assert abs(got[0, 0] - 1.0) < 1e-13
+
+
+def test_config3_shapes_sampled_rows_and_determinism(hip, oracle):
+    """4096^3, [4096,4096]@[4096,11008]+bias in fp32 and 4096^3 in fp64: the product is checked on
+    a stride of rows against the wide-accumulation truth; the whole output is compared bitwise
+    between two runs; linearity (A.(B1+B2) vs A.B1 + A.B2) is checked without the oracle."""
+    a = synth.uniform(2, "A", (4096, 4096), -1, 1)
+    b = synth.uniform(2, "B", (4096, 4096), -1, 1)
+    da, db = DeviceBuffer.from_host(a), DeviceBuffer.from_host(b)
+    dc, dc2 = DeviceBuffer((4096, 4096)), DeviceBuffer((4096, 4096))
+    rows = np.arange(5, 4096, 127)
+    for trans_b in (False, True):
+        d = hip.gemm_desc(4096, 4096, 4096, trans_b=trans_b)
+        hip.gemm(d, da, db, dc)
+        hip.gemm(d, da, db, dc2)
+        c = dc.to_host()
+        assert np.array_equal(c.view(np.uint32), dc2.to_host().view(np.uint32))
+        assert rel_err(c[rows], oracle.gemm(a[rows], b, trans_b)) <= TOL_GEMM_F32
+    # rectangular with bias
+    b2 = synth.uniform(2, "B2", (4096, 11008), -1, 1)
+    bias = synth.uniform(2, "bias2", (11008,), -1, 1)
+    db2, dbias = DeviceBuffer.from_host(b2), DeviceBuffer.from_host(bias)
+    dr = DeviceBuffer((4096, 11008))
+    hip.gemm(hip.gemm_desc(4096, 11008, 4096, epilogue=EPI_BIAS), da, db2, dr, dbias)
+    c = dr.to_host()
+    assert rel_err(c[rows], oracle.gemm(a[rows], b2) + bias) <= TOL_GEMM_F32
+    del dr, db2, c
+    # fp64 square
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    da64, db64 = DeviceBuffer.from_host(a64), DeviceBuffer.from_host(b64)
+    dc64 = DeviceBuffer((4096, 4096), np.float64)
+    hip.gemm(hip.gemm_desc(4096, 4096, 4096), da64, db64, dc64)
+    c64 = dc64.to_host()
+    r64 = rows[::4]
+    assert rel_err(c64[r64], oracle.gemm(a64[r64], b64)) <= TOL_F64
+    # linearity in B, fp64, no oracle: A.(B + B^T-ish perturbation) == A.B + A.P within rounding
+    p = np.roll(b64, 17, axis=1)
+    dp, dsum = DeviceBuffer.from_host(p), DeviceBuffer.from_host(b64 + p)
+    dcp, dcs = DeviceBuffer((4096, 4096), np.float64), DeviceBuffer((4096, 4096), np.float64)
+    hip.gemm(hip.gemm_desc(4096, 4096, 4096), da64, dp, dcp)
+    hip.gemm(hip.gemm_desc(4096, 4096, 4096), da64, dsum, dcs)
+    assert rel_err(dcs.to_host(), c64 + dcp.to_host()) <= 1e-12

@@ -1,0 +1,107 @@
+"""Integer-exact kernels: argmax, index_select / embedding gather, head split-merge permute.
+Bit-exact against the CPU checker."""
+import numpy as np
+import pytest
+
+from frankentorch_amd import synth
+from frankentorch_amd.device import DeviceBuffer
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_argmax_semantics_ties_nan_and_all_neg_inf(hip, oracle, dtype):
+    x = synth.normal(7, "am", (41, 50257)).astype(dtype)
+    x[3, 100] = np.nan
+    x[3, 40000] = np.nan          # the FIRST NaN wins
+    x[4, :] = -np.inf             # nothing is > -inf: index 0
+    x[5, 9000] = x[5, 7] = x[5].max() + 1  # tie: the first index wins
+    x[6, 50256] = 1e9             # last element
+    x[7, 0] = 1e9
+    x[8, 12] = np.inf
+    x[9, 5] = np.nan
+    x[9, 4] = np.inf              # a NaN beats +inf even when it comes later
+    dx = DeviceBuffer.from_host(x)
+    dy = DeviceBuffer((41,), dtype)
+    hip.argmax(dx, 41, 50257, 1, dy)
+    got = dy.to_host()
+    assert np.array_equal(got, oracle.argmax(x, 1))
+    assert got[3] == 100 and got[4] == 0 and got[5] == 7 and got[6] == 50256 and got[7] == 0 and got[8] == 12 and got[9] == 5
+
+
+@pytest.mark.parametrize("shape,dim", [((5, 17, 9), 1), ((64, 3), 0), ((2, 300, 4), 1), ((1, 7), 1), ((3, 1, 5), 1)])
+def test_argmax_any_dim(hip, oracle, shape, dim):
+    x = np.round(synth.normal(8, "am2", shape) * 2)  # many ties
+    x.ravel()[::13] = np.nan
+    outer = int(np.prod(shape[:dim], dtype=np.int64))
+    inner = int(np.prod(shape[dim + 1:], dtype=np.int64))
+    dx = DeviceBuffer.from_host(x)
+    dy = DeviceBuffer((outer * inner,))
+    hip.argmax(dx, outer, shape[dim], inner, dy)
+    assert np.array_equal(dy.to_host().reshape(oracle.argmax(x, dim).shape), oracle.argmax(x, dim))
+
+
+def test_argmax_empty_reduce_dim_is_an_error(hip):
+    from frankentorch_amd.core import KernelError
+
+    dx = DeviceBuffer((4,))
+    with pytest.raises(KernelError) as ei:
+        hip.argmax(dx, 3, 0, 1, dx)
+    assert ei.value.kind == "EmptyReductionDim"
+    hip.argmax(dx, 0, 0, 1, dx)  # empty output: nothing to do, as in the reference
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_index_select_rows_and_general(hip, oracle, dtype):
+    table = synth.normal(9, "tab", (1000, 768)).astype(dtype)
+    ids = synth.token_ids(9, "ids", (513,), 1000)
+    dt, di = DeviceBuffer.from_host(table), DeviceBuffer.from_host(ids)
+    do = DeviceBuffer((513, 768), dtype)
+    bad = DeviceBuffer((1,), np.int64)
+    hip.index_select(dt, 1, 1000, 768, di, 513, do, bad)
+    ref, rbad = oracle.index_select(table, 0, ids)
+    assert rbad == -1 and bad.to_host()[0] == -1
+    assert np.array_equal(do.to_host(), ref)
+    # middle dim, odd inner (scalar copy path)
+    t3 = synth.normal(9, "t3", (4, 11, 7)).astype(dtype)
+    idx = np.array([10.0, 0.0, 3.0, 3.0])
+    d3, di3 = DeviceBuffer.from_host(t3), DeviceBuffer.from_host(idx)
+    o3 = DeviceBuffer((4, 4, 7), dtype)
+    hip.index_select(d3, 4, 11, 7, di3, 4, o3, bad)
+    assert np.array_equal(o3.to_host(), oracle.index_select(t3, 1, idx)[0])
+
+
+def test_index_select_reports_first_invalid_index(hip, oracle):
+    table = synth.normal(9, "tab", (10, 8))
+    dt = DeviceBuffer.from_host(table)
+    bad = DeviceBuffer((1,), np.int64)
+    for idx, want in (([1.0, 2.5, 3.0], 1), ([1.0, 2.0, 10.0], 2), ([-1.0, 99.0], 0), ([np.nan], 0), ([1e300], 0), ([np.inf], 0)):
+        sentinel = np.full((len(idx), 8), 123.0, np.float32)
+        do = DeviceBuffer.from_host(sentinel)
+        di = DeviceBuffer.from_host(np.array(idx))
+        hip.index_select(dt, 1, 10, 8, di, len(idx), do, bad)
+        assert bad.to_host()[0] == want == oracle.index_select(table, 0, idx)[1]
+        out = do.to_host()
+        assert np.all(out[want] == 123.0)  # rows with an invalid index are left untouched
+
+
+def test_embedding_add_and_permute(hip, oracle):
+    vocab, maxpos, d, batch, seq = 777, 40, 768, 3, 32
+    wte = synth.normal(4, "wte", (vocab, d), 0.0, 0.02)
+    wpe = synth.normal(4, "wpe", (maxpos, d), 0.0, 0.02)
+    ids = synth.token_ids(4, "ids", (batch * seq,), vocab)
+    dwte, dwpe, dids = DeviceBuffer.from_host(wte), DeviceBuffer.from_host(wpe), DeviceBuffer.from_host(ids)
+    out = DeviceBuffer((batch * seq, d))
+    bad = DeviceBuffer((1,), np.int64)
+    hip.embedding_add(dwte, vocab, dwpe, maxpos, dids, batch * seq, seq, d, out, bad)
+    ref = wte[ids.astype(int)] + np.tile(wpe[:seq], (batch, 1))
+    assert np.array_equal(out.to_host(), ref) and bad.to_host()[0] == -1
+    for shape in ((2, 5, 3, 8), (3, 128, 12, 64), (1, 7, 2, 3)):
+        x = synth.normal(6, "perm", shape)
+        dx = DeviceBuffer.from_host(x)
+        dy = DeviceBuffer((shape[0], shape[2], shape[1], shape[3]))
+        hip.permute_0213(dx, dy, *shape)
+        assert np.array_equal(dy.to_host(), oracle.permute_0213(x))
+        back = DeviceBuffer(shape)
+        hip.permute_0213(dy, back, shape[0], shape[2], shape[1], shape[3])
+        assert np.array_equal(back.to_host(), x)  # split then merge is the identity

@@ -1,0 +1,164 @@
+"""Parity of the HIP row kernels with the CPU checker, through the device-pointer C ABI.
+
+fp32 row ops: max|d| / max|ref| <= 1e-5; fp64: <= 1e-12; add / bias add: bit-exact.
+"""
+import numpy as np
+import pytest
+
+from conftest import TOL_F64, TOL_ROW_F32, rel_err
+from frankentorch_amd import synth
+from frankentorch_amd.device import DeviceBuffer
+
+pytestmark = pytest.mark.gpu
+
+# register-resident one-wave rows, four-wave rows, streaming rows, ragged / unaligned lengths
+SHAPES = [(1, 1), (3, 7), (64, 256), (33, 768), (5, 1024), (16, 4100), (9, 4096), (8, 16384), (3, 20000), (4, 50257), (7, 513)]
+
+
+def _inputs(rows, cols, dtype, seed=11):
+    x = synth.normal(seed, "x", (rows, cols)).astype(dtype)
+    w = synth.uniform(seed, "gamma", (cols,), 0.5, 1.5).astype(dtype)
+    b = synth.normal(seed, "beta", (cols,), 0.0, 0.1).astype(dtype)
+    r = synth.normal(seed, "res", (rows, cols)).astype(dtype)
+    return x, w, b, r
+
+
+@pytest.mark.parametrize("rows,cols", SHAPES)
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_row_ops_match_oracle(hip, oracle, rows, cols, dtype):
+    tol = TOL_ROW_F32 if dtype == np.float32 else TOL_F64
+    x, w, b, r = _inputs(rows, cols, dtype)
+    dx, dw, db, dr = (DeviceBuffer.from_host(a) for a in (x, w, b, r))
+    dy = DeviceBuffer(x.shape, dtype)
+    hip.softmax_lastdim(dx, dy, rows, cols)
+    assert rel_err(dy.to_host(), oracle.softmax(x, 1)) <= tol
+    hip.layer_norm(dx, dw, db, dy, rows, cols, 1e-5)
+    assert rel_err(dy.to_host(), oracle.layer_norm(x, w, b, 1e-5)) <= tol
+    hip.layer_norm(dx, None, None, dy, rows, cols, 1e-5)
+    assert rel_err(dy.to_host(), oracle.layer_norm(x, None, None, 1e-5)) <= tol
+    hip.layer_norm(dx, dw, None, dy, rows, cols, 1e-5)
+    assert rel_err(dy.to_host(), oracle.layer_norm(x, w, None, 1e-5)) <= tol
+    hip.rms_norm(dx, dw, dy, rows, cols, 1e-6)
+    assert rel_err(dy.to_host(), oracle.rms_norm(x, w, 1e-6)) <= tol
+    hip.rms_norm(dx, None, dy, rows, cols, 1e-6)
+    assert rel_err(dy.to_host(), oracle.rms_norm(x, None, 1e-6)) <= tol
+    hip.gelu(dx, dy, rows * cols)
+    assert rel_err(dy.to_host(), oracle.gelu(x)) <= tol
+    hip.add(dx, dr, dy, rows * cols)
+    assert np.array_equal(dy.to_host(), oracle.add(x, r))  # exact IEEE
+    hip.bias_add(dx, db, dy, rows, cols)
+    assert np.array_equal(dy.to_host(), oracle.bias_add(x, b))
+    if dtype == np.float32:
+        hip.add_layer_norm(dx, dr, dw, db, dy, rows, cols, 1e-5)
+        assert rel_err(dy.to_host(), oracle.add_layer_norm(x, r, w, b, 1e-5)) <= tol
+        hip.bias_residual_add(dx, db, dr, dy, rows, cols)
+        assert np.array_equal(dy.to_host(), oracle.bias_add(x, b, r))
+
+
+def test_unaligned_pointers_take_the_scalar_path(hip, oracle):
+    """A storage offset of one element breaks 16-byte alignment: results must not change class."""
+    rows, cols = 6, 1024
+    x, w, b, r = _inputs(rows, cols + 0, np.float32)
+    pad = np.concatenate([np.zeros(1, np.float32), x.ravel()])
+    dpad = DeviceBuffer.from_host(pad)
+    dy = DeviceBuffer((rows * cols + 1,), np.float32)
+    dw, db = DeviceBuffer.from_host(w), DeviceBuffer.from_host(b)
+    hip.softmax_lastdim(dpad.view(1), dy.view(1), rows, cols)
+    assert rel_err(dy.to_host()[1:].reshape(rows, cols), oracle.softmax(x, 1)) <= TOL_ROW_F32
+    hip.layer_norm(dpad.view(1), dw, db, dy.view(1), rows, cols, 1e-5)
+    assert rel_err(dy.to_host()[1:].reshape(rows, cols), oracle.layer_norm(x, w, b, 1e-5)) <= TOL_ROW_F32
+    hip.gelu(dpad.view(1), dy.view(1), rows * cols)
+    assert rel_err(dy.to_host()[1:].reshape(rows, cols), oracle.gelu(x)) <= TOL_ROW_F32
+    hip.bias_add(dpad.view(1), db, dy.view(1), rows, cols)
+    assert np.array_equal(dy.to_host()[1:].reshape(rows, cols), x + b)
+
+
+def test_softmax_strided_dims(hip, oracle):
+    x = synth.normal(5, "s", (6, 37, 19))
+    dx = DeviceBuffer.from_host(x)
+    dy = DeviceBuffer(x.shape)
+    hip.softmax_strided(dx, dy, 6, 37, 19)
+    assert rel_err(dy.to_host(), oracle.softmax(x, 1)) <= TOL_ROW_F32
+    hip.softmax_strided(dx, dy, 1, 6, 37 * 19)
+    assert rel_err(dy.to_host(), oracle.softmax(x, 0)) <= TOL_ROW_F32
+    x64 = x.astype(np.float64)
+    dx64, dy64 = DeviceBuffer.from_host(x64), DeviceBuffer(x.shape, np.float64)
+    hip.softmax_strided(dx64, dy64, 6, 37, 19)
+    assert rel_err(dy64.to_host(), oracle.softmax(x64, 1)) <= TOL_F64
+
+
+def test_softmax_special_values(hip, oracle, vectors):
+    """inf -> all-NaN row, NaN -> all-NaN row, finite extremes -> exact 0 and 1, uniform -> exact 0.5
+    (crates/ft-kernel-cpu/src/lib.rs:65294-65317; golden bits 0x3f000000)."""
+    cols = 8
+    x = np.zeros((6, cols), np.float32)
+    x[0, 2] = np.inf
+    x[1, 3] = np.nan
+    x[2] = [-1000.0, 0.0, 1000.0, 0, 0, 0, 0, 0]
+    x[3] = -np.inf
+    x[4] = 5.0
+    x[5, 0] = -np.inf
+    dx = DeviceBuffer.from_host(x)
+    dy = DeviceBuffer(x.shape)
+    hip.softmax_lastdim(dx, dy, 6, cols)
+    y = dy.to_host()
+    ref = oracle.softmax(x, 1)
+    assert np.all(np.isnan(y[0])) and np.all(np.isnan(y[1])) and np.all(np.isnan(y[3]))
+    assert np.array_equal(np.isnan(y), np.isnan(ref))
+    assert y[2, 0] == 0.0 and y[2, 2] == 1.0
+    assert np.all(y[4].view(np.uint32) == 0x3E000000)  # 1/8 exactly
+    assert y[5, 0] == 0.0 and rel_err(y[5, 1:], ref[5, 1:]) <= TOL_ROW_F32
+    b = vectors["golden_text"]["softmax_parallel_bits"]
+    rows, c2 = b["meta"]["fast_rows"], b["meta"]["fast_cols"]
+    dz = DeviceBuffer.from_host(np.zeros((rows, c2), np.float32))
+    dzo = DeviceBuffer((rows, c2))
+    hip.softmax_lastdim(dz, dzo, rows, c2)
+    bits = dzo.to_host().ravel().view(np.uint32)
+    for i, v in b["bits"]["f32_softmax_fast_bits"].items():
+        assert bits[int(i)] == int(v, 16)
+
+
+def test_empty_inputs_are_no_ops(hip):
+    dx = DeviceBuffer((4,))
+    hip.softmax_lastdim(dx, dx, 0, 4)
+    hip.softmax_lastdim(dx, dx, 4, 0)
+    hip.layer_norm(dx, None, None, dx, 0, 16, 1e-5)
+    hip.gelu(dx, dx, 0)
+    hip.add(dx, dx, dx, 0)
+
+
+def test_full_size_row_ops_parity_determinism_and_properties(hip, oracle):
+    """Config 2: fp32 [8192, 4096], seed 1. Parity on the whole tensor, run-twice bitwise equality,
+    and properties that do not need the oracle (rows sum to 1, zero mean / unit variance, linearity)."""
+    rows, cols = 8192, 4096
+    x = synth.normal(1, "x", (rows, cols))
+    gamma = synth.uniform(1, "gamma", (cols,), 0.5, 1.5)
+    beta = synth.normal(1, "beta", (cols,), 0.0, 0.1)
+    bias = synth.normal(1, "bias", (cols,), 0.0, 0.1)
+    res = synth.normal(1, "residual", (rows, cols))
+    dx, dg, dbt, dbi, dr = (DeviceBuffer.from_host(a) for a in (x, gamma, beta, bias, res))
+    dy, dy2 = DeviceBuffer(x.shape), DeviceBuffer(x.shape)
+
+    def twice(launch):
+        launch(dy)
+        launch(dy2)
+        a, b = dy.to_host(), dy2.to_host()
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), "repeated runs differ bitwise"
+        return a
+
+    y = twice(lambda out: hip.softmax_lastdim(dx, out, rows, cols))
+    assert rel_err(y, oracle.softmax(x, 1)) <= TOL_ROW_F32
+    assert np.max(np.abs(y.sum(axis=1, dtype=np.float64) - 1.0)) < 1e-5 and y.min() >= 0 and y.max() <= 1
+    y = twice(lambda out: hip.layer_norm(dx, dg, dbt, out, rows, cols, 1e-5))
+    assert rel_err(y, oracle.layer_norm(x, gamma, beta, 1e-5)) <= TOL_ROW_F32
+    hip.layer_norm(dx, None, None, dy, rows, cols, 1e-5)
+    z = dy.to_host().astype(np.float64)
+    assert np.max(np.abs(z.mean(axis=1))) < 1e-5 and np.max(np.abs(z.var(axis=1) - 1.0)) < 1e-3
+    y = twice(lambda out: hip.rms_norm(dx, dg, out, rows, cols, 1e-6))
+    assert rel_err(y, oracle.rms_norm(x, gamma, 1e-6)) <= TOL_ROW_F32
+    y = twice(lambda out: hip.gelu(dx, out, rows * cols))
+    assert rel_err(y, oracle.gelu(x)) <= TOL_ROW_F32
+    y = twice(lambda out: hip.bias_residual_add(dx, dbi, dr, out, rows, cols))
+    assert np.array_equal(y, (x + bias) + res)
+    y = twice(lambda out: hip.add_layer_norm(dx, dr, dg, dbt, out, rows, cols, 1e-5))
+    assert rel_err(y, oracle.add_layer_norm(x, res, gamma, beta, 1e-5)) <= TOL_ROW_F32

@@ -1,0 +1,117 @@
+"""Fused causal SDPA against the CPU checker (the reference's row softmax between two
+wide-accumulation products). fp32: max|d| / max|ref| <= 2e-5; fp64: <= 1e-12."""
+import math
+
+import numpy as np
+import pytest
+
+from conftest import TOL_F64, TOL_GEMM_F32, rel_err
+from frankentorch_amd import _lib, synth
+from frankentorch_amd.device import DeviceBuffer
+
+pytestmark = pytest.mark.gpu
+
+
+def _qkv(seed, bh, sq, sk, dk, dv, dtype=np.float32):
+    s = 1.0 / math.sqrt(dk)
+    q = synth.normal(seed, "q", (bh, sq, dk), 0.0, s).astype(dtype)
+    k = synth.normal(seed, "k", (bh, sk, dk), 0.0, 1.0).astype(dtype)
+    v = synth.normal(seed, "v", (bh, sk, dv), 0.0, 1.0).astype(dtype)
+    return q, k, v
+
+
+def _run(hip, q, k, v, scale, causal):
+    bh, sq, dk = q.shape
+    sk, dv = k.shape[1], v.shape[2]
+    dq, dk_, dv_ = DeviceBuffer.from_host(q), DeviceBuffer.from_host(k), DeviceBuffer.from_host(v)
+    do = DeviceBuffer((bh, sq, dv), q.dtype)
+    hip.sdpa_forward(hip.sdpa_desc_contiguous(bh, sq, sk, dk, dv, causal), scale, dq, dk_, dv_, do)
+    return do.to_host()
+
+
+# MFMA variant (d 32 / 64 / 128), ragged sequence tails, seq_q != seq_k, one-row and one-key cases,
+# and head sizes that take the generic kernel (48, d_k != d_v)
+CASES = [(2, 64, 64, 64, 64, True), (3, 100, 100, 128, 128, True), (2, 130, 77, 64, 64, False), (2, 77, 130, 32, 32, True),
+         (2, 129, 129, 128, 128, False), (1, 1, 1, 64, 64, True), (2, 1, 300, 128, 128, False), (2, 300, 1, 64, 64, True),
+         (8, 256, 256, 128, 128, True), (2, 50, 50, 48, 48, True), (2, 40, 33, 16, 24, False), (4, 128, 128, 64, 64, True)]
+
+
+@pytest.mark.parametrize("bh,sq,sk,dk,dv,causal", CASES)
+def test_sdpa_f32_matches_oracle(hip, oracle, bh, sq, sk, dk, dv, causal):
+    q, k, v = _qkv(3, bh, sq, sk, dk, dv)
+    scale = 1.0 / math.sqrt(dk)
+    got = _run(hip, q, k, v, scale, causal)
+    assert rel_err(got, oracle.sdpa_forward(q, k, v, scale, causal)) <= TOL_GEMM_F32
+
+
+@pytest.mark.parametrize("bh,sq,sk,dk,dv,causal", [(2, 33, 33, 64, 64, True), (2, 20, 45, 16, 24, False), (1, 70, 70, 128, 128, True)])
+def test_sdpa_f64_matches_oracle(hip, oracle, bh, sq, sk, dk, dv, causal):
+    q, k, v = _qkv(3, bh, sq, sk, dk, dv, np.float64)
+    scale = 1.0 / math.sqrt(dk)
+    got = _run(hip, q, k, v, scale, causal)
+    assert rel_err(got, oracle.sdpa_forward(q, k, v, scale, causal)) <= TOL_F64
+
+
+def test_causal_independence_and_first_row(hip):
+    """Later keys cannot move earlier rows (crates/ft-nn/src/lib.rs:24403); row 0 of a causal
+    problem attends to key 0 only, so it equals v[0] exactly."""
+    q, k, v = _qkv(5, 2, 200, 200, 64, 64)
+    base = _run(hip, q, k, v, 0.125, True)
+    k2, v2 = k.copy(), v.copy()
+    k2[:, 131:] += 3.0
+    v2[:, 131:] -= 2.0
+    moved = _run(hip, q, k2, v2, 0.125, True)
+    assert np.array_equal(moved[:, :131], base[:, :131])
+    assert not np.array_equal(moved[:, 131:], base[:, 131:])
+    assert np.array_equal(base[:, 0], v[:, 0])
+
+
+def test_packed_qkv_strides_equal_the_permuted_copies(hip, oracle):
+    """Reading q/k/v head by head out of a packed [tokens, 3*d_model] projection and writing
+    [tokens, d_model] equals split-heads -> contiguous SDPA -> merge-heads, bit for bit."""
+    batch, seq, heads, hd = 2, 96, 4, 64
+    d = heads * hd
+    qkv = synth.normal(6, "qkv", (batch * seq, 3 * d), 0.0, 0.3)
+    dqkv = DeviceBuffer.from_host(qkv)
+    dout = DeviceBuffer((batch * seq, d))
+    desc = _lib.SdpaDesc()
+    desc.num_bh, desc.heads = batch * heads, heads
+    desc.seq_q = desc.seq_k = seq
+    desc.d_k = desc.d_v = hd
+    for p in "qkv":
+        setattr(desc, p + "_batch_stride", seq * 3 * d)
+        setattr(desc, p + "_head_stride", hd)
+        setattr(desc, p + "_row_stride", 3 * d)
+    desc.o_batch_stride, desc.o_head_stride, desc.o_row_stride = seq * d, hd, d
+    desc.causal = 1
+    scale = 1.0 / math.sqrt(hd)
+    hip.sdpa_forward(desc, scale, dqkv, dqkv.view(d), dqkv.view(2 * d), dout)
+    split = lambda t: oracle.permute_0213(np.ascontiguousarray(t).reshape(batch, seq, heads, hd)).reshape(batch * heads, seq, hd)
+    q, k, v = (split(qkv[:, i * d:(i + 1) * d]) for i in range(3))
+    ctx = _run(hip, q, k, v, scale, True)
+    merged = oracle.permute_0213(ctx.reshape(batch, heads, seq, hd)).reshape(batch * seq, d)
+    assert np.array_equal(dout.to_host(), merged)
+    assert rel_err(merged, oracle.permute_0213(oracle.sdpa_forward(q, k, v, scale, True).reshape(batch, heads, seq, hd)).reshape(batch * seq, d)) <= TOL_GEMM_F32
+
+
+def test_config4_full_size_sampled_heads_determinism_and_checksum(hip, oracle):
+    """B4 H32 S2048 D128, seed 3, causal. Two (batch, head) slices are compared with the oracle in
+    full; the whole output is bitwise equal across two runs; rows are convex combinations of V
+    rows, so every output lies inside V's per-head range (a property that needs no oracle)."""
+    B, H, S, D = 4, 32, 2048, 128
+    s = 1.0 / math.sqrt(D)
+    q = synth.normal(3, "Q", (B * H, S, D), 0.0, s)
+    k = synth.normal(3, "K", (B * H, S, D), 0.0, s)
+    v = synth.normal(3, "V", (B * H, S, D), 0.0, s)
+    dq, dk, dv = DeviceBuffer.from_host(q), DeviceBuffer.from_host(k), DeviceBuffer.from_host(v)
+    do, do2 = DeviceBuffer(q.shape), DeviceBuffer(q.shape)
+    desc = hip.sdpa_desc_contiguous(B * H, S, S, D, D, True)
+    hip.sdpa_forward(desc, s, dq, dk, dv, do)
+    hip.sdpa_forward(desc, s, dq, dk, dv, do2)
+    out = do.to_host()
+    assert np.array_equal(out.view(np.uint32), do2.to_host().view(np.uint32))
+    for bh in (0, 77):
+        ref = oracle.sdpa_forward(q[bh:bh + 1], k[bh:bh + 1], v[bh:bh + 1], s, True)
+        assert rel_err(out[bh:bh + 1], ref) <= TOL_GEMM_F32
+    assert np.all(out.max(axis=1) <= v.max(axis=1) + 1e-6) and np.all(out.min(axis=1) >= v.min(axis=1) - 1e-6)
+    assert np.array_equal(out[:, 0], v[:, 0])
