@@ -55,9 +55,9 @@ class DeviceBuffer:
             check(_lib.load().fth_memcpy_d2h(out.ctypes.data, self.ptr, self.nbytes))
         return out
 
-    def view(self, offset_elems: int) -> int:
-        """Device address of element `offset_elems`."""
-        return self.ptr + offset_elems * self.dtype.itemsize
+    def view(self, offset_elems: int) -> "DeviceView":
+        """A non-owning typed pointer to element `offset_elems` (keeps this buffer alive)."""
+        return DeviceView(self, offset_elems)
 
     def free(self) -> None:
         if self._owned and self.ptr:
@@ -70,6 +70,15 @@ class DeviceBuffer:
             self.free()
         except Exception:
             pass
+
+
+class DeviceView:
+    """Typed device address inside a DeviceBuffer; accepted wherever a DeviceBuffer operand is."""
+
+    def __init__(self, base: DeviceBuffer, offset_elems: int):
+        self.base = base
+        self.dtype = base.dtype
+        self.ptr = base.ptr + offset_elems * base.dtype.itemsize
 
 
 def synchronize() -> None:
@@ -109,7 +118,7 @@ def _sfx(buf: DeviceBuffer) -> str:
 
 
 def _ptr(buf):
-    return None if buf is None else (buf.ptr if isinstance(buf, DeviceBuffer) else int(buf))
+    return None if buf is None else (buf.ptr if hasattr(buf, "ptr") else int(buf))
 
 
 def _real(buf, v):
