@@ -1,0 +1,317 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X transformer-op backend.
+
+    python bench.py --gpus 1 --steps K --warmup W [--cases LIST] [--no-cpu]
+
+Prints ONE JSON line. The headline `value` is the row-op throughput on the configured fp32
+[8192, 4096] tensors (seed 1): one step = last-dim softmax + LayerNorm + RMSNorm + erf-GELU +
+bias+residual add, each reading its inputs from HBM and writing its output once; value =
+algorithmic bytes of the step / wall time, with every input already resident in HBM. The same line
+carries `roofline` (dominant kernel of the step, HIP-event timed), `cpu_baseline` (the CPU checker
+restating ft-kernel-cpu, timed on this host's cores), and `cases`: the other parts of the metric --
+fp32 / fp64 GEMM TFLOP/s, causal SDPA TFLOP/s, pre-LN block and GPT-2-shaped forward tokens/s --
+each with its own roofline fraction.
+
+Everything runs on one GPU. `--gpus N` with N > 1 exits: this backend has no multi-GPU path.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+FP32_MFMA_PEAK_TF = 157.3    # dense fp32 matrix
+FP64_MFMA_PEAK_TF = 78.6     # dense fp64 matrix
+
+ROWS, COLS = 8192, 4096
+ELEM = ROWS * COLS
+# Algorithmic bytes per launch: every input read once + the output written once.
+ROW_BYTES = {
+    "softmax": 2 * ELEM * 4,
+    "layer_norm": 2 * ELEM * 4 + 2 * COLS * 4,
+    "rms_norm": 2 * ELEM * 4 + COLS * 4,
+    "gelu": 2 * ELEM * 4,
+    "bias_residual_add": 3 * ELEM * 4 + COLS * 4,
+}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def event_time_ms(device, launch, iters):
+    """Average duration of `launch` over `iters` back-to-back launches, by HIP events recorded on
+    the stream the kernels run on (the library stream)."""
+    e0, e1 = device.Event(), device.Event()
+    e0.record()
+    for _ in range(iters):
+        launch()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_ms(e1) / iters
+
+
+def bench_rowops(device, synth, steps, warmup, with_cpu):
+    from frankentorch_amd.device import DeviceBuffer
+
+    log("[rowops] generating fp32 [%d, %d] inputs (seed 1)" % (ROWS, COLS))
+    x = synth.normal(1, "x", (ROWS, COLS))
+    gamma = synth.uniform(1, "gamma", (COLS,), 0.5, 1.5)
+    beta = synth.normal(1, "beta", (COLS,), 0.0, 0.1)
+    bias = synth.normal(1, "bias", (COLS,), 0.0, 0.1)
+    res = synth.normal(1, "residual", (ROWS, COLS))
+    dx, dg, dbt, dbi, dr = (DeviceBuffer.from_host(a) for a in (x, gamma, beta, bias, res))
+    outs = {k: DeviceBuffer((ROWS, COLS)) for k in ROW_BYTES}
+    launches = {
+        "softmax": lambda: device.softmax_lastdim(dx, outs["softmax"], ROWS, COLS),
+        "layer_norm": lambda: device.layer_norm(dx, dg, dbt, outs["layer_norm"], ROWS, COLS, 1e-5),
+        "rms_norm": lambda: device.rms_norm(dx, dg, outs["rms_norm"], ROWS, COLS, 1e-6),
+        "gelu": lambda: device.gelu(dx, outs["gelu"], ELEM),
+        "bias_residual_add": lambda: device.bias_residual_add(dx, dbi, dr, outs["bias_residual_add"], ROWS, COLS),
+    }
+
+    def step():
+        for fn in launches.values():
+            fn()
+
+    for _ in range(warmup):
+        step()
+    device.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    device.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / steps
+    step_bytes = sum(ROW_BYTES.values())
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    per_kernel = {}
+    for name, fn in launches.items():
+        fn()
+        device.synchronize()
+        ms = event_time_ms(device, fn, max(20, steps))
+        gbs = ROW_BYTES[name] / (ms * 1e-3) / 1e9
+        per_kernel[name] = {"ms": round(ms, 5), "GB/s": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
+                            "bytes": ROW_BYTES[name]}
+        log("[rowops] %-18s %.4f ms  %7.1f GB/s  %.1f%% of HBM peak" % (name, ms, gbs, 100 * gbs / HBM_PEAK_GBS))
+    dominant = max(per_kernel, key=lambda k: per_kernel[k]["ms"])
+    roof = {"bound": "hbm", "kernel": dominant, "achieved": per_kernel[dominant]["GB/s"], "peak": HBM_PEAK_GBS,
+            "unit": "GB/s", "frac": per_kernel[dominant]["frac"], "traffic": None}
+
+    cpu = None
+    if with_cpu:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import oracle as O  # CPU checker restating ft-kernel-cpu: the reported baseline only
+
+        def cpu_step():
+            O.softmax(x, 1)
+            O.layer_norm(x, gamma, beta, 1e-5)
+            O.rms_norm(x, gamma, 1e-6)
+            O.gelu(x)
+            O.bias_add(x, bias, res)
+
+        cpu_step()
+        best = float("inf")
+        t_all = time.perf_counter()
+        reps = 0
+        while reps < 3 or (time.perf_counter() - t_all < 10.0 and reps < 400):
+            t0 = time.perf_counter()
+            cpu_step()
+            best = min(best, time.perf_counter() - t0)
+            reps += 1
+        cpu = {"value": round(step_bytes / best / 1e9, 2), "unit": "GB/s", "cores": O.threads(), "kind": "port",
+               "sample": "the full config-2 step (5 row ops on fp32 [8192,4096]), best of %d runs, %.1f s of CPU work"
+                         % (reps, time.perf_counter() - t_all)}
+        log("[rowops] cpu baseline %.2f GB/s on %d threads" % (cpu["value"], cpu["cores"]))
+    return value, ms_per_step, roof, per_kernel, cpu
+
+
+def bench_gemm(device, synth, steps):
+    from frankentorch_amd.device import EPI_BIAS, DeviceBuffer
+
+    out = {}
+    a = synth.uniform(2, "A", (4096, 4096), -1, 1)
+    b = synth.uniform(2, "B", (4096, 4096), -1, 1)
+    da, db = DeviceBuffer.from_host(a), DeviceBuffer.from_host(b)
+    dc = DeviceBuffer((4096, 4096))
+    iters = max(10, steps)
+
+    def run(name, desc, A, B, Cc, bias, flop, peak):
+        fn = lambda: device.gemm(desc, A, B, Cc, bias)
+        for _ in range(3):
+            fn()
+        device.synchronize()
+        ms = event_time_ms(device, fn, iters)
+        tf = flop / (ms * 1e-3) / 1e12
+        out[name] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac": round(tf / peak, 4), "flop": flop,
+                     "peak_TFLOP/s": peak}
+        log("[gemm] %-34s %.3f ms  %6.2f TFLOP/s  %.1f%% of MFMA peak" % (name, ms, tf, 100 * tf / peak))
+
+    run("f32_4096x4096x4096_nn", device.gemm_desc(4096, 4096, 4096), da, db, dc, None, 2 * 4096 ** 3, FP32_MFMA_PEAK_TF)
+    run("f32_4096x4096x4096_nt", device.gemm_desc(4096, 4096, 4096, trans_b=True), da, db, dc, None, 2 * 4096 ** 3,
+        FP32_MFMA_PEAK_TF)
+    b2 = synth.uniform(2, "B2", (4096, 11008), -1, 1)
+    bias = synth.uniform(2, "bias2", (11008,), -1, 1)
+    db2, dbias = DeviceBuffer.from_host(b2), DeviceBuffer.from_host(bias)
+    dc2 = DeviceBuffer((4096, 11008))
+    run("f32_4096x11008x4096_bias", device.gemm_desc(4096, 11008, 4096, epilogue=EPI_BIAS), da, db2, dc2, dbias,
+        2 * 4096 * 4096 * 11008, FP32_MFMA_PEAK_TF)
+    del db2, dc2
+    ba = synth.uniform(2, "ba", (32, 512, 128), -1, 1)
+    bb = synth.uniform(2, "bb", (32, 128, 512), -1, 1)
+    dba, dbb = DeviceBuffer.from_host(ba), DeviceBuffer.from_host(bb)
+    dbc = DeviceBuffer((32, 512, 512))
+    run("f32_bmm_32x512x512x128", device.gemm_desc(512, 512, 128, batch=32), dba, dbb, dbc, None, 32 * 2 * 512 * 128 * 512,
+        FP32_MFMA_PEAK_TF)
+    da64, db64 = DeviceBuffer.from_host(a.astype(np.float64)), DeviceBuffer.from_host(b.astype(np.float64))
+    dc64 = DeviceBuffer((4096, 4096), np.float64)
+    run("f64_4096x4096x4096_nn", device.gemm_desc(4096, 4096, 4096), da64, db64, dc64, None, 2 * 4096 ** 3, FP64_MFMA_PEAK_TF)
+    return out
+
+
+def bench_sdpa(device, synth, steps):
+    from frankentorch_amd.device import DeviceBuffer
+
+    B, H, S, D = 4, 32, 2048, 128
+    s = 1.0 / math.sqrt(D)
+    q, k, v = (synth.normal(3, t, (B * H, S, D), 0.0, s) for t in ("Q", "K", "V"))
+    dq, dk, dv = DeviceBuffer.from_host(q), DeviceBuffer.from_host(k), DeviceBuffer.from_host(v)
+    do = DeviceBuffer(q.shape)
+    desc = device.sdpa_desc_contiguous(B * H, S, S, D, D, True)
+    fn = lambda: device.sdpa_forward(desc, s, dq, dk, dv, do)
+    for _ in range(2):
+        fn()
+    device.synchronize()
+    ms = event_time_ms(device, fn, max(5, steps // 2))
+    flop = B * H * 4 * D * (S * (S + 1) // 2)  # causal count: two products over the lower triangle
+    tf = flop / (ms * 1e-3) / 1e12
+    log("[sdpa] B4 H32 S2048 D128 causal  %.3f ms  %.2f TFLOP/s (causal count)  %.1f%% of MFMA peak" % (ms, tf, 100 * tf / FP32_MFMA_PEAK_TF))
+    return {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac": round(tf / FP32_MFMA_PEAK_TF, 4), "flop": flop,
+            "peak_TFLOP/s": FP32_MFMA_PEAK_TF, "workload": "B4 H32 S2048 D128 causal fp32"}
+
+
+def make_layer(synth, seed, li, d, f):
+    n = lambda tag, *s: synth.normal(seed, "L%d.%s" % (li, tag), s, 0.0, 0.02)
+    one, zero = (lambda m: np.ones(m, np.float32)), (lambda m: np.zeros(m, np.float32))
+    return {"ln1_w": one(d), "ln1_b": zero(d), "wq": n("wq", d, d), "bq": zero(d), "wk": n("wk", d, d), "bk": zero(d),
+            "wv": n("wv", d, d), "bv": zero(d), "wo": n("wo", d, d), "bo": zero(d), "ln2_w": one(d), "ln2_b": zero(d),
+            "w1": n("w1", f, d), "b1": zero(f), "w2": n("w2", d, f), "b2": zero(d)}
+
+
+def bench_block(device, synth, steps):
+    from frankentorch_amd import fused
+    from frankentorch_amd.device import DeviceBuffer
+
+    batch, seq, d, heads, f = 1, 128, 256, 4, 1024
+    enc = fused.EncoderHip(d, heads, f, [make_layer(synth, 0, 0, d, f)], 1e-5, causal=True)
+    x = synth.normal(0, "x", (batch * seq, d))
+    dx, dout = DeviceBuffer.from_host(x), DeviceBuffer((batch * seq, d))
+    res = {"workload": "pre-LN block B1 S128 d256 h4 ffn1024 causal fp32 (launch-latency-bound)"}
+    iters = max(50, steps)
+    for label, graph in (("eager", False), ("graph", True)):
+        fn = lambda: enc.forward_dev(dx, dout, batch, seq, graph=graph)
+        for _ in range(3):
+            fn()
+        device.synchronize()
+        ms = event_time_ms(device, fn, iters)
+        res[label] = {"ms": round(ms, 5), "tokens/s": round(batch * seq / (ms * 1e-3), 1)}
+        log("[block] %s %.4f ms  %.0f tokens/s" % (label, ms, batch * seq / (ms * 1e-3)))
+    flop = 2.10e8
+    res["flop"] = flop
+    res["frac"] = round(flop / (res["graph"]["ms"] * 1e-3) / 1e12 / FP32_MFMA_PEAK_TF, 5)
+    return res
+
+
+def bench_gpt2(device, synth, steps):
+    from frankentorch_amd import fused
+    from frankentorch_amd.device import DeviceBuffer
+
+    vocab, maxpos, d, heads, f, nl, batch, seq = 50257, 1024, 768, 12, 3072, 12, 8, 1024
+    log("[gpt2] generating GPT-2-small-shaped weights (seed 4)")
+    wte = synth.normal(4, "wte", (vocab, d), 0.0, 0.02)
+    wpe = synth.normal(4, "wpe", (maxpos, d), 0.0, 0.02)
+    layers = [make_layer(synth, 4, i, d, f) for i in range(nl)]
+    ids = synth.token_ids(4, "ids", (batch * seq,), vocab)
+    model = fused.Gpt2Hip(wte, wpe, layers, None, None, heads, 1e-5)
+    T = batch * seq
+    dids = DeviceBuffer.from_host(ids)
+    dlog, dam = DeviceBuffer((T, vocab)), DeviceBuffer((T,))
+    fn = lambda: model.forward_dev(dids, batch, seq, dlog, dam)
+    for _ in range(2):
+        fn()
+    device.synchronize()
+    ms = event_time_ms(device, fn, max(5, steps // 4))
+    flop = 12 * 2 * T * d * (3 * d + d + 2 * f) + 12 * (batch * heads) * 4 * (d // heads) * (seq * (seq + 1) // 2) + 2 * T * d * vocab
+    tf = flop / (ms * 1e-3) / 1e12
+    log("[gpt2] forward (logits + argmax) %.3f ms  %.0f tokens/s  %.2f TFLOP/s  %.1f%% of MFMA peak"
+        % (ms, T / (ms * 1e-3), tf, 100 * tf / FP32_MFMA_PEAK_TF))
+    return {"ms": round(ms, 3), "tokens/s": round(T / (ms * 1e-3), 1), "TFLOP/s": round(tf, 2), "frac": round(tf / FP32_MFMA_PEAK_TF, 4),
+            "flop": flop, "workload": "GPT-2-small shape: 12L d768 h12 ffn3072 vocab50257 B8 S1024 fp32, logits + argmax"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--cases", default="all", help="comma list of: gemm,sdpa,block,gpt2 (row ops always run); 'none' for row ops only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this backend runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding)" % args.gpus)
+
+    from frankentorch_amd import device, synth
+
+    if not device.is_available():
+        sys.exit("bench.py: no usable gfx950 device; the HIP library has no CPU fallback")
+    info = device.device_info()
+    log("[device] %s, %d CUs, %.0f GiB HBM, engine %d MHz" % (info["arch"], info["compute_units"], info["hbm_bytes"] / 2 ** 30,
+                                                               info["engine_clock_khz"] // 1000))
+    cases = {"gemm", "sdpa", "block", "gpt2"} if args.cases == "all" else set(c for c in args.cases.split(",") if c and c != "none")
+
+    value, ms_per_step, roof, per_kernel, cpu = bench_rowops(device, synth, args.steps, args.warmup, not args.no_cpu)
+    extra = {"row_ops": per_kernel}
+    if "gemm" in cases:
+        extra["gemm"] = bench_gemm(device, synth, args.steps)
+    if "sdpa" in cases:
+        extra["sdpa_causal"] = bench_sdpa(device, synth, args.steps)
+    if "block" in cases:
+        extra["block"] = bench_block(device, synth, args.steps)
+    if "gpt2" in cases:
+        extra["gpt2_forward"] = bench_gpt2(device, synth, args.steps)
+
+    line = {
+        "metric": "row-op GB/s (fp32, 1 MI355X)",
+        "metric_full": "GEMM TFLOP/s, row-op GB/s, fused-block tokens/s (fp32, 1 MI355X) + %roofline",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: row ops on fp32 [8192,4096], seed 1: softmax + LayerNorm + RMSNorm + erf-GELU + bias+residual add",
+                   "bytes_per_step": sum(ROW_BYTES.values()), "device": info["arch"], "compute_units": info["compute_units"]},
+        "roofline": roof,
+        "cpu_baseline": cpu,
+        "cases": extra,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
