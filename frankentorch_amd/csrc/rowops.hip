@@ -1,20 +1,24 @@
 // Memory-bound row kernels for gfx950: last-dim softmax, LayerNorm, add+LayerNorm, RMSNorm,
 // erf-GELU, add, bias add, bias+residual add.
 //
-// Shape of every row kernel: one 64-lane wavefront (or the four wavefronts of a 256-thread block,
-// for long rows) owns one row, pulls it from HBM once with 128-bit loads into registers, reduces
-// with a fixed xor-butterfly over the wavefront and a fixed left-to-right fold over the block's
-// wavefronts, and writes the row back once with 128-bit stores. No atomics anywhere: the
-// reduction tree is a function of (row length, kernel variant) only, so repeated runs are
-// bitwise identical. Rows whose base is not 16-byte aligned, whose length is not a multiple of
-// the vector width, or which do not fit the register budget take a block-per-row streaming
-// variant with the same fixed trees.
+// Shape of every row kernel: one, two or four 64-lane wavefronts of a 256-thread block own one
+// row (the fewest that keep a lane at <= 4 vectors; up to 16 vectors per lane for rows of up to
+// 16 Ki elements), pull it from HBM once with 128-bit loads into registers, reduce with a fixed
+// xor-butterfly over the wavefront and a fixed left-to-right fold over the row's wavefronts, and
+// write the row back once with 128-bit non-temporal stores. No atomics anywhere: the reduction
+// tree is a function of (row length, kernel variant) only, so repeated runs are bitwise
+// identical. Rows whose base is not 16-byte aligned, whose length is not a multiple of the
+// vector width, or which do not fit the register budget take a block-per-row streaming variant
+// with the same fixed trees.
 //
 // Arithmetic follows crates/ft-kernel-cpu/src/lib.rs step for step (separate multiplies and adds;
 // this file is compiled with -ffp-contract=off): softmax :39219-39229, LayerNorm :5886-5909,
 // add+LayerNorm :5946-5970, RMSNorm :6466-6480, GELU :36966-36969, add :36870-36877,
 // bias pass :17336-17351. Only the summation ORDER differs (tree instead of sequential /
 // pairwise-128), which is what the 1e-5 tolerance of the parity tests covers.
+
+#include <cstdlib>
+#include <initializer_list>
 
 #include "common.hpp"
 
@@ -23,11 +27,72 @@ namespace {
 constexpr int kWave = 64;
 constexpr int kBlock = 256;
 
+// Streaming stores carry the non-temporal hint: an output is written once and not re-read by the
+// kernel, so it should not displace the input (which a producer kernel may just have left in the
+// last-level cache) or the reusable gamma / beta / bias lines. Loads stay temporal: measured on
+// MI355X at fp32 [8192,4096], non-temporal loads cost 8-10 % on every kernel, non-temporal stores
+// gain 2-25 %.
+typedef float nat_f4 __attribute__((ext_vector_type(4)));
+typedef double nat_d2 __attribute__((ext_vector_type(2)));
+#ifndef FTH_NT_LOAD
+#define FTH_NT_LOAD 0
+#endif
+#ifndef FTH_NT_STORE
+#define FTH_NT_STORE 1
+#endif
+__device__ __forceinline__ float4 stream_load(const float4 *p) {
+#if FTH_NT_LOAD
+    nat_f4 v = __builtin_nontemporal_load(reinterpret_cast<const nat_f4 *>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
+#else
+    return *p;
+#endif
+}
+__device__ __forceinline__ double2 stream_load(const double2 *p) {
+#if FTH_NT_LOAD
+    nat_d2 v = __builtin_nontemporal_load(reinterpret_cast<const nat_d2 *>(p));
+    return make_double2(v.x, v.y);
+#else
+    return *p;
+#endif
+}
+__device__ __forceinline__ void stream_store(float4 *p, const float4 &v) {
+#if FTH_NT_STORE
+    nat_f4 n = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(n, reinterpret_cast<nat_f4 *>(p));
+#else
+    *p = v;
+#endif
+}
+__device__ __forceinline__ void stream_store(double2 *p, const double2 &v) {
+#if FTH_NT_STORE
+    nat_d2 n = {v.x, v.y};
+    __builtin_nontemporal_store(n, reinterpret_cast<nat_d2 *>(p));
+#else
+    *p = v;
+#endif
+}
+
 template <typename T> struct Vec128;
 template <> struct Vec128<float> { using type = float4; static constexpr int n = 4; };
 template <> struct Vec128<double> { using type = double2; static constexpr int n = 2; };
 
-__device__ __forceinline__ float dev_exp(float x) { return expf(x); }
+// exp(x) = 2^(x * log2 e) on the hardware exp2 unit. The product x * log2 e is carried in two
+// pieces (t + r, with the rounding error of the multiply recovered by an FMA and the low bits of
+// log2 e added), and 2^r is folded back as 1 + r ln 2, so the result stays within about 1.5 ULP
+// instead of the |x| * 2^-24 relative error of a bare exp2(x * log2e). -inf maps to exactly 0 and
+// NaN propagates, which the softmax special cases rely on. Results below 2^-126 flush to zero.
+__device__ __forceinline__ float dev_exp(float x) {
+    const float kL2eHi = 1.44269502162933349609375f;  // float(log2 e)
+    const float kL2eLo = 1.925963033500011e-8f;       // log2 e - float(log2 e)
+    const float kLn2 = 0.693147182464599609375f;
+    const float t = x * kL2eHi;
+    float r = __builtin_fmaf(x, kL2eHi, -t);
+    r = __builtin_fmaf(x, kL2eLo, r);
+    r = (x == -__builtin_inff()) ? 0.0f : r;
+    const float e = __builtin_amdgcn_exp2f(t);
+    return __builtin_fmaf(e * r, kLn2, e);
+}
 __device__ __forceinline__ double dev_exp(double x) { return exp(x); }
 __device__ __forceinline__ float dev_sqrt(float x) { return sqrtf(x); }
 __device__ __forceinline__ double dev_sqrt(double x) { return sqrt(x); }
@@ -57,8 +122,9 @@ template <typename T, class F> __device__ __forceinline__ T wave_reduce(T v, F f
     return v;
 }
 
-// Reduction over the WPR wavefronts that share a row (WPR == 1: the wavefront alone; WPR == 4:
-// the whole block, folded left to right through LDS).
+// Reduction over the WPR wavefronts that share a row (WPR == 1: the wavefront alone; WPR == 2 or
+// 4: the row's wavefronts inside the 256-thread block, folded left to right through LDS). Every
+// thread of the block reaches the barriers (blocks with WPR > 1 never exit early).
 template <int WPR, typename T, class F>
 __device__ __forceinline__ T group_reduce(T v, F f, T *smem) {
     v = wave_reduce(v, f);
@@ -66,12 +132,13 @@ __device__ __forceinline__ T group_reduce(T v, F f, T *smem) {
         return v;
     } else {
         const int wave = threadIdx.x / kWave;
+        const int first = (wave / WPR) * WPR;
         __syncthreads();
         if ((threadIdx.x & (kWave - 1)) == 0) smem[wave] = v;
         __syncthreads();
-        T r = smem[0];
+        T r = smem[first];
 #pragma unroll
-        for (int w = 1; w < WPR; ++w) r = f(r, smem[w]);
+        for (int w = 1; w < WPR; ++w) r = f(r, smem[first + w]);
         return r;
     }
 }
@@ -86,7 +153,7 @@ template <typename T, int VPL, int WPR> struct RowRegs {
     T e[VPL][EPV];
 
     __device__ __forceinline__ static int lane() {
-        return WPR == 1 ? (threadIdx.x & (kWave - 1)) : threadIdx.x;
+        return threadIdx.x & (kLanes - 1);
     }
     __device__ __forceinline__ void load(const T *row, int nvec, T fill) {
         const V *p = reinterpret_cast<const V *>(row);
@@ -94,7 +161,7 @@ template <typename T, int VPL, int WPR> struct RowRegs {
 #pragma unroll
         for (int i = 0; i < VPL; ++i) {
             int v = lane() + i * kLanes;
-            if (v < nvec) tmp[i] = p[v];
+            if (v < nvec) tmp[i] = stream_load(p + v);
         }
 #pragma unroll
         for (int i = 0; i < VPL; ++i) {
@@ -123,18 +190,25 @@ template <typename T, int VPL, int WPR> struct RowRegs {
 #pragma unroll
         for (int i = 0; i < VPL; ++i) {
             int v = lane() + i * kLanes;
-            if (v < nvec) p[v] = pack(e[i]);
+            if (v < nvec) stream_store(p + v, pack(e[i]));
         }
     }
 };
 
+// A 256-thread block holds 4 / WPR rows.
 template <int WPR> __device__ __forceinline__ int64_t row_of_block() {
-    if constexpr (WPR == 1) {
-        return (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
-    } else {
-        return (int64_t)blockIdx.x;
-    }
+    return (int64_t)blockIdx.x * (kBlock / (kWave * WPR)) + threadIdx.x / (kWave * WPR);
 }
+// Rows past the end are clamped (so every wavefront still reaches the block barriers) and their
+// stores are suppressed by passing nvec_store == 0.
+#define FTH_ROW_PROLOGUE(WPR_)                                  \
+    int64_t row = row_of_block<WPR_>();                         \
+    const bool row_live = row < rows;                           \
+    if constexpr (WPR_ == 1) {                                  \
+        if (!row_live) return;                                  \
+    } else {                                                    \
+        if (!row_live) row = rows - 1;                          \
+    }
 
 // ---- softmax ------------------------------------------------------------------------------
 template <typename T, int VPL, int WPR>
@@ -142,8 +216,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_kernel(const T *__restrict
                                                              int64_t rows, int cols) {
     __shared__ T smem[4];
     using R = RowRegs<T, VPL, WPR>;
-    const int64_t row = row_of_block<WPR>();
-    if (row >= rows) return;  // WPR == 1 only: whole wavefronts drop out, no barrier is used
+    FTH_ROW_PROLOGUE(WPR)
     const int nvec = cols / R::EPV;
     R r;
     r.load(x + row * cols, nvec, neg_inf<T>());
@@ -166,11 +239,15 @@ __global__ __launch_bounds__(kBlock) void softmax_row_kernel(const T *__restrict
         }
     }
     s = group_reduce<WPR>(s, SumOp{}, smem);
+    // One correctly rounded 1 / s per row, then a multiply per element (the reference divides each
+    // element: the two differ by at most one rounding, far inside the parity tolerance, and the
+    // per-element IEEE division sequence would make this kernel ALU-bound).
+    const T inv = T(1) / s;
 #pragma unroll
     for (int i = 0; i < VPL; ++i)
 #pragma unroll
-        for (int j = 0; j < R::EPV; ++j) r.e[i][j] = r.e[i][j] / s;
-    r.store(y + row * cols, nvec);
+        for (int j = 0; j < R::EPV; ++j) r.e[i][j] = r.e[i][j] * inv;
+    r.store(y + row * cols, row_live ? nvec : 0);
 }
 
 // ---- LayerNorm / add+LayerNorm ---------------------------------------------------------------
@@ -180,8 +257,7 @@ __global__ __launch_bounds__(kBlock) void layernorm_row_kernel(const T *__restri
                                                                T *__restrict__ y, int64_t rows, int cols, T eps) {
     __shared__ T smem[4];
     using R = RowRegs<T, VPL, WPR>;
-    const int64_t row = row_of_block<WPR>();
-    if (row >= rows) return;
+    FTH_ROW_PROLOGUE(WPR)
     const int nvec = cols / R::EPV;
     R r;
     r.load(x + row * cols, nvec, T(0));
@@ -229,7 +305,7 @@ __global__ __launch_bounds__(kBlock) void layernorm_row_kernel(const T *__restri
             }
         }
     }
-    r.store(y + row * cols, nvec);
+    r.store(y + row * cols, row_live ? nvec : 0);
 }
 
 // ---- RMSNorm ---------------------------------------------------------------------------------
@@ -238,8 +314,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_row_kernel(const T *__restrict
                                                              T *__restrict__ y, int64_t rows, int cols, T eps) {
     __shared__ T smem[4];
     using R = RowRegs<T, VPL, WPR>;
-    const int64_t row = row_of_block<WPR>();
-    if (row >= rows) return;
+    FTH_ROW_PROLOGUE(WPR)
     const int nvec = cols / R::EPV;
     R r;
     r.load(x + row * cols, nvec, T(0));
@@ -265,7 +340,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_row_kernel(const T *__restrict
             }
         }
     }
-    r.store(y + row * cols, nvec);
+    r.store(y + row * cols, row_live ? nvec : 0);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -390,8 +465,8 @@ __global__ __launch_bounds__(kBlock) void elementwise_vec_kernel(const T *__rest
     for (int u = 0; u < kUnr; ++u) {
         int64_t v = base + (int64_t)u * kBlock;
         if (v < nvec) {
-            va[u] = reinterpret_cast<const V *>(a)[v];
-            if constexpr (OP == Ew::Add) vb[u] = reinterpret_cast<const V *>(b)[v];
+            va[u] = stream_load(reinterpret_cast<const V *>(a) + v);
+            if constexpr (OP == Ew::Add) vb[u] = stream_load(reinterpret_cast<const V *>(b) + v);
         }
     }
 #pragma unroll
@@ -406,7 +481,7 @@ __global__ __launch_bounds__(kBlock) void elementwise_vec_kernel(const T *__rest
                 if constexpr (OP == Ew::Gelu) ea[j] = dev_gelu(ea[j]);
                 else ea[j] = ea[j] + eb[j];
             }
-            reinterpret_cast<V *>(y)[v] = R::pack(ea);
+            stream_store(reinterpret_cast<V *>(y) + v, R::pack(ea));
         }
     }
 }
@@ -441,9 +516,9 @@ __global__ __launch_bounds__(kBlock) void bias_row_kernel(const T *x, const T *_
         for (int u = 0; u < kUnr; ++u) {
             int v = v0 + u * kWave;
             if (v < nvec) {
-                vx[u] = xr[v];
+                vx[u] = stream_load(xr + v);
                 vb[u] = br[v];
-                if constexpr (RES) vr[u] = rr[v];
+                if constexpr (RES) vr[u] = stream_load(rr + v);
             }
         }
 #pragma unroll
@@ -460,7 +535,7 @@ __global__ __launch_bounds__(kBlock) void bias_row_kernel(const T *x, const T *_
                     if constexpr (RES) o = o + er[j];
                     ex[j] = o;
                 }
-                yr[v] = R::pack(ex);
+                stream_store(yr + v, R::pack(ex));
             }
         }
     }
@@ -484,21 +559,28 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 constexpr int64_t kMaxGrid = 2147483647LL;
 
 // Picks (VPL, WPR) for a register-resident row of `nvec` vectors, or returns false.
-inline bool pick_row_shape(int64_t nvec, int &vpl, int &wpr) {
-    if (nvec <= 0) return false;
-    if (nvec <= 64 * 16) {
-        wpr = 1;
-        int64_t need = fth::ceil_div(nvec, 64);
-        vpl = need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : need <= 8 ? 8 : 16;
-        return true;
+// Few vectors per lane and more wavefronts per row measured best on MI355X (fp32 [8192,4096]:
+// LayerNorm 74 % of HBM peak with 16 vectors x 1 wavefront, 85 % with 4 x 4), so the row is spread
+// over the fewest wavefronts that keep a lane at <= 4 vectors, and only longer rows grow the
+// per-lane count. `max_vpl` caps the vectors a lane may hold.
+inline bool pick_row_shape(int64_t nvec, int max_vpl, int &vpl, int &wpr) {
+    if (nvec <= 0 || nvec > 256 * (int64_t)max_vpl) return false;
+    static const int forced = [] {
+        const char *e = std::getenv("FT_HIP_ROW_WPR");  // tuning knob: wavefronts per row (1, 2 or 4)
+        return e ? std::atoi(e) : 0;
+    }();
+    int w = nvec <= 64 * 4 ? 1 : nvec <= 128 * 4 ? 2 : 4;
+    if (forced == 1 || forced == 2 || forced == 4) {
+        if (fth::ceil_div(nvec, 64 * forced) <= max_vpl) w = forced;
     }
-    if (nvec <= 256 * 16) {
-        wpr = 4;
-        int64_t need = fth::ceil_div(nvec, 256);
-        vpl = need <= 8 ? 8 : 16;
-        return true;
-    }
-    return false;
+    const int64_t need = fth::ceil_div(nvec, 64 * w);
+    int v = need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : need <= 8 ? 8 : 16;
+    // instantiated shapes: WPR 1 x {1,2,4,8,16}, WPR 2 x {4,8,16}, WPR 4 x {2,4,8,16}
+    if (w == 2 && v < 4) v = 4;
+    if (w == 4 && v < 2) v = 2;
+    vpl = v;
+    wpr = w;
+    return true;
 }
 
 #define FTH_ROW_DISPATCH(VPL_, WPR_, LAUNCH)                         \
@@ -511,12 +593,23 @@ inline bool pick_row_shape(int64_t nvec, int &vpl, int &wpr) {
                 case 8: { LAUNCH(8, 1); } break;                     \
                 default: { LAUNCH(16, 1); } break;                   \
             }                                                        \
+        } else if (WPR_ == 2) {                                      \
+            switch (VPL_) {                                          \
+                case 4: { LAUNCH(4, 2); } break;                     \
+                case 8: { LAUNCH(8, 2); } break;                     \
+                default: { LAUNCH(16, 2); } break;                   \
+            }                                                        \
         } else {                                                     \
-            if (VPL_ == 8) { LAUNCH(8, 4); } else { LAUNCH(16, 4); } \
+            switch (VPL_) {                                          \
+                case 2: { LAUNCH(2, 4); } break;                     \
+                case 4: { LAUNCH(4, 4); } break;                     \
+                case 8: { LAUNCH(8, 4); } break;                     \
+                default: { LAUNCH(16, 4); } break;                   \
+            }                                                        \
         }                                                            \
     } while (0)
 
-inline int64_t row_grid(int64_t rows, int wpr) { return wpr == 1 ? fth::ceil_div(rows, 4) : rows; }
+inline int64_t row_grid(int64_t rows, int wpr) { return fth::ceil_div(rows, 4 / wpr); }
 
 template <typename T>
 int32_t launch_softmax(const T *x, T *y, int64_t rows, int64_t cols, fth_stream s) {
@@ -527,7 +620,7 @@ int32_t launch_softmax(const T *x, T *y, int64_t rows, int64_t cols, fth_stream 
     hipStream_t st = fth::resolve_stream(s);
     constexpr int EPV = Vec128<T>::n;
     int vpl, wpr;
-    if (cols % EPV == 0 && aligned16(x) && aligned16(y) && pick_row_shape(cols / EPV, vpl, wpr) &&
+    if (cols % EPV == 0 && aligned16(x) && aligned16(y) && pick_row_shape(cols / EPV, 16, vpl, wpr) &&
         row_grid(rows, wpr) <= kMaxGrid) {
 #define L(V_, W_) softmax_row_kernel<T, V_, W_><<<dim3((unsigned)row_grid(rows, W_)), dim3(kBlock), 0, st>>>(x, y, rows, (int)cols)
         FTH_ROW_DISPATCH(vpl, wpr, L);
@@ -566,7 +659,7 @@ int32_t launch_layernorm(const T *x, const T *x2, const T *w, const T *b, T *y, 
     int vpl, wpr;
     bool vec_ok = cols % EPV == 0 && aligned16(x) && aligned16(y) && (!ADD || aligned16(x2)) &&
                   (!w || aligned16(w)) && (!b || aligned16(b));
-    if (vec_ok && pick_row_shape(cols / EPV, vpl, wpr) && row_grid(rows, wpr) <= kMaxGrid) {
+    if (vec_ok && pick_row_shape(cols / EPV, 16, vpl, wpr) && row_grid(rows, wpr) <= kMaxGrid) {
 #define L(V_, W_) layernorm_row_kernel<T, V_, W_, ADD><<<dim3((unsigned)row_grid(rows, W_)), dim3(kBlock), 0, st>>>(x, x2, w, b, y, rows, (int)cols, eps)
         FTH_ROW_DISPATCH(vpl, wpr, L);
 #undef L
@@ -588,7 +681,7 @@ int32_t launch_rmsnorm(const T *x, const T *w, T *y, int64_t rows, int64_t cols,
     constexpr int EPV = Vec128<T>::n;
     int vpl, wpr;
     if (cols % EPV == 0 && aligned16(x) && aligned16(y) && (!w || aligned16(w)) &&
-        pick_row_shape(cols / EPV, vpl, wpr) && row_grid(rows, wpr) <= kMaxGrid) {
+        pick_row_shape(cols / EPV, 16, vpl, wpr) && row_grid(rows, wpr) <= kMaxGrid) {
 #define L(V_, W_) rmsnorm_row_kernel<T, V_, W_><<<dim3((unsigned)row_grid(rows, W_)), dim3(kBlock), 0, st>>>(x, w, y, rows, (int)cols, eps)
         FTH_ROW_DISPATCH(vpl, wpr, L);
 #undef L
