@@ -15,27 +15,46 @@
 //   B stored [k, n]: each thread reads EPV consecutive k of ONE column with scalar loads (the
 //   wavefront covers 64 consecutive columns, so every load instruction is one 256-byte run) and
 //   writes them to LDS as a single vector. No transpose pass, no bank conflicts.
-// The accumulators never leave registers; K is never split, so the sum order of an output
-// element depends on the shape and the tile configuration only: bitwise repeatable.
+//
+// Scheduling. The kernel is persistent: the grid is (CUs x resident blocks per CU) workgroups,
+// and the linearised iteration space (output tiles x K-tiles) is cut into equal contiguous
+// ranges, one per workgroup ("stream-K"). A workgroup therefore runs whole tiles back to back
+// and at most one partial tile at each end of its range; no CU idles while another still has a
+// tile to finish, whatever the tile count. A tile whose K range is shared by several workgroups
+// is completed without spinning, fences or atomics: every contributor writes its accumulators to
+// a workspace slot, and a small second kernel (ordered after the first by the stream) adds the
+// slots of each split tile in K order and runs the epilogue. The split points depend only on
+// (shape, tile configuration, grid size) and the additions are in a fixed order, so results are
+// bitwise repeatable on a given device.
 //
 // Tile order. Consecutive workgroup ids land on different XCDs (8 per device, each with its own
-// L2), so the id is first remapped to give each XCD one contiguous range of tiles, and within
-// the range tiles are walked in groups of GROUP_M tile-rows so that concurrently resident blocks
+// L2), so the id is first remapped to give each XCD one contiguous range of the iteration space,
+// and tiles are numbered in groups of GROUP_M tile-rows so that workgroups that run concurrently
 // share A row-panels and B column-panels in that XCD's L2.
 //
 // replaces gemm::sgemm / dgemm / sgemm_bt / dgemm_bt (crates/ft-kernel-cpu/src/lib.rs:1310-1338,
 // 107-138, 1430-1481, 201-255), the per-batch loop of bmm (:38572-38606) and the bias pass of
 // linear_tensor_f32 (:17336-17351).
 
+#include <cstdlib>
+#include <map>
+#include <mutex>
 #include <type_traits>
 
 #include "common.hpp"
+#include "pool.hpp"
 
 namespace {
 
 constexpr int kWave = 64;
 constexpr int kXcds = 8;
 constexpr int kGroupM = 8;
+#ifndef FTH_F32_BK
+#define FTH_F32_BK 32
+#endif
+#ifndef FTH_F32_MINW
+#define FTH_F32_MINW 2
+#endif
 
 template <typename T> struct Mfma;
 template <> struct Mfma<float> {
@@ -86,25 +105,37 @@ template <typename T> struct GemmArgs {
     int tiles_m, tiles_n;
     int epilogue;
     int use_alpha;
+    // persistent schedule
+    int ktiles;              // K-tiles per output tile
+    int64_t tiles_per_batch; // tiles_m * tiles_n
+    int64_t total_iters;     // batch * tiles_per_batch * ktiles
+    T *partials;             // [grid][2][BM * BN] accumulator slots of split tiles
+    int grid;                // workgroups of the main kernel (the fix-up kernel needs it too)
 };
 
-// Maps the hardware workgroup id to a (tile_m, tile_n) pair: XCD-contiguous, then grouped.
-__device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int &tm, int &tn) {
-    const int nblk = tiles_m * tiles_n;
-    const int per = nblk / kXcds, rem = nblk % kXcds;
-    const int xcd = pid % kXcds, q = pid / kXcds;
-    const int id = q + xcd * per + (xcd < rem ? xcd : rem);
-    const int group = kGroupM * tiles_n;
-    const int g = id / group;
-    const int first_m = g * kGroupM;
+// Tile number -> (tile_m, tile_n): groups of kGroupM tile-rows, column-major inside a group.
+__device__ __forceinline__ void tile_of_id(int64_t id, int tiles_m, int tiles_n, int &tm, int &tn) {
+    const int64_t group = (int64_t)kGroupM * tiles_n;
+    const int64_t g = id / group;
+    const int first_m = (int)(g * kGroupM);
     const int gm = (tiles_m - first_m) < kGroupM ? (tiles_m - first_m) : kGroupM;
-    const int in_g = id - g * group;
+    const int in_g = (int)(id - g * group);
     tm = first_m + in_g % gm;
     tn = in_g / gm;
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, bool TRANS_B, bool VEC>
-__global__ __launch_bounds__(WM *WN *kWave) void gemm_kernel(const GemmArgs<T> p) {
+// Hardware workgroup id -> virtual id such that each XCD owns one contiguous run of virtual ids.
+__device__ __forceinline__ int xcd_contiguous_id(int pid, int grid) {
+    const int per = grid / kXcds, rem = grid % kXcds;
+    const int xcd = pid % kXcds, q = pid / kXcds;
+    return q + xcd * per + (xcd < rem ? xcd : rem);
+}
+
+// VEC:  128-bit global loads along k are legal for A (and for B when it is stored [n, k]).
+// VECB: B is stored [k, n] and 128-bit global loads along n are legal; the loader then moves
+//       EPV x EPV register blocks (EPV vector loads, transposed in registers, EPV vector LDS stores).
+template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool TRANS_B, bool VEC, bool VECB>
+__global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_kernel(const GemmArgs<T> p) {
     using M = Mfma<T>;
     using V = typename M::V;
     constexpr int MT = M::MT, KG = M::KG, EPV = M::EPV;
@@ -121,6 +152,12 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemm_kernel(const GemmArgs<T> p
     constexpr int B_VECS = BN * KV / NT;
     static_assert(BM * KV % NT == 0 && BN * KV % NT == 0, "tile must divide evenly over the threads");
     static_assert(NT % BN == 0 || TRANS_B, "[k,n] loader needs whole column sweeps");
+    // Register-block loader for [k, n] B: the tile holds B_BLOCKS blocks of EPV x EPV elements,
+    // B_BPT per thread (threads past the last block of a sweep carry none).
+    constexpr int B_BLOCKS = KV * (BN / EPV);
+    constexpr int B_BPT = (B_BLOCKS + NT - 1) / NT;
+    constexpr bool BLOCK_B = !TRANS_B && VECB && (NT % (BN / EPV) == 0);
+    constexpr int B_ST = BLOCK_B ? B_BPT * EPV : B_VECS;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *As = reinterpret_cast<T *>(smem_raw);  // [2][BM][S]
@@ -132,15 +169,13 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemm_kernel(const GemmArgs<T> p
     const int wm0 = (wave / WN) * WTM;
     const int wn0 = (wave % WN) * WTN;
 
-    int tile_m, tile_n;
-    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
-    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
-    const int64_t batch = blockIdx.y;
-    const T *A = p.a + batch * p.stride_a;
-    const T *B = p.b + batch * p.stride_b;
-    T *C = p.c + batch * p.stride_c;
+    // Per-segment state (set at the top of the persistent loop; the loaders read it by reference).
+    int64_t m0 = 0, n0 = 0, batch = 0;
+    const T *A = p.a;
+    const T *B = p.b;
+    T *C = p.c;
 
-    V a_st[A_VECS], b_st[B_VECS];
+    V a_st[A_VECS], b_st[B_ST];
 
     auto load_k_contig = [&](const T *base, int64_t ld, int64_t r0, int64_t rmax, int64_t k0, V *st, auto nvecs) {
 #pragma unroll
@@ -163,9 +198,37 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemm_kernel(const GemmArgs<T> p
             st[i] = v;
         }
     };
-    // B stored [k, n]: thread owns column (tid % BN) and k-vectors kv = tid / BN + i * (NT / BN).
+    // B stored [k, n], register-block form: thread owns EPV consecutive columns (4 * nv) and
+    // k-vectors kq = tid / (BN / EPV) + blk * (NT / (BN / EPV)); it loads EPV rows of EPV columns
+    // and regroups them into EPV vectors of EPV consecutive k, one per column.
+    auto load_b_blocks = [&](int64_t k0) {
+        if constexpr (BLOCK_B) {
+            constexpr int NV = BN / EPV, KQ_STEP = NT / NV;
+            const int nv = tid % NV, kq0 = tid / NV;
+            const int64_t gc = n0 + (int64_t)nv * EPV;
+#pragma unroll
+            for (int blk = 0; blk < B_BPT; ++blk) {
+                const int kq = kq0 + blk * KQ_STEP;
+                const int64_t gk = k0 + (int64_t)kq * EPV;
+                V rows[EPV];
+#pragma unroll
+                for (int j = 0; j < EPV; ++j) {
+                    // n % EPV == 0 and k % EPV == 0 are guaranteed by the launcher for this path
+                    rows[j] = (kq < KV && gc < p.n && gk + j < p.k) ? *reinterpret_cast<const V *>(B + (gk + j) * p.ldb + gc) : M::zero();
+                }
+#pragma unroll
+                for (int c = 0; c < EPV; ++c) {
+                    T e[EPV];
+#pragma unroll
+                    for (int j = 0; j < EPV; ++j) e[j] = M::elem(rows[j], c);
+                    b_st[blk * EPV + c] = M::make(e);
+                }
+            }
+        }
+    };
+    // B stored [k, n], scalar form: thread owns column (tid % BN) and k-vectors kv = tid / BN + i * (NT / BN).
     auto load_b_kn = [&](int64_t k0) {
-        if constexpr (!TRANS_B) {
+        if constexpr (!TRANS_B && !BLOCK_B) {
             constexpr int KV_STEP = NT / BN;
             const int col = tid % BN, kv0 = tid / BN;
             const int64_t gc = n0 + col;
@@ -182,6 +245,7 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemm_kernel(const GemmArgs<T> p
     auto load_tiles = [&](int64_t k0) {
         load_k_contig(A, p.lda, m0, p.m, k0, a_st, std::integral_constant<int, A_VECS>{});
         if constexpr (TRANS_B) load_k_contig(B, p.ldb, n0, p.n, k0, b_st, std::integral_constant<int, B_VECS>{});
+        else if constexpr (BLOCK_B) load_b_blocks(k0);
         else load_b_kn(k0);
     };
     auto store_tiles = [&](int buf) {
@@ -198,6 +262,17 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemm_kernel(const GemmArgs<T> p
                 const int vid = tid + i * NT;
                 *reinterpret_cast<V *>(bs + (vid / KV) * S + (vid % KV) * EPV) = b_st[i];
             }
+        } else if constexpr (BLOCK_B) {
+            constexpr int NV = BN / EPV, KQ_STEP = NT / NV;
+            const int nv = tid % NV, kq0 = tid / NV;
+#pragma unroll
+            for (int blk = 0; blk < B_BPT; ++blk) {
+                const int kq = kq0 + blk * KQ_STEP;
+                if (kq < KV) {
+#pragma unroll
+                    for (int c = 0; c < EPV; ++c) *reinterpret_cast<V *>(bs + (nv * EPV + c) * S + kq * EPV) = b_st[blk * EPV + c];
+                }
+            }
         } else {
             constexpr int KV_STEP = NT / BN;
             const int col = tid % BN, kv0 = tid / BN;
@@ -207,63 +282,167 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemm_kernel(const GemmArgs<T> p
     };
 
     typename M::Acc acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < M::ACC; ++r) acc[i][j][r] = T(0);
-
-    const int64_t ktiles = (p.k + BK - 1) / BK;
     const int lrow = lane % MT;           // row / column inside an MFMA tile
     const int lk = (lane / MT) * EPV;     // k offset of this lane's vector inside a fetch
-
-    if (ktiles > 0) {
-        load_tiles(0);
-        store_tiles(0);
-    }
-    __syncthreads();
-
-    for (int64_t kt = 0; kt < ktiles; ++kt) {
-        const int buf = (int)(kt & 1);
-        if (kt + 1 < ktiles) load_tiles((kt + 1) * BK);
-        const T *as = As + buf * BM * S + (wm0 + lrow) * S + lk;
-        const T *bs = Bs + buf * BN * S + (wn0 + lrow) * S + lk;
-#pragma unroll
-        for (int kc = 0; kc < BK / KCH; ++kc) {
-            V af[TM], bf[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const V *>(as + i * MT * S + kc * KCH);
-#pragma unroll
-            for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const V *>(bs + j * MT * S + kc * KCH);
-#pragma unroll
-            for (int e = 0; e < EPV; ++e)
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j) acc[i][j] = M::mma(M::elem(af[i], e), M::elem(bf[j], e), acc[i][j]);
-        }
-        if (kt + 1 < ktiles) store_tiles(buf ^ 1);
-        __syncthreads();
-    }
 
     // Epilogue: each rounding is its own step, in the order product -> alpha -> bias -> GELU ->
     // residual, which is the order the unfused reference ops would apply them.
     const bool has_bias = (p.epilogue & FTH_EPI_BIAS) != 0;
     const bool has_gelu = (p.epilogue & FTH_EPI_GELU) != 0;
     const bool has_res = (p.epilogue & FTH_EPI_RESIDUAL) != 0;
+    auto epilogue = [&]() {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int64_t col = n0 + wn0 + j * MT + lrow;
+            if (col >= p.n) continue;
+            const T bv = has_bias ? p.bias[col] : T(0);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                for (int r = 0; r < M::ACC; ++r) {
+                    const int64_t row = m0 + wm0 + i * MT + M::acc_row(r, lane);
+                    if (row < p.m) {
+                        T v = acc[i][j][r];
+                        if (p.use_alpha) v = p.alpha * v;
+                        if (has_bias) v = v + bv;
+                        if (has_gelu) v = M::gelu(v);
+                        if (has_res) v = v + p.residual[batch * p.stride_c + row * p.ldc + col];
+                        C[row * p.ldc + col] = v;
+                    }
+                }
+            }
+        }
+    };
+
+    const int grid = (int)gridDim.x;
+    const int vb = xcd_contiguous_id((int)blockIdx.x, grid);
+    const int64_t total = p.total_iters;
+    // Workgroup b owns iterations [b * total / grid, (b + 1) * total / grid).
+    int64_t it = (int64_t)vb * total / grid;
+    const int64_t it_end = (int64_t)(vb + 1) * total / grid;
+
+    while (it < it_end) {
+        const int64_t tile = it / p.ktiles;
+        const int k_lo = (int)(it - tile * p.ktiles);
+        const int64_t left = it_end - it;
+        const int nk = (int)((int64_t)(p.ktiles - k_lo) < left ? (int64_t)(p.ktiles - k_lo) : left);
+        batch = tile / p.tiles_per_batch;
+        int tile_m, tile_n;
+        tile_of_id(tile - batch * p.tiles_per_batch, p.tiles_m, p.tiles_n, tile_m, tile_n);
+        m0 = (int64_t)tile_m * BM;
+        n0 = (int64_t)tile_n * BN;
+        A = p.a + batch * p.stride_a;
+        B = p.b + batch * p.stride_b;
+        C = p.c + batch * p.stride_c;
+
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < M::ACC; ++r) acc[i][j][r] = T(0);
+
+        load_tiles((int64_t)k_lo * BK);
+        store_tiles(0);
+        __syncthreads();
+        for (int kt = 0; kt < nk; ++kt) {
+            const int buf = kt & 1;
+            if (kt + 1 < nk) load_tiles((int64_t)(k_lo + kt + 1) * BK);
+            const T *as = As + buf * BM * S + (wm0 + lrow) * S + lk;
+            const T *bs = Bs + buf * BN * S + (wn0 + lrow) * S + lk;
+#pragma unroll
+            for (int kc = 0; kc < BK / KCH; ++kc) {
+                V af[TM], bf[TN];
+#pragma unroll
+                for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const V *>(as + i * MT * S + kc * KCH);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const V *>(bs + j * MT * S + kc * KCH);
+#pragma unroll
+                for (int e = 0; e < EPV; ++e)
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) acc[i][j] = M::mma(M::elem(af[i], e), M::elem(bf[j], e), acc[i][j]);
+            }
+            if (kt + 1 < nk) store_tiles(buf ^ 1);
+            __syncthreads();
+        }
+
+        if (nk == p.ktiles) {
+            epilogue();
+        } else {
+            // Split tile: park the accumulators; gemm_fixup_kernel adds the contributions in K order.
+            constexpr int64_t SLOT = (int64_t)BM * BN;
+            T *mine = p.partials + ((int64_t)vb * 2 + (k_lo > 0 ? 0 : 1)) * SLOT;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int r = 0; r < M::ACC; ++r) mine[((i * TN + j) * M::ACC + r) * NT + tid] = acc[i][j][r];
+        }
+        it += nk;
+    }
+}
+
+// Completes the tiles whose K range was shared by several workgroups of gemm_kernel. Workgroup b
+// (1 <= b < grid) looks at the boundary between main-kernel workgroups b - 1 and b; if that
+// boundary falls inside a tile and is the FIRST such boundary of that tile, it adds the tile's
+// slots in K order (each thread owns the same accumulator elements as in the main kernel) and
+// applies the epilogue.
+template <typename T, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM *WN *kWave) void gemm_fixup_kernel(const GemmArgs<T> p) {
+    using M = Mfma<T>;
+    constexpr int MT = M::MT;
+    constexpr int NT = WM * WN * kWave;
+    constexpr int WTM = BM / WM, WTN = BN / WN;
+    constexpr int TM = WTM / MT, TN = WTN / MT;
+    constexpr int64_t SLOT = (int64_t)BM * BN;
+    const int grid = p.grid;
+    const int64_t total = p.total_iters;
+    const int b = (int)blockIdx.x + 1;
+    const int64_t x = (int64_t)b * total / grid;  // first iteration of main-kernel workgroup b
+    const int64_t tile = x / p.ktiles;
+    const int64_t it0 = tile * p.ktiles;
+    if (x == it0) return;  // boundary on a tile edge: nothing is split here
+    auto owner_of = [&](int64_t i) { return (int)(((i + 1) * grid - 1) / total); };
+    const int b_first = owner_of(it0), b_last = owner_of(it0 + p.ktiles - 1);
+    if (b != b_first + 1) return;  // a later boundary of the same tile
+    const int nseg = b_last - b_first + 1;
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int wm0 = (wave / WN) * WTM, wn0 = (wave % WN) * WTN, lrow = lane % MT;
+    const int64_t batch = tile / p.tiles_per_batch;
+    int tile_m, tile_n;
+    tile_of_id(tile - batch * p.tiles_per_batch, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+    T *C = p.c + batch * p.stride_c;
+    const bool has_bias = (p.epilogue & FTH_EPI_BIAS) != 0;
+    const bool has_gelu = (p.epilogue & FTH_EPI_GELU) != 0;
+    const bool has_res = (p.epilogue & FTH_EPI_RESIDUAL) != 0;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int64_t col = n0 + wn0 + j * MT + lrow;
-        if (col >= p.n) continue;
-        const T bv = has_bias ? p.bias[col] : T(0);
+        const T bv = (has_bias && col < p.n) ? p.bias[col] : T(0);
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
+            T sum[M::ACC];
+            for (int sgm = 0; sgm < nseg; ++sgm) {
+                const int ob = b_first + sgm;
+                const bool starts_inside = ((int64_t)ob * total / grid) > it0;
+                const T *src = p.partials + ((int64_t)ob * 2 + (starts_inside ? 0 : 1)) * SLOT;
+#pragma unroll
+                for (int r = 0; r < M::ACC; ++r) {
+                    const T v = src[((i * TN + j) * M::ACC + r) * NT + tid];
+                    sum[r] = sgm == 0 ? v : sum[r] + v;
+                }
+            }
+            if (col >= p.n) continue;
 #pragma unroll
             for (int r = 0; r < M::ACC; ++r) {
                 const int64_t row = m0 + wm0 + i * MT + M::acc_row(r, lane);
                 if (row < p.m) {
-                    T v = acc[i][j][r];
+                    T v = sum[r];
                     if (p.use_alpha) v = p.alpha * v;
                     if (has_bias) v = v + bv;
                     if (has_gelu) v = M::gelu(v);
@@ -290,39 +469,117 @@ __global__ __launch_bounds__(256) void gemm_k0_kernel(const GemmArgs<T> p) {
     p.c[batch * p.stride_c + row * p.ldc + col] = v;
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, bool TRANS_B, bool VEC>
-int32_t launch_config(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
-    using M = Mfma<T>;
-    constexpr int S = BK + M::EPV;
-    constexpr size_t smem = (size_t)2 * (BM + BN) * S * sizeof(T);
-    auto kern = gemm_kernel<T, BM, BN, BK, WM, WN, TRANS_B, VEC>;
-    static bool attr_set = false;  // benign race: the attribute call is idempotent
-    if (!attr_set) {
-        FTH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        attr_set = true;
+// Workspace of split tiles, one per stream (two GEMMs on different streams may overlap).
+struct StreamWorkspace {
+    void *partials = nullptr;
+    size_t partial_bytes = 0;
+};
+int32_t get_workspace(hipStream_t st, size_t partial_bytes, void **partials) {
+    static std::mutex mu;
+    static std::map<hipStream_t, StreamWorkspace> *table = new std::map<hipStream_t, StreamWorkspace>();
+    std::lock_guard<std::mutex> lock(mu);
+    StreamWorkspace &w = (*table)[st];
+    if (w.partial_bytes < partial_bytes) {
+        // The old block returns to the pool; kernels already queued on this stream that still use
+        // it are ordered before whatever reuses it on the same stream.
+        fth::pool_free(w.partials);
+        w.partials = nullptr;
+        w.partial_bytes = 0;
+        if (int32_t rc = fth::pool_alloc(&w.partials, partial_bytes)) return rc;
+        w.partial_bytes = partial_bytes;
     }
-    int64_t tm = fth::ceil_div(p.m, BM), tn = fth::ceil_div(p.n, BN);
-    FTH_ARG(tm * tn <= 2147483647LL && batch <= 65535, "gemm: grid too large (tiles %lld x %lld, batch %lld)",
-            (long long)tm, (long long)tn, (long long)batch);
-    p.tiles_m = (int)tm;
-    p.tiles_n = (int)tn;
-    kern<<<dim3((unsigned)(tm * tn), (unsigned)batch), dim3(WM * WN * kWave), smem, st>>>(p);
-    FTH_CHECK_LAUNCH("gemm");
+    *partials = w.partials;
     return FTH_OK;
 }
 
-template <typename T, bool TRANS_B, bool VEC>
+constexpr int kMinItersPerBlock = 4;  // never cut the iteration space finer than this many K-tiles
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool TRANS_B, bool VEC, bool VECB>
+int32_t launch_config(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
+    using M = Mfma<T>;
+    constexpr int S = BK + M::EPV;
+    constexpr int NT = WM * WN * kWave;
+    constexpr size_t smem = (size_t)2 * (BM + BN) * S * sizeof(T);
+    auto kern = gemm_kernel<T, BM, BN, BK, WM, WN, MINW, TRANS_B, VEC, VECB>;
+    static int blocks_per_cu = 0;  // benign race: both calls are idempotent
+    if (blocks_per_cu == 0) {
+        FTH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        int nb = 0;
+        FTH_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, kern, NT, smem));
+        blocks_per_cu = nb > 0 ? nb : 1;
+    }
+    const int64_t tm = fth::ceil_div(p.m, BM), tn = fth::ceil_div(p.n, BN);
+    const int64_t ktiles = fth::ceil_div(p.k, BK);
+    FTH_ARG(tm <= 2147483647LL && tn <= 2147483647LL && ktiles <= 2147483647LL, "gemm: extent too large");
+    int64_t tiles, total;
+    if (__builtin_mul_overflow(tm, tn, &tiles) || __builtin_mul_overflow(tiles, batch, &total) || total > 2147483647LL ||
+        __builtin_mul_overflow(total, ktiles, &total) || total > (int64_t)1 << 46)
+        return fth::set_error(FTH_ERR_SIZE_OVERFLOW, "gemm: too many tiles (%lld x %lld x batch %lld)", (long long)tm, (long long)tn,
+                              (long long)batch);
+    const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
+    int64_t grid = (int64_t)cus * blocks_per_cu;
+    const int64_t cap = total / kMinItersPerBlock > 0 ? total / kMinItersPerBlock : 1;
+    if (grid > cap) grid = cap;
+    p.tiles_m = (int)tm;
+    p.tiles_n = (int)tn;
+    p.ktiles = (int)ktiles;
+    p.tiles_per_batch = tm * tn;
+    p.total_iters = total;
+    p.grid = (int)grid;
+    // A tile is split when a workgroup boundary b * total / grid is not a multiple of ktiles.
+    bool any_split = false;
+    if (grid > 1) {
+        const int64_t per = total / grid;
+        any_split = !(total % grid == 0 && per % ktiles == 0);
+    }
+    void *partials = nullptr;
+    if (any_split)
+        if (int32_t rc = get_workspace(st, (size_t)grid * 2 * BM * BN * sizeof(T), &partials)) return rc;
+    p.partials = static_cast<T *>(partials);
+    kern<<<dim3((unsigned)grid), dim3(NT), smem, st>>>(p);
+    FTH_CHECK_LAUNCH("gemm");
+    if (any_split) {
+        gemm_fixup_kernel<T, BM, BN, WM, WN><<<dim3((unsigned)(grid - 1)), dim3(NT), 0, st>>>(p);
+        FTH_CHECK_LAUNCH("gemm_fixup");
+    }
+    return FTH_OK;
+}
+
+// Tile configurations. The choice depends on the shape only (never on timing), so a given problem
+// always runs the same kernel and reproduces its bits.
+enum class Tile { Big, Wide, Small };
+
+inline int forced_tile() {
+    static const int v = [] {
+        const char *e = std::getenv("FT_HIP_GEMM_TILE");  // tuning knob: 0 = 128x128, 1 = 256x128, 2 = 64x64
+        return e ? std::atoi(e) : -1;
+    }();
+    return v;
+}
+
+template <typename T, bool TRANS_B, bool VEC, bool VECB>
 int32_t launch_shape(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     // Large problems: 128x128 tiles (2x2 wavefronts of 64x64). Problems too small to give every
     // CU a large tile: 64x64 tiles (2x2 wavefronts of 32x32).
     const int64_t big_tiles = fth::ceil_div(p.m, 128) * fth::ceil_div(p.n, 128) * batch;
     const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
+    Tile t = big_tiles >= cus ? Tile::Big : Tile::Small;
+    const int f = forced_tile();
+    if (f == 0) t = Tile::Big;
+    if (f == 1) t = Tile::Wide;
+    if (f == 2) t = Tile::Small;
     if constexpr (std::is_same<T, float>::value) {
-        if (big_tiles >= cus) return launch_config<T, 128, 128, 32, 2, 2, TRANS_B, VEC>(p, batch, st);
-        return launch_config<T, 64, 64, 32, 2, 2, TRANS_B, VEC>(p, batch, st);
+        switch (t) {
+            case Tile::Big: return launch_config<T, 128, 128, FTH_F32_BK, 2, 2, FTH_F32_MINW, TRANS_B, VEC, VECB>(p, batch, st);
+            case Tile::Wide: return launch_config<T, 256, 128, 16, 2, 2, 2, TRANS_B, VEC, VECB>(p, batch, st);
+            default: return launch_config<T, 64, 64, 32, 2, 2, 1, TRANS_B, VEC, VECB>(p, batch, st);
+        }
     } else {
-        if (big_tiles >= cus) return launch_config<T, 128, 128, 16, 2, 2, TRANS_B, VEC>(p, batch, st);
-        return launch_config<T, 64, 64, 16, 2, 2, TRANS_B, VEC>(p, batch, st);
+        switch (t) {
+            case Tile::Big:
+            case Tile::Wide: return launch_config<T, 128, 128, 16, 2, 2, 1, TRANS_B, VEC, VECB>(p, batch, st);
+            default: return launch_config<T, 64, 64, 16, 2, 2, 1, TRANS_B, VEC, VECB>(p, batch, st);
+        }
     }
 }
 
@@ -364,9 +621,13 @@ int32_t gemm_entry(const fth_gemm_desc *d, T alpha, const T *a, const T *b, T *c
     bool vec = d->k % EPV == 0 && d->lda % EPV == 0 && al(a) && d->stride_a % EPV == 0;
     if (d->trans_b) vec = vec && d->ldb % EPV == 0 && al(b) && d->stride_b % EPV == 0;
     if (d->trans_b) {
-        return vec ? launch_shape<T, true, true>(p, d->batch, st) : launch_shape<T, true, false>(p, d->batch, st);
+        return vec ? launch_shape<T, true, true, false>(p, d->batch, st) : launch_shape<T, true, false, false>(p, d->batch, st);
     }
-    return vec ? launch_shape<T, false, true>(p, d->batch, st) : launch_shape<T, false, false>(p, d->batch, st);
+    // [k, n] B: 128-bit loads along n need n, ldb and the base to be vector multiples (and k, so
+    // that a register block never straddles the k edge).
+    const bool vecb = d->n % EPV == 0 && d->k % EPV == 0 && d->ldb % EPV == 0 && al(b) && d->stride_b % EPV == 0;
+    if (vec) return vecb ? launch_shape<T, false, true, true>(p, d->batch, st) : launch_shape<T, false, true, false>(p, d->batch, st);
+    return vecb ? launch_shape<T, false, false, true>(p, d->batch, st) : launch_shape<T, false, false, false>(p, d->batch, st);
 }
 
 }  // namespace
