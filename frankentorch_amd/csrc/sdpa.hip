@@ -5,7 +5,7 @@
 // limit = min(qi + 1, seq_k) keys when causal (all seq_k otherwise), entries past the limit are
 // exactly zero, out = P.V. The reference materialises a [64, seq_k] score tile per block and
 // normalises P before the second product; this kernel never materialises scores: it walks the
-// keys in tiles of 32 with an online softmax (running max m, running sum l, rescaled
+// keys in tiles of 32 or 64 with an online softmax (running max m, running sum l, rescaled
 // accumulator) and divides by l once at the end. Same mathematics, different rounding order:
 // covered by the 2e-5 tolerance of the parity tests.
 //
@@ -24,9 +24,11 @@
 //                                       feeding the NDT d-tiles.
 // No atomics, no split over keys across wavefronts: bitwise repeatable.
 //
-// Tile order: blocks of one (batch, head) are given to one XCD so that its K/V (<= a few MB)
-// stay in that XCD's L2, and the long (late) query blocks of a causal problem are issued first.
+// Work order: a causal workgroup runs a long query block and then the matching short one, so all
+// workgroups carry the same work; units are issued heaviest first across all heads; and a
+// (batch, head) always lands on the same XCD when the head count is a multiple of 8.
 
+#include <cstdlib>
 #include <type_traits>
 
 #include "common.hpp"
@@ -35,8 +37,6 @@ namespace {
 
 constexpr int kWave = 64;
 constexpr int kXcds = 8;
-constexpr int kBQ = 128;  // queries per block (4 wavefronts x 32)
-constexpr int kBC = 32;   // keys per tile
 
 using Acc16 = float __attribute__((ext_vector_type(16)));
 
@@ -48,6 +48,14 @@ struct SdpaArgs {
     int q_blocks;
 };
 
+// exp(x - m) for x <= m as 2^((x - m) * log2 e) on the hardware exp2 unit: subtract, multiply,
+// v_exp_f32. The subtraction is exact or nearly so; rounding the product costs a relative error of
+// about |x - m| * 2^-24 in the result, i.e. < 1e-6 for every weight that is not already
+// negligible, far inside the 2e-5 parity tolerance. x = -inf gives exactly 0.
+__device__ __forceinline__ float exp_diff(float x, float m) {
+    return __builtin_amdgcn_exp2f((x - m) * 1.44269502162933349609375f);
+}
+
 template <int N> struct VecN;
 template <> struct VecN<1> { using type = float; };
 template <> struct VecN<2> { using type = float2; };
@@ -57,15 +65,24 @@ __device__ __forceinline__ float vecn_get(const float2 &v, int e) { return e == 
 __device__ __forceinline__ float vecn_get(const float4 &v, int e) { return e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w; }
 __device__ __forceinline__ float f4_get(const float4 &v, int e) { return e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w; }
 
-template <int D>
-__global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs p) {
+// D: head size (32, 64, 128). NW: wavefronts per block (4 or 2); a block owns 32 * NW consecutive
+// queries per pass. PAIR: causal balancing -- the block runs two passes, query block
+// (q_blocks - 1 - p) and then query block p, so every block does the same amount of work.
+// BC: keys per tile (32, or 64 for the small head sizes, which halves the barriers and the
+// cross-lane softmax steps per key).
+template <int D, int NW, bool PAIR, int BC>
+__global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p) {
+    constexpr int kBC = BC;
+    constexpr int KS = BC / 32;        // 32-key sub-tiles per tile
+    constexpr int NTH = 64 * NW;
+    constexpr int BQ = 32 * NW;
     constexpr int NDT = D / 32;        // 32-wide d-tiles of the output
     constexpr int KP = D + 4;          // K tile row pitch (odd number of 16-byte vectors)
     constexpr int VP = D + 8;          // V tile row pitch (rows j and j+4 land 32 banks apart)
     constexpr int KT = kBC * KP;       // floats per K tile
     constexpr int VT = kBC * VP;
-    constexpr int NV = kBC * (D / 4) / 256;  // float4 per thread per tile
-    static_assert(kBC * (D / 4) % 256 == 0, "tile must divide over the block");
+    constexpr int NV = kBC * (D / 4) / NTH;  // float4 per thread per tile
+    static_assert(kBC * (D / 4) % NTH == 0, "tile must divide over the block");
     using VV = typename VecN<NDT>::type;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -76,20 +93,22 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs p) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lq = lane & 31, half = lane >> 5;
 
-    // ---- which (bh, query block) ----
+    // ---- which (bh, unit): a unit is a query block, or a (heavy, light) pair of them ----
+    const int units = PAIR ? (p.q_blocks + 1) / 2 : p.q_blocks;
     int64_t bh;
-    int qb;
+    int unit;
     {
+        // Units are issued heaviest first across ALL heads (unit index is the slow digit), and
+        // when the head count allows it a head always lands on the same XCD.
         const int64_t pid = blockIdx.x;
         if (d.num_bh % kXcds == 0) {
-            const int64_t xcd = pid % kXcds, w = pid / kXcds;
-            bh = (w / p.q_blocks) * kXcds + xcd;
-            qb = (int)(w % p.q_blocks);
+            const int64_t xcd = pid % kXcds, w = pid / kXcds, per = d.num_bh / kXcds;
+            unit = (int)(w / per);
+            bh = (w % per) * kXcds + xcd;
         } else {
-            bh = pid / p.q_blocks;
-            qb = (int)(pid % p.q_blocks);
+            unit = (int)(pid / d.num_bh);
+            bh = pid % d.num_bh;
         }
-        qb = p.q_blocks - 1 - qb;  // longest causal rows first
     }
     const int64_t b = bh / d.heads, h = bh % d.heads;
     const float *Q = static_cast<const float *>(p.q) + b * d.q_batch_stride + h * d.q_head_stride;
@@ -98,147 +117,176 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_kernel(const SdpaArgs p) {
     float *O = static_cast<float *>(p.out) + b * d.o_batch_stride + h * d.o_head_stride;
     const float scale = (float)p.scale;
 
-    const int64_t q_blk0 = (int64_t)qb * kBQ;
-    const int64_t q_wave0 = q_blk0 + wave * 32;
-    const int64_t qi = q_wave0 + lq;  // this lane's query
-    const bool q_live = qi < d.seq_q;
+    const int qb_first = p.q_blocks - 1 - unit;  // the long rows of a causal problem first
+    const int npass = (PAIR && unit != qb_first) ? 2 : 1;
 
-    // ---- Q rows into registers: lane holds Q[qi][8t + 4*half + e] ----
-    float4 qr[D / 8];
+    for (int pass = 0; pass < npass; ++pass) {
+        const int qb = pass == 0 ? qb_first : unit;
+        // Row indices inside one head fit 32 bits (the launcher checks seq_q, seq_k < 2^31).
+        const int q_blk0 = qb * BQ;
+        const int q_wave0 = q_blk0 + wave * 32;
+        const int qi = q_wave0 + lq;  // this lane's query
+        const int seq_q_i = (int)d.seq_q;
+        const bool q_live = qi < seq_q_i;
+
+        // ---- Q rows into registers: lane holds Q[qi][8t + 4*half + e] ----
+        float4 qr[D / 8];
 #pragma unroll
-    for (int t = 0; t < D / 8; ++t) {
-        qr[t] = q_live ? *reinterpret_cast<const float4 *>(Q + qi * d.q_row_stride + 8 * t + 4 * half)
-                       : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-
-    // ---- key range ----
-    int64_t blk_last_q = q_blk0 + kBQ - 1;
-    if (blk_last_q > d.seq_q - 1) blk_last_q = d.seq_q - 1;
-    int64_t k_end = d.seq_k;  // exclusive
-    if (d.causal && blk_last_q + 1 < k_end) k_end = blk_last_q + 1;
-    const int num_kt = (int)((k_end + kBC - 1) / kBC);
-    int64_t wave_last_q = q_wave0 + 31;
-    if (wave_last_q > d.seq_q - 1) wave_last_q = d.seq_q - 1;
-
-    float4 kst[NV], vst[NV];
-    auto load_tile = [&](int kt) {
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int vid = tid + i * 256;
-            const int row = vid / (D / 4), c = vid % (D / 4);
-            const int64_t key = (int64_t)kt * kBC + row;
-            if (key < d.seq_k) {
-                kst[i] = *reinterpret_cast<const float4 *>(K + key * d.k_row_stride + 4 * c);
-                vst[i] = *reinterpret_cast<const float4 *>(Vg + key * d.v_row_stride + 4 * c);
-            } else {
-                kst[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-                vst[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-            }
+        for (int t = 0; t < D / 8; ++t) {
+            qr[t] = q_live ? *reinterpret_cast<const float4 *>(Q + (int64_t)qi * d.q_row_stride + 8 * t + 4 * half)
+                           : make_float4(0.f, 0.f, 0.f, 0.f);
         }
-    };
-    auto store_tile = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int vid = tid + i * 256;
-            const int row = vid / (D / 4), c = vid % (D / 4);
-            *reinterpret_cast<float4 *>(Ks + buf * KT + row * KP + 4 * c) = kst[i];
-            *reinterpret_cast<float4 *>(Vs + buf * VT + row * VP + 4 * c) = vst[i];
-        }
-    };
 
-    Acc16 o[NDT];
-#pragma unroll
-    for (int e = 0; e < NDT; ++e)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) o[e][r] = 0.f;
-    float m_run = -__builtin_inff();
-    float l_run = 0.f;
+        // ---- key range ----
+        int blk_last_q = q_blk0 + BQ - 1;
+        if (blk_last_q > seq_q_i - 1) blk_last_q = seq_q_i - 1;
+        int k_end = (int)d.seq_k;  // exclusive
+        if (d.causal && blk_last_q + 1 < k_end) k_end = blk_last_q + 1;
+        const int num_kt = (k_end + kBC - 1) / kBC;
+        int wave_last_q = q_wave0 + 31;
+        if (wave_last_q > seq_q_i - 1) wave_last_q = seq_q_i - 1;
 
-    if (num_kt > 0) {
-        load_tile(0);
-        store_tile(0);
-    }
-    __syncthreads();
-
-    for (int kt = 0; kt < num_kt; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < num_kt) load_tile(kt + 1);
-        const int64_t key0 = (int64_t)kt * kBC;
-        // A wavefront whose every query precedes this tile's first key has nothing to add.
-        const bool wave_active = !d.causal || key0 <= wave_last_q;
-        if (wave_active) {
-            // ---- S^T = K_tile . Q^T ----
-            Acc16 s;
+        // Tile loader: thread owns column vector ld_c of rows ld_row + i * RS; everything that
+        // changes per tile or per i is wavefront-uniform, so the per-lane address is one base.
+        constexpr int RS = NTH / (D / 4);  // rows covered by one sweep of the block
+        const int ld_row = tid / (D / 4), ld_c = tid % (D / 4);
+        const int seq_k_i = (int)d.seq_k;
+        float4 kst[NV], vst[NV];
+        const float *kbase = K + (int64_t)ld_row * d.k_row_stride + 4 * ld_c;
+        const float *vbase = Vg + (int64_t)ld_row * d.v_row_stride + 4 * ld_c;
+        auto load_tile = [&](int kt) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s[r] = 0.f;
-            const float *kp = Ks + buf * KT + lq * KP + 4 * half;
-#pragma unroll
-            for (int t = 0; t < D / 8; ++t) {
-                const float4 kv = *reinterpret_cast<const float4 *>(kp + 8 * t);
-                s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.x, qr[t].x, s, 0, 0, 0);
-                s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.y, qr[t].y, s, 0, 0, 0);
-                s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.z, qr[t].z, s, 0, 0, 0);
-                s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.w, qr[t].w, s, 0, 0, 0);
-            }
-            // ---- scale, mask, online softmax (lane-local query) ----
-            const bool need_mask = (d.causal && key0 + kBC - 1 > q_wave0) || (key0 + kBC > d.seq_k);
-            float sv[16];
-            float mt = -__builtin_inff();
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float x = s[r] * scale;
-                if (need_mask) {
-                    const int64_t key = key0 + 8 * (r >> 2) + 4 * half + (r & 3);
-                    if ((d.causal && key > qi) || key >= d.seq_k) x = -__builtin_inff();
+            for (int i = 0; i < NV; ++i) {
+                const int row0 = kt * kBC + i * RS;  // uniform
+                if (row0 + ld_row < seq_k_i) {
+                    kst[i] = *reinterpret_cast<const float4 *>(kbase + (int64_t)row0 * d.k_row_stride);
+                    vst[i] = *reinterpret_cast<const float4 *>(vbase + (int64_t)row0 * d.v_row_stride);
+                } else {
+                    kst[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    vst[i] = make_float4(0.f, 0.f, 0.f, 0.f);
                 }
-                sv[r] = x;
-                mt = fmaxf(mt, x);
             }
-            mt = fmaxf(mt, __shfl_xor(mt, 32, kWave));
-            const float m_new = fmaxf(m_run, mt);
-            const float alpha = expf(m_run - m_new);
-            float psum = 0.f;
+        };
+        float *ks_st = Ks + ld_row * KP + 4 * ld_c;
+        float *vs_st = Vs + ld_row * VP + 4 * ld_c;
+        auto store_tile = [&](int buf) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float e = expf(sv[r] - m_new);
-                sv[r] = e;
-                psum += e;
+            for (int i = 0; i < NV; ++i) {
+                *reinterpret_cast<float4 *>(ks_st + buf * KT + i * RS * KP) = kst[i];
+                *reinterpret_cast<float4 *>(vs_st + buf * VT + i * RS * VP) = vst[i];
             }
-            psum += __shfl_xor(psum, 32, kWave);
-            l_run = l_run * alpha + psum;
-            m_run = m_new;
-            if (__any(alpha != 1.0f)) {
-#pragma unroll
-                for (int e = 0; e < NDT; ++e)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) o[e][r] *= alpha;
-            }
-            // ---- O^T += V_tile^T . P^T ----
-            const float *vp = Vs + buf * VT + (4 * half) * VP + NDT * lq;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const VV vv = *reinterpret_cast<const VV *>(vp + (8 * (r >> 2) + (r & 3)) * VP);
-#pragma unroll
-                for (int e = 0; e < NDT; ++e)
-                    o[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(vv, e), sv[r], o[e], 0, 0, 0);
-            }
-        }
-        if (kt + 1 < num_kt) store_tile(buf ^ 1);
-        __syncthreads();
-    }
+        };
 
-    // ---- normalise and store: lane owns query qi, d = NDT * rho + e ----
-    if (q_live) {
-        float *orow = O + qi * d.o_row_stride;
+        Acc16 o[NDT];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int rho = 8 * (r >> 2) + 4 * half + (r & 3);
-            float ov[NDT];
+        for (int e = 0; e < NDT; ++e)
 #pragma unroll
-            for (int e = 0; e < NDT; ++e) ov[e] = (num_kt > 0) ? o[e][r] / l_run : 0.f;
-            if constexpr (NDT == 4) *reinterpret_cast<float4 *>(orow + 4 * rho) = make_float4(ov[0], ov[1], ov[2], ov[3]);
-            else if constexpr (NDT == 2) *reinterpret_cast<float2 *>(orow + 2 * rho) = make_float2(ov[0], ov[1]);
-            else orow[rho] = ov[0];
+            for (int r = 0; r < 16; ++r) o[e][r] = 0.f;
+        float m_run = -__builtin_inff();
+        float l_run = 0.f;
+
+        if (num_kt > 0) {
+            load_tile(0);
+            store_tile(0);
+        }
+        __syncthreads();
+
+        for (int kt = 0; kt < num_kt; ++kt) {
+            const int buf = kt & 1;
+            const int key0 = kt * kBC;
+            // A wavefront whose every query precedes this tile's first key has nothing to add.
+            const bool wave_active = !d.causal || key0 <= wave_last_q;
+            // ---- S^T = K_tile . Q^T, one 32-key sub-tile per accumulator ----
+            Acc16 s[KS];
+            if (wave_active) {
+#pragma unroll
+                for (int j = 0; j < KS; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) s[j][r] = 0.f;
+                const float *kp = Ks + buf * KT + lq * KP + 4 * half;
+#pragma unroll
+                for (int t = 0; t < D / 8; ++t) {
+#pragma unroll
+                    for (int j = 0; j < KS; ++j) {
+                        const float4 kv = *reinterpret_cast<const float4 *>(kp + j * 32 * KP + 8 * t);
+                        s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.x, qr[t].x, s[j], 0, 0, 0);
+                        s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.y, qr[t].y, s[j], 0, 0, 0);
+                        s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.z, qr[t].z, s[j], 0, 0, 0);
+                        s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.w, qr[t].w, s[j], 0, 0, 0);
+                    }
+                }
+            }
+            // The next tile's global loads are issued here, after the score MFMAs and before the
+            // softmax: their latency is covered by the softmax and the P.V MFMAs, and their address
+            // temporaries cannot be handed the registers the score accumulator is about to claim
+            // (which makes the compiler wait for every load in flight before the first MFMA).
+            if (kt + 1 < num_kt) load_tile(kt + 1);
+            if (wave_active) {
+                // ---- scale, mask, online softmax (lane-local query) ----
+                const bool need_mask = (d.causal && key0 + kBC - 1 > q_wave0) || (key0 + kBC > seq_k_i);
+                float mt = -__builtin_inff();
+#pragma unroll
+                for (int j = 0; j < KS; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        float x = s[j][r] * scale;
+                        if (need_mask) {
+                            const int key = key0 + 32 * j + 8 * (r >> 2) + 4 * half + (r & 3);
+                            if ((d.causal && key > qi) || key >= seq_k_i) x = -__builtin_inff();
+                        }
+                        s[j][r] = x;
+                        mt = fmaxf(mt, x);
+                    }
+                mt = fmaxf(mt, __shfl_xor(mt, 32, kWave));
+                const float m_new = fmaxf(m_run, mt);
+                const float alpha = exp_diff(m_run, m_new);
+                float psum = 0.f;
+#pragma unroll
+                for (int j = 0; j < KS; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const float e = exp_diff(s[j][r], m_new);
+                        s[j][r] = e;
+                        psum += e;
+                    }
+                psum += __shfl_xor(psum, 32, kWave);
+                l_run = l_run * alpha + psum;
+                m_run = m_new;
+                if (__any(alpha != 1.0f)) {
+#pragma unroll
+                    for (int e = 0; e < NDT; ++e)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) o[e][r] *= alpha;
+                }
+                // ---- O^T += V_tile^T . P^T ----
+                const float *vp = Vs + buf * VT + (4 * half) * VP + NDT * lq;
+#pragma unroll
+                for (int j = 0; j < KS; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const VV vv = *reinterpret_cast<const VV *>(vp + (32 * j + 8 * (r >> 2) + (r & 3)) * VP);
+#pragma unroll
+                        for (int e = 0; e < NDT; ++e)
+                            o[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(vv, e), s[j][r], o[e], 0, 0, 0);
+                    }
+            }
+            if (kt + 1 < num_kt) store_tile(buf ^ 1);
+            __syncthreads();
+        }
+
+        // ---- normalise and store: lane owns query qi, d = NDT * rho + e ----
+        if (q_live) {
+            float *orow = O + (int64_t)qi * d.o_row_stride;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int rho = 8 * (r >> 2) + 4 * half + (r & 3);
+                float ov[NDT];
+#pragma unroll
+                for (int e = 0; e < NDT; ++e) ov[e] = (num_kt > 0) ? o[e][r] / l_run : 0.f;
+                if constexpr (NDT == 4) *reinterpret_cast<float4 *>(orow + 4 * rho) = make_float4(ov[0], ov[1], ov[2], ov[3]);
+                else if constexpr (NDT == 2) *reinterpret_cast<float2 *>(orow + 2 * rho) = make_float2(ov[0], ov[1]);
+                else orow[rho] = ov[0];
+            }
         }
     }
 }
@@ -318,19 +366,43 @@ __global__ __launch_bounds__(64) void sdpa_generic_kernel(const SdpaArgs p) {
     }
 }
 
-template <int D> int32_t launch_mfma(const SdpaArgs &a, hipStream_t st) {
-    constexpr size_t smem = (size_t)2 * kBC * ((D + 4) + (D + 8)) * sizeof(float);
-    auto kern = sdpa_mfma_kernel<D>;
+template <int D, int NW, bool PAIR> int32_t launch_mfma_cfg(SdpaArgs &a, hipStream_t st) {
+    constexpr int BC = (D <= 64 && (NW == 4 || D <= 32)) ? 64 : 32;  // 64-key tiles where the staging registers fit
+    constexpr size_t smem = (size_t)2 * BC * ((D + 4) + (D + 8)) * sizeof(float);
+    auto kern = sdpa_mfma_kernel<D, NW, PAIR, BC>;
     static bool attr_set = false;
     if (!attr_set) {
         FTH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    const int64_t grid = a.d.num_bh * a.q_blocks;
+    a.q_blocks = (int)fth::ceil_div(a.d.seq_q, 32 * NW);
+    const int64_t units = PAIR ? (a.q_blocks + 1) / 2 : a.q_blocks;
+    const int64_t grid = a.d.num_bh * units;
     FTH_ARG(grid <= 2147483647LL, "sdpa: grid too large");
-    kern<<<dim3((unsigned)grid), dim3(256), smem, st>>>(a);
+    kern<<<dim3((unsigned)grid), dim3(64 * NW), smem, st>>>(a);
     FTH_CHECK_LAUNCH("sdpa_mfma");
     return FTH_OK;
+}
+
+// Blocks of 128 queries (4 wavefronts) are used whenever they still give every other CU a
+// workgroup; shorter problems fall back to blocks of 64 queries. Workgroups are issued heaviest
+// first, which balances causal problems well enough that pairing a long with a short query
+// block per workgroup (kept behind the tuning knob) measured no faster.
+template <int D> int32_t launch_mfma(SdpaArgs &a, hipStream_t st) {
+    bool pair = false;
+    const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
+    const int64_t wg128 = a.d.num_bh * fth::ceil_div(a.d.seq_q, 128);
+    bool wide = D >= 128 || 2 * wg128 >= (int64_t)cus;  // D = 128 staging does not fit 2-wavefront blocks
+    static const int forced = [] {
+        const char *e = std::getenv("FT_HIP_SDPA_CFG");  // tuning knob: bit 0 = 4 wavefronts, bit 1 = pairing; -1 = auto
+        return e ? std::atoi(e) : -1;
+    }();
+    if (forced >= 0) {
+        wide = D >= 128 || (forced & 1);
+        pair = a.d.causal != 0 && (forced & 2);
+    }
+    if (pair) return wide ? launch_mfma_cfg<D, 4, true>(a, st) : launch_mfma_cfg<D, 2, true>(a, st);
+    return wide ? launch_mfma_cfg<D, 4, false>(a, st) : launch_mfma_cfg<D, 2, false>(a, st);
 }
 
 template <typename T>
@@ -342,10 +414,11 @@ int32_t sdpa_entry(const fth_sdpa_desc *d, double scale, const T *q, const T *k,
             (long long)d->heads, (long long)d->num_bh);
     if (d->num_bh == 0 || d->seq_q == 0 || d->d_v == 0) return FTH_OK;
     FTH_ARG(q && k && v && out, "sdpa: NULL operand");
+    FTH_ARG(d->seq_q < 2147483647LL - 256 && d->seq_k < 2147483647LL - 256, "sdpa: sequence too long");
     hipStream_t st = fth::resolve_stream(s);
     SdpaArgs a;
     a.q = q; a.k = k; a.v = v; a.out = out; a.d = *d; a.scale = scale;
-    a.q_blocks = (int)fth::ceil_div(d->seq_q, kBQ);
+    a.q_blocks = 0;  // set by the launcher of the chosen variant
     auto al16 = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; };
     auto m4 = [](int64_t x) { return x % 4 == 0; };
     if constexpr (std::is_same<T, float>::value) {
