@@ -60,6 +60,13 @@ def event_time_ms(device, launch, iters):
     return e0.elapsed_ms(e1) / iters
 
 
+# HBM bytes per launch at fp32 [8192,4096], from two rocprofv3 --pmc runs of this file (FETCH_SIZE, then WRITE_SIZE),
+# each scaled by what the same counter reads for the GELU kernel, a plain copy of 2 x 128 MiB (factors 0.5004 and 1.0006).
+# Counters cannot be read from inside the process, so these are the figures of the committed profile summary.
+MEASURED_HBM_TRAFFIC = {"softmax": 268778238, "layer_norm": 268800070, "rms_norm": 268650774, "gelu": 268435456,
+                        "bias_residual_add": 402521496}
+
+
 def bench_rowops(device, synth, steps, warmup, with_cpu):
     from frankentorch_amd.device import DeviceBuffer
 
@@ -106,7 +113,7 @@ def bench_rowops(device, synth, steps, warmup, with_cpu):
         log("[rowops] %-18s %.4f ms  %7.1f GB/s  %.1f%% of HBM peak" % (name, ms, gbs, 100 * gbs / HBM_PEAK_GBS))
     dominant = max(per_kernel, key=lambda k: per_kernel[k]["ms"])
     roof = {"bound": "hbm", "kernel": dominant, "achieved": per_kernel[dominant]["GB/s"], "peak": HBM_PEAK_GBS,
-            "unit": "GB/s", "frac": per_kernel[dominant]["frac"], "traffic": None}
+            "unit": "GB/s", "frac": per_kernel[dominant]["frac"], "traffic": MEASURED_HBM_TRAFFIC.get(dominant)}
 
     cpu = None
     if with_cpu:
