@@ -372,6 +372,8 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_kernel(const GemmArg
             epilogue();
         } else {
             // Split tile: park the accumulators; gemm_fixup_kernel adds the contributions in K order.
+            // Slot layout: the thread's TM * TN * ACC values in flat order e, as 16-byte vectors
+            // interleaved over the threads ([e / EPV][tid][e % EPV]), so both sides move whole vectors.
             constexpr int64_t SLOT = (int64_t)BM * BN;
             T *mine = p.partials + ((int64_t)vb * 2 + (k_lo > 0 ? 0 : 1)) * SLOT;
 #pragma unroll
@@ -379,24 +381,37 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_kernel(const GemmArg
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
 #pragma unroll
-                    for (int r = 0; r < M::ACC; ++r) mine[((i * TN + j) * M::ACC + r) * NT + tid] = acc[i][j][r];
+                    for (int r = 0; r < M::ACC; r += EPV) {
+                        T e[EPV];
+#pragma unroll
+                        for (int q = 0; q < EPV; ++q) e[q] = acc[i][j][r + q];
+                        const int ev = ((i * TN + j) * M::ACC + r) / EPV;
+                        *reinterpret_cast<V *>(mine + ((int64_t)ev * NT + tid) * EPV) = M::make(e);
+                    }
         }
         it += nk;
     }
 }
 
-// Completes the tiles whose K range was shared by several workgroups of gemm_kernel. Workgroup b
-// (1 <= b < grid) looks at the boundary between main-kernel workgroups b - 1 and b; if that
-// boundary falls inside a tile and is the FIRST such boundary of that tile, it adds the tile's
-// slots in K order (each thread owns the same accumulator elements as in the main kernel) and
-// applies the epilogue.
+// Completes the tiles whose K range was shared by several workgroups of gemm_kernel. Workgroup
+// (b, part) (1 <= b < grid) looks at the boundary between main-kernel workgroups b - 1 and b; if
+// that boundary falls inside a tile and is the FIRST such boundary of that tile, it adds the
+// tile's slots in K order and applies the epilogue for one of kFixupParts equal shares of the
+// values each thread owned in the main kernel.
+constexpr int kFixupParts = 4;
+
 template <typename T, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM *WN *kWave) void gemm_fixup_kernel(const GemmArgs<T> p) {
     using M = Mfma<T>;
-    constexpr int MT = M::MT;
+    using V = typename M::V;
+    constexpr int MT = M::MT, EPV = M::EPV;
     constexpr int NT = WM * WN * kWave;
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / MT, TN = WTN / MT;
+    constexpr int PER = TM * TN * M::ACC;   // values per thread and slot
+    constexpr int PV = PER / kFixupParts;   // values this workgroup sums per thread
+    constexpr int NV = PV / EPV;
+    static_assert(PER % (kFixupParts * EPV) == 0 && M::ACC % EPV == 0, "slot share must be whole vectors");
     constexpr int64_t SLOT = (int64_t)BM * BN;
     const int grid = p.grid;
     const int64_t total = p.total_iters;
@@ -412,6 +427,33 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemm_fixup_kernel(const GemmArg
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const int wm0 = (wave / WN) * WTM, wn0 = (wave % WN) * WTN, lrow = lane % MT;
+    const int ev0 = (int)blockIdx.y * NV;  // first vector of this workgroup's share
+    auto slot_of = [&](int ob) {
+        const bool starts_inside = ((int64_t)ob * total / grid) > it0;
+        return p.partials + ((int64_t)ob * 2 + (starts_inside ? 0 : 1)) * SLOT + ((int64_t)ev0 * NT + tid) * EPV;
+    };
+    // The first two contributions are fetched together (every split tile has at least two).
+    V s0[NV], s1[NV];
+    const T *src0 = slot_of(b_first), *src1 = slot_of(b_first + 1);
+#pragma unroll
+    for (int v = 0; v < NV; ++v) s0[v] = *reinterpret_cast<const V *>(src0 + (int64_t)v * NT * EPV);
+#pragma unroll
+    for (int v = 0; v < NV; ++v) s1[v] = *reinterpret_cast<const V *>(src1 + (int64_t)v * NT * EPV);
+    T sum[PV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+        for (int q = 0; q < EPV; ++q) sum[v * EPV + q] = M::elem(s0[v], q) + M::elem(s1[v], q);
+    for (int sgm = 2; sgm < nseg; ++sgm) {
+        const T *src = slot_of(b_first + sgm);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) s0[v] = *reinterpret_cast<const V *>(src + (int64_t)v * NT * EPV);
+#pragma unroll
+        for (int v = 0; v < NV; ++v)
+#pragma unroll
+            for (int q = 0; q < EPV; ++q) sum[v * EPV + q] = sum[v * EPV + q] + M::elem(s0[v], q);
+    }
+
     const int64_t batch = tile / p.tiles_per_batch;
     int tile_m, tile_n;
     tile_of_id(tile - batch * p.tiles_per_batch, p.tiles_m, p.tiles_n, tile_m, tile_n);
@@ -421,35 +463,18 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemm_fixup_kernel(const GemmArg
     const bool has_gelu = (p.epilogue & FTH_EPI_GELU) != 0;
     const bool has_res = (p.epilogue & FTH_EPI_RESIDUAL) != 0;
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
+    for (int u = 0; u < PV; ++u) {
+        const int e = (int)blockIdx.y * PV + u;  // flat index (i * TN + j) * ACC + r of the main kernel
+        const int r = e % M::ACC, j = (e / M::ACC) % TN, i = e / (M::ACC * TN);
         const int64_t col = n0 + wn0 + j * MT + lrow;
-        const T bv = (has_bias && col < p.n) ? p.bias[col] : T(0);
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            T sum[M::ACC];
-            for (int sgm = 0; sgm < nseg; ++sgm) {
-                const int ob = b_first + sgm;
-                const bool starts_inside = ((int64_t)ob * total / grid) > it0;
-                const T *src = p.partials + ((int64_t)ob * 2 + (starts_inside ? 0 : 1)) * SLOT;
-#pragma unroll
-                for (int r = 0; r < M::ACC; ++r) {
-                    const T v = src[((i * TN + j) * M::ACC + r) * NT + tid];
-                    sum[r] = sgm == 0 ? v : sum[r] + v;
-                }
-            }
-            if (col >= p.n) continue;
-#pragma unroll
-            for (int r = 0; r < M::ACC; ++r) {
-                const int64_t row = m0 + wm0 + i * MT + M::acc_row(r, lane);
-                if (row < p.m) {
-                    T v = sum[r];
-                    if (p.use_alpha) v = p.alpha * v;
-                    if (has_bias) v = v + bv;
-                    if (has_gelu) v = M::gelu(v);
-                    if (has_res) v = v + p.residual[batch * p.stride_c + row * p.ldc + col];
-                    C[row * p.ldc + col] = v;
-                }
-            }
+        const int64_t row = m0 + wm0 + i * MT + M::acc_row(r, lane);
+        if (col < p.n && row < p.m) {
+            T v = sum[u];
+            if (p.use_alpha) v = p.alpha * v;
+            if (has_bias) v = v + p.bias[col];
+            if (has_gelu) v = M::gelu(v);
+            if (has_res) v = v + p.residual[batch * p.stride_c + row * p.ldc + col];
+            C[row * p.ldc + col] = v;
         }
     }
 }
@@ -539,7 +564,7 @@ int32_t launch_config(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     kern<<<dim3((unsigned)grid), dim3(NT), smem, st>>>(p);
     FTH_CHECK_LAUNCH("gemm");
     if (any_split) {
-        gemm_fixup_kernel<T, BM, BN, WM, WN><<<dim3((unsigned)(grid - 1)), dim3(NT), 0, st>>>(p);
+        gemm_fixup_kernel<T, BM, BN, WM, WN><<<dim3((unsigned)(grid - 1), kFixupParts), dim3(NT), 0, st>>>(p);
         FTH_CHECK_LAUNCH("gemm_fixup");
     }
     return FTH_OK;
