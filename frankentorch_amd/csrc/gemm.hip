@@ -393,6 +393,193 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_kernel(const GemmArg
     }
 }
 
+// ---- direct-to-LDS variant for k-contiguous operands (A [m,k] and B stored [n,k]) ----
+//
+// Same tiling, schedule, accumulation order and slot format as gemm_kernel; only the way operand
+// tiles reach LDS and the LDS layout differ. A K-tile is 128 bytes of k per row (32 floats, 16
+// doubles). Tiles are written by global_load_lds (16 bytes per lane, no staging registers and no
+// LDS store instructions): one wavefront instruction fills 1 KiB of LDS in lane order, i.e.
+// 8 rows x 8 vectors, unpadded. To keep the MFMA operand reads conflict-free the vectors of a row
+// are stored XOR-swizzled: logical vector q of row r sits in slot q ^ (r & 7). The loader does the
+// swizzle on the global side (lane -> slot is fixed by the hardware, so lane (r, slot) fetches
+// vector slot ^ (r & 7) of its row); the 8 lanes of a row still cover one whole 128-byte line.
+// Rows past the m / n edge are clamped to the last valid row: a row of A (B) only feeds the same
+// row (column) of C, and those are never stored. The launcher guarantees k % BK == 0.
+// One wavefront-wide global -> LDS copy of 16 bytes per lane: lane L's 16 bytes land at
+// lds_chunk + 16 * L. Written as inline assembly so that the compiler's wait-count insertion does
+// not see an LDS write it cannot disambiguate (it would drain the load queue before every LDS
+// read and serialise the prefetch); the kernel waits for vmcnt(0) itself before each barrier.
+template <typename T> __device__ __forceinline__ void load_to_lds_16(const T *src, unsigned lds_chunk) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_chunk) : "memory", "m0");
+}
+
+template <typename T, int BM, int BN, int WM, int WN, int MINW>
+__global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const GemmArgs<T> p) {
+    using M = Mfma<T>;
+    using V = typename M::V;
+    constexpr int MT = M::MT, KG = M::KG, EPV = M::EPV;
+    constexpr int NW = WM * WN, NT = NW * kWave;
+    constexpr int BK = 128 / (int)sizeof(T);
+    constexpr int KCH = KG * EPV, NCH = BK / KCH;
+    constexpr int WTM = BM / WM, WTN = BN / WN;
+    constexpr int TM = WTM / MT, TN = WTN / MT;
+    constexpr int A_LD = BM / 8 / NW, B_LD = BN / 8 / NW;  // chunk loads per wavefront and K-tile
+    static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile rows must divide into 8-row chunks per wavefront");
+    static_assert(MT % 8 == 0, "swizzle assumes MFMA tile rows start on a multiple of 8");
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    T *As = reinterpret_cast<T *>(smem_raw);  // [2][BM][BK]
+    T *Bs = As + 2 * BM * BK;                 // [2][BN][BK]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const int wm0 = (wave / WN) * WTM;
+    const int wn0 = (wave % WN) * WTN;
+    const int lrow = lane % MT;
+    // low half of a flat LDS address = LDS offset
+    const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)reinterpret_cast<uintptr_t>(smem_raw));
+    const unsigned wave_u = __builtin_amdgcn_readfirstlane((unsigned)wave);
+    const int lr = lane >> 3;                           // loader: row inside the chunk
+    const int lvec = ((lane & 7) ^ lr) * EPV;           // loader: k offset of the vector this lane fetches
+    int roff[NCH];                                      // reader: swizzled k offset per operand fetch
+#pragma unroll
+    for (int kc = 0; kc < NCH; ++kc) roff[kc] = ((kc * KG + lane / MT) ^ (lrow & 7)) * EPV;
+
+    const bool has_bias = (p.epilogue & FTH_EPI_BIAS) != 0;
+    const bool has_gelu = (p.epilogue & FTH_EPI_GELU) != 0;
+    const bool has_res = (p.epilogue & FTH_EPI_RESIDUAL) != 0;
+
+    const int grid = (int)gridDim.x;
+    const int vb = xcd_contiguous_id((int)blockIdx.x, grid);
+    const int64_t total = p.total_iters;
+    int64_t it = (int64_t)vb * total / grid;
+    const int64_t it_end = (int64_t)(vb + 1) * total / grid;
+
+    typename M::Acc acc[TM][TN];
+
+    while (it < it_end) {
+        const int64_t tile = it / p.ktiles;
+        const int k_lo = (int)(it - tile * p.ktiles);
+        const int64_t left = it_end - it;
+        const int nk = (int)((int64_t)(p.ktiles - k_lo) < left ? (int64_t)(p.ktiles - k_lo) : left);
+        const int64_t batch = tile / p.tiles_per_batch;
+        int tile_m, tile_n;
+        tile_of_id(tile - batch * p.tiles_per_batch, p.tiles_m, p.tiles_n, tile_m, tile_n);
+        const int64_t m0 = (int64_t)tile_m * BM;
+        const int64_t n0 = (int64_t)tile_n * BN;
+        T *C = p.c + batch * p.stride_c;
+        // Uniform tile bases, advanced by BK per K-tile; per-lane offsets fit 32 bits (launcher check).
+        const T *ak = p.a + batch * p.stride_a + m0 * p.lda + (int64_t)k_lo * BK;
+        const T *bk = p.b + batch * p.stride_b + n0 * p.ldb + (int64_t)k_lo * BK;
+        unsigned a_off[A_LD], b_off[B_LD];
+        const int a_rows = (int)((p.m - m0) < BM ? (p.m - m0) : BM), b_rows = (int)((p.n - n0) < BN ? (p.n - n0) : BN);
+#pragma unroll
+        for (int i = 0; i < A_LD; ++i) {
+            int row = (wave * A_LD + i) * 8 + lr;
+            row = row < a_rows ? row : a_rows - 1;
+            a_off[i] = (unsigned)row * (unsigned)p.lda + (unsigned)lvec;
+        }
+#pragma unroll
+        for (int i = 0; i < B_LD; ++i) {
+            int row = (wave * B_LD + i) * 8 + lr;
+            row = row < b_rows ? row : b_rows - 1;
+            b_off[i] = (unsigned)row * (unsigned)p.ldb + (unsigned)lvec;
+        }
+        auto issue = [&](int buf) {
+            // LDS byte offsets of this wavefront's chunks (wavefront-uniform scalars)
+            const unsigned as = lds0 + (unsigned)(buf * BM * BK * (int)sizeof(T)) + wave_u * (A_LD * 1024u);
+            const unsigned bs = lds0 + (unsigned)((2 * BM + buf * BN) * BK * (int)sizeof(T)) + wave_u * (B_LD * 1024u);
+#pragma unroll
+            for (int i = 0; i < A_LD; ++i) load_to_lds_16(ak + a_off[i], as + i * 1024u);
+#pragma unroll
+            for (int i = 0; i < B_LD; ++i) load_to_lds_16(bk + b_off[i], bs + i * 1024u);
+            ak += BK;
+            bk += BK;
+        };
+
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < M::ACC; ++r) acc[i][j][r] = T(0);
+
+        issue(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's tile parts have landed
+        __syncthreads();
+        for (int kt = 0; kt < nk; ++kt) {
+            const int buf = kt & 1;
+            if (kt + 1 < nk) issue(buf ^ 1);
+            const T *as = As + buf * BM * BK + (wm0 + lrow) * BK;
+            const T *bs = Bs + buf * BN * BK + (wn0 + lrow) * BK;
+            V af[2][TM], bf[2][TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) af[0][i] = *reinterpret_cast<const V *>(as + i * MT * BK + roff[0]);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) bf[0][j] = *reinterpret_cast<const V *>(bs + j * MT * BK + roff[0]);
+#pragma unroll
+            for (int kc = 0; kc < NCH; ++kc) {
+                const int cur = kc & 1, nxt = cur ^ 1;
+                if (kc + 1 < NCH) {
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) af[nxt][i] = *reinterpret_cast<const V *>(as + i * MT * BK + roff[kc + 1]);
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) bf[nxt][j] = *reinterpret_cast<const V *>(bs + j * MT * BK + roff[kc + 1]);
+                }
+#pragma unroll
+                for (int e = 0; e < EPV; ++e)
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) acc[i][j] = M::mma(M::elem(af[cur][i], e), M::elem(bf[cur][j], e), acc[i][j]);
+            }
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            __syncthreads();
+        }
+
+        if (nk == p.ktiles) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int64_t col = n0 + wn0 + j * MT + lrow;
+                if (col >= p.n) continue;
+                const T bv = has_bias ? p.bias[col] : T(0);
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                    for (int r = 0; r < M::ACC; ++r) {
+                        const int64_t row = m0 + wm0 + i * MT + M::acc_row(r, lane);
+                        if (row < p.m) {
+                            T v = acc[i][j][r];
+                            if (p.use_alpha) v = p.alpha * v;
+                            if (has_bias) v = v + bv;
+                            if (has_gelu) v = M::gelu(v);
+                            if (has_res) v = v + p.residual[batch * p.stride_c + row * p.ldc + col];
+                            C[row * p.ldc + col] = v;
+                        }
+                    }
+                }
+            }
+        } else {
+            constexpr int64_t SLOT = (int64_t)BM * BN;
+            T *mine = p.partials + ((int64_t)vb * 2 + (k_lo > 0 ? 0 : 1)) * SLOT;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int r = 0; r < M::ACC; r += EPV) {
+                        T e[EPV];
+#pragma unroll
+                        for (int q = 0; q < EPV; ++q) e[q] = acc[i][j][r + q];
+                        const int ev = ((i * TN + j) * M::ACC + r) / EPV;
+                        *reinterpret_cast<V *>(mine + ((int64_t)ev * NT + tid) * EPV) = M::make(e);
+                    }
+        }
+        it += nk;
+    }
+}
+
 // Completes the tiles whose K range was shared by several workgroups of gemm_kernel. Workgroup
 // (b, part) (1 <= b < grid) looks at the boundary between main-kernel workgroups b - 1 and b; if
 // that boundary falls inside a tile and is the FIRST such boundary of that tile, it adds the
@@ -519,15 +706,12 @@ int32_t get_workspace(hipStream_t st, size_t partial_bytes, void **partials) {
 
 constexpr int kMinItersPerBlock = 4;  // never cut the iteration space finer than this many K-tiles
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool TRANS_B, bool VEC, bool VECB>
-int32_t launch_config(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
-    using M = Mfma<T>;
-    constexpr int S = BK + M::EPV;
+// Launches a persistent main kernel over the stream-K schedule, then the fix-up kernel if any
+// tile is split. `blocks_per_cu` caches the kernel's occupancy (one static per kernel).
+template <typename T, int BM, int BN, int WM, int WN, typename Kern>
+int32_t launch_persistent(Kern kern, size_t smem, int BK, int &blocks_per_cu, GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     constexpr int NT = WM * WN * kWave;
-    constexpr size_t smem = (size_t)2 * (BM + BN) * S * sizeof(T);
-    auto kern = gemm_kernel<T, BM, BN, BK, WM, WN, MINW, TRANS_B, VEC, VECB>;
-    static int blocks_per_cu = 0;  // benign race: both calls are idempotent
-    if (blocks_per_cu == 0) {
+    if (blocks_per_cu == 0) {  // benign race: both calls are idempotent
         FTH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         int nb = 0;
         FTH_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, kern, NT, smem));
@@ -570,6 +754,23 @@ int32_t launch_config(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     return FTH_OK;
 }
 
+template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool TRANS_B, bool VEC, bool VECB>
+int32_t launch_config(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
+    constexpr int S = BK + Mfma<T>::EPV;
+    constexpr size_t smem = (size_t)2 * (BM + BN) * S * sizeof(T);
+    static int blocks_per_cu = 0;
+    return launch_persistent<T, BM, BN, WM, WN>(gemm_kernel<T, BM, BN, BK, WM, WN, MINW, TRANS_B, VEC, VECB>, smem, BK, blocks_per_cu, p,
+                                                 batch, st);
+}
+
+template <typename T, int BM, int BN, int WM, int WN, int MINW>
+int32_t launch_direct(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
+    constexpr int BK = 128 / (int)sizeof(T);
+    constexpr size_t smem = (size_t)2 * (BM + BN) * BK * sizeof(T);
+    static int blocks_per_cu = 0;
+    return launch_persistent<T, BM, BN, WM, WN>(gemm_direct_kernel<T, BM, BN, WM, WN, MINW>, smem, BK, blocks_per_cu, p, batch, st);
+}
+
 // Tile configurations. The choice depends on the shape only (never on timing), so a given problem
 // always runs the same kernel and reproduces its bits.
 enum class Tile { Big, Wide, Small };
@@ -593,6 +794,20 @@ int32_t launch_shape(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     if (f == 0) t = Tile::Big;
     if (f == 1) t = Tile::Wide;
     if (f == 2) t = Tile::Small;
+    if constexpr (TRANS_B && VEC) {
+        // Both operands k-contiguous and 16-byte aligned: direct-to-LDS kernel when K is a whole
+        // number of 128-byte K-tiles and a tile's row offsets fit 32 bits.
+        constexpr int64_t DBK = 128 / (int64_t)sizeof(T);
+        static const bool direct_off = [] {
+            const char *e = std::getenv("FT_HIP_GEMM_DIRECT");  // tuning knob: 0 disables the direct-to-LDS kernels
+            return e && std::atoi(e) == 0;
+        }();
+        const int64_t lim = ((int64_t)1 << 31) / 128 - DBK;
+        if (!direct_off && t != Tile::Wide && p.k % DBK == 0 && p.lda <= lim && p.ldb <= lim) {
+            if (t == Tile::Big) return launch_direct<T, 128, 128, 2, 2, std::is_same<T, float>::value ? 2 : 1>(p, batch, st);
+            return launch_direct<T, 64, 64, 2, 2, 2>(p, batch, st);
+        }
+    }
     if constexpr (std::is_same<T, float>::value) {
         switch (t) {
             case Tile::Big: return launch_config<T, 128, 128, FTH_F32_BK, 2, 2, FTH_F32_MINW, TRANS_B, VEC, VECB>(p, batch, st);
