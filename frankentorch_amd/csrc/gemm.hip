@@ -52,6 +52,12 @@ constexpr int kGroupM = 8;
 #ifndef FTH_F32_BK
 #define FTH_F32_BK 32
 #endif
+#ifndef FTH_GD_ROTATE
+#define FTH_GD_ROTATE 1
+#endif
+#ifndef FTH_GD_SCHED
+#define FTH_GD_SCHED 1
+#endif
 #ifndef FTH_F32_MINW
 #define FTH_F32_MINW 2
 #endif
@@ -393,27 +399,32 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_kernel(const GemmArg
     }
 }
 
-// ---- direct-to-LDS variant for k-contiguous operands (A [m,k] and B stored [n,k]) ----
+// ---- direct-to-LDS variant (A [m,k] with 16-byte aligned rows; B stored [n,k] or [k,n]) ----
 //
 // Same tiling, schedule, accumulation order and slot format as gemm_kernel; only the way operand
 // tiles reach LDS and the LDS layout differ. A K-tile is 128 bytes of k per row (32 floats, 16
 // doubles). Tiles are written by global_load_lds (16 bytes per lane, no staging registers and no
-// LDS store instructions): one wavefront instruction fills 1 KiB of LDS in lane order, i.e.
-// 8 rows x 8 vectors, unpadded. To keep the MFMA operand reads conflict-free the vectors of a row
-// are stored XOR-swizzled: logical vector q of row r sits in slot q ^ (r & 7). The loader does the
-// swizzle on the global side (lane -> slot is fixed by the hardware, so lane (r, slot) fetches
-// vector slot ^ (r & 7) of its row); the 8 lanes of a row still cover one whole 128-byte line.
-// Rows past the m / n edge are clamped to the last valid row: a row of A (B) only feeds the same
-// row (column) of C, and those are never stored. The launcher guarantees k % BK == 0.
-// One wavefront-wide global -> LDS copy of 16 bytes per lane: lane L's 16 bytes land at
-// lds_chunk + 16 * L. Written as inline assembly so that the compiler's wait-count insertion does
-// not see an LDS write it cannot disambiguate (it would drain the load queue before every LDS
-// read and serialise the prefetch); the kernel waits for vmcnt(0) itself before each barrier.
+// LDS store instructions): one wavefront instruction fills 1 KiB of LDS in lane order.
+//   k-contiguous operands (A, and B stored [n,k]): a chunk is 8 rows x 8 vectors, unpadded. To
+//   keep the MFMA operand reads conflict-free the vectors of a row are stored XOR-swizzled:
+//   logical vector q of row r sits in slot q ^ ((r >> 1) & 7). The loader does the swizzle on the
+//   global side (lane -> slot is fixed by the hardware, so lane (r, slot) fetches vector
+//   slot ^ ((r >> 1) & 7) of its row); the 8 lanes of a row still cover one whole 128-byte line.
+//   B stored [k,n]: the tile is kept [k][n] as it is in memory (a chunk is 1 KiB of consecutive
+//   n of one or more k rows) and a lane reads its MFMA operand element by element; consecutive
+//   lanes read consecutive n, which is conflict-free without padding.
+// Rows (columns) past the m / n edge are clamped to the last valid one: a row of A (column of B)
+// only feeds the same row (column) of C, and those are never stored. The launcher guarantees
+// k % BK == 0. The loader runs one K-tile ahead of the MFMAs across output-tile boundaries too,
+// so the first K-tile of the next output tile is in flight during the epilogue of this one.
 template <typename T> __device__ __forceinline__ void load_to_lds_16(const T *src, unsigned lds_chunk) {
+    // Inline assembly so that the compiler's wait-count insertion does not see an LDS write it
+    // cannot disambiguate (it would drain the load queue before every LDS read and serialise the
+    // prefetch); the kernel waits for vmcnt(0) itself before each barrier.
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_chunk) : "memory", "m0");
 }
 
-template <typename T, int BM, int BN, int WM, int WN, int MINW>
+template <typename T, int BM, int BN, int WM, int WN, int MINW, bool TRANS_B>
 __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const GemmArgs<T> p) {
     using M = Mfma<T>;
     using V = typename M::V;
@@ -423,13 +434,17 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
     constexpr int KCH = KG * EPV, NCH = BK / KCH;
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / MT, TN = WTN / MT;
-    constexpr int A_LD = BM / 8 / NW, B_LD = BN / 8 / NW;  // chunk loads per wavefront and K-tile
+    constexpr int A_LD = BM / 8 / NW;                         // chunk loads per wavefront and K-tile
+    constexpr int B_LD = BN * BK * (int)sizeof(T) / 1024 / NW;
+    constexpr int LPR = BN * (int)sizeof(T) / 16;             // [k,n] B: lanes per k row of the tile
+    constexpr int RPC = kWave / LPR;                          // [k,n] B: k rows per chunk
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile rows must divide into 8-row chunks per wavefront");
-    static_assert(MT % 8 == 0, "swizzle assumes MFMA tile rows start on a multiple of 8");
+    static_assert(MT % 16 == 0, "swizzle assumes MFMA tile rows start on a multiple of 16");
+    static_assert(LPR <= kWave && kWave % LPR == 0, "a chunk must hold whole k rows of B");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *As = reinterpret_cast<T *>(smem_raw);  // [2][BM][BK]
-    T *Bs = As + 2 * BM * BK;                 // [2][BN][BK]
+    T *Bs = As + 2 * BM * BK;                 // [2][BN][BK] or [2][BK][BN]
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -441,10 +456,15 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
     const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)reinterpret_cast<uintptr_t>(smem_raw));
     const unsigned wave_u = __builtin_amdgcn_readfirstlane((unsigned)wave);
     const int lr = lane >> 3;                           // loader: row inside the chunk
-    const int lvec = ((lane & 7) ^ lr) * EPV;           // loader: k offset of the vector this lane fetches
+    // Swizzle term of tile row r. The LDS serves a 128-bit read 16 lanes at a time over 64 banks
+    // (256 bytes), so 16 consecutive rows at the same logical vector must differ in
+    // (row parity, slot): slot = q ^ ((r >> 1) & 7).
+    auto swz = [](int r) { return (r >> 1) & 7; };
+    // loader: k offset of the vector this lane fetches for 8-row chunk c of the tile
+    auto lvec = [&](int c) { return ((lane & 7) ^ swz(c * 8 + lr)) * EPV; };
     int roff[NCH];                                      // reader: swizzled k offset per operand fetch
 #pragma unroll
-    for (int kc = 0; kc < NCH; ++kc) roff[kc] = ((kc * KG + lane / MT) ^ (lrow & 7)) * EPV;
+    for (int kc = 0; kc < NCH; ++kc) roff[kc] = ((kc * KG + lane / MT) ^ swz(lrow)) * EPV;
 
     const bool has_bias = (p.epilogue & FTH_EPI_BIAS) != 0;
     const bool has_gelu = (p.epilogue & FTH_EPI_GELU) != 0;
@@ -455,48 +475,115 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
     const int64_t total = p.total_iters;
     int64_t it = (int64_t)vb * total / grid;
     const int64_t it_end = (int64_t)(vb + 1) * total / grid;
+    if (it >= it_end) return;
+
+    // ---- loader state: runs one K-tile ahead of the MFMAs ----
+    int n_iter = (int)(it_end - it);  // K-tiles this workgroup still has to multiply (fits: launcher check)
+    int ld_left = n_iter;             // K-tiles it still has to request
+    int64_t ld_tile = it / p.ktiles;
+    int ld_k = (int)(it - ld_tile * p.ktiles);
+    const T *ak = nullptr, *bk = nullptr;  // uniform bases of the next K-tile to load; lane offsets fit 32 bits (launcher check)
+    unsigned a_off[A_LD], b_off[B_LD];
+    auto setup_loader = [&]() {
+        const int64_t batch = ld_tile / p.tiles_per_batch;
+        int tile_m, tile_n;
+        tile_of_id(ld_tile - batch * p.tiles_per_batch, p.tiles_m, p.tiles_n, tile_m, tile_n);
+        const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+        ak = p.a + batch * p.stride_a + m0 * p.lda + (int64_t)ld_k * BK;
+        const int a_rows = (int)((p.m - m0) < BM ? (p.m - m0) : BM), b_cols = (int)((p.n - n0) < BN ? (p.n - n0) : BN);
+#pragma unroll
+        for (int i = 0; i < A_LD; ++i) {
+            int row = (wave * A_LD + i) * 8 + lr;
+            row = row < a_rows ? row : a_rows - 1;
+            a_off[i] = (unsigned)row * (unsigned)p.lda + (unsigned)lvec(wave * A_LD + i);
+        }
+        if constexpr (TRANS_B) {
+            bk = p.b + batch * p.stride_b + n0 * p.ldb + (int64_t)ld_k * BK;
+#pragma unroll
+            for (int i = 0; i < B_LD; ++i) {
+                int row = (wave * B_LD + i) * 8 + lr;
+                row = row < b_cols ? row : b_cols - 1;
+                b_off[i] = (unsigned)row * (unsigned)p.ldb + (unsigned)lvec(wave * B_LD + i);
+            }
+        } else {
+            bk = p.b + batch * p.stride_b + (int64_t)ld_k * BK * p.ldb + n0;
+            int col = (lane % LPR) * EPV;
+            col = col < b_cols ? col : b_cols - EPV;  // n is a multiple of EPV on this path
+#pragma unroll
+            for (int i = 0; i < B_LD; ++i) {
+                const int krow = (wave * B_LD + i) * RPC + lane / LPR;
+                b_off[i] = (unsigned)krow * (unsigned)p.ldb + (unsigned)col;
+            }
+        }
+    };
+    auto issue = [&](int buf) {
+        // LDS byte offsets of this wavefront's chunks (wavefront-uniform scalars)
+        const unsigned as = lds0 + (unsigned)(buf * BM * BK * (int)sizeof(T)) + wave_u * (A_LD * 1024u);
+        const unsigned bs = lds0 + (unsigned)((2 * BM + buf * BN) * BK * (int)sizeof(T)) + wave_u * (B_LD * 1024u);
+#pragma unroll
+        for (int i = 0; i < A_LD; ++i) load_to_lds_16(ak + a_off[i], as + i * 1024u);
+#pragma unroll
+        for (int i = 0; i < B_LD; ++i) load_to_lds_16(bk + b_off[i], bs + i * 1024u);
+        ak += BK;
+        bk += TRANS_B ? (int64_t)BK : (int64_t)BK * p.ldb;
+        --ld_left;
+        if (++ld_k == p.ktiles) {
+            ld_k = 0;
+            ++ld_tile;
+            if (ld_left > 0) setup_loader();  // the next load starts a new output tile
+        }
+    };
+
+    // ---- operand fetch: LDS -> registers, one k-chunk ahead of the MFMAs (two register slots) ----
+    T af[2][TM][EPV], bf[2][TN][EPV];
+    auto fetch = [&](int buf, int kc, int slot) {
+        const T *as = As + buf * BM * BK + (wm0 + lrow) * BK;
+        // B operand base of this lane: row (wn0 + lrow) of the [n][k] tile, or column
+        // (wn0 + lrow) and k row (lane / MT) * EPV of the [k][n] tile.
+        const T *bs = TRANS_B ? Bs + buf * BN * BK + (wn0 + lrow) * BK : Bs + buf * BK * BN + (lane / MT) * EPV * BN + wn0 + lrow;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const V v = *reinterpret_cast<const V *>(as + i * MT * BK + roff[kc]);
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) af[slot][i][e] = M::elem(v, e);
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            if constexpr (TRANS_B) {
+                const V v = *reinterpret_cast<const V *>(bs + j * MT * BK + roff[kc]);
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) bf[slot][j][e] = M::elem(v, e);
+            } else {
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) bf[slot][j][e] = bs[(kc * KCH + e) * BN + j * MT];
+            }
+        }
+    };
+    static_assert(NCH % 2 == 0, "the register slot of chunk 0 must be the same in every K-tile");
+    // Pinning the source order (operand reads of chunk c + 1 ahead of the MFMAs of chunk c) pays for
+    // fp64, whose 16x16x4 MFMAs leave little room behind them; for fp32 the compiler's own placement
+    // (reads a few MFMAs before the end of a chunk) measures faster.
+    constexpr bool kRotate = FTH_GD_ROTATE != 0, kSched = FTH_GD_SCHED != 0 && std::is_same<T, double>::value;
+
+    setup_loader();
+    issue(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's tile parts have landed
+    __syncthreads();
+    int cbuf = 0;
+    if constexpr (kRotate) fetch(0, 0, 0);
 
     typename M::Acc acc[TM][TN];
 
-    while (it < it_end) {
+    while (n_iter > 0) {
         const int64_t tile = it / p.ktiles;
         const int k_lo = (int)(it - tile * p.ktiles);
-        const int64_t left = it_end - it;
-        const int nk = (int)((int64_t)(p.ktiles - k_lo) < left ? (int64_t)(p.ktiles - k_lo) : left);
+        const int nk = (p.ktiles - k_lo) < n_iter ? (p.ktiles - k_lo) : n_iter;
         const int64_t batch = tile / p.tiles_per_batch;
         int tile_m, tile_n;
         tile_of_id(tile - batch * p.tiles_per_batch, p.tiles_m, p.tiles_n, tile_m, tile_n);
         const int64_t m0 = (int64_t)tile_m * BM;
         const int64_t n0 = (int64_t)tile_n * BN;
         T *C = p.c + batch * p.stride_c;
-        // Uniform tile bases, advanced by BK per K-tile; per-lane offsets fit 32 bits (launcher check).
-        const T *ak = p.a + batch * p.stride_a + m0 * p.lda + (int64_t)k_lo * BK;
-        const T *bk = p.b + batch * p.stride_b + n0 * p.ldb + (int64_t)k_lo * BK;
-        unsigned a_off[A_LD], b_off[B_LD];
-        const int a_rows = (int)((p.m - m0) < BM ? (p.m - m0) : BM), b_rows = (int)((p.n - n0) < BN ? (p.n - n0) : BN);
-#pragma unroll
-        for (int i = 0; i < A_LD; ++i) {
-            int row = (wave * A_LD + i) * 8 + lr;
-            row = row < a_rows ? row : a_rows - 1;
-            a_off[i] = (unsigned)row * (unsigned)p.lda + (unsigned)lvec;
-        }
-#pragma unroll
-        for (int i = 0; i < B_LD; ++i) {
-            int row = (wave * B_LD + i) * 8 + lr;
-            row = row < b_rows ? row : b_rows - 1;
-            b_off[i] = (unsigned)row * (unsigned)p.ldb + (unsigned)lvec;
-        }
-        auto issue = [&](int buf) {
-            // LDS byte offsets of this wavefront's chunks (wavefront-uniform scalars)
-            const unsigned as = lds0 + (unsigned)(buf * BM * BK * (int)sizeof(T)) + wave_u * (A_LD * 1024u);
-            const unsigned bs = lds0 + (unsigned)((2 * BM + buf * BN) * BK * (int)sizeof(T)) + wave_u * (B_LD * 1024u);
-#pragma unroll
-            for (int i = 0; i < A_LD; ++i) load_to_lds_16(ak + a_off[i], as + i * 1024u);
-#pragma unroll
-            for (int i = 0; i < B_LD; ++i) load_to_lds_16(bk + b_off[i], bs + i * 1024u);
-            ak += BK;
-            bk += BK;
-        };
 
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -505,37 +592,38 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
 #pragma unroll
                 for (int r = 0; r < M::ACC; ++r) acc[i][j][r] = T(0);
 
-        issue(0);
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's tile parts have landed
-        __syncthreads();
         for (int kt = 0; kt < nk; ++kt) {
-            const int buf = kt & 1;
-            if (kt + 1 < nk) issue(buf ^ 1);
-            const T *as = As + buf * BM * BK + (wm0 + lrow) * BK;
-            const T *bs = Bs + buf * BN * BK + (wn0 + lrow) * BK;
-            V af[2][TM], bf[2][TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) af[0][i] = *reinterpret_cast<const V *>(as + i * MT * BK + roff[0]);
-#pragma unroll
-            for (int j = 0; j < TN; ++j) bf[0][j] = *reinterpret_cast<const V *>(bs + j * MT * BK + roff[0]);
+            if (ld_left > 0) issue(cbuf ^ 1);
+            if constexpr (!kRotate) fetch(cbuf, 0, 0);
 #pragma unroll
             for (int kc = 0; kc < NCH; ++kc) {
-                const int cur = kc & 1, nxt = cur ^ 1;
+                const int cur = kc & 1;
                 if (kc + 1 < NCH) {
-#pragma unroll
-                    for (int i = 0; i < TM; ++i) af[nxt][i] = *reinterpret_cast<const V *>(as + i * MT * BK + roff[kc + 1]);
-#pragma unroll
-                    for (int j = 0; j < TN; ++j) bf[nxt][j] = *reinterpret_cast<const V *>(bs + j * MT * BK + roff[kc + 1]);
+                    fetch(cbuf, kc + 1, cur ^ 1);
+                } else if constexpr (kRotate) {
+                    // Last chunk: its operands are already in registers. Close the K-tile (own loads
+                    // landed, everyone done reading this buffer) and fetch the first chunk of the next
+                    // K-tile before this chunk's MFMAs, so the matrix pipe never waits on LDS latency.
+                    __builtin_amdgcn_s_waitcnt(0x0F70);
+                    __syncthreads();
+                    cbuf ^= 1;
+                    if (--n_iter > 0) fetch(cbuf, 0, 0);
                 }
+                if constexpr (kSched) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int e = 0; e < EPV; ++e)
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
 #pragma unroll
-                        for (int j = 0; j < TN; ++j) acc[i][j] = M::mma(M::elem(af[cur][i], e), M::elem(bf[cur][j], e), acc[i][j]);
+                        for (int j = 0; j < TN; ++j) acc[i][j] = M::mma(af[cur][i][e], bf[cur][j][e], acc[i][j]);
+                if constexpr (kSched) __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_s_waitcnt(0x0F70);
-            __syncthreads();
+            if constexpr (!kRotate) {
+                __builtin_amdgcn_s_waitcnt(0x0F70);
+                __syncthreads();
+                cbuf ^= 1;
+                --n_iter;
+            }
         }
 
         if (nk == p.ktiles) {
@@ -763,12 +851,13 @@ int32_t launch_config(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
                                                  batch, st);
 }
 
-template <typename T, int BM, int BN, int WM, int WN, int MINW>
+template <typename T, int BM, int BN, int WM, int WN, int MINW, bool TRANS_B>
 int32_t launch_direct(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     constexpr int BK = 128 / (int)sizeof(T);
     constexpr size_t smem = (size_t)2 * (BM + BN) * BK * sizeof(T);
     static int blocks_per_cu = 0;
-    return launch_persistent<T, BM, BN, WM, WN>(gemm_direct_kernel<T, BM, BN, WM, WN, MINW>, smem, BK, blocks_per_cu, p, batch, st);
+    return launch_persistent<T, BM, BN, WM, WN>(gemm_direct_kernel<T, BM, BN, WM, WN, MINW, TRANS_B>, smem, BK, blocks_per_cu, p, batch,
+                                                 st);
 }
 
 // Tile configurations. The choice depends on the shape only (never on timing), so a given problem
@@ -794,18 +883,19 @@ int32_t launch_shape(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     if (f == 0) t = Tile::Big;
     if (f == 1) t = Tile::Wide;
     if (f == 2) t = Tile::Small;
-    if constexpr (TRANS_B && VEC) {
-        // Both operands k-contiguous and 16-byte aligned: direct-to-LDS kernel when K is a whole
-        // number of 128-byte K-tiles and a tile's row offsets fit 32 bits.
+    if constexpr (VEC && (TRANS_B || VECB)) {
+        // 16-byte aligned operand rows: direct-to-LDS kernel when K is a whole number of 128-byte
+        // K-tiles and a tile's lane offsets fit 32 bits.
         constexpr int64_t DBK = 128 / (int64_t)sizeof(T);
         static const bool direct_off = [] {
             const char *e = std::getenv("FT_HIP_GEMM_DIRECT");  // tuning knob: 0 disables the direct-to-LDS kernels
             return e && std::atoi(e) == 0;
         }();
-        const int64_t lim = ((int64_t)1 << 31) / 128 - DBK;
+        const int64_t lim = ((int64_t)1 << 31) / 128 - 128;
         if (!direct_off && t != Tile::Wide && p.k % DBK == 0 && p.lda <= lim && p.ldb <= lim) {
-            if (t == Tile::Big) return launch_direct<T, 128, 128, 2, 2, std::is_same<T, float>::value ? 2 : 1>(p, batch, st);
-            return launch_direct<T, 64, 64, 2, 2, 2>(p, batch, st);
+            constexpr int MINW_BIG = std::is_same<T, float>::value ? 2 : 1;
+            if (t == Tile::Big) return launch_direct<T, 128, 128, 2, 2, MINW_BIG, TRANS_B>(p, batch, st);
+            return launch_direct<T, 64, 64, 2, 2, 2, TRANS_B>(p, batch, st);
         }
     }
     if constexpr (std::is_same<T, float>::value) {
