@@ -893,7 +893,7 @@ int32_t launch_shape(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
         }();
         const int64_t lim = ((int64_t)1 << 31) / 128 - 128;
         if (!direct_off && t != Tile::Wide && p.k % DBK == 0 && p.lda <= lim && p.ldb <= lim) {
-            constexpr int MINW_BIG = std::is_same<T, float>::value ? 2 : 1;
+            constexpr int MINW_BIG = 2;
             if (t == Tile::Big) return launch_direct<T, 128, 128, 2, 2, MINW_BIG, TRANS_B>(p, batch, st);
             return launch_direct<T, 64, 64, 2, 2, 2, TRANS_B>(p, batch, st);
         }
