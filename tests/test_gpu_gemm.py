@@ -37,6 +37,58 @@ def test_gemm_matches_oracle(hip, oracle, m, n, k, trans_b, dtype):
     assert rel_err(got, oracle.gemm(a, b, trans_b)) <= tol
 
 
+# K a whole number of 128-byte K-tiles with 16-byte aligned rows: the global->LDS direct kernels.
+# Ragged m / n (clamped edge rows and columns), one-row and one-vector extents, tile counts that
+# leave every workgroup a mix of whole and split tiles (several tiles per workgroup, K split 2-3 ways).
+DIRECT_SHAPES = [(200, 300, 96), (77, 52, 64), (130, 132, 512), (1, 4, 32), (1000, 8, 32), (129, 257 * 4, 160),
+                 (2048, 2304, 768), (4096, 3072, 256), (2050, 1540, 288)]
+
+
+@pytest.mark.parametrize("m,n,k", DIRECT_SHAPES)
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_direct_to_lds_kernels(hip, oracle, m, n, k, trans_b, dtype):
+    tol = TOL_GEMM_F32 if dtype == np.float32 else TOL_F64
+    a = synth.uniform(2, "da", (m, k), -1, 1, dtype=dtype)
+    b = synth.uniform(2, "db", (n, k) if trans_b else (k, n), -1, 1, dtype=dtype)
+    bias = synth.normal(2, "dbias", (n,), dtype=dtype)
+    res = synth.normal(2, "dres", (m, n), dtype=dtype)
+    rows = np.unique(np.concatenate([np.arange(0, m, max(1, m // 37)), [m - 1]]))
+    ref = oracle.gemm(a[rows], b, trans_b)
+    plain = _run(hip, a, b, trans_b)
+    assert rel_err(plain[rows], ref) <= tol
+    again = _run(hip, a, b, trans_b)
+    assert np.array_equal(plain.view(np.uint8), again.view(np.uint8))          # fixed summation order
+    got = _run(hip, a, b, trans_b, bias, res, EPI_BIAS | EPI_RESIDUAL)
+    assert np.array_equal(got, (plain + bias) + res)                             # same roundings as the separate ops
+    got = _run(hip, a, b, trans_b, bias, None, EPI_BIAS | EPI_GELU)
+    assert rel_err(got[rows], oracle.gelu(ref + bias)) <= tol
+
+
+def test_direct_to_lds_kernels_with_row_pitch_and_batches(hip, oracle):
+    """Sub-blocks of larger buffers (pitch > row, 16-byte aligned offsets) and a batched problem whose
+    tiles straddle workgroup ranges, through the direct kernels."""
+    big_a = synth.uniform(2, "qa", (300, 264), -1, 1)
+    big_b = synth.uniform(2, "qb", (280, 200), -1, 1)
+    dA, dB = DeviceBuffer.from_host(big_a), DeviceBuffer.from_host(big_b)
+    dC = DeviceBuffer.from_host(np.zeros((300, 212), np.float32))
+    # A sub-block [290, 256] at element offset 4 (pitch 264); B^T sub-block [270, 256]... stored [n, k] with pitch 200 would
+    # not hold k = 256, so B is taken as [k, n] = [256, 196] at offset 4 with pitch 200.
+    hip.gemm(hip.gemm_desc(290, 196, 256, lda=264, ldb=200, ldc=212), dA.view(4), dB.view(4), dC.view(8))
+    a_sub = big_a.ravel()[4:][: 290 * 264].reshape(290, 264)[:, :256]
+    b_sub = big_b.ravel()[4:][: 256 * 200].reshape(256, 200)[:, :196]
+    got = dC.to_host().ravel()[8:][: 290 * 212].reshape(290, 212)[:, :196]
+    assert rel_err(got, oracle.gemm(np.ascontiguousarray(a_sub), np.ascontiguousarray(b_sub))) <= TOL_GEMM_F32
+    untouched = dC.to_host().ravel()[8:][: 290 * 212].reshape(290, 212)[:, 196:]
+    assert np.all(untouched == 0.0)
+    a = synth.uniform(2, "qba", (24, 384, 96), -1, 1)
+    w = synth.uniform(2, "qbw", (24, 320, 96), -1, 1)
+    da, dw = DeviceBuffer.from_host(a), DeviceBuffer.from_host(w)
+    dc = DeviceBuffer((24, 384, 320))
+    hip.gemm(hip.gemm_desc(384, 320, 96, batch=24, trans_b=True), da, dw, dc)
+    assert rel_err(dc.to_host(), oracle.bmm(a, np.ascontiguousarray(w.transpose(0, 2, 1)))) <= TOL_GEMM_F32
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_epilogues_keep_their_own_roundings(hip, oracle, dtype):
     """bias, GELU and residual applied in the epilogue equal the separate ops applied to the
