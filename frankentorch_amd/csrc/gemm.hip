@@ -52,6 +52,9 @@ constexpr int kGroupM = 8;
 #ifndef FTH_F32_BK
 #define FTH_F32_BK 32
 #endif
+#ifndef FTH_EP_CHUNK
+#define FTH_EP_CHUNK 0
+#endif
 #ifndef FTH_GD_ROTATE
 #define FTH_GD_ROTATE 1
 #endif
@@ -434,7 +437,9 @@ template <typename T> __device__ __forceinline__ void load_to_lds_16(const T *sr
                  : "memory", "m0");
 }
 
-template <typename T, int BM, int BN, int WM, int WN, int MINW, bool TRANS_B>
+// EPI >= 0: the epilogue flags are this compile-time mask and alpha is 1 (straight-line output code);
+// EPI < 0: flags and alpha are read from the arguments.
+template <typename T, int BM, int BN, int WM, int WN, int MINW, bool TRANS_B, int EPI>
 __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const GemmArgs<T> p) {
     using M = Mfma<T>;
     using V = typename M::V;
@@ -476,9 +481,11 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
 #pragma unroll
     for (int kc = 0; kc < NCH; ++kc) roff[kc] = ((kc * KG + lane / MT) ^ swz(lrow)) * EPV;
 
-    const bool has_bias = (p.epilogue & FTH_EPI_BIAS) != 0;
-    const bool has_gelu = (p.epilogue & FTH_EPI_GELU) != 0;
-    const bool has_res = (p.epilogue & FTH_EPI_RESIDUAL) != 0;
+    const int epi = EPI >= 0 ? EPI : p.epilogue;
+    const bool has_bias = (epi & FTH_EPI_BIAS) != 0;
+    const bool has_gelu = (epi & FTH_EPI_GELU) != 0;
+    const bool has_res = (epi & FTH_EPI_RESIDUAL) != 0;
+    const bool use_alpha = EPI >= 0 ? false : p.use_alpha != 0;
 
     const int grid = (int)gridDim.x;
     const int vb = xcd_contiguous_id((int)blockIdx.x, grid);
@@ -601,48 +608,80 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
     T res[DEFER ? TILES_PP : 1][DEFER ? M::ACC : 1];  // residual values of the share being written
     T bias_v[DEFER ? TILES_PP : 1];
 
+    // Interior tiles (no m / n edge inside) address C and the residual as a wavefront-uniform row
+    // base plus one per-lane offset: acc_row(r, lane) = acc_row(r, 0) + acc_row(0, lane), so the r
+    // term moves into the scalar base and every store is `base[lane_off]` with no bounds test.
+    const unsigned lane_off = (unsigned)M::acc_row(0, lane) * (unsigned)p.ldc + (unsigned)lrow;
+    auto is_interior = [&](int64_t m0_, int64_t n0_) __attribute__((always_inline)) { return m0_ + BM <= p.m && n0_ + BN <= p.n; };
+
     // Loads the bias and residual values a share needs (ahead of the K-tile loads of the iteration
     // that will use them, so that waiting for them does not wait for those).
     auto out_load = [&](auto S, bool full, int64_t m0_, int64_t n0_, int64_t batch_) __attribute__((always_inline)) {
         constexpr int sidx = decltype(S)::value;
-        if (!DEFER || !full) return;
+        if (!DEFER || !full || !(has_bias || has_res)) return;
+        const bool interior = is_interior(m0_, n0_);
 #pragma unroll
         for (int u = 0; u < TILES_PP; ++u) {
             const int t = sidx * TILES_PP + u, i = t / TN, j = t % TN;
             const int64_t col = n0_ + wn0 + j * MT + lrow;
             bias_v[u] = (has_bias && col < p.n) ? p.bias[col] : T(0);
             if (has_res) {
+                if (interior) {
+                    const T *rb = p.residual + batch_ * p.stride_c + (m0_ + wm0 + i * MT) * p.ldc + (n0_ + wn0 + j * MT);
 #pragma unroll
-                for (int r = 0; r < M::ACC; ++r) {
-                    const int64_t row = m0_ + wm0 + i * MT + M::acc_row(r, lane);
-                    res[u][r] = (col < p.n && row < p.m) ? p.residual[batch_ * p.stride_c + row * p.ldc + col] : T(0);
+                    for (int r = 0; r < M::ACC; ++r) res[u][r] = (rb + (int64_t)M::acc_row(r, 0) * p.ldc)[lane_off];
+                } else {
+#pragma unroll
+                    for (int r = 0; r < M::ACC; ++r) {
+                        const int64_t row = m0_ + wm0 + i * MT + M::acc_row(r, lane);
+                        res[u][r] = (col < p.n && row < p.m) ? p.residual[batch_ * p.stride_c + row * p.ldc + col] : T(0);
+                    }
                 }
             }
         }
     };
+    auto finish = [&](T v, T bv, T rv) __attribute__((always_inline)) {
+        if (use_alpha) v = p.alpha * v;
+        if (has_bias) v = v + bv;
+        if (has_gelu) v = M::gelu(v);
+        if (has_res) v = v + rv;
+        return v;
+    };
     auto out_store = [&](auto S, auto &src, bool full, int64_t m0_, int64_t n0_, int64_t batch_, T *slot_) __attribute__((always_inline)) {
         constexpr int sidx = decltype(S)::value;
+        if (full) {
+            const bool interior = is_interior(m0_, n0_);
 #pragma unroll
-        for (int u = 0; u < TILES_PP; ++u) {
-            const int t = sidx * TILES_PP + u, i = t / TN, j = t % TN;
-            if (full) {
+            for (int u = 0; u < TILES_PP; ++u) {
+                const int t = sidx * TILES_PP + u, i = t / TN, j = t % TN;
                 const int64_t col = n0_ + wn0 + j * MT + lrow;
-                T *C = p.c + batch_ * p.stride_c;
-                if (col < p.n) {
+                if (interior) {
+                    const int64_t tile_off = batch_ * p.stride_c + (m0_ + wm0 + i * MT) * p.ldc + (n0_ + wn0 + j * MT);
+                    T *cb = p.c + tile_off;
+                    const T bv = DEFER ? bias_v[u] : (has_bias ? p.bias[col] : T(0));
+#pragma unroll
+                    for (int r = 0; r < M::ACC; ++r) {
+                        const int64_t row_off = (int64_t)M::acc_row(r, 0) * p.ldc;
+                        const T rv = !has_res ? T(0) : DEFER ? res[u][r] : (p.residual + tile_off + row_off)[lane_off];
+                        (cb + row_off)[lane_off] = finish(src[i][j][r], bv, rv);
+                    }
+                } else if (col < p.n) {
+                    T *C = p.c + batch_ * p.stride_c;
+                    const T bv = DEFER ? bias_v[u] : (has_bias ? p.bias[col] : T(0));
 #pragma unroll
                     for (int r = 0; r < M::ACC; ++r) {
                         const int64_t row = m0_ + wm0 + i * MT + M::acc_row(r, lane);
                         if (row < p.m) {
-                            T v = src[i][j][r];
-                            if (p.use_alpha) v = p.alpha * v;
-                            if (has_bias) v = v + (DEFER ? bias_v[u] : p.bias[col]);
-                            if (has_gelu) v = M::gelu(v);
-                            if (has_res) v = v + (DEFER ? res[u][r] : p.residual[batch_ * p.stride_c + row * p.ldc + col]);
-                            C[row * p.ldc + col] = v;
+                            const T rv = !has_res ? T(0) : DEFER ? res[u][r] : p.residual[batch_ * p.stride_c + row * p.ldc + col];
+                            C[row * p.ldc + col] = finish(src[i][j][r], bv, rv);
                         }
                     }
                 }
-            } else {
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < TILES_PP; ++u) {
+                const int t = sidx * TILES_PP + u, i = t / TN, j = t % TN;
 #pragma unroll
                 for (int r = 0; r < M::ACC; r += EPV) {
                     T e[EPV];
@@ -694,7 +733,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
                 }
             }
             if constexpr (ep >= 0) {
-                if (kc == 0) out_store(EP, old, pend_full, pm0, pn0, pbatch, pslot);
+                if (kc == FTH_EP_CHUNK) out_store(EP, old, pend_full, pm0, pn0, pbatch, pslot);
             }
         }
         if constexpr (!kRotate) {
@@ -958,13 +997,33 @@ int32_t launch_config(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
                                                  batch, st);
 }
 
-template <typename T, int BM, int BN, int WM, int WN, int MINW, bool TRANS_B>
-int32_t launch_direct(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
+template <typename T, int BM, int BN, int WM, int WN, int MINW, bool TRANS_B, int EPI>
+int32_t launch_direct_epi(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     constexpr int BK = 128 / (int)sizeof(T);
     constexpr size_t smem = (size_t)2 * (BM + BN) * BK * sizeof(T);
     static int blocks_per_cu = 0;
-    return launch_persistent<T, BM, BN, WM, WN>(gemm_direct_kernel<T, BM, BN, WM, WN, MINW, TRANS_B>, smem, BK, blocks_per_cu, p, batch,
-                                                 st);
+    return launch_persistent<T, BM, BN, WM, WN>(gemm_direct_kernel<T, BM, BN, WM, WN, MINW, TRANS_B, EPI>, smem, BK, blocks_per_cu, p,
+                                                 batch, st);
+}
+
+// SPECIALIZE: pick a kernel with the epilogue flags compiled in for the combinations the
+// transformer block uses (none, bias, bias+GELU, bias+residual; alpha = 1).
+template <typename T, int BM, int BN, int WM, int WN, int MINW, bool TRANS_B, bool SPECIALIZE>
+int32_t launch_direct(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
+    if constexpr (SPECIALIZE) {
+        if (!p.use_alpha) {
+            switch (p.epilogue) {
+                case 0: return launch_direct_epi<T, BM, BN, WM, WN, MINW, TRANS_B, 0>(p, batch, st);
+                case FTH_EPI_BIAS: return launch_direct_epi<T, BM, BN, WM, WN, MINW, TRANS_B, FTH_EPI_BIAS>(p, batch, st);
+                case FTH_EPI_BIAS | FTH_EPI_GELU:
+                    return launch_direct_epi<T, BM, BN, WM, WN, MINW, TRANS_B, FTH_EPI_BIAS | FTH_EPI_GELU>(p, batch, st);
+                case FTH_EPI_BIAS | FTH_EPI_RESIDUAL:
+                    return launch_direct_epi<T, BM, BN, WM, WN, MINW, TRANS_B, FTH_EPI_BIAS | FTH_EPI_RESIDUAL>(p, batch, st);
+                default: break;
+            }
+        }
+    }
+    return launch_direct_epi<T, BM, BN, WM, WN, MINW, TRANS_B, -1>(p, batch, st);
 }
 
 // Tile configurations. The choice depends on the shape only (never on timing), so a given problem
@@ -999,10 +1058,10 @@ int32_t launch_shape(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
             return e && std::atoi(e) == 0;
         }();
         const int64_t lim = ((int64_t)1 << 31) / 128 - 128;
-        if (!direct_off && t != Tile::Wide && p.k % DBK == 0 && p.lda <= lim && p.ldb <= lim) {
+        if (!direct_off && t != Tile::Wide && p.k % DBK == 0 && p.lda <= lim && p.ldb <= lim && p.ldc <= lim) {
             constexpr int MINW_BIG = 2;
-            if (t == Tile::Big) return launch_direct<T, 128, 128, 2, 2, MINW_BIG, TRANS_B>(p, batch, st);
-            return launch_direct<T, 64, 64, 2, 2, 2, TRANS_B>(p, batch, st);
+            if (t == Tile::Big) return launch_direct<T, 128, 128, 2, 2, MINW_BIG, TRANS_B, std::is_same<T, float>::value>(p, batch, st);
+            return launch_direct<T, 64, 64, 2, 2, 2, TRANS_B, false>(p, batch, st);
         }
     }
     if constexpr (std::is_same<T, float>::value) {
