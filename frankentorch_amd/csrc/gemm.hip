@@ -1028,11 +1028,11 @@ int32_t launch_direct(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
 
 // Tile configurations. The choice depends on the shape only (never on timing), so a given problem
 // always runs the same kernel and reproduces its bits.
-enum class Tile { Big, Wide, Small };
+enum class Tile { Big, Wide, Small, Tall };
 
 inline int forced_tile() {
     static const int v = [] {
-        const char *e = std::getenv("FT_HIP_GEMM_TILE");  // tuning knob: 0 = 128x128, 1 = 256x128, 2 = 64x64
+        const char *e = std::getenv("FT_HIP_GEMM_TILE");  // tuning knob: 0 = 128x128, 1 = 256x128, 2 = 64x64, 3 = 128x64 (direct fp32 only)
         return e ? std::atoi(e) : -1;
     }();
     return v;
@@ -1060,6 +1060,17 @@ int32_t launch_shape(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
         const int64_t lim = ((int64_t)1 << 31) / 128 - 128;
         if (!direct_off && t != Tile::Wide && p.k % DBK == 0 && p.lda <= lim && p.ldb <= lim && p.ldc <= lim) {
             constexpr int MINW_BIG = 2;
+            if constexpr (std::is_same<T, float>::value) {
+                // Fewer 128x128 tiles than resident workgroups would split every tile over K; 128x64
+                // tiles (three workgroups per CU) give each workgroup whole tiles instead. Their main
+                // loop is about 8 % slower, which costs more than the fix-up pass (about 25 us) once
+                // the problem exceeds some 30 GFLOP.
+                const int64_t tall_tiles = fth::ceil_div(p.m, 128) * fth::ceil_div(p.n, 64) * batch;
+                const double flop = 2.0 * (double)p.m * (double)p.n * (double)p.k * (double)batch;
+                if (f < 0 && t == Tile::Big && big_tiles < 2 * (int64_t)cus && tall_tiles >= 2 * (int64_t)cus && flop < 30e9) t = Tile::Tall;
+                if (f == 3) t = Tile::Tall;
+                if (t == Tile::Tall) return launch_direct<T, 128, 64, 2, 2, 3, TRANS_B, true>(p, batch, st);
+            }
             if (t == Tile::Big) return launch_direct<T, 128, 128, 2, 2, MINW_BIG, TRANS_B, std::is_same<T, float>::value>(p, batch, st);
             return launch_direct<T, 64, 64, 2, 2, 2, TRANS_B, false>(p, batch, st);
         }
