@@ -3,18 +3,22 @@
 //   fp32: v_mfma_f32_32x32x2_f32   (32x32 output tile per wavefront instruction, k = 2)
 //   fp64: v_mfma_f64_16x16x4_f64   (16x16 output tile, k = 4)
 //
-// Data path. A block owns a BM x BN tile of C. Both operands are staged in LDS K-CONTIGUOUS
-// (As[BM][BK+pad], Bs[BN][BK+pad]), so a lane fetches its MFMA operands with one 128-bit LDS
-// read: that vector holds EPV consecutive k for the lane's row, and feeds EPV successive MFMAs.
+// Two kernels share the tiling, the schedule and the accumulation order:
+//   gemm_direct_kernel  operand tiles go global -> LDS directly (global_load_lds); used whenever the
+//                       operand rows are 16-byte aligned and K is a whole number of 128-byte K-tiles.
+//                       Its header comment describes the LDS layout and the pipeline.
+//   gemm_kernel         any K and alignment: global -> registers -> LDS, described next.
+//
+// Data path of gemm_kernel. A block owns a BM x BN tile of C. Both operands are staged in LDS
+// K-CONTIGUOUS (As[BM][BK+pad], Bs[BN][BK+pad]), so a lane fetches its MFMA operands with one 128-bit
+// LDS read: that vector holds EPV consecutive k for the lane's row, and feeds EPV successive MFMAs.
 // Which k lands in which MFMA is irrelevant as long as A and B agree, and they do because both
 // use the same (lane / MT, element) -> k map. The pad (one vector per row) makes the row pitch
-// an odd number of vectors, which spreads the 16 rows of a read pass over all 64 banks.
-// Global -> LDS goes through registers, one K-tile ahead (two LDS buffers, one barrier per
-// K-tile): the loads of tile t+1 are issued before the MFMAs of tile t.
+// an odd number of vectors. Global -> LDS goes through registers, one K-tile ahead (two LDS
+// buffers, one barrier per K-tile): the loads of tile t+1 are issued before the MFMAs of tile t.
 //   A, and B stored [n, k] (trans_b): 128-bit global loads along k.
-//   B stored [k, n]: each thread reads EPV consecutive k of ONE column with scalar loads (the
-//   wavefront covers 64 consecutive columns, so every load instruction is one 256-byte run) and
-//   writes them to LDS as a single vector. No transpose pass, no bank conflicts.
+//   B stored [k, n]: EPV x EPV register blocks (EPV vector loads along n, regrouped in registers
+//   into EPV vectors along k), or element loads when n is not a vector multiple.
 //
 // Scheduling. The kernel is persistent: the grid is (CUs x resident blocks per CU) workgroups,
 // and the linearised iteration space (output tiles x K-tiles) is cut into equal contiguous

@@ -37,6 +37,9 @@ namespace {
 
 constexpr int kWave = 64;
 constexpr int kXcds = 8;
+#ifndef FTH_SDPA_DIRECT
+#define FTH_SDPA_DIRECT 1
+#endif
 
 using Acc16 = float __attribute__((ext_vector_type(16)));
 
@@ -56,6 +59,15 @@ __device__ __forceinline__ float exp_diff(float x, float m) {
     return __builtin_amdgcn_exp2f((x - m) * 1.44269502162933349609375f);
 }
 
+// One wavefront-wide global -> LDS copy of 16 bytes per lane: lane L's bytes land at
+// lds_chunk + 16 * L. Inline assembly so that the compiler's wait-count insertion does not see an
+// LDS write it cannot disambiguate (it would wait for the load before every LDS read); the kernel
+// waits for vmcnt(0) itself before each barrier.
+__device__ __forceinline__ void load_to_lds_16(const float *src, unsigned lds_chunk) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(__builtin_amdgcn_readfirstlane(lds_chunk))
+                 : "memory", "m0");
+}
+
 template <int N> struct VecN;
 template <> struct VecN<1> { using type = float; };
 template <> struct VecN<2> { using type = float2; };
@@ -70,15 +82,24 @@ __device__ __forceinline__ float f4_get(const float4 &v, int e) { return e == 0 
 // (q_blocks - 1 - p) and then query block p, so every block does the same amount of work.
 // BC: keys per tile (32, or 64 for the small head sizes, which halves the barriers and the
 // cross-lane softmax steps per key).
-template <int D, int NW, bool PAIR, int BC>
+// DIRECT: K/V tiles go global -> LDS with global_load_lds (no staging registers, no LDS stores; the
+// loads stay in flight under the MFMAs). A wavefront instruction fills 1 KiB of LDS in lane order,
+// so the tiles are unpadded. V rows are read whole (consecutive lanes, consecutive d) and need
+// nothing more. K rows are read one 16-byte vector per lane with 16 consecutive lanes on 16
+// consecutive rows, which would all hit the same banks (the LDS serves such a read 16 lanes at a
+// time over 64 banks); logical vector q of tile row r is therefore stored in slot q ^ (r & 15), the
+// permutation being applied on the global side by choosing which vector each lane fetches. Rows
+// past seq_k are clamped to the last row (their scores are masked, their weights are zero).
+template <int D, int NW, bool PAIR, int BC, bool DIRECT>
 __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p) {
     constexpr int kBC = BC;
     constexpr int KS = BC / 32;        // 32-key sub-tiles per tile
     constexpr int NTH = 64 * NW;
     constexpr int BQ = 32 * NW;
     constexpr int NDT = D / 32;        // 32-wide d-tiles of the output
-    constexpr int KP = D + 4;          // K tile row pitch (odd number of 16-byte vectors)
-    constexpr int VP = D + 8;          // V tile row pitch (rows j and j+4 land 32 banks apart)
+    constexpr int KP = DIRECT ? D : D + 4;  // K tile row pitch (padded: odd number of 16-byte vectors)
+    constexpr int VP = DIRECT ? D : D + 8;  // V tile row pitch (padded: rows j and j+4 land 32 banks apart)
+    static_assert(!DIRECT || D >= 64, "the direct layout assumes rows of at least 256 bytes");
     constexpr int KT = kBC * KP;       // floats per K tile
     constexpr int VT = kBC * VP;
     constexpr int NV = kBC * (D / 4) / NTH;  // float4 per thread per tile
@@ -151,10 +172,33 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
         constexpr int RS = NTH / (D / 4);  // rows covered by one sweep of the block
         const int ld_row = tid / (D / 4), ld_c = tid % (D / 4);
         const int seq_k_i = (int)d.seq_k;
-        float4 kst[NV], vst[NV];
+        float4 kst[DIRECT ? 1 : NV], vst[DIRECT ? 1 : NV];
         const float *kbase = K + (int64_t)ld_row * d.k_row_stride + 4 * ld_c;
         const float *vbase = Vg + (int64_t)ld_row * d.v_row_stride + 4 * ld_c;
+        // Direct loader: this wavefront owns CPW 1 KiB chunks of each tile; lane L of chunk c covers
+        // tile row c * RPC + L / VPR, vector slot L % VPR.
+        constexpr int VPR = D / 4, RPC = 64 / VPR, CPW = kBC / RPC / NW;
+        static_assert(!DIRECT || kBC % (RPC * NW) == 0, "tile rows must divide into chunks per wavefront");
+        const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)reinterpret_cast<uintptr_t>(smem_raw));
+        const unsigned wave_u = __builtin_amdgcn_readfirstlane((unsigned)wave);
+        auto issue_tile = [&](int kt, int buf) __attribute__((always_inline)) {
+            if constexpr (DIRECT) {
+                const int row_t0 = kt * kBC;
+#pragma unroll
+                for (int ci = 0; ci < CPW; ++ci) {
+                    const int trow = (wave * CPW + ci) * RPC + lane / VPR;  // row inside the tile
+                    const int slot = lane % VPR;
+                    int grow = row_t0 + trow;
+                    grow = grow < seq_k_i ? grow : seq_k_i - 1;
+                    const int kq = (slot & ~15) | ((slot ^ trow) & 15);
+                    const unsigned chunk = (wave_u * CPW + ci) * 1024u;
+                    load_to_lds_16(K + (int64_t)grow * d.k_row_stride + 4 * kq, lds0 + (unsigned)(buf * KT * 4) + chunk);
+                    load_to_lds_16(Vg + (int64_t)grow * d.v_row_stride + 4 * slot, lds0 + (unsigned)((2 * KT + buf * VT) * 4) + chunk);
+                }
+            }
+        };
         auto load_tile = [&](int kt) {
+            if constexpr (DIRECT) return;
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
                 const int row0 = kt * kBC + i * RS;  // uniform
@@ -170,6 +214,7 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
         float *ks_st = Ks + ld_row * KP + 4 * ld_c;
         float *vs_st = Vs + ld_row * VP + 4 * ld_c;
         auto store_tile = [&](int buf) {
+            if constexpr (DIRECT) return;
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
                 *reinterpret_cast<float4 *>(ks_st + buf * KT + i * RS * KP) = kst[i];
@@ -186,14 +231,18 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
         float l_run = 0.f;
 
         if (num_kt > 0) {
+            issue_tile(0, 0);
             load_tile(0);
             store_tile(0);
         }
+        if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): own tile parts have landed
         __syncthreads();
 
         for (int kt = 0; kt < num_kt; ++kt) {
             const int buf = kt & 1;
             const int key0 = kt * kBC;
+            // The other buffer was released by the barrier that ended the previous tile.
+            if (kt + 1 < num_kt) issue_tile(kt + 1, buf ^ 1);
             // A wavefront whose every query precedes this tile's first key has nothing to add.
             const bool wave_active = !d.causal || key0 <= wave_last_q;
             // ---- S^T = K_tile . Q^T, one 32-key sub-tile per accumulator ----
@@ -203,12 +252,14 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
                 for (int j = 0; j < KS; ++j)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) s[j][r] = 0.f;
-                const float *kp = Ks + buf * KT + lq * KP + 4 * half;
+                const float *kp = Ks + buf * KT + lq * KP + (DIRECT ? 0 : 4 * half);
+                // direct layout: vector 2t + half of row lq sits in slot (2t + half) ^ (lq & 15) = 2t ^ lx
+                const int lx = half ^ (lq & 15);
 #pragma unroll
                 for (int t = 0; t < D / 8; ++t) {
 #pragma unroll
                     for (int j = 0; j < KS; ++j) {
-                        const float4 kv = *reinterpret_cast<const float4 *>(kp + j * 32 * KP + 8 * t);
+                        const float4 kv = *reinterpret_cast<const float4 *>(kp + j * 32 * KP + (DIRECT ? 4 * ((2 * t) ^ lx) : 8 * t));
                         s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.x, qr[t].x, s[j], 0, 0, 0);
                         s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.y, qr[t].y, s[j], 0, 0, 0);
                         s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.z, qr[t].z, s[j], 0, 0, 0);
@@ -271,6 +322,7 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
                     }
             }
             if (kt + 1 < num_kt) store_tile(buf ^ 1);
+            if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0x0F70);
             __syncthreads();
         }
 
@@ -367,9 +419,10 @@ __global__ __launch_bounds__(64) void sdpa_generic_kernel(const SdpaArgs p) {
 }
 
 template <int D, int NW, bool PAIR> int32_t launch_mfma_cfg(SdpaArgs &a, hipStream_t st) {
-    constexpr int BC = (D <= 64 && (NW == 4 || D <= 32)) ? 64 : 32;  // 64-key tiles where the staging registers fit
-    constexpr size_t smem = (size_t)2 * BC * ((D + 4) + (D + 8)) * sizeof(float);
-    auto kern = sdpa_mfma_kernel<D, NW, PAIR, BC>;
+    constexpr int BC = (D <= 64 && (NW == 4 || D <= 32)) ? 64 : 32;  // 64-key tiles where two workgroups still fit a CU
+    constexpr bool DIRECT = D >= 64 && FTH_SDPA_DIRECT;
+    constexpr size_t smem = DIRECT ? (size_t)2 * BC * 2 * D * sizeof(float) : (size_t)2 * BC * ((D + 4) + (D + 8)) * sizeof(float);
+    auto kern = sdpa_mfma_kernel<D, NW, PAIR, BC, DIRECT>;
     static bool attr_set = false;
     if (!attr_set) {
         FTH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
