@@ -117,8 +117,7 @@ def bench_rowops(device, synth, steps, warmup, with_cpu):
 
     cpu = None
     if with_cpu:
-        sys.path.insert(0, os.path.join(ROOT, "oracle"))
-        import oracle as O  # CPU checker restating ft-kernel-cpu: the reported baseline only
+        O = cpu_oracle()
 
         def cpu_step():
             O.softmax(x, 1)
@@ -143,7 +142,26 @@ def bench_rowops(device, synth, steps, warmup, with_cpu):
     return value, ms_per_step, roof, per_kernel, cpu
 
 
-def bench_gemm(device, synth, steps):
+def cpu_oracle():
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle as O  # CPU checker restating ft-kernel-cpu: the reported baseline only
+
+    return O
+
+
+def cpu_time(fn, budget_s, min_reps=2, max_reps=50):
+    """Best-of-N wall time of a CPU call inside a time budget (one untimed warm-up first)."""
+    fn()
+    best, reps, t_all = float("inf"), 0, time.perf_counter()
+    while reps < min_reps or (time.perf_counter() - t_all < budget_s and reps < max_reps):
+        t0 = time.perf_counter()
+        fn()
+        best = min(best, time.perf_counter() - t0)
+        reps += 1
+    return best, reps
+
+
+def bench_gemm(device, synth, steps, with_cpu):
     from frankentorch_amd.device import EPI_BIAS, DeviceBuffer
 
     out = {}
@@ -183,10 +201,17 @@ def bench_gemm(device, synth, steps):
     da64, db64 = DeviceBuffer.from_host(a.astype(np.float64)), DeviceBuffer.from_host(b.astype(np.float64))
     dc64 = DeviceBuffer((4096, 4096), np.float64)
     run("f64_4096x4096x4096_nn", device.gemm_desc(4096, 4096, 4096), da64, db64, dc64, None, 2 * 4096 ** 3, FP64_MFMA_PEAK_TF)
+    if with_cpu:
+        O = cpu_oracle()
+        if O.sgemm_blocked(a[:64], b) is not None:
+            best, reps = cpu_time(lambda: O.sgemm_blocked(a, b), 4.0)
+            out["cpu"] = {"value": round(2 * 4096 ** 3 / best / 1e12, 3), "unit": "TFLOP/s", "cores": O.threads(), "kind": "port",
+                          "sample": "fp32 4096^3 [m,k].[k,n] with the blocked AVX2 kernel that stands in for matrixmultiply, best of %d" % reps}
+            log("[gemm] cpu baseline %.3f TFLOP/s on %d threads" % (out["cpu"]["value"], O.threads()))
     return out
 
 
-def bench_sdpa(device, synth, steps):
+def bench_sdpa(device, synth, steps, with_cpu):
     from frankentorch_amd.device import DeviceBuffer
 
     B, H, S, D = 4, 32, 2048, 128
@@ -203,8 +228,16 @@ def bench_sdpa(device, synth, steps):
     flop = B * H * 4 * D * (S * (S + 1) // 2)  # causal count: two products over the lower triangle
     tf = flop / (ms * 1e-3) / 1e12
     log("[sdpa] B4 H32 S2048 D128 causal  %.3f ms  %.2f TFLOP/s (causal count)  %.1f%% of MFMA peak" % (ms, tf, 100 * tf / FP32_MFMA_PEAK_TF))
-    return {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac": round(tf / FP32_MFMA_PEAK_TF, 4), "flop": flop,
-            "peak_TFLOP/s": FP32_MFMA_PEAK_TF, "workload": "B4 H32 S2048 D128 causal fp32"}
+    res = {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac": round(tf / FP32_MFMA_PEAK_TF, 4), "flop": flop,
+           "peak_TFLOP/s": FP32_MFMA_PEAK_TF, "workload": "B4 H32 S2048 D128 causal fp32"}
+    if with_cpu:
+        O = cpu_oracle()
+        nh = 16  # heads of the 128 timed on the CPU (one per thread); same causal flop count per head
+        best, reps = cpu_time(lambda: O.sdpa_forward(q[:nh], k[:nh], v[:nh], s, True), 4.0, min_reps=1)
+        res["cpu"] = {"value": round(flop * nh / (B * H) / best / 1e12, 4), "unit": "TFLOP/s", "cores": O.threads(), "kind": "port",
+                      "sample": "%d of the %d heads, best of %d" % (nh, B * H, reps)}
+        log("[sdpa] cpu baseline %.4f TFLOP/s (causal count) on %d threads" % (res["cpu"]["value"], O.threads()))
+    return res
 
 
 def make_layer(synth, seed, li, d, f):
@@ -215,7 +248,7 @@ def make_layer(synth, seed, li, d, f):
             "w1": n("w1", f, d), "b1": zero(f), "w2": n("w2", d, f), "b2": zero(d)}
 
 
-def bench_block(device, synth, steps):
+def bench_block(device, synth, steps, with_cpu):
     from frankentorch_amd import fused
     from frankentorch_amd.device import DeviceBuffer
 
@@ -236,6 +269,13 @@ def bench_block(device, synth, steps):
     flop = 2.10e8
     res["flop"] = flop
     res["frac"] = round(flop / (res["graph"]["ms"] * 1e-3) / 1e12 / FP32_MFMA_PEAK_TF, 5)
+    if with_cpu:
+        O = cpu_oracle()
+        layer = make_layer(synth, 0, 0, d, f)
+        best, reps = cpu_time(lambda: O.encoder_layer(layer, x, batch, seq, heads, 1e-5, True), 2.0, max_reps=200)
+        res["cpu"] = {"value": round(batch * seq / best, 1), "unit": "tokens/s", "cores": O.threads(), "kind": "port",
+                      "sample": "the same block and input, best of %d" % reps}
+        log("[block] cpu baseline %.0f tokens/s on %d threads" % (res["cpu"]["value"], O.threads()))
     return res
 
 
@@ -289,11 +329,11 @@ def main():
     value, ms_per_step, roof, per_kernel, cpu = bench_rowops(device, synth, args.steps, args.warmup, not args.no_cpu)
     extra = {"row_ops": per_kernel}
     if "gemm" in cases:
-        extra["gemm"] = bench_gemm(device, synth, args.steps)
+        extra["gemm"] = bench_gemm(device, synth, args.steps, not args.no_cpu)
     if "sdpa" in cases:
-        extra["sdpa_causal"] = bench_sdpa(device, synth, args.steps)
+        extra["sdpa_causal"] = bench_sdpa(device, synth, args.steps, not args.no_cpu)
     if "block" in cases:
-        extra["block"] = bench_block(device, synth, args.steps)
+        extra["block"] = bench_block(device, synth, args.steps, not args.no_cpu)
     if "gpt2" in cases:
         extra["gpt2_forward"] = bench_gpt2(device, synth, args.steps)
 

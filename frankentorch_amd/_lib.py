@@ -51,6 +51,8 @@ class GemmDesc(C.Structure):
     _fields_ = [(n, C.c_int64) for n in ("m", "n", "k", "lda", "ldb", "ldc", "batch", "stride_a", "stride_b", "stride_c")] + [
         ("trans_b", C.c_int32),
         ("epilogue", C.c_int32),
+        ("trans_a", C.c_int32),
+        ("reserved", C.c_int32),
     ]
 
 

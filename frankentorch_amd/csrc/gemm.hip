@@ -443,7 +443,8 @@ template <typename T> __device__ __forceinline__ void load_to_lds_16(const T *sr
 
 // EPI >= 0: the epilogue flags are this compile-time mask and alpha is 1 (straight-line output code);
 // EPI < 0: flags and alpha are read from the arguments.
-template <typename T, int BM, int BN, int WM, int WN, int MINW, bool TRANS_B, int EPI>
+// TRANS_A: A is stored [k, m] (its tile is kept [k][m] in LDS and read element-wise, like a [k,n] B).
+template <typename T, int BM, int BN, int WM, int WN, int MINW, bool TRANS_A, bool TRANS_B, int EPI>
 __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const GemmArgs<T> p) {
     using M = Mfma<T>;
     using V = typename M::V;
@@ -457,6 +458,9 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
     constexpr int B_LD = BN * BK * (int)sizeof(T) / 1024 / NW;
     constexpr int LPR = BN * (int)sizeof(T) / 16;             // [k,n] B: lanes per k row of the tile
     constexpr int RPC = kWave / LPR;                          // [k,n] B: k rows per chunk
+    constexpr int LPR_A = BM * (int)sizeof(T) / 16;           // [k,m] A: the same for A
+    constexpr int RPC_A = kWave / LPR_A;
+    static_assert(LPR_A <= kWave && kWave % LPR_A == 0, "a chunk must hold whole k rows of A");
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile rows must divide into 8-row chunks per wavefront");
     static_assert(MT % 16 == 0, "swizzle assumes MFMA tile rows start on a multiple of 16");
     static_assert(LPR <= kWave && kWave % LPR == 0, "a chunk must hold whole k rows of B");
@@ -510,13 +514,24 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
         int tile_m, tile_n;
         tile_of_id(ld_tile - batch * p.tiles_per_batch, p.tiles_m, p.tiles_n, tile_m, tile_n);
         const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
-        ak = p.a + batch * p.stride_a + m0 * p.lda + (int64_t)ld_k * BK;
         const int a_rows = (int)((p.m - m0) < BM ? (p.m - m0) : BM), b_cols = (int)((p.n - n0) < BN ? (p.n - n0) : BN);
+        if constexpr (!TRANS_A) {
+            ak = p.a + batch * p.stride_a + m0 * p.lda + (int64_t)ld_k * BK;
 #pragma unroll
-        for (int i = 0; i < A_LD; ++i) {
-            int row = (wave * A_LD + i) * 8 + lr;
-            row = row < a_rows ? row : a_rows - 1;
-            a_off[i] = (unsigned)row * (unsigned)p.lda + (unsigned)lvec(wave * A_LD + i);
+            for (int i = 0; i < A_LD; ++i) {
+                int row = (wave * A_LD + i) * 8 + lr;
+                row = row < a_rows ? row : a_rows - 1;
+                a_off[i] = (unsigned)row * (unsigned)p.lda + (unsigned)lvec(wave * A_LD + i);
+            }
+        } else {
+            ak = p.a + batch * p.stride_a + (int64_t)ld_k * BK * p.lda + m0;
+            int col = (lane % LPR_A) * EPV;
+            col = col < a_rows ? col : a_rows - EPV;  // m is a multiple of EPV on this path
+#pragma unroll
+            for (int i = 0; i < A_LD; ++i) {
+                const int krow = (wave * A_LD + i) * RPC_A + lane / LPR_A;
+                a_off[i] = (unsigned)krow * (unsigned)p.lda + (unsigned)col;
+            }
         }
         if constexpr (TRANS_B) {
             bk = p.b + batch * p.stride_b + n0 * p.ldb + (int64_t)ld_k * BK;
@@ -545,7 +560,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
         for (int i = 0; i < A_LD; ++i) load_to_lds_16(ak + a_off[i], as + i * 1024u);
 #pragma unroll
         for (int i = 0; i < B_LD; ++i) load_to_lds_16(bk + b_off[i], bs + i * 1024u);
-        ak += BK;
+        ak += TRANS_A ? (int64_t)BK * p.lda : (int64_t)BK;
         bk += TRANS_B ? (int64_t)BK : (int64_t)BK * p.ldb;
         --ld_left;
         if (++ld_k == p.ktiles) {
@@ -558,15 +573,20 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
     // ---- operand fetch: LDS -> registers, one k-chunk ahead of the MFMAs (two register slots) ----
     T af[2][TM][EPV], bf[2][TN][EPV];
     auto fetch = [&](int buf, int kc, int slot) __attribute__((always_inline)) {
-        const T *as = As + buf * BM * BK + (wm0 + lrow) * BK;
-        // B operand base of this lane: row (wn0 + lrow) of the [n][k] tile, or column
-        // (wn0 + lrow) and k row (lane / MT) * EPV of the [k][n] tile.
+        // Operand base of this lane: row (w0 + lrow) of a k-contiguous [rows][k] tile, or column
+        // (w0 + lrow) and k row (lane / MT) * EPV of a [k][rows] tile.
+        const T *as = !TRANS_A ? As + buf * BM * BK + (wm0 + lrow) * BK : As + buf * BK * BM + (lane / MT) * EPV * BM + wm0 + lrow;
         const T *bs = TRANS_B ? Bs + buf * BN * BK + (wn0 + lrow) * BK : Bs + buf * BK * BN + (lane / MT) * EPV * BN + wn0 + lrow;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            const V v = *reinterpret_cast<const V *>(as + i * MT * BK + roff[kc]);
+            if constexpr (!TRANS_A) {
+                const V v = *reinterpret_cast<const V *>(as + i * MT * BK + roff[kc]);
 #pragma unroll
-            for (int e = 0; e < EPV; ++e) af[slot][i][e] = M::elem(v, e);
+                for (int e = 0; e < EPV; ++e) af[slot][i][e] = M::elem(v, e);
+            } else {
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) af[slot][i][e] = as[(kc * KCH + e) * BM + i * MT];
+            }
         }
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
@@ -924,11 +944,12 @@ struct StreamWorkspace {
     void *partials = nullptr;
     size_t partial_bytes = 0;
 };
-int32_t get_workspace(hipStream_t st, size_t partial_bytes, void **partials) {
+// slot 0: split-tile accumulators; slot 1: transposed copy of a [k, m] A operand.
+int32_t get_workspace(hipStream_t st, size_t partial_bytes, void **partials, int slot = 0) {
     static std::mutex mu;
-    static std::map<hipStream_t, StreamWorkspace> *table = new std::map<hipStream_t, StreamWorkspace>();
+    static std::map<std::pair<hipStream_t, int>, StreamWorkspace> *table = new std::map<std::pair<hipStream_t, int>, StreamWorkspace>();
     std::lock_guard<std::mutex> lock(mu);
-    StreamWorkspace &w = (*table)[st];
+    StreamWorkspace &w = (*table)[std::make_pair(st, slot)];
     if (w.partial_bytes < partial_bytes) {
         // The old block returns to the pool; kernels already queued on this stream that still use
         // it are ordered before whatever reuses it on the same stream.
@@ -1001,12 +1022,12 @@ int32_t launch_config(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
                                                  batch, st);
 }
 
-template <typename T, int BM, int BN, int WM, int WN, int MINW, bool TRANS_B, int EPI>
+template <typename T, int BM, int BN, int WM, int WN, int MINW, bool TRANS_A, bool TRANS_B, int EPI>
 int32_t launch_direct_epi(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     constexpr int BK = 128 / (int)sizeof(T);
     constexpr size_t smem = (size_t)2 * (BM + BN) * BK * sizeof(T);
     static int blocks_per_cu = 0;
-    return launch_persistent<T, BM, BN, WM, WN>(gemm_direct_kernel<T, BM, BN, WM, WN, MINW, TRANS_B, EPI>, smem, BK, blocks_per_cu, p,
+    return launch_persistent<T, BM, BN, WM, WN>(gemm_direct_kernel<T, BM, BN, WM, WN, MINW, TRANS_A, TRANS_B, EPI>, smem, BK, blocks_per_cu, p,
                                                  batch, st);
 }
 
@@ -1017,17 +1038,17 @@ int32_t launch_direct(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     if constexpr (SPECIALIZE) {
         if (!p.use_alpha) {
             switch (p.epilogue) {
-                case 0: return launch_direct_epi<T, BM, BN, WM, WN, MINW, TRANS_B, 0>(p, batch, st);
-                case FTH_EPI_BIAS: return launch_direct_epi<T, BM, BN, WM, WN, MINW, TRANS_B, FTH_EPI_BIAS>(p, batch, st);
+                case 0: return launch_direct_epi<T, BM, BN, WM, WN, MINW, false, TRANS_B, 0>(p, batch, st);
+                case FTH_EPI_BIAS: return launch_direct_epi<T, BM, BN, WM, WN, MINW, false, TRANS_B, FTH_EPI_BIAS>(p, batch, st);
                 case FTH_EPI_BIAS | FTH_EPI_GELU:
-                    return launch_direct_epi<T, BM, BN, WM, WN, MINW, TRANS_B, FTH_EPI_BIAS | FTH_EPI_GELU>(p, batch, st);
+                    return launch_direct_epi<T, BM, BN, WM, WN, MINW, false, TRANS_B, FTH_EPI_BIAS | FTH_EPI_GELU>(p, batch, st);
                 case FTH_EPI_BIAS | FTH_EPI_RESIDUAL:
-                    return launch_direct_epi<T, BM, BN, WM, WN, MINW, TRANS_B, FTH_EPI_BIAS | FTH_EPI_RESIDUAL>(p, batch, st);
+                    return launch_direct_epi<T, BM, BN, WM, WN, MINW, false, TRANS_B, FTH_EPI_BIAS | FTH_EPI_RESIDUAL>(p, batch, st);
                 default: break;
             }
         }
     }
-    return launch_direct_epi<T, BM, BN, WM, WN, MINW, TRANS_B, -1>(p, batch, st);
+    return launch_direct_epi<T, BM, BN, WM, WN, MINW, false, TRANS_B, -1>(p, batch, st);
 }
 
 // Tile configurations. The choice depends on the shape only (never on timing), so a given problem
@@ -1094,6 +1115,33 @@ int32_t launch_shape(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     }
 }
 
+// dst[b][i][j] = src[b][j][i]: src is [rows, cols] with pitch ld_src, dst is [cols, rows] contiguous.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(const T *src, T *dst, int64_t rows, int64_t cols, int64_t ld_src,
+                                                        int64_t stride_src, int64_t stride_dst) {
+    __shared__ T tile[32][33];
+    const int tx = threadIdx.x % 32, ty = threadIdx.x / 32;  // 32 x 8
+    const int64_t r0 = (int64_t)blockIdx.y * 32, c0 = (int64_t)blockIdx.x * 32;
+    src += (int64_t)blockIdx.z * stride_src;
+    dst += (int64_t)blockIdx.z * stride_dst;
+#pragma unroll
+    for (int i = 0; i < 32; i += 8) {
+        const int64_t r = r0 + ty + i, c = c0 + tx;
+        tile[ty + i][tx] = (r < rows && c < cols) ? src[r * ld_src + c] : T(0);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 32; i += 8) {
+        const int64_t c = c0 + ty + i, r = r0 + tx;
+        if (c < cols && r < rows) dst[c * rows + r] = tile[tx][ty + i];
+    }
+}
+
+// A stored [k, m]: gemm::sgemm_tb / dgemm_tb (crates/ft-kernel-cpu/src/lib.rs:1484-1524, 262-345).
+// With 16-byte aligned rows of both operands and K a whole number of K-tiles the direct-to-LDS
+// kernel reads A as stored; other shapes go through a transposed copy and the [m, k] path.
+template <typename T> int32_t launch_trans_a(GemmArgs<T> &p, const fth_gemm_desc *d, hipStream_t st);
+
 template <typename T>
 int32_t gemm_entry(const fth_gemm_desc *d, T alpha, const T *a, const T *b, T *c, const T *bias, const T *residual,
                    fth_stream s) {
@@ -1103,9 +1151,10 @@ int32_t gemm_entry(const fth_gemm_desc *d, T alpha, const T *a, const T *b, T *c
     if (d->m == 0 || d->n == 0 || d->batch == 0) return FTH_OK;  // crates/ft-kernel-cpu/src/lib.rs:1311-1313
     FTH_ARG(c != nullptr, "gemm: C is NULL");
     FTH_ARG(d->k == 0 || (a && b), "gemm: NULL operand");
-    FTH_ARG(d->lda >= d->k && d->ldc >= d->n && d->ldb >= (d->trans_b ? d->k : d->n),
+    FTH_ARG(d->lda >= (d->trans_a ? d->m : d->k) && d->ldc >= d->n && d->ldb >= (d->trans_b ? d->k : d->n),
             "gemm: row pitch smaller than the row (lda %lld ldb %lld ldc %lld)", (long long)d->lda, (long long)d->ldb,
             (long long)d->ldc);
+    FTH_ARG(!(d->trans_a && d->trans_b), "gemm: trans_a together with trans_b is not supported");
     FTH_ARG(!(d->epilogue & FTH_EPI_BIAS) || bias, "gemm: bias epilogue without a bias pointer");
     FTH_ARG(!(d->epilogue & FTH_EPI_RESIDUAL) || residual, "gemm: residual epilogue without a residual pointer");
     FTH_ARG((d->epilogue & ~(FTH_EPI_BIAS | FTH_EPI_GELU | FTH_EPI_RESIDUAL)) == 0, "gemm: unknown epilogue bits");
@@ -1126,6 +1175,7 @@ int32_t gemm_entry(const fth_gemm_desc *d, T alpha, const T *a, const T *b, T *c
         FTH_CHECK_LAUNCH("gemm_k0");
         return FTH_OK;
     }
+    if (d->trans_a) return launch_trans_a<T>(p, d, st);
     constexpr int EPV = Mfma<T>::EPV;
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
     // 128-bit global loads along k need 16-byte aligned rows in every batch.
@@ -1139,6 +1189,38 @@ int32_t gemm_entry(const fth_gemm_desc *d, T alpha, const T *a, const T *b, T *c
     const bool vecb = d->n % EPV == 0 && d->k % EPV == 0 && d->ldb % EPV == 0 && al(b) && d->stride_b % EPV == 0;
     if (vec) return vecb ? launch_shape<T, false, true, true>(p, d->batch, st) : launch_shape<T, false, true, false>(p, d->batch, st);
     return vecb ? launch_shape<T, false, false, true>(p, d->batch, st) : launch_shape<T, false, false, false>(p, d->batch, st);
+}
+
+template <typename T> int32_t launch_trans_a(GemmArgs<T> &p, const fth_gemm_desc *d, hipStream_t st) {
+    constexpr int EPV = Mfma<T>::EPV;
+    constexpr int64_t DBK = 128 / (int64_t)sizeof(T);
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    const int64_t lim = ((int64_t)1 << 31) / 128 - 128;
+    const bool direct = d->m % EPV == 0 && d->n % EPV == 0 && d->k % DBK == 0 && d->lda % EPV == 0 && d->ldb % EPV == 0 &&
+                        d->stride_a % EPV == 0 && d->stride_b % EPV == 0 && al(p.a) && al(p.b) && d->lda <= lim && d->ldb <= lim &&
+                        d->ldc <= lim;
+    if (direct) {
+        const int64_t big_tiles = fth::ceil_div(p.m, 128) * fth::ceil_div(p.n, 128) * d->batch;
+        const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
+        if (big_tiles >= cus) return launch_direct_epi<T, 128, 128, 2, 2, 2, true, false, -1>(p, d->batch, st);
+        return launch_direct_epi<T, 64, 64, 2, 2, 2, true, false, -1>(p, d->batch, st);
+    }
+    // Transposed copy A^T [batch][m][k], then the ordinary [m, k] path.
+    size_t elems;
+    if (__builtin_mul_overflow((size_t)d->m, (size_t)d->k, &elems) || __builtin_mul_overflow(elems, (size_t)d->batch, &elems) ||
+        elems > ((size_t)1 << 40))
+        return fth::set_error(FTH_ERR_SIZE_OVERFLOW, "gemm: transposed copy of A too large");
+    void *ws = nullptr;
+    if (int32_t rc = get_workspace(st, elems * sizeof(T), &ws, 1)) return rc;
+    FTH_ARG(d->batch <= 65535 && fth::ceil_div(d->k, 32) <= 65535, "gemm: transposed copy grid too large");
+    transpose_kernel<T><<<dim3((unsigned)fth::ceil_div(d->m, 32), (unsigned)fth::ceil_div(d->k, 32), (unsigned)d->batch), dim3(256), 0, st>>>(
+        p.a, static_cast<T *>(ws), d->k, d->m, d->lda, d->stride_a, d->m * d->k);
+    FTH_CHECK_LAUNCH("gemm_transpose_a");
+    fth_gemm_desc d2 = *d;
+    d2.trans_a = 0;
+    d2.lda = d->k;
+    d2.stride_a = d->m * d->k;
+    return gemm_entry<T>(&d2, p.alpha, static_cast<const T *>(ws), p.b, p.c, p.bias, p.residual, reinterpret_cast<fth_stream>(st));
 }
 
 }  // namespace

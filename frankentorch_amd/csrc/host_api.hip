@@ -198,7 +198,7 @@ template <> struct Dev<double> {
 };
 
 fth_gemm_desc gemm_desc(int64_t m, int64_t n, int64_t k, int trans_b, int64_t batch, int epi) {
-    fth_gemm_desc d;
+    fth_gemm_desc d{};
     d.m = m; d.n = n; d.k = k;
     d.lda = k; d.ldb = trans_b ? k : n; d.ldc = n;
     d.batch = batch;

@@ -157,7 +157,7 @@ int32_t tensor_new(int64_t rows, int64_t cols, fth_tensor **out) {
 }
 
 fth_gemm_desc linear_desc(int64_t m, int64_t n, int64_t k, int epi) {
-    fth_gemm_desc d;
+    fth_gemm_desc d{};
     d.m = m; d.n = n; d.k = k;
     d.lda = k; d.ldb = k; d.ldc = n;
     d.batch = 1;

@@ -183,10 +183,11 @@ def permute_0213(src, dst, d0, d1, d2, d3, stream=None):
 
 
 def gemm_desc(m, n, k, trans_b=False, batch=1, epilogue=EPI_NONE, lda=None, ldb=None, ldc=None, stride_a=None,
-              stride_b=None, stride_c=None) -> _lib.GemmDesc:
+              stride_b=None, stride_c=None, trans_a=False) -> _lib.GemmDesc:
     d = _lib.GemmDesc()
     d.m, d.n, d.k = m, n, k
-    d.lda = k if lda is None else lda
+    d.trans_a = 1 if trans_a else 0
+    d.lda = (m if trans_a else k) if lda is None else lda
     d.ldb = (k if trans_b else n) if ldb is None else ldb
     d.ldc = n if ldc is None else ldc
     d.batch = batch

@@ -224,6 +224,8 @@ typedef struct fth_gemm_desc {
     int64_t stride_a, stride_b, stride_c;
     int32_t trans_b;
     int32_t epilogue; /* bit set of FTH_EPI_* */
+    int32_t trans_a;  /* 1: A is [k, m] row-major (lda >= m) -> gemm::sgemm_tb / dgemm_tb (:1484, :262); not with trans_b */
+    int32_t reserved; /* 0 */
 } fth_gemm_desc;
 int32_t fth_dev_gemm_f32(const fth_gemm_desc *d, float alpha, const float *a, const float *b, float *c,
                          const float *bias, const float *residual, fth_stream s);

@@ -65,6 +65,29 @@ def test_direct_to_lds_kernels(hip, oracle, m, n, k, trans_b, dtype):
     assert rel_err(got[rows], oracle.gelu(ref + bias)) <= tol
 
 
+# A stored [k, m] (gemm::sgemm_tb / dgemm_tb): direct-to-LDS shapes, a ragged shape that goes through
+# the transposed copy, scaled (alpha) and batched.
+@pytest.mark.parametrize("m,n,k", [(256, 384, 128), (200, 300, 96), (72, 40, 96), (77, 50, 33), (1024, 2304, 512), (4, 8, 16)])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_gemm_with_a_stored_k_by_m(hip, oracle, m, n, k, dtype):
+    tol = TOL_GEMM_F32 if dtype == np.float32 else TOL_F64
+    at = synth.uniform(2, "ta", (k, m), -1, 1, dtype=dtype)
+    b = synth.uniform(2, "tb", (k, n), -1, 1, dtype=dtype)
+    da, db = DeviceBuffer.from_host(at), DeviceBuffer.from_host(b)
+    dc = DeviceBuffer((m, n), dtype)
+    hip.gemm(hip.gemm_desc(m, n, k, trans_a=True), da, db, dc)
+    ref = oracle.gemm(np.ascontiguousarray(at.T), b)
+    got = dc.to_host()
+    assert rel_err(got, ref) <= tol
+    hip.gemm(hip.gemm_desc(m, n, k, trans_a=True), da, db, dc, alpha=0.25)
+    assert np.array_equal(dc.to_host(), dtype(0.25) * got)
+    # batched with a shared right operand
+    at3 = synth.uniform(2, "ta3", (3, k, m), -1, 1, dtype=dtype)
+    da3, dc3 = DeviceBuffer.from_host(at3), DeviceBuffer((3, m, n), dtype)
+    hip.gemm(hip.gemm_desc(m, n, k, trans_a=True, batch=3, stride_b=0), da3, db, dc3)
+    assert rel_err(dc3.to_host()[2], oracle.gemm(np.ascontiguousarray(at3[2].T), b)) <= tol
+
+
 def test_direct_to_lds_kernels_with_row_pitch_and_batches(hip, oracle):
     """Sub-blocks of larger buffers (pitch > row, 16-byte aligned offsets) and a batched problem whose
     tiles straddle workgroup ranges, through the direct kernels."""
