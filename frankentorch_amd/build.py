@@ -24,6 +24,7 @@ HIP_SOURCES = [
     "indexops.hip",
     "gemm.hip",
     "sdpa.hip",
+    "backward.hip",
     "host_api.hip",
     "resident.hip",
 ]

@@ -1,0 +1,651 @@
+// Backward kernels of the transformer forward ops: LayerNorm, RMSNorm, linear and scaled-dot-product
+// attention. Every reduction has a fixed order (no atomics), so results are bitwise repeatable.
+//
+// replaces layer_norm_backward_f32 / _f64 (crates/ft-kernel-cpu/src/lib.rs:6189-6322, 6052-6183),
+// rms_norm_backward_f32 / _f64 (:6574-6646, 6503-6570), linear_backward_f64 (:17226-17302) and its
+// f32 use through the same formulas, sdpa_backward_f32 / _f64 (:5539-5650, 5300-5414).
+//
+// Norm backward. One workgroup owns a run of consecutive rows. A row's x and dy are loaded once
+// into registers (128-bit loads), the row statistics and the two dot products are reduced with a
+// fixed butterfly per wavefront and a fixed left-to-right fold across the four wavefronts, dx is
+// stored once, and the column sums (dweight, dbias) of the workgroup's rows are accumulated in
+// registers in row order. Each workgroup then writes one row of partial column sums; a second
+// kernel adds the partials in workgroup order. The reference sums the rows serially in one chain;
+// this is the same sum re-associated into (rows of a workgroup) then (workgroups), which the
+// 1e-5 / 1e-12 parity tolerances cover. Row lengths that do not fit the register layout take a
+// streaming kernel (x and dy re-read from cache per pass) plus a separate column-sum pass.
+//
+// Linear backward is two MFMA GEMMs (dx = dy.W as stored, dweight = dy^T.x with dy read as stored
+// through the [k, m] operand path) and a column sum of dy. SDPA backward follows the reference's
+// own structure on the device: P = softmax(scale * Q.K^T) and dU are materialised per
+// (batch*head) in a caller-provided workspace (2 * num_bh * seq_q * seq_k elements), the five
+// products are batched MFMA GEMMs and the two row passes are HBM-bound row kernels.
+
+#include <type_traits>
+
+#include "common.hpp"
+
+namespace {
+
+constexpr int kWave = 64;
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / kWave;
+
+template <typename T> struct Vec16;
+template <> struct Vec16<float> {
+    using type = float4;
+    static constexpr int N = 4;
+};
+template <> struct Vec16<double> {
+    using type = double2;
+    static constexpr int N = 2;
+};
+__device__ __forceinline__ float vget(const float4 &v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+__device__ __forceinline__ double vget(const double2 &v, int i) { return i == 0 ? v.x : v.y; }
+__device__ __forceinline__ void vset(float4 &v, int i, float x) {
+    if (i == 0) v.x = x;
+    else if (i == 1) v.y = x;
+    else if (i == 2) v.z = x;
+    else v.w = x;
+}
+__device__ __forceinline__ void vset(double2 &v, int i, double x) {
+    if (i == 0) v.x = x;
+    else v.y = x;
+}
+
+template <typename T> __device__ __forceinline__ T wave_sum(T v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// Sum of NV values per thread over the workgroup: butterfly inside each wavefront, then wavefront 0..3
+// added left to right by every thread (same result in all threads). `red` holds kWaves * NV values.
+template <typename T, int NV> __device__ __forceinline__ void block_sum(T (&v)[NV], T *red) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) v[i] = wave_sum(v[i]);
+    __syncthreads();  // the previous use of `red` is over
+    if (lane == 0) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) red[wave * NV + i] = v[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        T s = red[i];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) s += red[w * NV + i];
+        v[i] = s;
+    }
+}
+
+template <typename T> __device__ __forceinline__ T t_rsqrt_of(T v) { return T(1) / sqrt(v); }
+
+// ---- register-resident norm backward ----
+// RMS = false: LayerNorm (weight required, partial dbias written); RMS = true: RMSNorm (weight optional).
+// VPT: 16-byte vectors per thread; cols <= kThreads * VPT * N and cols % N == 0.
+template <typename T, int VPT, bool RMS>
+__global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__restrict__ dy, const T *__restrict__ x,
+                                                                 const T *__restrict__ w, int64_t rows, int cols, T eps,
+                                                                 T *__restrict__ dx, T *__restrict__ part_w,
+                                                                 T *__restrict__ part_b, int rows_per_block) {
+    using V = typename Vec16<T>::type;
+    constexpr int N = Vec16<T>::N;
+    __shared__ T red[kWaves * 2];
+    const int tid = threadIdx.x;
+    const int nvec = cols / N;
+    const T inv_n = T(1) / (T)cols;
+    V wv[VPT];
+    T aw[VPT][N], ab[VPT][N];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int v = tid + i * kThreads;
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+            aw[i][e] = T(0);
+            ab[i][e] = T(0);
+            vset(wv[i], e, T(1));
+        }
+        if (w != nullptr && v < nvec) wv[i] = reinterpret_cast<const V *>(w)[v];
+    }
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
+    for (int64_t r = r0; r < r1; ++r) {
+        const V *xr = reinterpret_cast<const V *>(x + r * cols);
+        const V *dyr = reinterpret_cast<const V *>(dy + r * cols);
+        V xv[VPT], gv[VPT];
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) {
+            const int v = tid + i * kThreads;
+            if (v < nvec) {
+                xv[i] = xr[v];
+                gv[i] = dyr[v];
+            } else {
+#pragma unroll
+                for (int e = 0; e < N; ++e) {
+                    vset(xv[i], e, T(0));
+                    vset(gv[i], e, T(0));
+                }
+            }
+        }
+        if constexpr (!RMS) {
+            T s[1] = {T(0)};
+#pragma unroll
+            for (int i = 0; i < VPT; ++i)
+#pragma unroll
+                for (int e = 0; e < N; ++e) s[0] += vget(xv[i], e);
+            block_sum<T, 1>(s, red);
+            const T mean = s[0] * inv_n;
+            T q[1] = {T(0)};
+#pragma unroll
+            for (int i = 0; i < VPT; ++i) {
+                const bool live = tid + i * kThreads < nvec;
+#pragma unroll
+                for (int e = 0; e < N; ++e) {
+                    const T d = vget(xv[i], e) - mean;
+                    if (live) q[0] += d * d;
+                }
+            }
+            block_sum<T, 1>(q, red);
+            const T rstd = t_rsqrt_of(q[0] * inv_n + eps);
+            T c[2] = {T(0), T(0)};
+#pragma unroll
+            for (int i = 0; i < VPT; ++i) {
+                const bool live = tid + i * kThreads < nvec;
+#pragma unroll
+                for (int e = 0; e < N; ++e) {
+                    const T xhat = (vget(xv[i], e) - mean) * rstd;
+                    const T dxhat = vget(gv[i], e) * vget(wv[i], e);
+                    if (live) {
+                        c[0] += dxhat;
+                        c[1] += dxhat * xhat;
+                    }
+                }
+            }
+            block_sum<T, 2>(c, red);
+            V *dxr = reinterpret_cast<V *>(dx + r * cols);
+#pragma unroll
+            for (int i = 0; i < VPT; ++i) {
+                const int v = tid + i * kThreads;
+                V o;
+#pragma unroll
+                for (int e = 0; e < N; ++e) {
+                    const T xhat = (vget(xv[i], e) - mean) * rstd;
+                    const T dxhat = vget(gv[i], e) * vget(wv[i], e);
+                    vset(o, e, rstd * (dxhat - (c[0] + xhat * c[1]) * inv_n));
+                    aw[i][e] += vget(gv[i], e) * xhat;
+                    ab[i][e] += vget(gv[i], e);
+                }
+                if (v < nvec) dxr[v] = o;
+            }
+        } else {
+            T s[1] = {T(0)};
+#pragma unroll
+            for (int i = 0; i < VPT; ++i)
+#pragma unroll
+                for (int e = 0; e < N; ++e) s[0] += vget(xv[i], e) * vget(xv[i], e);
+            block_sum<T, 1>(s, red);
+            const T rstd = t_rsqrt_of(s[0] * inv_n + eps);
+            T c[1] = {T(0)};
+#pragma unroll
+            for (int i = 0; i < VPT; ++i)
+#pragma unroll
+                for (int e = 0; e < N; ++e) c[0] += (vget(gv[i], e) * vget(wv[i], e)) * vget(xv[i], e);
+            block_sum<T, 1>(c, red);
+            const T coef = rstd * rstd * rstd * c[0] * inv_n;
+            V *dxr = reinterpret_cast<V *>(dx + r * cols);
+#pragma unroll
+            for (int i = 0; i < VPT; ++i) {
+                const int v = tid + i * kThreads;
+                V o;
+#pragma unroll
+                for (int e = 0; e < N; ++e) {
+                    const T g = vget(gv[i], e) * vget(wv[i], e);
+                    vset(o, e, rstd * g - coef * vget(xv[i], e));
+                    aw[i][e] += vget(gv[i], e) * vget(xv[i], e) * rstd;
+                }
+                if (v < nvec) dxr[v] = o;
+            }
+        }
+    }
+    // one row of partial column sums per workgroup
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int v = tid + i * kThreads;
+        if (v < nvec) {
+            V ow, ob;
+#pragma unroll
+            for (int e = 0; e < N; ++e) {
+                vset(ow, e, aw[i][e]);
+                vset(ob, e, ab[i][e]);
+            }
+            if (part_w) reinterpret_cast<V *>(part_w + (int64_t)blockIdx.x * cols)[v] = ow;
+            if (part_b) reinterpret_cast<V *>(part_b + (int64_t)blockIdx.x * cols)[v] = ob;
+        }
+    }
+}
+
+// ---- streaming norm backward (any row length): one workgroup per row, x / dy re-read per pass ----
+// Writes dx and the row statistics (mean, rstd; mean = 0 for RMSNorm) for the column-sum pass.
+template <typename T, bool RMS>
+__global__ __launch_bounds__(kThreads) void norm_backward_stream_kernel(const T *__restrict__ dy, const T *__restrict__ x,
+                                                                        const T *__restrict__ w, int64_t cols, T eps,
+                                                                        T *__restrict__ dx, T *__restrict__ stats) {
+    __shared__ T red[kWaves * 2];
+    const int64_t r = blockIdx.x;
+    const T *xr = x + r * cols, *dyr = dy + r * cols;
+    T *dxr = dx + r * cols;
+    const T inv_n = T(1) / (T)cols;
+    T mean = T(0), rstd;
+    if constexpr (!RMS) {
+        T s[1] = {T(0)};
+        for (int64_t j = threadIdx.x; j < cols; j += kThreads) s[0] += xr[j];
+        block_sum<T, 1>(s, red);
+        mean = s[0] * inv_n;
+        T q[1] = {T(0)};
+        for (int64_t j = threadIdx.x; j < cols; j += kThreads) {
+            const T d = xr[j] - mean;
+            q[0] += d * d;
+        }
+        block_sum<T, 1>(q, red);
+        rstd = t_rsqrt_of(q[0] * inv_n + eps);
+        T c[2] = {T(0), T(0)};
+        for (int64_t j = threadIdx.x; j < cols; j += kThreads) {
+            const T xhat = (xr[j] - mean) * rstd;
+            const T dxhat = dyr[j] * w[j];
+            c[0] += dxhat;
+            c[1] += dxhat * xhat;
+        }
+        block_sum<T, 2>(c, red);
+        for (int64_t j = threadIdx.x; j < cols; j += kThreads) {
+            const T xhat = (xr[j] - mean) * rstd;
+            const T dxhat = dyr[j] * w[j];
+            dxr[j] = rstd * (dxhat - (c[0] + xhat * c[1]) * inv_n);
+        }
+    } else {
+        T s[1] = {T(0)};
+        for (int64_t j = threadIdx.x; j < cols; j += kThreads) s[0] += xr[j] * xr[j];
+        block_sum<T, 1>(s, red);
+        rstd = t_rsqrt_of(s[0] * inv_n + eps);
+        T c[1] = {T(0)};
+        for (int64_t j = threadIdx.x; j < cols; j += kThreads) c[0] += (dyr[j] * (w ? w[j] : T(1))) * xr[j];
+        block_sum<T, 1>(c, red);
+        const T coef = rstd * rstd * rstd * c[0] * inv_n;
+        for (int64_t j = threadIdx.x; j < cols; j += kThreads) dxr[j] = rstd * (dyr[j] * (w ? w[j] : T(1))) - coef * xr[j];
+    }
+    if (threadIdx.x == 0 && stats) {
+        stats[2 * r] = mean;
+        stats[2 * r + 1] = rstd;
+    }
+}
+
+// Partial column sums over a run of rows, one thread per column (coalesced), rows in order.
+// MODE 0: sum of src; MODE 1: LayerNorm dweight, sum of dy * (x - mean) * rstd; MODE 2: RMSNorm
+// dweight, sum of dy * x * rstd. part[blockIdx.y][col].
+template <typename T, int MODE>
+__global__ __launch_bounds__(kThreads) void col_partial_kernel(const T *__restrict__ src, const T *__restrict__ x,
+                                                               const T *__restrict__ stats, int64_t rows, int64_t cols,
+                                                               int64_t ld, int rows_per_block, T *__restrict__ part) {
+    const int64_t col = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (col >= cols) return;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
+    T acc = T(0);
+    for (int64_t r = r0; r < r1; ++r) {
+        const T g = src[r * ld + col];
+        if constexpr (MODE == 0) acc += g;
+        else if constexpr (MODE == 1) acc += g * ((x[r * ld + col] - stats[2 * r]) * stats[2 * r + 1]);
+        else acc += g * x[r * ld + col] * stats[2 * r + 1];
+    }
+    part[(int64_t)blockIdx.y * cols + col] = acc;
+}
+
+// out[col] = part[0][col] + part[1][col] + ... in that order.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void col_final_kernel(const T *__restrict__ part, int nparts, int64_t cols, T *__restrict__ out) {
+    const int64_t col = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (col >= cols) return;
+    T acc = T(0);
+    for (int b = 0; b < nparts; ++b) acc += part[(int64_t)b * cols + col];
+    out[col] = acc;
+}
+
+// Zero fill as a kernel (memset nodes are avoided so that callers can capture these entry points).
+template <typename T> __global__ __launch_bounds__(kThreads) void zero_kernel(T *dst, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (i < n) dst[i] = T(0);
+}
+template <typename T> int32_t zero_fill(T *dst, int64_t n, hipStream_t st) {
+    if (n <= 0) return FTH_OK;
+    FTH_ARG(fth::ceil_div(n, kThreads) <= 2147483647LL, "zero fill: extent too large");
+    zero_kernel<T><<<dim3((unsigned)fth::ceil_div(n, kThreads)), dim3(kThreads), 0, st>>>(dst, n);
+    FTH_CHECK_LAUNCH("zero_fill");
+    return FTH_OK;
+}
+
+inline int pick_rows_per_block(int64_t rows) {
+    // enough workgroups to fill the chip several times over, at most 64 rows each
+    const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
+    int64_t r = rows / ((int64_t)cus * 4);
+    if (r < 1) r = 1;
+    if (r > 64) r = 64;
+    return (int)r;
+}
+
+template <typename T> bool norm_fast_path(int64_t cols, const void *a, const void *b, const void *c, const void *d) {
+    constexpr int N = Vec16<T>::N;
+    auto al = [](const void *q) { return q == nullptr || (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    return cols % N == 0 && cols <= (int64_t)kThreads * 16 * N && al(a) && al(b) && al(c) && al(d);
+}
+
+template <typename T> size_t norm_backward_workspace(int64_t rows, int64_t cols) {
+    // fast path: 2 partial arrays of [blocks, cols]; streaming path: stats [rows, 2] + 2 partial arrays
+    const int rpb = pick_rows_per_block(rows);
+    const int64_t blocks = fth::ceil_div(rows, rpb);
+    return (size_t)(2 * blocks * cols + 2 * rows + 64) * sizeof(T);
+}
+
+template <typename T, bool RMS>
+int32_t norm_backward_entry(const T *dy, const T *x, const T *w, int64_t rows, int64_t cols, T eps, T *dx, T *dw, T *db,
+                            void *workspace, size_t workspace_bytes, fth_stream s) {
+    FTH_REQUIRE_DEVICE();
+    FTH_ARG(rows >= 0 && cols >= 0, "norm backward: negative extent");
+    FTH_ARG(RMS || w != nullptr, "layer_norm backward: weight is required");
+    FTH_ARG(RMS || (dw != nullptr && db != nullptr), "layer_norm backward: dweight and dbias are required");
+    FTH_ARG(!(RMS && w == nullptr && dw != nullptr), "rms_norm backward: dweight without a weight");
+    hipStream_t st = fth::resolve_stream(s);
+    if (cols == 0) return FTH_OK;
+    const bool want_w = dw != nullptr;
+    if (rows == 0) {
+        if (want_w) if (int32_t rc = zero_fill<T>(dw, cols, st)) return rc;
+        if (db) if (int32_t rc = zero_fill<T>(db, cols, st)) return rc;
+        return FTH_OK;
+    }
+    FTH_ARG(dy && x && dx, "norm backward: NULL operand");
+    FTH_ARG(cols <= 2147483647LL && rows <= 2147483647LL, "norm backward: extent too large");
+    FTH_ARG(workspace_bytes >= norm_backward_workspace<T>(rows, cols) && (workspace != nullptr),
+            "norm backward: workspace of %zu bytes needed, %zu given", norm_backward_workspace<T>(rows, cols), workspace_bytes);
+    const int rpb = pick_rows_per_block(rows);
+    const int64_t blocks = fth::ceil_div(rows, rpb);
+    T *part_w = static_cast<T *>(workspace);
+    T *part_b = part_w + blocks * cols;
+    T *stats = part_b + blocks * cols;
+    const int64_t col_blocks = fth::ceil_div(cols, kThreads);
+    if (norm_fast_path<T>(cols, dy, x, w, dx)) {
+        constexpr int N = Vec16<T>::N;
+        const int64_t nvec = cols / N;
+        const int vpt = (int)fth::ceil_div(nvec, kThreads);
+        T *pw = want_w ? part_w : nullptr, *pb = db ? part_b : nullptr;
+#define FTH_NORM_BWD(V) \
+    norm_backward_kernel<T, V, RMS><<<dim3((unsigned)blocks), dim3(kThreads), 0, st>>>(dy, x, w, rows, (int)cols, eps, dx, pw, pb, rpb)
+        if (vpt <= 1) FTH_NORM_BWD(1);
+        else if (vpt <= 2) FTH_NORM_BWD(2);
+        else if (vpt <= 4) FTH_NORM_BWD(4);
+        else if (vpt <= 8) FTH_NORM_BWD(8);
+        else FTH_NORM_BWD(16);
+#undef FTH_NORM_BWD
+        FTH_CHECK_LAUNCH("norm_backward");
+    } else {
+        norm_backward_stream_kernel<T, RMS><<<dim3((unsigned)rows), dim3(kThreads), 0, st>>>(dy, x, w, cols, eps, dx, stats);
+        FTH_CHECK_LAUNCH("norm_backward_stream");
+        if (want_w) {
+            col_partial_kernel<T, RMS ? 2 : 1><<<dim3((unsigned)col_blocks, (unsigned)blocks), dim3(kThreads), 0, st>>>(
+                dy, x, stats, rows, cols, cols, rpb, part_w);
+            FTH_CHECK_LAUNCH("norm_backward_dweight");
+        }
+        if (db) {
+            col_partial_kernel<T, 0><<<dim3((unsigned)col_blocks, (unsigned)blocks), dim3(kThreads), 0, st>>>(
+                dy, nullptr, nullptr, rows, cols, cols, rpb, part_b);
+            FTH_CHECK_LAUNCH("norm_backward_dbias");
+        }
+    }
+    if (want_w) {
+        col_final_kernel<T><<<dim3((unsigned)col_blocks), dim3(kThreads), 0, st>>>(part_w, (int)blocks, cols, dw);
+        FTH_CHECK_LAUNCH("norm_backward_dweight_sum");
+    }
+    if (db) {
+        col_final_kernel<T><<<dim3((unsigned)col_blocks), dim3(kThreads), 0, st>>>(part_b, (int)blocks, cols, db);
+        FTH_CHECK_LAUNCH("norm_backward_dbias_sum");
+    }
+    return FTH_OK;
+}
+
+// ---- linear backward ----
+template <typename T> size_t linear_backward_workspace(int64_t batch, int64_t out_f) {
+    const int rpb = pick_rows_per_block(batch);
+    return (size_t)(fth::ceil_div(batch > 0 ? batch : 1, rpb) * out_f + 64) * sizeof(T);
+}
+
+template <typename T> int32_t dev_gemm(const fth_gemm_desc *d, T alpha, const T *a, const T *b, T *c, fth_stream s);
+template <> int32_t dev_gemm<float>(const fth_gemm_desc *d, float alpha, const float *a, const float *b, float *c, fth_stream s) {
+    return fth_dev_gemm_f32(d, alpha, a, b, c, nullptr, nullptr, s);
+}
+template <> int32_t dev_gemm<double>(const fth_gemm_desc *d, double alpha, const double *a, const double *b, double *c, fth_stream s) {
+    return fth_dev_gemm_f64(d, alpha, a, b, c, nullptr, nullptr, s);
+}
+
+inline fth_gemm_desc make_desc(int64_t m, int64_t n, int64_t k, int trans_a, int trans_b, int64_t batch) {
+    fth_gemm_desc d{};
+    d.m = m; d.n = n; d.k = k;
+    d.lda = trans_a ? m : k;
+    d.ldb = trans_b ? k : n;
+    d.ldc = n;
+    d.batch = batch;
+    d.stride_a = m * k; d.stride_b = k * n; d.stride_c = m * n;
+    d.trans_a = trans_a; d.trans_b = trans_b;
+    return d;
+}
+
+template <typename T>
+int32_t linear_backward_entry(const T *dy, const T *x, const T *w, int64_t batch, int64_t in_f, int64_t out_f, T *dx, T *dw,
+                              T *db, void *workspace, size_t workspace_bytes, fth_stream s) {
+    FTH_REQUIRE_DEVICE();
+    FTH_ARG(batch >= 0 && in_f >= 0 && out_f >= 0, "linear backward: negative extent");
+    hipStream_t st = fth::resolve_stream(s);
+    fth_stream fs = reinterpret_cast<fth_stream>(st);
+    // dx = dy . W : [batch, out] . [out, in]
+    if (batch > 0 && in_f > 0) {
+        FTH_ARG(dx != nullptr, "linear backward: dx is NULL");
+        fth_gemm_desc d = make_desc(batch, in_f, out_f, 0, 0, 1);
+        if (int32_t rc = dev_gemm<T>(&d, T(1), dy, w, dx, fs)) return rc;
+    }
+    // dweight = dy^T . x : dy [batch, out] read as the [k, m] operand
+    if (out_f > 0 && in_f > 0) {
+        FTH_ARG(dw != nullptr, "linear backward: dweight is NULL");
+        fth_gemm_desc d = make_desc(out_f, in_f, batch, 1, 0, 1);
+        if (int32_t rc = dev_gemm<T>(&d, T(1), dy, x, dw, fs)) return rc;
+    }
+    if (db && out_f > 0) {
+        if (batch == 0) {
+            if (int32_t rc = zero_fill<T>(db, out_f, st)) return rc;
+            return FTH_OK;
+        }
+        FTH_ARG(workspace != nullptr && workspace_bytes >= linear_backward_workspace<T>(batch, out_f),
+                "linear backward: workspace of %zu bytes needed, %zu given", linear_backward_workspace<T>(batch, out_f), workspace_bytes);
+        const int rpb = pick_rows_per_block(batch);
+        const int64_t blocks = fth::ceil_div(batch, rpb), col_blocks = fth::ceil_div(out_f, kThreads);
+        T *part = static_cast<T *>(workspace);
+        col_partial_kernel<T, 0><<<dim3((unsigned)col_blocks, (unsigned)blocks), dim3(kThreads), 0, st>>>(dy, nullptr, nullptr, batch,
+                                                                                                         out_f, out_f, rpb, part);
+        FTH_CHECK_LAUNCH("linear_backward_dbias");
+        col_final_kernel<T><<<dim3((unsigned)col_blocks), dim3(kThreads), 0, st>>>(part, (int)blocks, out_f, db);
+        FTH_CHECK_LAUNCH("linear_backward_dbias_sum");
+    }
+    return FTH_OK;
+}
+
+// ---- SDPA backward row passes ----
+// In place on the score rows: scale, strict-max scan over the first `limit` entries, exp, sum,
+// divide, zero tail (the forward's row loop, crates/ft-kernel-cpu/src/lib.rs:5594-5616). One
+// wavefront per row; limit = min(i + 1, seq_k) when causal, i = row % seq_q.
+template <typename T> __device__ __forceinline__ T dev_exp_t(T v);
+template <> __device__ __forceinline__ float dev_exp_t<float>(float v) { return expf(v); }
+template <> __device__ __forceinline__ double dev_exp_t<double>(double v) { return exp(v); }
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void sdpa_softmax_rows_kernel(T *__restrict__ p, int64_t rows, int64_t seq_q, int64_t seq_k,
+                                                                    T scale, int causal) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t r = (int64_t)blockIdx.x * kWaves + threadIdx.x / kWave;
+    if (r >= rows) return;
+    const int64_t i = r % seq_q;
+    const int64_t limit = causal ? (i + 1 < seq_k ? i + 1 : seq_k) : seq_k;
+    T *row = p + r * seq_k;
+    T m = -__builtin_inf();
+    for (int64_t j = lane; j < limit; j += kWave) {
+        const T v = row[j] * scale;
+        m = v > m ? v : m;
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const T o = __shfl_xor(m, off, kWave);
+        m = o > m ? o : m;
+    }
+    T sum = T(0);
+    for (int64_t j = lane; j < limit; j += kWave) {
+        const T e = dev_exp_t<T>(row[j] * scale - m);
+        row[j] = e;
+        sum += e;
+    }
+    sum = wave_sum(sum);
+    for (int64_t j = lane; j < limit; j += kWave) row[j] = row[j] / sum;
+    for (int64_t j = limit + lane; j < seq_k; j += kWave) row[j] = T(0);
+}
+
+// dU_ij = P_ij * (dU_ij - sum_j P_ij dU_ij), in place on dU (:5637-5647).
+template <typename T>
+__global__ __launch_bounds__(kThreads) void sdpa_softmax_backward_rows_kernel(const T *__restrict__ p, T *__restrict__ du, int64_t rows,
+                                                                             int64_t seq_k) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t r = (int64_t)blockIdx.x * kWaves + threadIdx.x / kWave;
+    if (r >= rows) return;
+    const T *pr = p + r * seq_k;
+    T *dr = du + r * seq_k;
+    T dot = T(0);
+    for (int64_t j = lane; j < seq_k; j += kWave) dot += pr[j] * dr[j];
+    dot = wave_sum(dot);
+    for (int64_t j = lane; j < seq_k; j += kWave) dr[j] = pr[j] * (dr[j] - dot);
+}
+
+template <typename T> size_t sdpa_backward_workspace(int64_t num_bh, int64_t seq_q, int64_t seq_k) {
+    return (size_t)(2 * num_bh * seq_q * seq_k + 64) * sizeof(T);
+}
+
+template <typename T>
+int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, int64_t num_bh, int64_t seq_q, int64_t seq_k,
+                            int64_t d_k, int64_t d_v, T scale, int causal, T *dq, T *dk, T *dv, void *workspace,
+                            size_t workspace_bytes, fth_stream s) {
+    FTH_REQUIRE_DEVICE();
+    FTH_ARG(num_bh >= 0 && seq_q >= 0 && seq_k >= 0 && d_k >= 0 && d_v >= 0, "sdpa backward: negative extent");
+    hipStream_t st = fth::resolve_stream(s);
+    fth_stream fs = reinterpret_cast<fth_stream>(st);
+    if (num_bh == 0) return FTH_OK;
+    // Degenerate extents: the gradients that exist are all zero (crates/ft-kernel-cpu/src/lib.rs:5552-5554).
+    if (seq_q == 0 || seq_k == 0 || (d_k == 0 && d_v == 0)) {
+        if (dq && num_bh * seq_q * d_k > 0) if (int32_t rc = zero_fill<T>(dq, num_bh * seq_q * d_k, st)) return rc;
+        if (dk && num_bh * seq_k * d_k > 0) if (int32_t rc = zero_fill<T>(dk, num_bh * seq_k * d_k, st)) return rc;
+        if (dv && num_bh * seq_k * d_v > 0) if (int32_t rc = zero_fill<T>(dv, num_bh * seq_k * d_v, st)) return rc;
+        return FTH_OK;
+    }
+    FTH_ARG(q && k && v && dout && dq && dk && dv, "sdpa backward: NULL operand");
+    int64_t pe;
+    FTH_ARG(!__builtin_mul_overflow(num_bh, seq_q, &pe) && !__builtin_mul_overflow(pe, seq_k, &pe) && pe < ((int64_t)1 << 40),
+            "sdpa backward: score matrix too large");
+    FTH_ARG(workspace != nullptr && workspace_bytes >= sdpa_backward_workspace<T>(num_bh, seq_q, seq_k),
+            "sdpa backward: workspace of %zu bytes needed, %zu given", sdpa_backward_workspace<T>(num_bh, seq_q, seq_k), workspace_bytes);
+    T *p = static_cast<T *>(workspace);
+    T *du = p + pe;
+    const int64_t rows = num_bh * seq_q;
+    FTH_ARG(fth::ceil_div(rows, kWaves) <= 2147483647LL, "sdpa backward: too many rows");
+    // P = Q . K^T  (scores; scaled inside the row pass)
+    if (d_k > 0) {
+        fth_gemm_desc d = make_desc(seq_q, seq_k, d_k, 0, 1, num_bh);
+        if (int32_t rc = dev_gemm<T>(&d, T(1), q, k, p, fs)) return rc;
+    } else {
+        if (int32_t rc = zero_fill<T>(p, pe, st)) return rc;
+    }
+    sdpa_softmax_rows_kernel<T><<<dim3((unsigned)fth::ceil_div(rows, kWaves)), dim3(kThreads), 0, st>>>(p, rows, seq_q, seq_k, scale, causal);
+    FTH_CHECK_LAUNCH("sdpa_backward_softmax");
+    // dU = dOut . V^T
+    if (d_v > 0) {
+        fth_gemm_desc d = make_desc(seq_q, seq_k, d_v, 0, 1, num_bh);
+        if (int32_t rc = dev_gemm<T>(&d, T(1), dout, v, du, fs)) return rc;
+    } else {
+        if (int32_t rc = zero_fill<T>(du, pe, st)) return rc;
+    }
+    // dV = P^T . dOut  (P read as the [k, m] operand) -- before dU is overwritten? dV does not use dU.
+    if (d_v > 0) {
+        fth_gemm_desc d = make_desc(seq_k, d_v, seq_q, 1, 0, num_bh);
+        if (int32_t rc = dev_gemm<T>(&d, T(1), p, dout, dv, fs)) return rc;
+    }
+    sdpa_softmax_backward_rows_kernel<T><<<dim3((unsigned)fth::ceil_div(rows, kWaves)), dim3(kThreads), 0, st>>>(p, du, rows, seq_k);
+    FTH_CHECK_LAUNCH("sdpa_backward_softmax_grad");
+    if (d_k > 0) {
+        // dQ = scale * dU . K ; dK = scale * dU^T . Q
+        fth_gemm_desc dqd = make_desc(seq_q, d_k, seq_k, 0, 0, num_bh);
+        if (int32_t rc = dev_gemm<T>(&dqd, scale, du, k, dq, fs)) return rc;
+        fth_gemm_desc dkd = make_desc(seq_k, d_k, seq_q, 1, 0, num_bh);
+        if (int32_t rc = dev_gemm<T>(&dkd, scale, du, q, dk, fs)) return rc;
+    }
+    return FTH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t fth_dev_norm_backward_workspace_bytes(int64_t rows, int64_t cols, int32_t dtype) {
+    if (rows < 0 || cols < 0) return 0;
+    return dtype == FTH_DTYPE_F64 ? norm_backward_workspace<double>(rows, cols) : norm_backward_workspace<float>(rows, cols);
+}
+int32_t fth_dev_layer_norm_backward_f32(const float *dy, const float *x, const float *weight, int64_t rows, int64_t cols, float eps,
+                                        float *dx, float *dweight, float *dbias, void *workspace, size_t workspace_bytes,
+                                        fth_stream s) {
+    return norm_backward_entry<float, false>(dy, x, weight, rows, cols, eps, dx, dweight, dbias, workspace, workspace_bytes, s);
+}
+int32_t fth_dev_layer_norm_backward_f64(const double *dy, const double *x, const double *weight, int64_t rows, int64_t cols, double eps,
+                                        double *dx, double *dweight, double *dbias, void *workspace, size_t workspace_bytes,
+                                        fth_stream s) {
+    return norm_backward_entry<double, false>(dy, x, weight, rows, cols, eps, dx, dweight, dbias, workspace, workspace_bytes, s);
+}
+int32_t fth_dev_rms_norm_backward_f32(const float *dy, const float *x, const float *weight, int64_t rows, int64_t cols, float eps,
+                                      float *dx, float *dweight, void *workspace, size_t workspace_bytes, fth_stream s) {
+    return norm_backward_entry<float, true>(dy, x, weight, rows, cols, eps, dx, dweight, nullptr, workspace, workspace_bytes, s);
+}
+int32_t fth_dev_rms_norm_backward_f64(const double *dy, const double *x, const double *weight, int64_t rows, int64_t cols, double eps,
+                                      double *dx, double *dweight, void *workspace, size_t workspace_bytes, fth_stream s) {
+    return norm_backward_entry<double, true>(dy, x, weight, rows, cols, eps, dx, dweight, nullptr, workspace, workspace_bytes, s);
+}
+
+size_t fth_dev_linear_backward_workspace_bytes(int64_t batch, int64_t out_features, int32_t dtype) {
+    if (batch < 0 || out_features < 0) return 0;
+    return dtype == FTH_DTYPE_F64 ? linear_backward_workspace<double>(batch, out_features) : linear_backward_workspace<float>(batch, out_features);
+}
+int32_t fth_dev_linear_backward_f32(const float *dy, const float *x, const float *weight, int64_t batch, int64_t in_features,
+                                    int64_t out_features, float *dx, float *dweight, float *dbias, void *workspace,
+                                    size_t workspace_bytes, fth_stream s) {
+    return linear_backward_entry<float>(dy, x, weight, batch, in_features, out_features, dx, dweight, dbias, workspace, workspace_bytes, s);
+}
+int32_t fth_dev_linear_backward_f64(const double *dy, const double *x, const double *weight, int64_t batch, int64_t in_features,
+                                    int64_t out_features, double *dx, double *dweight, double *dbias, void *workspace,
+                                    size_t workspace_bytes, fth_stream s) {
+    return linear_backward_entry<double>(dy, x, weight, batch, in_features, out_features, dx, dweight, dbias, workspace, workspace_bytes, s);
+}
+
+size_t fth_dev_sdpa_backward_workspace_bytes(int64_t num_bh, int64_t seq_q, int64_t seq_k, int32_t dtype) {
+    if (num_bh < 0 || seq_q < 0 || seq_k < 0) return 0;
+    return dtype == FTH_DTYPE_F64 ? sdpa_backward_workspace<double>(num_bh, seq_q, seq_k) : sdpa_backward_workspace<float>(num_bh, seq_q, seq_k);
+}
+int32_t fth_dev_sdpa_backward_f32(const float *q, const float *k, const float *v, const float *dout, int64_t num_bh, int64_t seq_q,
+                                  int64_t seq_k, int64_t d_k, int64_t d_v, float scale, int32_t causal, float *dq, float *dk,
+                                  float *dv, void *workspace, size_t workspace_bytes, fth_stream s) {
+    return sdpa_backward_entry<float>(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dk, dv, workspace, workspace_bytes, s);
+}
+int32_t fth_dev_sdpa_backward_f64(const double *q, const double *k, const double *v, const double *dout, int64_t num_bh, int64_t seq_q,
+                                  int64_t seq_k, int64_t d_k, int64_t d_v, double scale, int32_t causal, double *dq, double *dk,
+                                  double *dv, void *workspace, size_t workspace_bytes, fth_stream s) {
+    return sdpa_backward_entry<double>(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dk, dv, workspace, workspace_bytes, s);
+}
+
+}  // extern "C"

@@ -205,6 +205,54 @@ def gemm(desc, a, b, c, bias=None, residual=None, alpha=1.0, stream=None):
                                                           _ptr(bias), _ptr(residual), stream))
 
 
+def _dtype_code(buf) -> int:
+    return 0 if buf.dtype == np.float64 else 1  # FTH_DTYPE_F64 / FTH_DTYPE_F32
+
+
+def _workspace(nbytes, workspace):
+    """The caller's workspace buffer, or a fresh one of the size the library asks for."""
+    if workspace is not None:
+        return workspace
+    return DeviceBuffer((max(int(nbytes), 16) + 3) // 4, np.float32)
+
+
+def norm_backward_workspace_bytes(rows, cols, dtype=np.float32) -> int:
+    return _lib.load().fth_dev_norm_backward_workspace_bytes(rows, cols, 0 if np.dtype(dtype) == np.float64 else 1)
+
+
+def layer_norm_backward(dy, x, weight, dx, dweight, dbias, rows, cols, eps, workspace=None, stream=None):
+    """layer_norm_backward_f32 / _f64: dx [rows, cols], dweight / dbias [cols]; mean / rstd recomputed from x."""
+    ws = _workspace(_lib.load().fth_dev_norm_backward_workspace_bytes(rows, cols, _dtype_code(x)), workspace)
+    check(getattr(_lib.load(), "fth_dev_layer_norm_backward_" + _sfx(x))(_ptr(dy), _ptr(x), _ptr(weight), rows, cols, _real(x, eps),
+                                                                         _ptr(dx), _ptr(dweight), _ptr(dbias), ws.ptr, ws.nbytes, stream))
+    return ws
+
+
+def rms_norm_backward(dy, x, weight, dx, dweight, rows, cols, eps, workspace=None, stream=None):
+    """rms_norm_backward_f32 / _f64: weight and dweight may both be None."""
+    ws = _workspace(_lib.load().fth_dev_norm_backward_workspace_bytes(rows, cols, _dtype_code(x)), workspace)
+    check(getattr(_lib.load(), "fth_dev_rms_norm_backward_" + _sfx(x))(_ptr(dy), _ptr(x), _ptr(weight), rows, cols, _real(x, eps),
+                                                                       _ptr(dx), _ptr(dweight), ws.ptr, ws.nbytes, stream))
+    return ws
+
+
+def linear_backward(dy, x, weight, dx, dweight, dbias, batch, in_features, out_features, workspace=None, stream=None):
+    """linear_backward: dx = dy . W, dweight = dy^T . x, dbias = column sums of dy (None: not wanted)."""
+    ws = _workspace(_lib.load().fth_dev_linear_backward_workspace_bytes(batch, out_features, _dtype_code(x)), workspace)
+    check(getattr(_lib.load(), "fth_dev_linear_backward_" + _sfx(x))(_ptr(dy), _ptr(x), _ptr(weight), batch, in_features, out_features,
+                                                                     _ptr(dx), _ptr(dweight), _ptr(dbias), ws.ptr, ws.nbytes, stream))
+    return ws
+
+
+def sdpa_backward(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dk, dv, workspace=None, stream=None):
+    """sdpa_backward_f32 / _f64 on contiguous [num_bh, seq, d] operands."""
+    ws = _workspace(_lib.load().fth_dev_sdpa_backward_workspace_bytes(num_bh, seq_q, seq_k, _dtype_code(q)), workspace)
+    check(getattr(_lib.load(), "fth_dev_sdpa_backward_" + _sfx(q))(_ptr(q), _ptr(k), _ptr(v), _ptr(dout), num_bh, seq_q, seq_k, d_k, d_v,
+                                                                   _real(q, scale), 1 if causal else 0, _ptr(dq), _ptr(dk), _ptr(dv),
+                                                                   ws.ptr, ws.nbytes, stream))
+    return ws
+
+
 def sdpa_desc_contiguous(num_bh, seq_q, seq_k, d_k, d_v, causal) -> _lib.SdpaDesc:
     d = _lib.SdpaDesc()
     _lib.load().fth_sdpa_desc_contiguous(C.byref(d), num_bh, seq_q, seq_k, d_k, d_v, 1 if causal else 0)

@@ -232,6 +232,47 @@ int32_t fth_dev_gemm_f32(const fth_gemm_desc *d, float alpha, const float *a, co
 int32_t fth_dev_gemm_f64(const fth_gemm_desc *d, double alpha, const double *a, const double *b, double *c,
                          const double *bias, const double *residual, fth_stream s);
 
+/* ---- backward kernels of the same ops (device pointers; caller-provided workspace) ----
+ * Each entry point needs scratch memory for its fixed-order partial sums (and, for SDPA, for the
+ * probability and score-gradient matrices the reference materialises per head): ask the matching
+ * *_workspace_bytes function and pass a device buffer of at least that size. dtype is FTH_DTYPE_*. */
+
+/* layer_norm_backward_f32 / _f64 (crates/ft-kernel-cpu/src/lib.rs:6189-6322, 6052-6183): dy, x, dx are
+ * [rows, cols]; weight, dweight, dbias are [cols]; mean / rstd are recomputed from x. */
+size_t fth_dev_norm_backward_workspace_bytes(int64_t rows, int64_t cols, int32_t dtype);
+int32_t fth_dev_layer_norm_backward_f32(const float *dy, const float *x, const float *weight, int64_t rows, int64_t cols, float eps,
+                                        float *dx, float *dweight, float *dbias, void *workspace, size_t workspace_bytes,
+                                        fth_stream s);
+int32_t fth_dev_layer_norm_backward_f64(const double *dy, const double *x, const double *weight, int64_t rows, int64_t cols, double eps,
+                                        double *dx, double *dweight, double *dbias, void *workspace, size_t workspace_bytes,
+                                        fth_stream s);
+/* rms_norm_backward_f32 / _f64 (:6574-6646, 6503-6570): weight and dweight may both be NULL. */
+int32_t fth_dev_rms_norm_backward_f32(const float *dy, const float *x, const float *weight, int64_t rows, int64_t cols, float eps,
+                                      float *dx, float *dweight, void *workspace, size_t workspace_bytes, fth_stream s);
+int32_t fth_dev_rms_norm_backward_f64(const double *dy, const double *x, const double *weight, int64_t rows, int64_t cols, double eps,
+                                      double *dx, double *dweight, void *workspace, size_t workspace_bytes, fth_stream s);
+
+/* linear_backward_f64 (:17226-17302) and the same formulas in f32: dy [batch, out], x [batch, in],
+ * weight [out, in] -> dx = dy . weight [batch, in], dweight = dy^T . x [out, in],
+ * dbias = column sums of dy [out] (skipped when dbias is NULL, the reference's need_bias = false). */
+size_t fth_dev_linear_backward_workspace_bytes(int64_t batch, int64_t out_features, int32_t dtype);
+int32_t fth_dev_linear_backward_f32(const float *dy, const float *x, const float *weight, int64_t batch, int64_t in_features,
+                                    int64_t out_features, float *dx, float *dweight, float *dbias, void *workspace,
+                                    size_t workspace_bytes, fth_stream s);
+int32_t fth_dev_linear_backward_f64(const double *dy, const double *x, const double *weight, int64_t batch, int64_t in_features,
+                                    int64_t out_features, double *dx, double *dweight, double *dbias, void *workspace,
+                                    size_t workspace_bytes, fth_stream s);
+
+/* sdpa_backward_f32 / _f64 (:5539-5650, 5300-5414): contiguous q [num_bh, seq_q, d_k], k [num_bh, seq_k, d_k],
+ * v [num_bh, seq_k, d_v], dout [num_bh, seq_q, d_v] -> dq, dk, dv of the shapes of q, k, v. */
+size_t fth_dev_sdpa_backward_workspace_bytes(int64_t num_bh, int64_t seq_q, int64_t seq_k, int32_t dtype);
+int32_t fth_dev_sdpa_backward_f32(const float *q, const float *k, const float *v, const float *dout, int64_t num_bh, int64_t seq_q,
+                                  int64_t seq_k, int64_t d_k, int64_t d_v, float scale, int32_t causal, float *dq, float *dk,
+                                  float *dv, void *workspace, size_t workspace_bytes, fth_stream s);
+int32_t fth_dev_sdpa_backward_f64(const double *q, const double *k, const double *v, const double *dout, int64_t num_bh, int64_t seq_q,
+                                  int64_t seq_k, int64_t d_k, int64_t d_v, double scale, int32_t causal, double *dq, double *dk,
+                                  double *dv, void *workspace, size_t workspace_bytes, fth_stream s);
+
 /* Fused scaled-dot-product attention forward, q [num_bh, seq_q, d_k], k [num_bh, seq_k, d_k],
  * v [num_bh, seq_k, d_v] -> out [num_bh, seq_q, d_v]; causal limit = min(qi + 1, seq_k)
  * (sdpa_forward_f32, crates/ft-kernel-cpu/src/lib.rs:5200-5284; _f64 :4572-4651).

@@ -12,7 +12,10 @@
 //   pinned by the reference's own fixtures / closed forms (tests/test_oracle_golden.py):
 //     softmax, gelu, add, matmul (small exact + stored f64 checksums), bmm, addmm, linear,
 //     index_select, argmax, layer_norm / rms_norm (closed form + textbook), sdpa (textbook
-//     attention + brute force), permute.
+//     attention + brute force), permute;
+//     layer_norm / rms_norm / linear / sdpa backward: central differences of the pinned forward
+//     functions in f64, the reference's own test inputs (KC:43862-43911, 64200-64360) and the
+//     identities those tests assert (unit-dy shortcut, dbias = column sums).
 //   third-party arithmetic that is NOT in the reference tree:
 //     * GEMM: `matrixmultiply 0.3.11` (Cargo.lock:1420-1423; call sites KC:1645, KC:1673). Its
 //       f32 accumulation order is unspecified and the reference's own test shows it is not the
@@ -470,7 +473,199 @@ __attribute__((target("avx2,fma"))) void sgemm_blocked_avx2(int64_t m, int64_t n
 
 }  // namespace
 
+// ------------------------------------------------------------------------------------------
+// Backward kernels of the same ops (the rows the forward path widens into next).
+
+// layer_norm_backward_f32 / _f64 (KC:6189-6322, 6052-6183): recomputes mean / rstd per row with the
+// forward's sequential sums, c1 = sum_j dxhat, c2 = sum_j dxhat * xhat,
+// dx = rstd * (dxhat - (c1 + xhat * c2) * inv_n); dweight / dbias are serial sums over the rows.
+// (The unit-dy shortcut KC:6198-6254 computes the same values with dy = 1 and is not restated.)
+template <typename T>
+void layer_norm_backward_impl(const T *dy, const T *x, const T *w, int64_t batch, int64_t n, T eps, T *dx, T *dw, T *db) {
+    const T inv_n = T(1) / (T)n;
+    std::vector<T> means((size_t)std::max<int64_t>(batch, 1)), rstds((size_t)std::max<int64_t>(batch, 1));
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < batch; ++r) {
+        const T *xr = x + r * n, *dyr = dy + r * n;
+        T sum = 0;
+        for (int64_t j = 0; j < n; ++j) sum += xr[j];
+        const T mean = sum * inv_n;
+        T vsum = 0;
+        for (int64_t j = 0; j < n; ++j) {
+            const T d = xr[j] - mean;
+            vsum += d * d;
+        }
+        const T rstd = T(1) / std::sqrt(vsum * inv_n + eps);
+        means[(size_t)r] = mean;
+        rstds[(size_t)r] = rstd;
+        T c1 = 0, c2 = 0;
+        for (int64_t j = 0; j < n; ++j) {
+            const T xhat = (xr[j] - mean) * rstd;
+            const T dxhat = dyr[j] * w[j];
+            c1 += dxhat;
+            c2 += dxhat * xhat;
+        }
+        for (int64_t j = 0; j < n; ++j) {
+            const T xhat = (xr[j] - mean) * rstd;
+            const T dxhat = dyr[j] * w[j];
+            dx[r * n + j] = rstd * (dxhat - (c1 + xhat * c2) * inv_n);
+        }
+    }
+    for (int64_t j = 0; j < n; ++j) dw[j] = db[j] = 0;
+    for (int64_t r = 0; r < batch; ++r) {
+        const T *xr = x + r * n, *dyr = dy + r * n;
+        const T mean = means[(size_t)r], rstd = rstds[(size_t)r];
+        for (int64_t j = 0; j < n; ++j) {
+            const T xhat = (xr[j] - mean) * rstd;
+            dw[j] += dyr[j] * xhat;
+            db[j] += dyr[j];
+        }
+    }
+}
+
+// rms_norm_backward_f32 / _f64 (KC:6574-6646, 6503-6570): g = dy * w (w optional),
+// rstd = 1 / sqrt(mean(x^2) + eps), c = sum_j g * x, dx = rstd * g - (rstd^3 * c / n) * x,
+// dweight[j] = sum_rows dy * x * rstd (serial over the rows), only when a weight is given.
+template <typename T>
+void rms_norm_backward_impl(const T *dy, const T *x, const T *w, int64_t batch, int64_t n, T eps, T *dx, T *dw) {
+    const T inv_n = T(1) / (T)n;
+    std::vector<T> rstds((size_t)std::max<int64_t>(batch, 1));
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < batch; ++r) {
+        const T *xr = x + r * n, *dyr = dy + r * n;
+        T ss = 0;
+        for (int64_t j = 0; j < n; ++j) ss += xr[j] * xr[j];
+        const T rstd = T(1) / std::sqrt(ss * inv_n + eps);
+        rstds[(size_t)r] = rstd;
+        T c = 0;
+        for (int64_t j = 0; j < n; ++j) {
+            const T g = dyr[j] * (w ? w[j] : T(1));
+            c += g * xr[j];
+        }
+        const T coef = rstd * rstd * rstd * c * inv_n;
+        for (int64_t j = 0; j < n; ++j) {
+            const T g = dyr[j] * (w ? w[j] : T(1));
+            dx[r * n + j] = rstd * g - coef * xr[j];
+        }
+    }
+    if (w && dw) {
+        for (int64_t j = 0; j < n; ++j) dw[j] = 0;
+        for (int64_t r = 0; r < batch; ++r) {
+            const T *xr = x + r * n, *dyr = dy + r * n;
+            const T rstd = rstds[(size_t)r];
+            for (int64_t j = 0; j < n; ++j) dw[j] += dyr[j] * xr[j] * rstd;
+        }
+    }
+}
+
+// Wide-accumulation product with A stored [k, m] (gemm::sgemm_tb / dgemm_tb, KC:1484-1524, 262-345).
+template <typename T> void gemm_tb_any(int64_t m, int64_t n, int64_t k, T alpha, const T *a_km, const T *b_kn, T *c) {
+    if (m <= 0 || n <= 0) return;
+    std::vector<T> at((size_t)m * (size_t)std::max<int64_t>(k, 1));
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < m; ++i)
+        for (int64_t p = 0; p < k; ++p) at[(size_t)i * k + p] = a_km[p * m + i];
+    gemm_any(0, m, n, k, at.data(), k, b_kn, n, c, n);
+    if (alpha != T(1))
+        for (int64_t i = 0; i < m * n; ++i) c[i] = alpha * c[i];
+}
+
+// linear_backward_f64 (KC:17226-17302) and its f32 twin by the same formulas:
+// dx = dy . W ([batch,out] . [out,in]), dweight = dy^T . x, dbias = serial sum of dy over the rows.
+template <typename T>
+void linear_backward_impl(const T *dy, const T *x, const T *w, int64_t batch, int64_t in_f, int64_t out_f, T *dx, T *dw, T *db) {
+    if (batch > 0 && in_f > 0) gemm_any(0, batch, in_f, out_f, dy, out_f, w, in_f, dx, in_f);
+    if (out_f > 0 && in_f > 0) gemm_tb_any<T>(out_f, in_f, batch, T(1), dy, x, dw);
+    if (db) {
+        for (int64_t o = 0; o < out_f; ++o) db[o] = 0;
+        for (int64_t b = 0; b < batch; ++b)
+            for (int64_t o = 0; o < out_f; ++o) db[o] += dy[b * out_f + o];
+    }
+}
+
+// sdpa_backward_f32 / _f64 (KC:5539-5650, 5300-5414): per (batch*head) P = softmax(scale * Q.K^T)
+// with the forward's row loop (strict max scan over the first `limit` entries, exp, sequential
+// sum, divide, zero tail), dU = dOut.V^T, dot_i = sum_j P_ij dU_ij, dU_ij = P_ij (dU_ij - dot_i),
+// dV = P^T.dOut, dQ = scale * dU.K, dK = scale * dU^T.Q. The products are the wide-accumulation
+// truth; the alpha of the scaled products is applied to the rounded product.
+template <typename T>
+void sdpa_backward_impl(const T *q, const T *k, const T *v, const T *dout, int64_t num_bh, int64_t seq_q, int64_t seq_k,
+                        int64_t d_k, int64_t d_v, T scale, int causal, T *dq, T *dk, T *dv) {
+    std::vector<T> p((size_t)std::max<int64_t>(seq_q * seq_k, 1)), du((size_t)std::max<int64_t>(seq_q * seq_k, 1));
+    for (int64_t bh = 0; bh < num_bh; ++bh) {
+        const T *qh = q + bh * seq_q * d_k, *kh = k + bh * seq_k * d_k, *vh = v + bh * seq_k * d_v;
+        const T *doh = dout + bh * seq_q * d_v;
+        T *dqh = dq + bh * seq_q * d_k, *dkh = dk + bh * seq_k * d_k, *dvh = dv + bh * seq_k * d_v;
+        if (seq_q > 0 && seq_k > 0) gemm_any(1, seq_q, seq_k, d_k, qh, d_k, kh, d_k, p.data(), seq_k);
+        for (int64_t i = 0; i < seq_q; ++i) {
+            const int64_t limit = causal ? std::min<int64_t>(i + 1, seq_k) : seq_k;
+            T *row = p.data() + i * seq_k;
+            T m = -std::numeric_limits<T>::infinity();
+            for (int64_t j = 0; j < limit; ++j) {
+                row[j] *= scale;
+                if (row[j] > m) m = row[j];
+            }
+            T sum = 0;
+            for (int64_t j = 0; j < limit; ++j) {
+                const T e = std::exp(row[j] - m);
+                row[j] = e;
+                sum += e;
+            }
+            for (int64_t j = 0; j < limit; ++j) row[j] /= sum;
+            for (int64_t j = limit; j < seq_k; ++j) row[j] = 0;
+        }
+        if (seq_q > 0 && seq_k > 0) gemm_any(1, seq_q, seq_k, d_v, doh, d_v, vh, d_v, du.data(), seq_k);
+        for (int64_t i = 0; i < seq_q; ++i) {
+            const T *pr = p.data() + i * seq_k;
+            T *dr = du.data() + i * seq_k;
+            T dot = 0;
+            for (int64_t j = 0; j < seq_k; ++j) dot += pr[j] * dr[j];
+            for (int64_t j = 0; j < seq_k; ++j) dr[j] = pr[j] * (dr[j] - dot);
+        }
+        gemm_tb_any<T>(seq_k, d_v, seq_q, T(1), p.data(), doh, dvh);
+        if (seq_q > 0 && d_k > 0) {
+            gemm_any(0, seq_q, d_k, seq_k, du.data(), seq_k, kh, d_k, dqh, d_k);
+            for (int64_t i = 0; i < seq_q * d_k; ++i) dqh[i] = scale * dqh[i];
+        }
+        gemm_tb_any<T>(seq_k, d_k, seq_q, scale, du.data(), qh, dkh);
+    }
+}
+
 extern "C" {
+
+void fto_layer_norm_backward_f32(const float *dy, const float *x, const float *w, int64_t batch, int64_t n, float eps,
+                                 float *dx, float *dw, float *db) {
+    layer_norm_backward_impl<float>(dy, x, w, batch, n, eps, dx, dw, db);
+}
+void fto_layer_norm_backward_f64(const double *dy, const double *x, const double *w, int64_t batch, int64_t n, double eps,
+                                 double *dx, double *dw, double *db) {
+    layer_norm_backward_impl<double>(dy, x, w, batch, n, eps, dx, dw, db);
+}
+void fto_rms_norm_backward_f32(const float *dy, const float *x, const float *w, int64_t batch, int64_t n, float eps,
+                               float *dx, float *dw) {
+    rms_norm_backward_impl<float>(dy, x, w, batch, n, eps, dx, dw);
+}
+void fto_rms_norm_backward_f64(const double *dy, const double *x, const double *w, int64_t batch, int64_t n, double eps,
+                               double *dx, double *dw) {
+    rms_norm_backward_impl<double>(dy, x, w, batch, n, eps, dx, dw);
+}
+void fto_linear_backward_f32(const float *dy, const float *x, const float *w, int64_t batch, int64_t in_f, int64_t out_f,
+                             float *dx, float *dw, float *db) {
+    linear_backward_impl<float>(dy, x, w, batch, in_f, out_f, dx, dw, db);
+}
+void fto_linear_backward_f64(const double *dy, const double *x, const double *w, int64_t batch, int64_t in_f, int64_t out_f,
+                             double *dx, double *dw, double *db) {
+    linear_backward_impl<double>(dy, x, w, batch, in_f, out_f, dx, dw, db);
+}
+void fto_sdpa_backward_f32(const float *q, const float *k, const float *v, const float *dout, int64_t num_bh, int64_t seq_q,
+                           int64_t seq_k, int64_t d_k, int64_t d_v, float scale, int causal, float *dq, float *dk, float *dv) {
+    sdpa_backward_impl<float>(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dk, dv);
+}
+void fto_sdpa_backward_f64(const double *q, const double *k, const double *v, const double *dout, int64_t num_bh,
+                           int64_t seq_q, int64_t seq_k, int64_t d_k, int64_t d_v, double scale, int causal, double *dq,
+                           double *dk, double *dv) {
+    sdpa_backward_impl<double>(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dk, dv);
+}
 
 void fto_softmax_f32(const float *x, float *y, int64_t outer, int64_t reduce, int64_t inner) {
     softmax_impl<float>(x, y, outer, reduce, inner);

@@ -204,6 +204,51 @@ def sdpa_forward(q, k, v, scale, causal):
     return out
 
 
+def layer_norm_backward(dy, x, weight, eps):
+    """Returns (dx, dweight, dbias) for y = layer_norm(x) * weight + bias over the last dim."""
+    dy, x, weight = _c(dy), _c(x), _c(weight)
+    sfx, ct = _sfx(x.dtype)
+    batch, n = x.reshape(-1, x.shape[-1]).shape
+    dx, dw, db = np.empty_like(x), np.empty(n, x.dtype), np.empty(n, x.dtype)
+    getattr(lib(), "fto_layer_norm_backward_" + sfx)(_p(dy), _p(x), _p(weight), _i64(batch), _i64(n), ct(eps), _p(dx), _p(dw), _p(db))
+    return dx, dw, db
+
+
+def rms_norm_backward(dy, x, weight, eps):
+    """Returns (dx, dweight or None)."""
+    dy, x, weight = _c(dy), _c(x), _c(weight)
+    sfx, ct = _sfx(x.dtype)
+    batch, n = x.reshape(-1, x.shape[-1]).shape
+    dx = np.empty_like(x)
+    dw = None if weight is None else np.empty(n, x.dtype)
+    getattr(lib(), "fto_rms_norm_backward_" + sfx)(_p(dy), _p(x), _p(weight), _i64(batch), _i64(n), ct(eps), _p(dx), _p(dw))
+    return dx, dw
+
+
+def linear_backward(dy, x, weight, need_bias=True):
+    """Returns (dx, dweight, dbias or None) for y = x . weight^T + bias."""
+    dy, x, weight = _c(dy), _c(x), _c(weight)
+    sfx, _ = _sfx(x.dtype)
+    batch, in_f = x.shape
+    out_f = weight.shape[0]
+    dx, dw = np.zeros((batch, in_f), x.dtype), np.zeros((out_f, in_f), x.dtype)
+    db = np.zeros(out_f, x.dtype) if need_bias else None
+    getattr(lib(), "fto_linear_backward_" + sfx)(_p(dy), _p(x), _p(weight), _i64(batch), _i64(in_f), _i64(out_f), _p(dx), _p(dw), _p(db))
+    return dx, dw, db
+
+
+def sdpa_backward(q, k, v, dout, scale, causal):
+    """Returns (dq, dk, dv) for out = sdpa_forward(q, k, v, scale, causal)."""
+    q, k, v, dout = _c(q), _c(k), _c(v), _c(dout)
+    sfx, ct = _sfx(q.dtype)
+    num_bh, seq_q, d_k = q.shape
+    seq_k, d_v = k.shape[1], v.shape[2]
+    dq, dk, dv = np.zeros_like(q), np.zeros_like(k), np.zeros_like(v)
+    getattr(lib(), "fto_sdpa_backward_" + sfx)(_p(q), _p(k), _p(v), _p(dout), _i64(num_bh), _i64(seq_q), _i64(seq_k), _i64(d_k),
+                                               _i64(d_v), ct(scale), C.c_int(1 if causal else 0), _p(dq), _p(dk), _p(dv))
+    return dq, dk, dv
+
+
 def index_select(x, dim, indices):
     """Returns (out, bad): bad is the position of the first invalid index, or -1."""
     x = _c(x)

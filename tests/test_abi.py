@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_struct_layouts_match_the_header():
     assert C.sizeof(_lib.Meta) == 16 + 8 * 8 * 2 + 8
-    assert C.sizeof(_lib.GemmDesc) == 10 * 8 + 8
+    assert C.sizeof(_lib.GemmDesc) == 10 * 8 + 16
     assert C.sizeof(_lib.SdpaDesc) == 18 * 8 + 8
     assert C.sizeof(_lib.LayerWeights) == 16 * 8
     assert C.sizeof(_lib.ErrorInfo) == 16 + 64 + 64 + 16 + 16 + 200

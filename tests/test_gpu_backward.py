@@ -1,0 +1,135 @@
+"""Backward kernels against the CPU checker: fp32 row work <= 1e-5, fp32 products <= 2e-5, fp64 <= 1e-12
+(max|d| / max|ref|), bitwise repeatable, and a size-independent property at the benchmark shape."""
+import math
+
+import numpy as np
+import pytest
+
+from conftest import TOL_F64, TOL_GEMM_F32, TOL_ROW_F32, rel_err
+from frankentorch_amd import synth
+from frankentorch_amd.device import DeviceBuffer
+
+pytestmark = pytest.mark.gpu
+
+
+def _up(*arrays):
+    return [None if a is None else DeviceBuffer.from_host(a) for a in arrays]
+
+
+# register-resident path (cols a vector multiple, up to 16 vectors per thread), ragged / long rows (streaming path)
+NORM_SHAPES = [(64, 256), (37, 768), (300, 4096), (5, 7), (3, 16), (9, 16384), (4, 20000), (130, 1026), (1, 4)]
+
+
+@pytest.mark.parametrize("rows,cols", NORM_SHAPES)
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_layer_norm_backward(hip, oracle, rows, cols, dtype):
+    tol = TOL_ROW_F32 if dtype == np.float32 else TOL_F64
+    x = synth.normal(11, "x", (rows, cols), dtype=dtype)
+    dy = synth.normal(11, "dy", (rows, cols), dtype=dtype)
+    w = synth.uniform(11, "w", (cols,), 0.5, 1.5, dtype=dtype)
+    dx_r, dw_r, db_r = oracle.layer_norm_backward(dy, x, w, dtype(1e-5))
+    ddy, dx_, dw_ = _up(dy, x, w)
+    ddx, ddw, ddb = DeviceBuffer((rows, cols), dtype), DeviceBuffer((cols,), dtype), DeviceBuffer((cols,), dtype)
+    hip.layer_norm_backward(ddy, dx_, dw_, ddx, ddw, ddb, rows, cols, 1e-5)
+    got = (ddx.to_host(), ddw.to_host(), ddb.to_host())
+    assert rel_err(got[0], dx_r) <= tol and rel_err(got[1], dw_r) <= tol * 4 and rel_err(got[2], db_r) <= tol * 4
+    hip.layer_norm_backward(ddy, dx_, dw_, ddx, ddw, ddb, rows, cols, 1e-5)
+    for a, b in zip(got, (ddx.to_host(), ddw.to_host(), ddb.to_host())):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
+@pytest.mark.parametrize("rows,cols", NORM_SHAPES)
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("with_weight", [True, False])
+def test_rms_norm_backward(hip, oracle, rows, cols, dtype, with_weight):
+    tol = TOL_ROW_F32 if dtype == np.float32 else TOL_F64
+    x = synth.normal(12, "x", (rows, cols), dtype=dtype)
+    dy = synth.normal(12, "dy", (rows, cols), dtype=dtype)
+    w = synth.uniform(12, "w", (cols,), 0.5, 1.5, dtype=dtype) if with_weight else None
+    dx_r, dw_r = oracle.rms_norm_backward(dy, x, w, dtype(1e-6))
+    ddy, dx_, dw_ = _up(dy, x, w)
+    ddx = DeviceBuffer((rows, cols), dtype)
+    ddw = DeviceBuffer((cols,), dtype) if with_weight else None
+    hip.rms_norm_backward(ddy, dx_, dw_, ddx, ddw, rows, cols, 1e-6)
+    assert rel_err(ddx.to_host(), dx_r) <= tol
+    if with_weight:
+        assert rel_err(ddw.to_host(), dw_r) <= tol * 4
+
+
+@pytest.mark.parametrize("batch,in_f,out_f", [(96, 40, 72), (128, 256, 1024), (200, 300, 100), (1024, 768, 2304), (1, 5, 3), (33, 64, 64)])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_linear_backward(hip, oracle, batch, in_f, out_f, dtype):
+    tol = TOL_GEMM_F32 if dtype == np.float32 else TOL_F64
+    dy = synth.normal(13, "dy", (batch, out_f), dtype=dtype)
+    x = synth.normal(13, "x", (batch, in_f), dtype=dtype)
+    w = synth.normal(13, "w", (out_f, in_f), dtype=dtype)
+    dx_r, dw_r, db_r = oracle.linear_backward(dy, x, w, True)
+    ddy, dx_, dw_ = _up(dy, x, w)
+    ddx, ddw, ddb = DeviceBuffer((batch, in_f), dtype), DeviceBuffer((out_f, in_f), dtype), DeviceBuffer((out_f,), dtype)
+    hip.linear_backward(ddy, dx_, dw_, ddx, ddw, ddb, batch, in_f, out_f)
+    assert rel_err(ddx.to_host(), dx_r) <= tol and rel_err(ddw.to_host(), dw_r) <= tol and rel_err(ddb.to_host(), db_r) <= tol
+    # need_bias = false
+    ddb2 = DeviceBuffer.from_host(np.full((out_f,), 7, dtype))
+    hip.linear_backward(ddy, dx_, dw_, ddx, ddw, None, batch, in_f, out_f)
+    assert np.all(ddb2.to_host() == 7)
+
+
+def test_linear_backward_reference_test_inputs(hip, oracle):
+    """The inputs of the reference's own dweight test (crates/ft-kernel-cpu/src/lib.rs:43862-43911), fp64."""
+    batch, in_f, out_f = 96, 40, 72
+    dy = ((np.arange(batch * out_f) % 101) * 0.01 - 0.5).reshape(batch, out_f)
+    x = ((np.arange(batch * in_f) % 89) * 0.02 - 0.7).reshape(batch, in_f)
+    w = ((np.arange(out_f * in_f) % 53) * 0.03 - 0.4).reshape(out_f, in_f)
+    ddy, dx_, dw_ = _up(dy, x, w)
+    ddx, ddw, ddb = DeviceBuffer((batch, in_f), np.float64), DeviceBuffer((out_f, in_f), np.float64), DeviceBuffer((out_f,), np.float64)
+    hip.linear_backward(ddy, dx_, dw_, ddx, ddw, ddb, batch, in_f, out_f)
+    assert np.allclose(ddw.to_host(), dy.T @ x, rtol=0, atol=1e-11)
+    assert np.allclose(ddb.to_host(), dy.sum(0), rtol=0, atol=1e-12)
+
+
+@pytest.mark.parametrize("bh,sq,sk,dk,dv", [(2, 64, 64, 64, 64), (3, 100, 70, 32, 48), (4, 128, 128, 128, 128), (1, 5, 6, 4, 3), (2, 33, 200, 16, 16)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_sdpa_backward(hip, oracle, bh, sq, sk, dk, dv, causal, dtype):
+    tol = TOL_GEMM_F32 if dtype == np.float32 else TOL_F64
+    s = 1.0 / math.sqrt(dk)
+    q = synth.normal(14, "q", (bh, sq, dk), dtype=dtype)
+    k = synth.normal(14, "k", (bh, sk, dk), dtype=dtype)
+    v = synth.normal(14, "v", (bh, sk, dv), dtype=dtype)
+    do = synth.normal(14, "do", (bh, sq, dv), dtype=dtype)
+    ref = oracle.sdpa_backward(q, k, v, do, dtype(s), causal)
+    dq_, dk_, dv_, ddo = _up(q, k, v, do)
+    gq, gk, gv = DeviceBuffer(q.shape, dtype), DeviceBuffer(k.shape, dtype), DeviceBuffer(v.shape, dtype)
+    hip.sdpa_backward(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, s, causal, gq, gk, gv)
+    got = (gq.to_host(), gk.to_host(), gv.to_host())
+    for g, r in zip(got, ref):
+        assert rel_err(g, r) <= tol * 2
+    hip.sdpa_backward(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, s, causal, gq, gk, gv)
+    for a, b in zip(got, (gq.to_host(), gk.to_host(), gv.to_host())):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
+def test_norm_backward_at_the_row_op_benchmark_shape(hip, oracle):
+    """fp32 [8192, 4096]: sampled rows against the checker, column sums against an f64 numpy sum, and the
+    property that dx rows of LayerNorm sum to zero."""
+    rows, cols = 8192, 4096
+    x = synth.normal(1, "x", (rows, cols))
+    dy = synth.normal(1, "dyb", (rows, cols))
+    w = synth.uniform(1, "gamma", (cols,), 0.5, 1.5)
+    ddy, dx_, dw_ = _up(dy, x, w)
+    ddx, ddw, ddb = DeviceBuffer((rows, cols)), DeviceBuffer((cols,)), DeviceBuffer((cols,))
+    hip.layer_norm_backward(ddy, dx_, dw_, ddx, ddw, ddb, rows, cols, 1e-5)
+    dx = ddx.to_host()
+    pick = np.arange(3, rows, 509)
+    dx_r, _, _ = oracle.layer_norm_backward(dy[pick], x[pick], w, np.float32(1e-5))
+    assert rel_err(dx[pick], dx_r) <= TOL_ROW_F32
+    assert np.max(np.abs(dx.astype(np.float64).sum(1))) <= 1e-3
+    x64, dy64 = x.astype(np.float64), dy.astype(np.float64)
+    xhat = (x64 - x64.mean(1, keepdims=True)) / np.sqrt(x64.var(1, keepdims=True) + 1e-5)
+    assert rel_err(ddw.to_host(), (dy64 * xhat).sum(0)) <= 4 * TOL_ROW_F32
+    assert rel_err(ddb.to_host(), dy64.sum(0)) <= 4 * TOL_ROW_F32
+    hip.rms_norm_backward(ddy, dx_, dw_, ddx, ddw, rows, cols, 1e-6)
+    dxr, _ = oracle.rms_norm_backward(dy[pick], x[pick], w, np.float32(1e-6))
+    assert rel_err(ddx.to_host()[pick], dxr) <= TOL_ROW_F32
+    rstd = 1.0 / np.sqrt((x64 * x64).mean(1, keepdims=True) + 1e-6)
+    assert rel_err(ddw.to_host(), (dy64 * x64 * rstd).sum(0)) <= 4 * TOL_ROW_F32

@@ -1,0 +1,107 @@
+"""Pins the CPU checker's backward functions without running the reference: central differences of
+the already pinned forward functions in f64 (a dropped term, a wrong sign or a transposed operand
+fails them), the identities the reference's own tests assert, and its test inputs
+(crates/ft-kernel-cpu/src/lib.rs:43862-43911, 64200-64360)."""
+import numpy as np
+import pytest
+
+
+def _num_grad(f, x, dy, h=1e-6):
+    """d/dx sum(dy * f(x)) by central differences, f64."""
+    g = np.zeros_like(x)
+    flat, gf = x.reshape(-1), g.reshape(-1)
+    for i in range(flat.size):
+        old = flat[i]
+        flat[i] = old + h
+        up = float(np.sum(dy * f(x)))
+        flat[i] = old - h
+        dn = float(np.sum(dy * f(x)))
+        flat[i] = old
+        gf[i] = (up - dn) / (2 * h)
+    return g
+
+
+def test_layer_norm_backward_is_the_gradient_of_the_forward(oracle):
+    rng = np.random.default_rng(5)
+    batch, n, eps = 4, 9, 1e-5
+    x, dy = rng.standard_normal((batch, n)), rng.standard_normal((batch, n))
+    w, b = rng.uniform(0.5, 1.5, n), rng.standard_normal(n)
+    dx, dw, db = oracle.layer_norm_backward(dy, x, w, eps)
+    assert np.allclose(dx, _num_grad(lambda t: oracle.layer_norm(t, w, b, eps), x.copy(), dy), atol=1e-7)
+    assert np.allclose(dw, _num_grad(lambda t: oracle.layer_norm(x, t, b, eps), w.copy(), dy), atol=1e-7)
+    assert np.allclose(db, _num_grad(lambda t: oracle.layer_norm(x, w, t, eps), b.copy(), dy), atol=1e-7)
+    assert np.array_equal(db, np.add.reduce(dy, axis=0))  # serial sum over the rows in row order
+    assert np.allclose(dx.sum(1), 0, atol=1e-12)  # a shift of the whole row leaves the output unchanged
+
+
+def test_layer_norm_backward_reference_test_inputs(oracle):
+    """Inputs of layer_norm_f32_unit_dy_matches_general_reference_bits (KC:64300-64360): with dy = 1 the
+    shortcut the reference takes must equal the general formula, i.e. dbias = batch and
+    dweight = sum of xhat over the rows."""
+    for batch, n in [(5, 7), (3, 16)]:
+        i = np.arange(batch * n)
+        x = (((i % 23).astype(np.float32) - 11.0) * np.float32(0.03125) + i.astype(np.float32) * np.float32(0.00091)).reshape(batch, n)
+        w = (0.75 + (np.arange(n) % 5) * 0.046875).astype(np.float32)
+        dy = np.ones_like(x)
+        dx, dw, db = oracle.layer_norm_backward(dy, x, w, np.float32(1e-5))
+        assert np.all(db == np.float32(batch))
+        x64 = x.astype(np.float64)
+        xhat = (x64 - x64.mean(1, keepdims=True)) / np.sqrt(x64.var(1, keepdims=True) + 1e-5)
+        assert np.allclose(dw, xhat.sum(0), atol=2e-5)
+        dx64, _, _ = oracle.layer_norm_backward(dy.astype(np.float64), x64, w.astype(np.float64), 1e-5)
+        assert np.allclose(dx, dx64, atol=2e-5)
+
+
+def test_rms_norm_backward_is_the_gradient_of_the_forward(oracle):
+    rng = np.random.default_rng(6)
+    batch, n, eps = 3, 8, 1e-6
+    x, dy, w = rng.standard_normal((batch, n)), rng.standard_normal((batch, n)), rng.uniform(0.5, 1.5, n)
+    dx, dw = oracle.rms_norm_backward(dy, x, w, eps)
+    assert np.allclose(dx, _num_grad(lambda t: oracle.rms_norm(t, w, eps), x.copy(), dy), atol=1e-7)
+    assert np.allclose(dw, _num_grad(lambda t: oracle.rms_norm(x, t, eps), w.copy(), dy), atol=1e-7)
+    dx1, dw1 = oracle.rms_norm_backward(dy, x, None, eps)
+    assert dw1 is None
+    assert np.allclose(dx1, _num_grad(lambda t: oracle.rms_norm(t, None, eps), x.copy(), dy), atol=1e-7)
+
+
+def test_linear_backward_reference_test_inputs_and_gradient(oracle):
+    """Inputs of linear_backward_dgemm_tb_dweight_matches_materialized_transpose_bit_exact (KC:43862-43911):
+    dweight must equal dy^T . x computed through an explicit transpose, dbias the column sums of dy."""
+    batch, in_f, out_f = 96, 40, 72
+    dy = ((np.arange(batch * out_f) % 101) * 0.01 - 0.5).reshape(batch, out_f)
+    x = ((np.arange(batch * in_f) % 89) * 0.02 - 0.7).reshape(batch, in_f)
+    w = ((np.arange(out_f * in_f) % 53) * 0.03 - 0.4).reshape(out_f, in_f)
+    dx, dw, db = oracle.linear_backward(dy, x, w, True)
+    assert np.allclose(dw, oracle.gemm(np.ascontiguousarray(dy.T), x), rtol=0, atol=1e-12)
+    assert np.allclose(dw, dy.T @ x, atol=1e-11) and np.allclose(dx, dy @ w, atol=1e-11)
+    ref_db = np.zeros(out_f)
+    for b in range(batch):
+        ref_db += dy[b]
+    assert np.array_equal(db, ref_db)
+    # gradient of the forward on a small case
+    rng = np.random.default_rng(7)
+    xs, ws, bs, dys = rng.standard_normal((3, 4)), rng.standard_normal((5, 4)), rng.standard_normal(5), rng.standard_normal((3, 5))
+    dxs, dws, dbs = oracle.linear_backward(dys, xs, ws, True)
+    assert np.allclose(dxs, _num_grad(lambda t: oracle.linear(t, ws, bs), xs.copy(), dys), atol=1e-8)
+    assert np.allclose(dws, _num_grad(lambda t: oracle.linear(xs, t, bs), ws.copy(), dys), atol=1e-8)
+    assert np.allclose(dbs, _num_grad(lambda t: oracle.linear(xs, ws, t), bs.copy(), dys), atol=1e-8)
+    assert oracle.linear_backward(dys, xs, ws, False)[2] is None
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_sdpa_backward_is_the_gradient_of_the_forward(oracle, causal):
+    rng = np.random.default_rng(8)
+    bh, sq, sk, dk, dv = 2, 5, 6, 4, 3
+    q, k, v = rng.standard_normal((bh, sq, dk)), rng.standard_normal((bh, sk, dk)), rng.standard_normal((bh, sk, dv))
+    dout = rng.standard_normal((bh, sq, dv))
+    scale = 0.37
+    dq, dk_, dv_ = oracle.sdpa_backward(q, k, v, dout, scale, causal)
+    assert np.allclose(dq, _num_grad(lambda t: oracle.sdpa_forward(t, k, v, scale, causal), q.copy(), dout), atol=1e-7)
+    assert np.allclose(dk_, _num_grad(lambda t: oracle.sdpa_forward(q, t, v, scale, causal), k.copy(), dout), atol=1e-7)
+    assert np.allclose(dv_, _num_grad(lambda t: oracle.sdpa_forward(q, k, t, scale, causal), v.copy(), dout), atol=1e-7)
+    if causal:  # a key no query can see gets no gradient
+        assert np.all(dk_[:, sq:, :] == 0) and np.all(dv_[:, sq:, :] == 0)
+    # f32 twin agrees with f64 to f32 rounding
+    f = np.float32
+    dq32, dk32, dv32 = oracle.sdpa_backward(q.astype(f), k.astype(f), v.astype(f), dout.astype(f), f(scale), causal)
+    assert np.allclose(dq32, dq, atol=2e-5) and np.allclose(dk32, dk_, atol=2e-5) and np.allclose(dv32, dv_, atol=2e-5)
