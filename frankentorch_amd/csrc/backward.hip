@@ -111,23 +111,41 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
     }
     const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
     const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
-    for (int64_t r = r0; r < r1; ++r) {
+    // Rows are loaded one ahead (a second register set) when the row is short enough to afford it.
+    constexpr bool PREFETCH = VPT * N <= 16;
+    V xn[PREFETCH ? VPT : 1], gn[PREFETCH ? VPT : 1];
+    auto load_row = [&](int64_t r, V *xd, V *gd) __attribute__((always_inline)) {
         const V *xr = reinterpret_cast<const V *>(x + r * cols);
         const V *dyr = reinterpret_cast<const V *>(dy + r * cols);
-        V xv[VPT], gv[VPT];
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
             const int v = tid + i * kThreads;
             if (v < nvec) {
-                xv[i] = xr[v];
-                gv[i] = dyr[v];
+                xd[i] = xr[v];
+                gd[i] = dyr[v];
             } else {
 #pragma unroll
                 for (int e = 0; e < N; ++e) {
-                    vset(xv[i], e, T(0));
-                    vset(gv[i], e, T(0));
+                    vset(xd[i], e, T(0));
+                    vset(gd[i], e, T(0));
                 }
             }
+        }
+    };
+    if constexpr (PREFETCH) {
+        if (r0 < r1) load_row(r0, xn, gn);
+    }
+    for (int64_t r = r0; r < r1; ++r) {
+        V xv[VPT], gv[VPT];
+        if constexpr (PREFETCH) {
+#pragma unroll
+            for (int i = 0; i < VPT; ++i) {
+                xv[i] = xn[i];
+                gv[i] = gn[i];
+            }
+            if (r + 1 < r1) load_row(r + 1, xn, gn);
+        } else {
+            load_row(r, xv, gv);
         }
         if constexpr (!RMS) {
             T s[1] = {T(0)};
@@ -301,14 +319,35 @@ __global__ __launch_bounds__(kThreads) void col_partial_kernel(const T *__restri
     part[(int64_t)blockIdx.y * cols + col] = acc;
 }
 
-// out[col] = part[0][col] + part[1][col] + ... in that order.
+// out[col] = sum over the parts. A workgroup owns 32 columns; its 8 part-lanes each add every 8th
+// part in ascending order (loads eight deep, independent of the adds), then the 8 lane sums are
+// added lane 0..7. The order is a function of (nparts) only.
 template <typename T>
 __global__ __launch_bounds__(kThreads) void col_final_kernel(const T *__restrict__ part, int nparts, int64_t cols, T *__restrict__ out) {
-    const int64_t col = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-    if (col >= cols) return;
+    constexpr int CW = 32, PL = kThreads / CW;
+    __shared__ T red[PL][CW];
+    const int c = threadIdx.x % CW, pl = threadIdx.x / CW;
+    const int64_t col = (int64_t)blockIdx.x * CW + c;
     T acc = T(0);
-    for (int b = 0; b < nparts; ++b) acc += part[(int64_t)b * cols + col];
-    out[col] = acc;
+    if (col < cols) {
+        int b = pl;
+        for (; b + 7 * PL < nparts; b += 8 * PL) {
+            T v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = part[(int64_t)(b + u * PL) * cols + col];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc += v[u];
+        }
+        for (; b < nparts; b += PL) acc += part[(int64_t)b * cols + col];
+    }
+    red[pl][c] = acc;
+    __syncthreads();
+    if (pl == 0 && col < cols) {
+        T s = red[0][c];
+#pragma unroll
+        for (int l = 1; l < PL; ++l) s += red[l][c];
+        out[col] = s;
+    }
 }
 
 // Zero fill as a kernel (memset nodes are avoided so that callers can capture these entry points).
@@ -327,7 +366,7 @@ template <typename T> int32_t zero_fill(T *dst, int64_t n, hipStream_t st) {
 inline int pick_rows_per_block(int64_t rows) {
     // enough workgroups to fill the chip several times over, at most 64 rows each
     const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
-    int64_t r = rows / ((int64_t)cus * 4);
+    int64_t r = rows / ((int64_t)cus * 2);
     if (r < 1) r = 1;
     if (r > 64) r = 64;
     return (int)r;
@@ -401,11 +440,11 @@ int32_t norm_backward_entry(const T *dy, const T *x, const T *w, int64_t rows, i
         }
     }
     if (want_w) {
-        col_final_kernel<T><<<dim3((unsigned)col_blocks), dim3(kThreads), 0, st>>>(part_w, (int)blocks, cols, dw);
+        col_final_kernel<T><<<dim3((unsigned)fth::ceil_div(cols, 32)), dim3(kThreads), 0, st>>>(part_w, (int)blocks, cols, dw);
         FTH_CHECK_LAUNCH("norm_backward_dweight_sum");
     }
     if (db) {
-        col_final_kernel<T><<<dim3((unsigned)col_blocks), dim3(kThreads), 0, st>>>(part_b, (int)blocks, cols, db);
+        col_final_kernel<T><<<dim3((unsigned)fth::ceil_div(cols, 32)), dim3(kThreads), 0, st>>>(part_b, (int)blocks, cols, db);
         FTH_CHECK_LAUNCH("norm_backward_dbias_sum");
     }
     return FTH_OK;
@@ -469,7 +508,7 @@ int32_t linear_backward_entry(const T *dy, const T *x, const T *w, int64_t batch
         col_partial_kernel<T, 0><<<dim3((unsigned)col_blocks, (unsigned)blocks), dim3(kThreads), 0, st>>>(dy, nullptr, nullptr, batch,
                                                                                                          out_f, out_f, rpb, part);
         FTH_CHECK_LAUNCH("linear_backward_dbias");
-        col_final_kernel<T><<<dim3((unsigned)col_blocks), dim3(kThreads), 0, st>>>(part, (int)blocks, out_f, db);
+        col_final_kernel<T><<<dim3((unsigned)fth::ceil_div(out_f, 32)), dim3(kThreads), 0, st>>>(part, (int)blocks, out_f, db);
         FTH_CHECK_LAUNCH("linear_backward_dbias_sum");
     }
     return FTH_OK;

@@ -1051,6 +1051,12 @@ int32_t launch_direct(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     return launch_direct_epi<T, BM, BN, WM, WN, MINW, false, TRANS_B, -1>(p, batch, st);
 }
 
+// 128x128 tiles when there is one per CU, or when K is long enough that the stream-K split still
+// leaves every resident workgroup a run of at least 16 K-tiles (few tiles, deep K: weight gradients).
+inline bool use_big_tiles(int64_t big_tiles, int64_t k, int cus) {
+    return big_tiles >= cus || big_tiles * fth::ceil_div(k, 32) >= (int64_t)cus * 2 * 16;
+}
+
 // Tile configurations. The choice depends on the shape only (never on timing), so a given problem
 // always runs the same kernel and reproduces its bits.
 enum class Tile { Big, Wide, Small, Tall };
@@ -1069,7 +1075,7 @@ int32_t launch_shape(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     // CU a large tile: 64x64 tiles (2x2 wavefronts of 32x32).
     const int64_t big_tiles = fth::ceil_div(p.m, 128) * fth::ceil_div(p.n, 128) * batch;
     const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
-    Tile t = big_tiles >= cus ? Tile::Big : Tile::Small;
+    Tile t = use_big_tiles(big_tiles, p.k, cus) ? Tile::Big : Tile::Small;
     const int f = forced_tile();
     if (f == 0) t = Tile::Big;
     if (f == 1) t = Tile::Wide;
@@ -1202,7 +1208,7 @@ template <typename T> int32_t launch_trans_a(GemmArgs<T> &p, const fth_gemm_desc
     if (direct) {
         const int64_t big_tiles = fth::ceil_div(p.m, 128) * fth::ceil_div(p.n, 128) * d->batch;
         const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
-        if (big_tiles >= cus) return launch_direct_epi<T, 128, 128, 2, 2, 2, true, false, -1>(p, d->batch, st);
+        if (use_big_tiles(big_tiles, p.k, cus)) return launch_direct_epi<T, 128, 128, 2, 2, 2, true, false, -1>(p, d->batch, st);
         return launch_direct_epi<T, 64, 64, 2, 2, 2, true, false, -1>(p, d->batch, st);
     }
     // Transposed copy A^T [batch][m][k], then the ordinary [m, k] path.
