@@ -633,6 +633,138 @@ int32_t argmax_impl(const T *input, size_t input_len, const fth_meta *meta, size
     return fetch(out, dy, (size_t)out_numel);
 }
 
+// ---- backward entry points on host slices ----
+// Several outputs per call, each with its own capacity; every output the call produces must fit.
+template <typename T> int32_t fetch_no_sync(T *host, const T *dev, size_t n) {
+    if (n) FTH_HIP(hipMemcpyAsync(host, dev, n * sizeof(T), hipMemcpyDeviceToHost, fth::resolve_stream(nullptr)));
+    return FTH_OK;
+}
+
+// layer_norm_backward (crates/ft-kernel-cpu/src/lib.rs:6189-6322 / 6052-6183), rms_norm_backward (:6574-6646 / 6503-6570)
+template <typename T, bool RMS>
+int32_t norm_backward_impl(const T *dy, size_t dy_len, const T *x, size_t x_len, const T *w, size_t batch, size_t n, T eps, T *dx,
+                           size_t dx_cap, T *dw, size_t dw_cap, T *db, size_t db_cap) {
+    uint64_t total;
+    FTH_ARG(checked_mul(batch, n, &total), "norm backward: batch * norm_size overflows");
+    FTH_ARG(RMS || w != nullptr, "layer_norm backward: weight is required");
+    const bool want_w = w != nullptr;
+    if (int32_t rc = check_out(dx, dx_cap, (size_t)total)) return rc;
+    if (want_w)
+        if (int32_t rc = check_out(dw, dw_cap, n)) return rc;
+    if (!RMS)
+        if (int32_t rc = check_out(db, db_cap, n)) return rc;
+    FTH_ARG(dy_len >= total && x_len >= total, "norm backward: input slice shorter than batch * norm_size");
+    if (n == 0) return FTH_OK;
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *ddy = nullptr, *dxin = nullptr, *dwt = nullptr, *ddx = nullptr, *ddw = nullptr, *ddb = nullptr;
+    void *ws = nullptr;
+    if (int32_t rc = stage_in(sc, dy, (size_t)total, &ddy)) return rc;
+    if (int32_t rc = stage_in(sc, x, (size_t)total, &dxin)) return rc;
+    if (w)
+        if (int32_t rc = stage_in(sc, w, n, &dwt)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)total, &ddx)) return rc;
+    if (want_w)
+        if (int32_t rc = stage_out(sc, n, &ddw)) return rc;
+    if (!RMS)
+        if (int32_t rc = stage_out(sc, n, &ddb)) return rc;
+    const size_t wsb = fth_dev_norm_backward_workspace_bytes((int64_t)batch, (int64_t)n, Dev<T>::dtype);
+    if (int32_t rc = sc.get(&ws, wsb)) return rc;
+    int32_t rc;
+    if constexpr (std::is_same<T, float>::value) {
+        rc = RMS ? fth_dev_rms_norm_backward_f32(ddy, dxin, dwt, (int64_t)batch, (int64_t)n, eps, ddx, ddw, ws, wsb, nullptr)
+                 : fth_dev_layer_norm_backward_f32(ddy, dxin, dwt, (int64_t)batch, (int64_t)n, eps, ddx, ddw, ddb, ws, wsb, nullptr);
+    } else {
+        rc = RMS ? fth_dev_rms_norm_backward_f64(ddy, dxin, dwt, (int64_t)batch, (int64_t)n, eps, ddx, ddw, ws, wsb, nullptr)
+                 : fth_dev_layer_norm_backward_f64(ddy, dxin, dwt, (int64_t)batch, (int64_t)n, eps, ddx, ddw, ddb, ws, wsb, nullptr);
+    }
+    if (rc) return rc;
+    if (want_w)
+        if (int32_t r2 = fetch_no_sync(dw, ddw, n)) return r2;
+    if (!RMS)
+        if (int32_t r2 = fetch_no_sync(db, ddb, n)) return r2;
+    return fetch(dx, ddx, (size_t)total);
+}
+
+// linear_backward (crates/ft-kernel-cpu/src/lib.rs:17226-17302)
+template <typename T>
+int32_t linear_backward_impl(const T *dy, size_t dy_len, const T *x, size_t x_len, const T *w, size_t w_len, size_t batch, size_t in_f,
+                             size_t out_f, int32_t need_bias, T *dx, size_t dx_cap, T *dw, size_t dw_cap, T *db, size_t db_cap) {
+    uint64_t n_dy, n_x, n_w;
+    FTH_ARG(checked_mul(batch, out_f, &n_dy) && checked_mul(batch, in_f, &n_x) && checked_mul(out_f, in_f, &n_w),
+            "linear backward: extents overflow");
+    if (int32_t rc = check_out(dx, dx_cap, (size_t)n_x)) return rc;
+    if (int32_t rc = check_out(dw, dw_cap, (size_t)n_w)) return rc;
+    if (need_bias)
+        if (int32_t rc = check_out(db, db_cap, out_f)) return rc;
+    FTH_ARG(dy_len >= n_dy && x_len >= n_x && w_len >= n_w, "linear backward: input slice shorter than its shape");
+    if (n_x == 0 && n_w == 0 && (!need_bias || out_f == 0)) return FTH_OK;
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *ddy = nullptr, *dxin = nullptr, *dwt = nullptr, *ddx = nullptr, *ddw = nullptr, *ddb = nullptr;
+    void *ws = nullptr;
+    if (int32_t rc = stage_in(sc, dy, (size_t)n_dy, &ddy)) return rc;
+    if (int32_t rc = stage_in(sc, x, (size_t)n_x, &dxin)) return rc;
+    if (int32_t rc = stage_in(sc, w, (size_t)n_w, &dwt)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)n_x, &ddx)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)n_w, &ddw)) return rc;
+    if (need_bias)
+        if (int32_t rc = stage_out(sc, out_f, &ddb)) return rc;
+    const size_t wsb = fth_dev_linear_backward_workspace_bytes((int64_t)batch, (int64_t)out_f, Dev<T>::dtype);
+    if (int32_t rc = sc.get(&ws, wsb)) return rc;
+    // dweight of an empty batch is all zeros (the product over k = 0), which the k == 0 GEMM path writes.
+    int32_t rc;
+    if constexpr (std::is_same<T, float>::value)
+        rc = fth_dev_linear_backward_f32(ddy, dxin, dwt, (int64_t)batch, (int64_t)in_f, (int64_t)out_f, ddx, ddw, ddb, ws, wsb, nullptr);
+    else
+        rc = fth_dev_linear_backward_f64(ddy, dxin, dwt, (int64_t)batch, (int64_t)in_f, (int64_t)out_f, ddx, ddw, ddb, ws, wsb, nullptr);
+    if (rc) return rc;
+    if (int32_t r2 = fetch_no_sync(dw, ddw, (size_t)n_w)) return r2;
+    if (need_bias)
+        if (int32_t r2 = fetch_no_sync(db, ddb, out_f)) return r2;
+    return fetch(dx, ddx, (size_t)n_x);
+}
+
+// sdpa_backward (crates/ft-kernel-cpu/src/lib.rs:5539-5650 / 5300-5414)
+template <typename T>
+int32_t sdpa_backward_impl(const T *q, size_t q_len, const T *k, size_t k_len, const T *v, size_t v_len, const T *dout, size_t do_len,
+                           size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, T scale, int32_t causal, T *dq,
+                           size_t dq_cap, T *dk, size_t dk_cap, T *dv, size_t dv_cap) {
+    uint64_t nq, nk, nv, no, t;
+    FTH_ARG(checked_mul(num_bh, seq_q, &t) && checked_mul(t, d_k, &nq) && checked_mul(t, d_v, &no) && checked_mul(num_bh, seq_k, &t) &&
+                checked_mul(t, d_k, &nk) && checked_mul(t, d_v, &nv),
+            "sdpa backward: extents overflow");
+    if (int32_t rc = check_out(dq, dq_cap, (size_t)nq)) return rc;
+    if (int32_t rc = check_out(dk, dk_cap, (size_t)nk)) return rc;
+    if (int32_t rc = check_out(dv, dv_cap, (size_t)nv)) return rc;
+    FTH_ARG(q_len >= nq && k_len >= nk && v_len >= nv && do_len >= no, "sdpa backward: input slice shorter than its shape");
+    if (nq == 0 && nk == 0 && nv == 0) return FTH_OK;
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *dqi = nullptr, *dki = nullptr, *dvi = nullptr, *ddo = nullptr, *gq = nullptr, *gk = nullptr, *gv = nullptr;
+    void *ws = nullptr;
+    if (int32_t rc = stage_in(sc, q, (size_t)nq, &dqi)) return rc;
+    if (int32_t rc = stage_in(sc, k, (size_t)nk, &dki)) return rc;
+    if (int32_t rc = stage_in(sc, v, (size_t)nv, &dvi)) return rc;
+    if (int32_t rc = stage_in(sc, dout, (size_t)no, &ddo)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)nq, &gq)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)nk, &gk)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)nv, &gv)) return rc;
+    const size_t wsb = fth_dev_sdpa_backward_workspace_bytes((int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, Dev<T>::dtype);
+    if (int32_t rc = sc.get(&ws, wsb)) return rc;
+    int32_t rc;
+    if constexpr (std::is_same<T, float>::value)
+        rc = fth_dev_sdpa_backward_f32(dqi, dki, dvi, ddo, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k, (int64_t)d_v, scale,
+                                       causal, gq, gk, gv, ws, wsb, nullptr);
+    else
+        rc = fth_dev_sdpa_backward_f64(dqi, dki, dvi, ddo, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k, (int64_t)d_v, scale,
+                                       causal, gq, gk, gv, ws, wsb, nullptr);
+    if (rc) return rc;
+    if (int32_t r2 = fetch_no_sync(dk, gk, (size_t)nk)) return r2;
+    if (int32_t r2 = fetch_no_sync(dv, gv, (size_t)nv)) return r2;
+    return fetch(dq, gq, (size_t)nq);
+}
+
 }  // namespace
 
 extern "C" {
@@ -749,6 +881,49 @@ int32_t fth_argmax_dim_tensor_contiguous_f32(const float *input, size_t input_le
 int32_t fth_argmax_dim_tensor_contiguous_f64(const double *input, size_t input_len, const fth_meta *meta, size_t dim,
                                              double *out, size_t out_cap, size_t *out_len) {
     return argmax_impl<double>(input, input_len, meta, dim, out, out_cap, out_len);
+}
+
+int32_t fth_layer_norm_backward_f32(const float *dy, size_t dy_len, const float *x, size_t x_len, const float *weight, size_t batch,
+                                    size_t norm_size, float eps, float *dx, size_t dx_cap, float *dweight, size_t dweight_cap,
+                                    float *dbias, size_t dbias_cap) {
+    return norm_backward_impl<float, false>(dy, dy_len, x, x_len, weight, batch, norm_size, eps, dx, dx_cap, dweight, dweight_cap, dbias, dbias_cap);
+}
+int32_t fth_layer_norm_backward_f64(const double *dy, size_t dy_len, const double *x, size_t x_len, const double *weight, size_t batch,
+                                    size_t norm_size, double eps, double *dx, size_t dx_cap, double *dweight, size_t dweight_cap,
+                                    double *dbias, size_t dbias_cap) {
+    return norm_backward_impl<double, false>(dy, dy_len, x, x_len, weight, batch, norm_size, eps, dx, dx_cap, dweight, dweight_cap, dbias, dbias_cap);
+}
+int32_t fth_rms_norm_backward_f32(const float *dy, size_t dy_len, const float *x, size_t x_len, const float *weight, size_t batch,
+                                  size_t norm_size, float eps, float *dx, size_t dx_cap, float *dweight, size_t dweight_cap) {
+    return norm_backward_impl<float, true>(dy, dy_len, x, x_len, weight, batch, norm_size, eps, dx, dx_cap, dweight, dweight_cap, nullptr, 0);
+}
+int32_t fth_rms_norm_backward_f64(const double *dy, size_t dy_len, const double *x, size_t x_len, const double *weight, size_t batch,
+                                  size_t norm_size, double eps, double *dx, size_t dx_cap, double *dweight, size_t dweight_cap) {
+    return norm_backward_impl<double, true>(dy, dy_len, x, x_len, weight, batch, norm_size, eps, dx, dx_cap, dweight, dweight_cap, nullptr, 0);
+}
+int32_t fth_linear_backward_f32(const float *dy, size_t dy_len, const float *x, size_t x_len, const float *weight, size_t weight_len,
+                                size_t batch, size_t in_features, size_t out_features, int32_t need_bias, float *dx, size_t dx_cap,
+                                float *dweight, size_t dweight_cap, float *dbias, size_t dbias_cap) {
+    return linear_backward_impl<float>(dy, dy_len, x, x_len, weight, weight_len, batch, in_features, out_features, need_bias, dx, dx_cap,
+                                       dweight, dweight_cap, dbias, dbias_cap);
+}
+int32_t fth_linear_backward_f64(const double *dy, size_t dy_len, const double *x, size_t x_len, const double *weight, size_t weight_len,
+                                size_t batch, size_t in_features, size_t out_features, int32_t need_bias, double *dx, size_t dx_cap,
+                                double *dweight, size_t dweight_cap, double *dbias, size_t dbias_cap) {
+    return linear_backward_impl<double>(dy, dy_len, x, x_len, weight, weight_len, batch, in_features, out_features, need_bias, dx, dx_cap,
+                                        dweight, dweight_cap, dbias, dbias_cap);
+}
+int32_t fth_sdpa_backward_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len, const float *dout,
+                              size_t dout_len, size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, float scale,
+                              int32_t causal, float *dq, size_t dq_cap, float *dk, size_t dk_cap, float *dv, size_t dv_cap) {
+    return sdpa_backward_impl<float>(q, q_len, k, k_len, v, v_len, dout, dout_len, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dq_cap,
+                                     dk, dk_cap, dv, dv_cap);
+}
+int32_t fth_sdpa_backward_f64(const double *q, size_t q_len, const double *k, size_t k_len, const double *v, size_t v_len, const double *dout,
+                              size_t dout_len, size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, double scale,
+                              int32_t causal, double *dq, size_t dq_cap, double *dk, size_t dk_cap, double *dv, size_t dv_cap) {
+    return sdpa_backward_impl<double>(q, q_len, k, k_len, v, v_len, dout, dout_len, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dq_cap,
+                                      dk, dk_cap, dv, dv_cap);
 }
 
 }  // extern "C"

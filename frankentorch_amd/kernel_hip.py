@@ -208,6 +208,82 @@ def rms_norm_forward_f64(x, weight, batch, norm_size, eps):
     return out
 
 
+def _layer_norm_backward(sfx, dtype, dy, x, weight, batch, norm_size, eps):
+    dy, x, weight = _slice(dy, dtype), _slice(x, dtype), _slice(weight, dtype)
+    dx = np.empty(batch * norm_size, dtype=dtype)
+    dw, db = np.empty(norm_size, dtype=dtype), np.empty(norm_size, dtype=dtype)
+    check(getattr(_lib.load(), "fth_layer_norm_backward_" + sfx)(_p(dy), dy.size, _p(x), x.size, _p(weight), batch, norm_size, eps,
+                                                                 _p(dx), dx.size, _p(dw), dw.size, _p(db), db.size))
+    return dx, dw, db
+
+
+def layer_norm_backward_f32(dy, x, weight, batch, norm_size, eps):
+    """(dx, dweight, dbias), crates/ft-kernel-cpu/src/lib.rs:6189."""
+    return _layer_norm_backward("f32", np.float32, dy, x, weight, batch, norm_size, eps)
+
+
+def layer_norm_backward_f64(dy, x, weight, batch, norm_size, eps):
+    return _layer_norm_backward("f64", np.float64, dy, x, weight, batch, norm_size, eps)
+
+
+def _rms_norm_backward(sfx, dtype, dy, x, weight, batch, norm_size, eps):
+    dy, x, weight = _slice(dy, dtype), _slice(x, dtype), _opt(weight, dtype)
+    dx = np.empty(batch * norm_size, dtype=dtype)
+    dw = None if weight is None else np.empty(norm_size, dtype=dtype)
+    check(getattr(_lib.load(), "fth_rms_norm_backward_" + sfx)(_p(dy), dy.size, _p(x), x.size, _p(weight), batch, norm_size, eps,
+                                                               _p(dx), dx.size, _p(dw), 0 if dw is None else dw.size))
+    return dx, dw
+
+
+def rms_norm_backward_f32(dy, x, weight, batch, norm_size, eps):
+    """(dx, Option<dweight>), crates/ft-kernel-cpu/src/lib.rs:6574."""
+    return _rms_norm_backward("f32", np.float32, dy, x, weight, batch, norm_size, eps)
+
+
+def rms_norm_backward_f64(dy, x, weight, batch, norm_size, eps):
+    return _rms_norm_backward("f64", np.float64, dy, x, weight, batch, norm_size, eps)
+
+
+def _linear_backward(sfx, dtype, dy, x, weight, batch, in_features, out_features, need_bias):
+    dy, x, weight = _slice(dy, dtype), _slice(x, dtype), _slice(weight, dtype)
+    dx = np.empty(batch * in_features, dtype=dtype)
+    dw = np.empty(out_features * in_features, dtype=dtype)
+    db = np.empty(out_features, dtype=dtype) if need_bias else None
+    check(getattr(_lib.load(), "fth_linear_backward_" + sfx)(_p(dy), dy.size, _p(x), x.size, _p(weight), weight.size, batch, in_features,
+                                                             out_features, 1 if need_bias else 0, _p(dx), dx.size, _p(dw), dw.size,
+                                                             _p(db), 0 if db is None else db.size))
+    return dx, dw, db
+
+
+def linear_backward_f64(dy, x, weight, batch, in_features, out_features, need_bias):
+    """(dx, dweight, Option<dbias>), crates/ft-kernel-cpu/src/lib.rs:17226."""
+    return _linear_backward("f64", np.float64, dy, x, weight, batch, in_features, out_features, need_bias)
+
+
+def linear_backward_f32(dy, x, weight, batch, in_features, out_features, need_bias):
+    return _linear_backward("f32", np.float32, dy, x, weight, batch, in_features, out_features, need_bias)
+
+
+def _sdpa_backward(sfx, dtype, q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal):
+    q, k, v, dout = _slice(q, dtype), _slice(k, dtype), _slice(v, dtype), _slice(dout, dtype)
+    dq = np.empty(num_bh * seq_q * d_k, dtype=dtype)
+    dk = np.empty(num_bh * seq_k * d_k, dtype=dtype)
+    dv = np.empty(num_bh * seq_k * d_v, dtype=dtype)
+    check(getattr(_lib.load(), "fth_sdpa_backward_" + sfx)(_p(q), q.size, _p(k), k.size, _p(v), v.size, _p(dout), dout.size, num_bh, seq_q,
+                                                           seq_k, d_k, d_v, scale, 1 if causal else 0, _p(dq), dq.size, _p(dk), dk.size,
+                                                           _p(dv), dv.size))
+    return dq, dk, dv
+
+
+def sdpa_backward_f32(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal):
+    """(dq, dk, dv), crates/ft-kernel-cpu/src/lib.rs:5539."""
+    return _sdpa_backward("f32", np.float32, q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal)
+
+
+def sdpa_backward_f64(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal):
+    return _sdpa_backward("f64", np.float64, q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal)
+
+
 def _sdpa(name, dtype, q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal):
     q, k, v = _slice(q, dtype), _slice(k, dtype), _slice(v, dtype)
     out = np.empty(num_bh * seq_q * d_v, dtype=dtype)

@@ -362,6 +362,33 @@ int32_t fth_rms_norm_forward_f32(const float *x, size_t x_len, const float *weig
                                  size_t norm_size, float eps, float *out, size_t out_cap);
 int32_t fth_rms_norm_forward_f64(const double *x, size_t x_len, const double *weight, size_t batch,
                                  size_t norm_size, double eps, double *out, size_t out_cap);
+/* Backward of the fused ops on host slices. Every output has its own capacity (in elements) and must hold its result:
+ * layer_norm_backward_f32 (:6189) / _f64 (:6052) -> dx [batch*norm_size], dweight, dbias [norm_size];
+ * rms_norm_backward_f32 (:6574) / _f64 (:6503) -> dx, dweight (weight == NULL: no dweight, pass NULL / 0);
+ * linear_backward_f64 (:17226) and the same formulas in f32 -> dx [batch*in], dweight [out*in], dbias [out] when need_bias;
+ * sdpa_backward_f32 (:5539) / _f64 (:5300) -> dq, dk, dv of the shapes of q, k, v. */
+int32_t fth_layer_norm_backward_f32(const float *dy, size_t dy_len, const float *x, size_t x_len, const float *weight, size_t batch,
+                                    size_t norm_size, float eps, float *dx, size_t dx_cap, float *dweight, size_t dweight_cap,
+                                    float *dbias, size_t dbias_cap);
+int32_t fth_layer_norm_backward_f64(const double *dy, size_t dy_len, const double *x, size_t x_len, const double *weight, size_t batch,
+                                    size_t norm_size, double eps, double *dx, size_t dx_cap, double *dweight, size_t dweight_cap,
+                                    double *dbias, size_t dbias_cap);
+int32_t fth_rms_norm_backward_f32(const float *dy, size_t dy_len, const float *x, size_t x_len, const float *weight, size_t batch,
+                                  size_t norm_size, float eps, float *dx, size_t dx_cap, float *dweight, size_t dweight_cap);
+int32_t fth_rms_norm_backward_f64(const double *dy, size_t dy_len, const double *x, size_t x_len, const double *weight, size_t batch,
+                                  size_t norm_size, double eps, double *dx, size_t dx_cap, double *dweight, size_t dweight_cap);
+int32_t fth_linear_backward_f32(const float *dy, size_t dy_len, const float *x, size_t x_len, const float *weight, size_t weight_len,
+                                size_t batch, size_t in_features, size_t out_features, int32_t need_bias, float *dx, size_t dx_cap,
+                                float *dweight, size_t dweight_cap, float *dbias, size_t dbias_cap);
+int32_t fth_linear_backward_f64(const double *dy, size_t dy_len, const double *x, size_t x_len, const double *weight, size_t weight_len,
+                                size_t batch, size_t in_features, size_t out_features, int32_t need_bias, double *dx, size_t dx_cap,
+                                double *dweight, size_t dweight_cap, double *dbias, size_t dbias_cap);
+int32_t fth_sdpa_backward_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len, const float *dout,
+                              size_t dout_len, size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, float scale,
+                              int32_t causal, float *dq, size_t dq_cap, float *dk, size_t dk_cap, float *dv, size_t dv_cap);
+int32_t fth_sdpa_backward_f64(const double *q, size_t q_len, const double *k, size_t k_len, const double *v, size_t v_len, const double *dout,
+                              size_t dout_len, size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, double scale,
+                              int32_t causal, double *dq, size_t dq_cap, double *dk, size_t dk_cap, double *dv, size_t dv_cap);
 /* gelu_tensor_contiguous_f32 (:37123) / _f64 (:3657); add_tensor_contiguous_f32 (:36870) / _f64 */
 int32_t fth_gelu_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta,
                                        float *out, size_t out_cap, size_t *out_len);

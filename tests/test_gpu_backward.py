@@ -133,3 +133,33 @@ def test_norm_backward_at_the_row_op_benchmark_shape(hip, oracle):
     assert rel_err(ddx.to_host()[pick], dxr) <= TOL_ROW_F32
     rstd = 1.0 / np.sqrt((x64 * x64).mean(1, keepdims=True) + 1e-6)
     assert rel_err(ddw.to_host(), (dy64 * x64 * rstd).sum(0)) <= 4 * TOL_ROW_F32
+
+
+def test_host_slice_backward_entry_points(oracle):
+    """The ft_kernel_cpu-named functions on host slices (upload, kernels, download), and their error statuses."""
+    from frankentorch_amd import kernel_hip as K
+    from frankentorch_amd.core import HipError, KernelError
+
+    rows, cols = 33, 96
+    x, dy = synth.normal(21, "x", (rows, cols)), synth.normal(21, "dy", (rows, cols))
+    w = synth.uniform(21, "w", (cols,), 0.5, 1.5)
+    dx, dw, db = K.layer_norm_backward_f32(dy.ravel(), x.ravel(), w, rows, cols, 1e-5)
+    rx, rw, rb = oracle.layer_norm_backward(dy, x, w, np.float32(1e-5))
+    assert rel_err(dx, rx.ravel()) <= TOL_ROW_F32 and rel_err(dw, rw) <= 4 * TOL_ROW_F32 and rel_err(db, rb) <= 4 * TOL_ROW_F32
+    dx, dw = K.rms_norm_backward_f64(dy.astype(np.float64).ravel(), x.astype(np.float64).ravel(), None, rows, cols, 1e-6)
+    assert dw is None
+    assert rel_err(dx, oracle.rms_norm_backward(dy.astype(np.float64), x.astype(np.float64), None, 1e-6)[0].ravel()) <= TOL_F64
+    batch, in_f, out_f = 40, 24, 56
+    dyl, xl, wl = synth.normal(22, "dy", (batch, out_f)), synth.normal(22, "x", (batch, in_f)), synth.normal(22, "w", (out_f, in_f))
+    gx, gw, gb = K.linear_backward_f32(dyl.ravel(), xl.ravel(), wl.ravel(), batch, in_f, out_f, True)
+    ox, ow, ob = oracle.linear_backward(dyl, xl, wl, True)
+    assert rel_err(gx, ox.ravel()) <= TOL_GEMM_F32 and rel_err(gw, ow.ravel()) <= TOL_GEMM_F32 and rel_err(gb, ob) <= TOL_GEMM_F32
+    assert K.linear_backward_f32(dyl.ravel(), xl.ravel(), wl.ravel(), batch, in_f, out_f, False)[2] is None
+    bh, sq, sk, dk, dv = 2, 17, 23, 16, 8
+    q, k, v = synth.normal(23, "q", (bh, sq, dk)), synth.normal(23, "k", (bh, sk, dk)), synth.normal(23, "v", (bh, sk, dv))
+    do = synth.normal(23, "do", (bh, sq, dv))
+    got = K.sdpa_backward_f32(q.ravel(), k.ravel(), v.ravel(), do.ravel(), bh, sq, sk, dk, dv, 0.25, True)
+    for g, r in zip(got, oracle.sdpa_backward(q, k, v, do, np.float32(0.25), True)):
+        assert rel_err(g, r.ravel()) <= 2 * TOL_GEMM_F32
+    with pytest.raises((KernelError, HipError)):  # a slice shorter than batch * norm_size
+        K.layer_norm_backward_f32(dy.ravel()[:10], x.ravel(), w, rows, cols, 1e-5)
