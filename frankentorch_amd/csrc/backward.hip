@@ -27,6 +27,9 @@
 
 namespace {
 
+#ifndef FTH_BWD_BLOCKS_PER_CU
+#define FTH_BWD_BLOCKS_PER_CU 2
+#endif
 constexpr int kWave = 64;
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
@@ -53,6 +56,18 @@ __device__ __forceinline__ void vset(double2 &v, int i, double x) {
     else v.y = x;
 }
 
+// Streaming (non-temporal) 16-byte stores for outputs the kernel never re-reads.
+typedef float nat_f4 __attribute__((ext_vector_type(4)));
+typedef double nat_d2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void stream_store(float4 *p, const float4 &v) {
+    nat_f4 n = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(n, reinterpret_cast<nat_f4 *>(p));
+}
+__device__ __forceinline__ void stream_store(double2 *p, const double2 &v) {
+    nat_d2 n = {v.x, v.y};
+    __builtin_nontemporal_store(n, reinterpret_cast<nat_d2 *>(p));
+}
+
 template <typename T> __device__ __forceinline__ T wave_sum(T v) {
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
@@ -60,22 +75,26 @@ template <typename T> __device__ __forceinline__ T wave_sum(T v) {
 }
 
 // Sum of NV values per thread over the workgroup: butterfly inside each wavefront, then wavefront 0..3
-// added left to right by every thread (same result in all threads). `red` holds kWaves * NV values.
-template <typename T, int NV> __device__ __forceinline__ void block_sum(T (&v)[NV], T *red) {
+// added left to right by every thread (same result in all threads). `red` holds 2 * kWaves * 2
+// values: consecutive calls alternate between its halves (`phase`), so one barrier per call is
+// enough -- a wavefront can only reach the write of call n + 2 after passing the barrier of call
+// n + 1, which every wavefront reaches only after its reads of call n.
+template <typename T, int NV> __device__ __forceinline__ void block_sum(T (&v)[NV], T *red, int &phase) {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    T *buf = red + phase * (kWaves * 2);
+    phase ^= 1;
 #pragma unroll
     for (int i = 0; i < NV; ++i) v[i] = wave_sum(v[i]);
-    __syncthreads();  // the previous use of `red` is over
     if (lane == 0) {
 #pragma unroll
-        for (int i = 0; i < NV; ++i) red[wave * NV + i] = v[i];
+        for (int i = 0; i < NV; ++i) buf[wave * NV + i] = v[i];
     }
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-        T s = red[i];
+        T s = buf[i];
 #pragma unroll
-        for (int w = 1; w < kWaves; ++w) s += red[w * NV + i];
+        for (int w = 1; w < kWaves; ++w) s += buf[w * NV + i];
         v[i] = s;
     }
 }
@@ -92,7 +111,8 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
                                                                  T *__restrict__ part_b, int rows_per_block) {
     using V = typename Vec16<T>::type;
     constexpr int N = Vec16<T>::N;
-    __shared__ T red[kWaves * 2];
+    __shared__ T red[2 * kWaves * 2];
+    int phase = 0;
     const int tid = threadIdx.x;
     const int nvec = cols / N;
     const T inv_n = T(1) / (T)cols;
@@ -153,7 +173,7 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
             for (int i = 0; i < VPT; ++i)
 #pragma unroll
                 for (int e = 0; e < N; ++e) s[0] += vget(xv[i], e);
-            block_sum<T, 1>(s, red);
+            block_sum<T, 1>(s, red, phase);
             const T mean = s[0] * inv_n;
             T q[1] = {T(0)};
 #pragma unroll
@@ -165,7 +185,7 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
                     if (live) q[0] += d * d;
                 }
             }
-            block_sum<T, 1>(q, red);
+            block_sum<T, 1>(q, red, phase);
             const T rstd = t_rsqrt_of(q[0] * inv_n + eps);
             T c[2] = {T(0), T(0)};
 #pragma unroll
@@ -181,7 +201,7 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
                     }
                 }
             }
-            block_sum<T, 2>(c, red);
+            block_sum<T, 2>(c, red, phase);
             V *dxr = reinterpret_cast<V *>(dx + r * cols);
 #pragma unroll
             for (int i = 0; i < VPT; ++i) {
@@ -195,7 +215,7 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
                     aw[i][e] += vget(gv[i], e) * xhat;
                     ab[i][e] += vget(gv[i], e);
                 }
-                if (v < nvec) dxr[v] = o;
+                if (v < nvec) stream_store(dxr + v, o);
             }
         } else {
             T s[1] = {T(0)};
@@ -203,14 +223,14 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
             for (int i = 0; i < VPT; ++i)
 #pragma unroll
                 for (int e = 0; e < N; ++e) s[0] += vget(xv[i], e) * vget(xv[i], e);
-            block_sum<T, 1>(s, red);
+            block_sum<T, 1>(s, red, phase);
             const T rstd = t_rsqrt_of(s[0] * inv_n + eps);
             T c[1] = {T(0)};
 #pragma unroll
             for (int i = 0; i < VPT; ++i)
 #pragma unroll
                 for (int e = 0; e < N; ++e) c[0] += (vget(gv[i], e) * vget(wv[i], e)) * vget(xv[i], e);
-            block_sum<T, 1>(c, red);
+            block_sum<T, 1>(c, red, phase);
             const T coef = rstd * rstd * rstd * c[0] * inv_n;
             V *dxr = reinterpret_cast<V *>(dx + r * cols);
 #pragma unroll
@@ -223,7 +243,7 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
                     vset(o, e, rstd * g - coef * vget(xv[i], e));
                     aw[i][e] += vget(gv[i], e) * vget(xv[i], e) * rstd;
                 }
-                if (v < nvec) dxr[v] = o;
+                if (v < nvec) stream_store(dxr + v, o);
             }
         }
     }
@@ -250,7 +270,8 @@ template <typename T, bool RMS>
 __global__ __launch_bounds__(kThreads) void norm_backward_stream_kernel(const T *__restrict__ dy, const T *__restrict__ x,
                                                                         const T *__restrict__ w, int64_t cols, T eps,
                                                                         T *__restrict__ dx, T *__restrict__ stats) {
-    __shared__ T red[kWaves * 2];
+    __shared__ T red[2 * kWaves * 2];
+    int phase = 0;
     const int64_t r = blockIdx.x;
     const T *xr = x + r * cols, *dyr = dy + r * cols;
     T *dxr = dx + r * cols;
@@ -259,14 +280,14 @@ __global__ __launch_bounds__(kThreads) void norm_backward_stream_kernel(const T 
     if constexpr (!RMS) {
         T s[1] = {T(0)};
         for (int64_t j = threadIdx.x; j < cols; j += kThreads) s[0] += xr[j];
-        block_sum<T, 1>(s, red);
+        block_sum<T, 1>(s, red, phase);
         mean = s[0] * inv_n;
         T q[1] = {T(0)};
         for (int64_t j = threadIdx.x; j < cols; j += kThreads) {
             const T d = xr[j] - mean;
             q[0] += d * d;
         }
-        block_sum<T, 1>(q, red);
+        block_sum<T, 1>(q, red, phase);
         rstd = t_rsqrt_of(q[0] * inv_n + eps);
         T c[2] = {T(0), T(0)};
         for (int64_t j = threadIdx.x; j < cols; j += kThreads) {
@@ -275,7 +296,7 @@ __global__ __launch_bounds__(kThreads) void norm_backward_stream_kernel(const T 
             c[0] += dxhat;
             c[1] += dxhat * xhat;
         }
-        block_sum<T, 2>(c, red);
+        block_sum<T, 2>(c, red, phase);
         for (int64_t j = threadIdx.x; j < cols; j += kThreads) {
             const T xhat = (xr[j] - mean) * rstd;
             const T dxhat = dyr[j] * w[j];
@@ -284,11 +305,11 @@ __global__ __launch_bounds__(kThreads) void norm_backward_stream_kernel(const T 
     } else {
         T s[1] = {T(0)};
         for (int64_t j = threadIdx.x; j < cols; j += kThreads) s[0] += xr[j] * xr[j];
-        block_sum<T, 1>(s, red);
+        block_sum<T, 1>(s, red, phase);
         rstd = t_rsqrt_of(s[0] * inv_n + eps);
         T c[1] = {T(0)};
         for (int64_t j = threadIdx.x; j < cols; j += kThreads) c[0] += (dyr[j] * (w ? w[j] : T(1))) * xr[j];
-        block_sum<T, 1>(c, red);
+        block_sum<T, 1>(c, red, phase);
         const T coef = rstd * rstd * rstd * c[0] * inv_n;
         for (int64_t j = threadIdx.x; j < cols; j += kThreads) dxr[j] = rstd * (dyr[j] * (w ? w[j] : T(1))) - coef * xr[j];
     }
@@ -366,7 +387,7 @@ template <typename T> int32_t zero_fill(T *dst, int64_t n, hipStream_t st) {
 inline int pick_rows_per_block(int64_t rows) {
     // enough workgroups to fill the chip several times over, at most 64 rows each
     const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
-    int64_t r = rows / ((int64_t)cus * 2);
+    int64_t r = rows / ((int64_t)cus * FTH_BWD_BLOCKS_PER_CU);
     if (r < 1) r = 1;
     if (r > 64) r = 64;
     return (int)r;
