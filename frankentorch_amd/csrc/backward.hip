@@ -588,6 +588,115 @@ __global__ __launch_bounds__(kThreads) void sdpa_softmax_backward_rows_kernel(co
     for (int64_t j = lane; j < seq_k; j += kWave) dr[j] = pr[j] * (dr[j] - dot);
 }
 
+// Register-resident forms of the two row passes for rows of up to 64 * VPL 16-byte vectors: the row is
+// read once (only its first `limit` entries matter for the softmax; the rest is written as zeros)
+// and written once. Same arithmetic as the streaming kernels above, lane-strided partial sums.
+template <typename T, int VPL>
+__global__ __launch_bounds__(kThreads) void sdpa_softmax_rows_vec_kernel(T *__restrict__ p, int64_t rows, int64_t seq_q, int seq_k,
+                                                                        T scale, int causal) {
+    using V = typename Vec16<T>::type;
+    constexpr int N = Vec16<T>::N;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t r = (int64_t)blockIdx.x * kWaves + threadIdx.x / kWave;
+    if (r >= rows) return;
+    const int64_t i = r % seq_q;
+    const int limit = causal ? (int)(i + 1 < seq_k ? i + 1 : seq_k) : seq_k;
+    const int nvec = seq_k / N;
+    V *row = reinterpret_cast<V *>(p + r * seq_k);
+    T e[VPL][N];
+    T m = -__builtin_inf();
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+        const int v = lane + u * kWave;
+        if (v < nvec && v * N < limit) {
+            const V x = row[v];
+#pragma unroll
+            for (int c = 0; c < N; ++c) {
+                e[u][c] = vget(x, c) * scale;
+                if (v * N + c < limit) m = e[u][c] > m ? e[u][c] : m;
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < N; ++c) e[u][c] = T(0);
+        }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const T o = __shfl_xor(m, off, kWave);
+        m = o > m ? o : m;
+    }
+    T sum = T(0);
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+        const int v = lane + u * kWave;
+#pragma unroll
+        for (int c = 0; c < N; ++c) {
+            if (v * N + c < limit) {
+                e[u][c] = dev_exp_t<T>(e[u][c] - m);
+                sum += e[u][c];
+            } else {
+                e[u][c] = T(0);
+            }
+        }
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+        const int v = lane + u * kWave;
+        if (v < nvec) {
+            V o;
+#pragma unroll
+            for (int c = 0; c < N; ++c) vset(o, c, (v * N + c < limit) ? e[u][c] / sum : T(0));
+            row[v] = o;
+        }
+    }
+}
+
+template <typename T, int VPL>
+__global__ __launch_bounds__(kThreads) void sdpa_softmax_backward_rows_vec_kernel(const T *__restrict__ p, T *__restrict__ du, int64_t rows,
+                                                                                 int seq_k) {
+    using V = typename Vec16<T>::type;
+    constexpr int N = Vec16<T>::N;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t r = (int64_t)blockIdx.x * kWaves + threadIdx.x / kWave;
+    if (r >= rows) return;
+    const int nvec = seq_k / N;
+    const V *pr = reinterpret_cast<const V *>(p + r * seq_k);
+    V *dr = reinterpret_cast<V *>(du + r * seq_k);
+    V pv[VPL], dv[VPL];
+    T dot = T(0);
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+        const int v = lane + u * kWave;
+        if (v < nvec) {
+            pv[u] = pr[v];
+            dv[u] = dr[v];
+#pragma unroll
+            for (int c = 0; c < N; ++c) dot += vget(pv[u], c) * vget(dv[u], c);
+        }
+    }
+    dot = wave_sum(dot);
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+        const int v = lane + u * kWave;
+        if (v < nvec) {
+            V o;
+#pragma unroll
+            for (int c = 0; c < N; ++c) vset(o, c, vget(pv[u], c) * (vget(dv[u], c) - dot));
+            dr[v] = o;
+        }
+    }
+}
+
+// 0 when the rows do not fit the register-resident kernels, else the vectors per lane to use.
+template <typename T> int sdpa_row_vpl(int64_t seq_k, const void *a, const void *b) {
+    constexpr int N = Vec16<T>::N;
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    if (seq_k % N != 0 || seq_k > (int64_t)kWave * 16 * N || !al(a) || !al(b)) return 0;
+    const int64_t per = fth::ceil_div(seq_k / N, kWave);
+    return per <= 1 ? 1 : per <= 2 ? 2 : per <= 4 ? 4 : per <= 8 ? 8 : 16;
+}
+
 template <typename T> size_t sdpa_backward_workspace(int64_t num_bh, int64_t seq_q, int64_t seq_k) {
     return (size_t)(2 * num_bh * seq_q * seq_k + 64) * sizeof(T);
 }
@@ -625,7 +734,21 @@ int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, i
     } else {
         if (int32_t rc = zero_fill<T>(p, pe, st)) return rc;
     }
-    sdpa_softmax_rows_kernel<T><<<dim3((unsigned)fth::ceil_div(rows, kWaves)), dim3(kThreads), 0, st>>>(p, rows, seq_q, seq_k, scale, causal);
+    const int vpl = sdpa_row_vpl<T>(seq_k, p, du);
+    const dim3 row_grid((unsigned)fth::ceil_div(rows, kWaves));
+#define FTH_ROWS_VEC(KERN, ...)                                                         \
+    switch (vpl) {                                                                      \
+        case 1: KERN<T, 1><<<row_grid, dim3(kThreads), 0, st>>>(__VA_ARGS__); break;     \
+        case 2: KERN<T, 2><<<row_grid, dim3(kThreads), 0, st>>>(__VA_ARGS__); break;     \
+        case 4: KERN<T, 4><<<row_grid, dim3(kThreads), 0, st>>>(__VA_ARGS__); break;     \
+        case 8: KERN<T, 8><<<row_grid, dim3(kThreads), 0, st>>>(__VA_ARGS__); break;     \
+        default: KERN<T, 16><<<row_grid, dim3(kThreads), 0, st>>>(__VA_ARGS__); break;   \
+    }
+    if (vpl > 0) {
+        FTH_ROWS_VEC(sdpa_softmax_rows_vec_kernel, p, rows, seq_q, (int)seq_k, scale, causal)
+    } else {
+        sdpa_softmax_rows_kernel<T><<<row_grid, dim3(kThreads), 0, st>>>(p, rows, seq_q, seq_k, scale, causal);
+    }
     FTH_CHECK_LAUNCH("sdpa_backward_softmax");
     // dU = dOut . V^T
     if (d_v > 0) {
@@ -639,7 +762,12 @@ int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, i
         fth_gemm_desc d = make_desc(seq_k, d_v, seq_q, 1, 0, num_bh);
         if (int32_t rc = dev_gemm<T>(&d, T(1), p, dout, dv, fs)) return rc;
     }
-    sdpa_softmax_backward_rows_kernel<T><<<dim3((unsigned)fth::ceil_div(rows, kWaves)), dim3(kThreads), 0, st>>>(p, du, rows, seq_k);
+    if (vpl > 0) {
+        FTH_ROWS_VEC(sdpa_softmax_backward_rows_vec_kernel, p, du, rows, (int)seq_k)
+    } else {
+        sdpa_softmax_backward_rows_kernel<T><<<row_grid, dim3(kThreads), 0, st>>>(p, du, rows, seq_k);
+    }
+#undef FTH_ROWS_VEC
     FTH_CHECK_LAUNCH("sdpa_backward_softmax_grad");
     if (d_k > 0) {
         // dQ = scale * dU . K ; dK = scale * dU^T . Q
