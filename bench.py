@@ -240,6 +240,85 @@ def bench_sdpa(device, synth, steps, with_cpu):
     return res
 
 
+def bench_backward(device, synth, steps, with_cpu):
+    """Backward kernels of the same ops at the forward benchmark shapes."""
+    from frankentorch_amd.device import DeviceBuffer
+
+    out = {}
+    iters = max(10, steps // 2)
+    O = cpu_oracle() if with_cpu else None
+
+    def timed(fn, n=iters):
+        for _ in range(3):
+            fn()
+        device.synchronize()
+        return event_time_ms(device, fn, n)
+
+    # LayerNorm / RMSNorm backward, fp32 [8192,4096]: read x and dy, write dx (+ weight, dweight, dbias once)
+    x = synth.normal(1, "x", (ROWS, COLS))
+    dy = synth.normal(1, "dy", (ROWS, COLS))
+    gamma = synth.uniform(1, "gamma", (COLS,), 0.5, 1.5)
+    dx_, ddy, dg = DeviceBuffer.from_host(x), DeviceBuffer.from_host(dy), DeviceBuffer.from_host(gamma)
+    gx, gw, gb = DeviceBuffer((ROWS, COLS)), DeviceBuffer((COLS,)), DeviceBuffer((COLS,))
+    ws = device.layer_norm_backward(ddy, dx_, dg, gx, gw, gb, ROWS, COLS, 1e-5)
+    for name, nbytes, fn, cpu_fn in (
+        ("layer_norm_backward", 3 * ELEM * 4 + 3 * COLS * 4,
+         lambda: device.layer_norm_backward(ddy, dx_, dg, gx, gw, gb, ROWS, COLS, 1e-5, workspace=ws),
+         lambda: O.layer_norm_backward(dy, x, gamma, np.float32(1e-5))),
+        ("rms_norm_backward", 3 * ELEM * 4 + 2 * COLS * 4,
+         lambda: device.rms_norm_backward(ddy, dx_, dg, gx, gw, ROWS, COLS, 1e-6, workspace=ws),
+         lambda: O.rms_norm_backward(dy, x, gamma, np.float32(1e-6))),
+    ):
+        ms = timed(fn)
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        out[name] = {"ms": round(ms, 5), "GB/s": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4), "bytes": nbytes,
+                     "workload": "fp32 [8192,4096], dx + dweight (+ dbias), all launches of the entry point"}
+        log("[backward] %-20s %.4f ms  %7.1f GB/s  %.1f%% of HBM peak" % (name, ms, gbs, 100 * gbs / HBM_PEAK_GBS))
+        if with_cpu:
+            best, reps = cpu_time(cpu_fn, 2.0)
+            out[name]["cpu"] = {"value": round(nbytes / best / 1e9, 2), "unit": "GB/s", "cores": O.threads(), "kind": "port",
+                                "sample": "the same tensors, best of %d" % reps}
+    del dx_, ddy, gx
+    # linear backward at the GPT-2 FC1 shape: dx and dweight products + dbias
+    batch, in_f, out_f = 8192, 768, 3072
+    dyl, xl = synth.normal(4, "dyl", (batch, out_f)), synth.normal(4, "xl", (batch, in_f))
+    wl = synth.normal(4, "wl", (out_f, in_f), 0.0, 0.02)
+    a, b, c = DeviceBuffer.from_host(dyl), DeviceBuffer.from_host(xl), DeviceBuffer.from_host(wl)
+    lx, lw, lb = DeviceBuffer((batch, in_f)), DeviceBuffer((out_f, in_f)), DeviceBuffer((out_f,))
+    ws2 = device.linear_backward(a, b, c, lx, lw, lb, batch, in_f, out_f)
+    ms = timed(lambda: device.linear_backward(a, b, c, lx, lw, lb, batch, in_f, out_f, workspace=ws2))
+    flop = 4 * batch * in_f * out_f
+    tf = flop / (ms * 1e-3) / 1e12
+    out["linear_backward"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac": round(tf / FP32_MFMA_PEAK_TF, 4), "flop": flop,
+                              "workload": "fp32 batch 8192, 768 -> 3072: dx = dy.W, dweight = dy^T.x, dbias"}
+    log("[backward] linear_backward      %.4f ms  %6.2f TFLOP/s  %.1f%% of MFMA peak" % (ms, tf, 100 * tf / FP32_MFMA_PEAK_TF))
+    if with_cpu:
+        nb = 512  # rows of the batch timed on the CPU (the checker's products accumulate wide and are slow)
+        best, reps = cpu_time(lambda: O.linear_backward(dyl[:nb], xl[:nb], wl, True), 3.0, min_reps=1)
+        out["linear_backward"]["cpu"] = {"value": round(4 * nb * in_f * out_f / best / 1e12, 4), "unit": "TFLOP/s", "cores": O.threads(),
+                                         "kind": "port", "sample": "%d of the 8192 rows, wide-accumulation products, best of %d" % (nb, reps)}
+    del a, b, c, lx, lw
+    # SDPA backward at the config-4 shape; flop count of the reference's five full-rectangle products per head
+    B, H, S, D = 4, 32, 2048, 128
+    sc = 1.0 / math.sqrt(D)
+    q, k, v = (synth.normal(3, t, (B * H, S, D), 0.0, sc) for t in ("Q", "K", "V"))
+    do = synth.normal(3, "dO", (B * H, S, D))
+    dq, dk, dv, ddo = (DeviceBuffer.from_host(t) for t in (q, k, v, do))
+    gq, gk, gv = DeviceBuffer(q.shape), DeviceBuffer(q.shape), DeviceBuffer(q.shape)
+    ws3 = device.sdpa_backward(dq, dk, dv, ddo, B * H, S, S, D, D, sc, True, gq, gk, gv)
+    ms = timed(lambda: device.sdpa_backward(dq, dk, dv, ddo, B * H, S, S, D, D, sc, True, gq, gk, gv, workspace=ws3), max(3, steps // 10))
+    flop = 5 * 2 * B * H * S * S * D
+    tf = flop / (ms * 1e-3) / 1e12
+    out["sdpa_backward"] = {"ms": round(ms, 3), "TFLOP/s": round(tf, 2), "frac": round(tf / FP32_MFMA_PEAK_TF, 4), "flop": flop,
+                            "workload": "B4 H32 S2048 D128 causal fp32; flop = the reference's five full [S,S] products per head"}
+    log("[backward] sdpa_backward        %.3f ms  %6.2f TFLOP/s  %.1f%% of MFMA peak" % (ms, tf, 100 * tf / FP32_MFMA_PEAK_TF))
+    if with_cpu:
+        best, reps = cpu_time(lambda: O.sdpa_backward(q[:1], k[:1], v[:1], do[:1], np.float32(sc), True), 3.0, min_reps=1)
+        out["sdpa_backward"]["cpu"] = {"value": round(flop / (B * H) / best / 1e12, 4), "unit": "TFLOP/s", "cores": O.threads(),
+                                       "kind": "port", "sample": "1 of the 128 heads, wide-accumulation products, best of %d" % reps}
+    return out
+
+
 def make_layer(synth, seed, li, d, f):
     n = lambda tag, *s: synth.normal(seed, "L%d.%s" % (li, tag), s, 0.0, 0.02)
     one, zero = (lambda m: np.ones(m, np.float32)), (lambda m: np.zeros(m, np.float32))
@@ -311,7 +390,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--cases", default="all", help="comma list of: gemm,sdpa,block,gpt2 (row ops always run); 'none' for row ops only")
+    ap.add_argument("--cases", default="all", help="comma list of: gemm,sdpa,block,gpt2,backward (row ops always run); 'none' for row ops only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -324,7 +403,7 @@ def main():
     info = device.device_info()
     log("[device] %s, %d CUs, %.0f GiB HBM, engine %d MHz" % (info["arch"], info["compute_units"], info["hbm_bytes"] / 2 ** 30,
                                                                info["engine_clock_khz"] // 1000))
-    cases = {"gemm", "sdpa", "block", "gpt2"} if args.cases == "all" else set(c for c in args.cases.split(",") if c and c != "none")
+    cases = {"gemm", "sdpa", "block", "gpt2", "backward"} if args.cases == "all" else set(c for c in args.cases.split(",") if c and c != "none")
 
     value, ms_per_step, roof, per_kernel, cpu = bench_rowops(device, synth, args.steps, args.warmup, not args.no_cpu)
     extra = {"row_ops": per_kernel}
@@ -336,6 +415,8 @@ def main():
         extra["block"] = bench_block(device, synth, args.steps, not args.no_cpu)
     if "gpt2" in cases:
         extra["gpt2_forward"] = bench_gpt2(device, synth, args.steps)
+    if "backward" in cases:
+        extra["backward"] = bench_backward(device, synth, args.steps, not args.no_cpu)
 
     line = {
         "metric": "row-op GB/s (fp32, 1 MI355X)",
