@@ -137,6 +137,7 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
     const float *Vg = static_cast<const float *>(p.v) + b * d.v_batch_stride + h * d.v_head_stride;
     float *O = static_cast<float *>(p.out) + b * d.o_batch_stride + h * d.o_head_stride;
     const float scale = (float)p.scale;
+    const float c2 = scale * 1.44269502162933349609375f;  // scale * log2(e)
 
     const int qb_first = p.q_blocks - 1 - unit;  // the long rows of a causal problem first
     const int npass = (PAIR && unit != qb_first) ? 2 : 1;
@@ -275,31 +276,60 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
             if (wave_active) {
                 // ---- scale, mask, online softmax (lane-local query) ----
                 const bool need_mask = (d.causal && key0 + kBC - 1 > q_wave0) || (key0 + kBC > seq_k_i);
-                float mt = -__builtin_inff();
+                float mt = -__builtin_inff(), m_new, alpha, psum = 0.f;
+                if (scale > 0.f) {
+                    // Positive scale (every real caller): the row max is taken on the raw scores (scaling
+                    // by a positive constant keeps the order), and scale * log2(e) is folded into one FMA
+                    // per score, 2^(s * c2 - m) with the running max m kept in those log2 units.
 #pragma unroll
-                for (int j = 0; j < KS; ++j)
+                    for (int j = 0; j < KS; ++j)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        float x = s[j][r] * scale;
-                        if (need_mask) {
-                            const int key = key0 + 32 * j + 8 * (r >> 2) + 4 * half + (r & 3);
-                            if ((d.causal && key > qi) || key >= seq_k_i) x = -__builtin_inff();
+                        for (int r = 0; r < 16; ++r) {
+                            float x = s[j][r];
+                            if (need_mask) {
+                                const int key = key0 + 32 * j + 8 * (r >> 2) + 4 * half + (r & 3);
+                                if ((d.causal && key > qi) || key >= seq_k_i) x = -__builtin_inff();
+                            }
+                            s[j][r] = x;
+                            mt = fmaxf(mt, x);
                         }
-                        s[j][r] = x;
-                        mt = fmaxf(mt, x);
-                    }
-                mt = fmaxf(mt, __shfl_xor(mt, 32, kWave));
-                const float m_new = fmaxf(m_run, mt);
-                const float alpha = exp_diff(m_run, m_new);
-                float psum = 0.f;
+                    mt = fmaxf(mt, __shfl_xor(mt, 32, kWave));
+                    m_new = fmaxf(m_run, mt * c2);
+                    alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                    const float neg_m = -m_new;
 #pragma unroll
-                for (int j = 0; j < KS; ++j)
+                    for (int j = 0; j < KS; ++j)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const float e = exp_diff(s[j][r], m_new);
-                        s[j][r] = e;
-                        psum += e;
-                    }
+                        for (int r = 0; r < 16; ++r) {
+                            const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][r], c2, neg_m));
+                            s[j][r] = e;
+                            psum += e;
+                        }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < KS; ++j)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            float x = s[j][r] * scale;
+                            if (need_mask) {
+                                const int key = key0 + 32 * j + 8 * (r >> 2) + 4 * half + (r & 3);
+                                if ((d.causal && key > qi) || key >= seq_k_i) x = -__builtin_inff();
+                            }
+                            s[j][r] = x;
+                            mt = fmaxf(mt, x);
+                        }
+                    mt = fmaxf(mt, __shfl_xor(mt, 32, kWave));
+                    m_new = fmaxf(m_run, mt);
+                    alpha = exp_diff(m_run, m_new);
+#pragma unroll
+                    for (int j = 0; j < KS; ++j)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const float e = exp_diff(s[j][r], m_new);
+                            s[j][r] = e;
+                            psum += e;
+                        }
+                }
                 psum += __shfl_xor(psum, 32, kWave);
                 l_run = l_run * alpha + psum;
                 m_run = m_new;
