@@ -139,6 +139,26 @@ def bench_rowops(device, synth, steps, warmup, with_cpu):
                "sample": "the full config-2 step (5 row ops on fp32 [8192,4096]), best of %d runs, %.1f s of CPU work"
                          % (reps, time.perf_counter() - t_all)}
         log("[rowops] cpu baseline %.2f GB/s on %d threads" % (cpu["value"], cpu["cores"]))
+        # Context only, clearly labelled: the same five ops through PyTorch's own CPU kernels.
+        try:
+            import torch
+
+            tx, tg, tb = torch.from_numpy(x), torch.from_numpy(gamma), torch.from_numpy(beta)
+            tbias, tres = torch.from_numpy(bias), torch.from_numpy(res)
+
+            def torch_step():
+                torch.softmax(tx, 1)
+                torch.nn.functional.layer_norm(tx, (COLS,), tg, tb, 1e-5)
+                tx * torch.rsqrt(tx.pow(2).mean(1, keepdim=True) + 1e-6) * tg
+                torch.nn.functional.gelu(tx)
+                tx + tbias + tres
+
+            best_t, reps_t = cpu_time(torch_step, 4.0)
+            cpu["torch_cpu_context"] = {"value": round(step_bytes / best_t / 1e9, 2), "unit": "GB/s", "threads": torch.get_num_threads(),
+                                        "note": "PyTorch %s CPU kernels on the same tensors, best of %d; not the reference" % (torch.__version__, reps_t)}
+            log("[rowops] torch CPU context %.2f GB/s" % cpu["torch_cpu_context"]["value"])
+        except Exception as exc:  # context line only
+            log("[rowops] torch CPU context skipped: %s" % exc)
     return value, ms_per_step, roof, per_kernel, cpu
 
 
@@ -316,6 +336,37 @@ def bench_backward(device, synth, steps, with_cpu):
         best, reps = cpu_time(lambda: O.sdpa_backward(q[:1], k[:1], v[:1], do[:1], np.float32(sc), True), 3.0, min_reps=1)
         out["sdpa_backward"]["cpu"] = {"value": round(flop / (B * H) / best / 1e12, 4), "unit": "TFLOP/s", "cores": O.threads(),
                                        "kind": "port", "sample": "1 of the 128 heads, wide-accumulation products, best of %d" % reps}
+    del dq, dk, dv, ddo, gq, gk, gv, ws3
+    # log-softmax and the fused cross-entropy on the forward's logits [8192, 50257] (made on the device by the LM-head product)
+    rows, vocab, width = 8192, 50257, 768
+    hid = synth.normal(5, "hidden", (rows, width)) * np.float32(0.25)
+    wte = synth.normal(5, "wte", (vocab, width))
+    tgt = synth.token_ids(5, "target", (rows,), vocab).astype(np.int64)
+    dh, dwte, dtgt = DeviceBuffer.from_host(hid), DeviceBuffer.from_host(wte), DeviceBuffer.from_host(tgt)
+    lg, lo = DeviceBuffer((rows, vocab)), DeviceBuffer((rows, vocab))
+    loss, dloss = DeviceBuffer((rows,)), DeviceBuffer.from_host(np.ones(rows, np.float32))
+    device.gemm(device.gemm_desc(rows, vocab, width, trans_b=True), dh, dwte, lg)
+    nel = rows * vocab * 4
+    sample = None
+    if with_cpu:
+        nb = 64
+        sample = (hid[:nb].astype(np.float64) @ wte.T.astype(np.float64)).astype(np.float32)
+    for name, nbytes, fn, cpu_fn in (
+        ("log_softmax", 2 * nel, lambda: device.log_softmax_strided(lg, lo, rows, vocab, 1), lambda: O.log_softmax(sample, 1)),
+        ("cross_entropy_forward", nel + rows * 12, lambda: device.cross_entropy_forward(lg, dtgt, rows, vocab, loss),
+         lambda: O.cross_entropy_forward(sample, tgt[:64])),
+        ("cross_entropy_backward", 2 * nel + rows * 12, lambda: device.cross_entropy_backward(lg, dtgt, dloss, rows, vocab, lo),
+         lambda: O.cross_entropy_backward(sample, tgt[:64], np.ones(64, np.float32))),
+    ):
+        ms = timed(fn, max(5, steps // 5))
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        out[name] = {"ms": round(ms, 4), "GB/s": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4), "bytes": nbytes,
+                     "workload": "fp32 logits [8192,50257], int64 targets"}
+        log("[backward] %-22s %.4f ms  %7.1f GB/s  %.1f%% of HBM peak" % (name, ms, gbs, 100 * gbs / HBM_PEAK_GBS))
+        if with_cpu:
+            best, reps = cpu_time(cpu_fn, 2.0)
+            out[name]["cpu"] = {"value": round(nbytes * 64 / rows / best / 1e9, 2), "unit": "GB/s", "cores": O.threads(), "kind": "port",
+                                "sample": "64 of the 8192 rows, best of %d" % reps}
     return out
 
 

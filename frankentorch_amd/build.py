@@ -25,6 +25,7 @@ HIP_SOURCES = [
     "gemm.hip",
     "sdpa.hip",
     "backward.hip",
+    "lossops.hip",
     "host_api.hip",
     "resident.hip",
 ]

@@ -173,6 +173,9 @@ template <> struct Dev<float> {
         return fth_dev_gemm_f32(d, al, a, b, c, bias, nullptr, nullptr);
     }
     static int32_t softmax(const float *x, float *y, int64_t o, int64_t r, int64_t i) { return fth_dev_softmax_strided_f32(x, y, o, r, i, nullptr); }
+    static int32_t log_softmax(const float *x, float *y, int64_t o, int64_t r, int64_t i) { return fth_dev_log_softmax_strided_f32(x, y, o, r, i, nullptr); }
+    static int32_t ce_fwd(const float *l, const int64_t *t, int64_t b, int64_t c, float *o, int64_t *bad) { return fth_dev_cross_entropy_forward_f32(l, t, b, c, o, bad, nullptr); }
+    static int32_t ce_bwd(const float *l, const int64_t *t, const float *g, int64_t b, int64_t c, float *o, int64_t *bad) { return fth_dev_cross_entropy_backward_f32(l, t, g, b, c, o, bad, nullptr); }
     static int32_t layer_norm(const float *x, const float *w, const float *b, float *y, int64_t n, int64_t c, float e) { return fth_dev_layer_norm_f32(x, w, b, y, n, c, e, nullptr); }
     static int32_t rms_norm(const float *x, const float *w, float *y, int64_t n, int64_t c, float e) { return fth_dev_rms_norm_f32(x, w, y, n, c, e, nullptr); }
     static int32_t gelu(const float *x, float *y, int64_t n) { return fth_dev_gelu_f32(x, y, n, nullptr); }
@@ -187,6 +190,9 @@ template <> struct Dev<double> {
         return fth_dev_gemm_f64(d, al, a, b, c, bias, nullptr, nullptr);
     }
     static int32_t softmax(const double *x, double *y, int64_t o, int64_t r, int64_t i) { return fth_dev_softmax_strided_f64(x, y, o, r, i, nullptr); }
+    static int32_t log_softmax(const double *x, double *y, int64_t o, int64_t r, int64_t i) { return fth_dev_log_softmax_strided_f64(x, y, o, r, i, nullptr); }
+    static int32_t ce_fwd(const double *l, const int64_t *t, int64_t b, int64_t c, double *o, int64_t *bad) { return fth_dev_cross_entropy_forward_f64(l, t, b, c, o, bad, nullptr); }
+    static int32_t ce_bwd(const double *l, const int64_t *t, const double *g, int64_t b, int64_t c, double *o, int64_t *bad) { return fth_dev_cross_entropy_backward_f64(l, t, g, b, c, o, bad, nullptr); }
     static int32_t layer_norm(const double *x, const double *w, const double *b, double *y, int64_t n, int64_t c, double e) { return fth_dev_layer_norm_f64(x, w, b, y, n, c, e, nullptr); }
     static int32_t rms_norm(const double *x, const double *w, double *y, int64_t n, int64_t c, double e) { return fth_dev_rms_norm_f64(x, w, y, n, c, e, nullptr); }
     static int32_t gelu(const double *x, double *y, int64_t n) { return fth_dev_gelu_f64(x, y, n, nullptr); }
@@ -420,7 +426,7 @@ int32_t ensure_unary(size_t len, const fth_meta *m) {
 // softmax_dim_tensor_contiguous (crates/ft-kernel-cpu/src/lib.rs:39193-39296 / 18350-18461)
 template <typename T>
 int32_t softmax_impl(const T *input, size_t input_len, const fth_meta *meta, size_t dim, T *out, size_t out_cap,
-                     size_t *out_len) {
+                     size_t *out_len, bool log_form = false) {
     FTH_ARG(meta_ok(meta), "softmax: bad meta");
     if (out_len) *out_len = 0;
     if (int32_t rc = ensure_unary(input_len, meta)) return rc;
@@ -436,7 +442,10 @@ int32_t softmax_impl(const T *input, size_t input_len, const fth_meta *meta, siz
     T *dx, *dy;
     if (int32_t rc = stage_in(sc, input + meta->storage_offset, (size_t)numel, &dx)) return rc;
     if (int32_t rc = stage_out(sc, (size_t)numel, &dy)) return rc;
-    if (int32_t rc = Dev<T>::softmax(dx, dy, (int64_t)outer, (int64_t)meta->shape[dim], (int64_t)inner)) return rc;
+    // log_softmax_dim_tensor_contiguous (crates/ft-kernel-cpu/src/lib.rs:39298-39375 / 18504-18590) shares the validation
+    if (int32_t rc = log_form ? Dev<T>::log_softmax(dx, dy, (int64_t)outer, (int64_t)meta->shape[dim], (int64_t)inner)
+                              : Dev<T>::softmax(dx, dy, (int64_t)outer, (int64_t)meta->shape[dim], (int64_t)inner))
+        return rc;
     return fetch(out, dy, (size_t)numel);
 }
 
@@ -631,6 +640,35 @@ int32_t argmax_impl(const T *input, size_t input_len, const fth_meta *meta, size
     if (int32_t rc = stage_out(sc, (size_t)out_numel, &dy)) return rc;
     if (int32_t rc = Dev<T>::argmax(dx, (int64_t)outer, (int64_t)reduce, (int64_t)inner, dy)) return rc;
     return fetch(out, dy, (size_t)out_numel);
+}
+
+// cross_entropy_forward / _backward (crates/ft-kernel-cpu/src/lib.rs:6717-6781 / 6649-6712). `target` holds class
+// indices (the reference's &[usize]); an index >= classes makes the reference panic on the slice index and is
+// reported here as InvalidArgument naming the row.
+template <typename T>
+int32_t cross_entropy_impl(bool backward, const T *logits, size_t logits_len, const uint64_t *target, size_t target_len, const T *dloss,
+                           size_t dloss_len, size_t batch, size_t classes, T *out, size_t out_cap) {
+    uint64_t total;
+    FTH_ARG(checked_mul(batch, classes, &total), "cross_entropy: batch * classes overflows");
+    const size_t n_out = backward ? (size_t)total : batch;
+    if (int32_t rc = check_out(out, out_cap, n_out)) return rc;
+    FTH_ARG(logits_len >= total && target_len >= batch && (!backward || dloss_len >= batch), "cross_entropy: input slice shorter than its shape");
+    if (batch == 0) return FTH_OK;
+    for (size_t i = 0; i < batch; ++i)
+        FTH_ARG(target[i] < classes, "cross_entropy: target %llu of row %zu is outside [0, %zu)", (unsigned long long)target[i], i, classes);
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *dl = nullptr, *dg = nullptr, *dout = nullptr;
+    int64_t *dt = nullptr;
+    if (int32_t rc = stage_in(sc, logits, (size_t)total, &dl)) return rc;
+    if (int32_t rc = stage_in(sc, reinterpret_cast<const int64_t *>(target), batch, &dt)) return rc;
+    if (backward)
+        if (int32_t rc = stage_in(sc, dloss, batch, &dg)) return rc;
+    if (int32_t rc = stage_out(sc, n_out, &dout)) return rc;
+    if (int32_t rc = backward ? Dev<T>::ce_bwd(dl, dt, dg, (int64_t)batch, (int64_t)classes, dout, nullptr)
+                              : Dev<T>::ce_fwd(dl, dt, (int64_t)batch, (int64_t)classes, dout, nullptr))
+        return rc;
+    return fetch(out, dout, n_out);
 }
 
 // ---- backward entry points on host slices ----
@@ -924,6 +962,31 @@ int32_t fth_sdpa_backward_f64(const double *q, size_t q_len, const double *k, si
                               int32_t causal, double *dq, size_t dq_cap, double *dk, size_t dk_cap, double *dv, size_t dv_cap) {
     return sdpa_backward_impl<double>(q, q_len, k, k_len, v, v_len, dout, dout_len, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dq_cap,
                                       dk, dk_cap, dv, dv_cap);
+}
+
+int32_t fth_log_softmax_dim_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta, size_t dim, float *out,
+                                                  size_t out_cap, size_t *out_len) {
+    return softmax_impl<float>(input, input_len, meta, dim, out, out_cap, out_len, true);
+}
+int32_t fth_log_softmax_dim_tensor_contiguous_f64(const double *input, size_t input_len, const fth_meta *meta, size_t dim, double *out,
+                                                  size_t out_cap, size_t *out_len) {
+    return softmax_impl<double>(input, input_len, meta, dim, out, out_cap, out_len, true);
+}
+int32_t fth_cross_entropy_forward_f32(const float *logits, size_t logits_len, const uint64_t *target, size_t target_len, size_t batch,
+                                      size_t classes, float *loss, size_t loss_cap) {
+    return cross_entropy_impl<float>(false, logits, logits_len, target, target_len, nullptr, 0, batch, classes, loss, loss_cap);
+}
+int32_t fth_cross_entropy_forward_f64(const double *logits, size_t logits_len, const uint64_t *target, size_t target_len, size_t batch,
+                                      size_t classes, double *loss, size_t loss_cap) {
+    return cross_entropy_impl<double>(false, logits, logits_len, target, target_len, nullptr, 0, batch, classes, loss, loss_cap);
+}
+int32_t fth_cross_entropy_backward_f32(const float *logits, size_t logits_len, const uint64_t *target, size_t target_len, const float *dloss,
+                                       size_t dloss_len, size_t batch, size_t classes, float *dlogits, size_t dlogits_cap) {
+    return cross_entropy_impl<float>(true, logits, logits_len, target, target_len, dloss, dloss_len, batch, classes, dlogits, dlogits_cap);
+}
+int32_t fth_cross_entropy_backward_f64(const double *logits, size_t logits_len, const uint64_t *target, size_t target_len, const double *dloss,
+                                       size_t dloss_len, size_t batch, size_t classes, double *dlogits, size_t dlogits_cap) {
+    return cross_entropy_impl<double>(true, logits, logits_len, target, target_len, dloss, dloss_len, batch, classes, dlogits, dlogits_cap);
 }
 
 }  // extern "C"

@@ -133,6 +133,21 @@ def softmax_strided(x, y, outer, reduce, inner, stream=None):
     check(getattr(_lib.load(), "fth_dev_softmax_strided_" + _sfx(x))(_ptr(x), _ptr(y), outer, reduce, inner, stream))
 
 
+def log_softmax_strided(x, y, outer, reduce, inner, stream=None):
+    check(getattr(_lib.load(), "fth_dev_log_softmax_strided_" + _sfx(x))(_ptr(x), _ptr(y), outer, reduce, inner, stream))
+
+
+def cross_entropy_forward(logits, target, batch, classes, loss, bad_index=None, stream=None):
+    """loss[i] = lse(logits[i]) - logits[i][target[i]]; target is an int64 tensor of class indices."""
+    check(getattr(_lib.load(), "fth_dev_cross_entropy_forward_" + _sfx(logits))(_ptr(logits), _ptr(target), batch, classes,
+                                                                                _ptr(loss), _ptr(bad_index), stream))
+
+
+def cross_entropy_backward(logits, target, dloss, batch, classes, dlogits, bad_index=None, stream=None):
+    check(getattr(_lib.load(), "fth_dev_cross_entropy_backward_" + _sfx(logits))(_ptr(logits), _ptr(target), _ptr(dloss), batch,
+                                                                                 classes, _ptr(dlogits), _ptr(bad_index), stream))
+
+
 def layer_norm(x, weight, bias, y, batch, norm_size, eps, stream=None):
     check(getattr(_lib.load(), "fth_dev_layer_norm_" + _sfx(x))(_ptr(x), _ptr(weight), _ptr(bias), _ptr(y), batch,
                                                                 norm_size, _real(x, eps), stream))

@@ -134,6 +134,50 @@ def softmax_dim_tensor_contiguous_f64(inp, meta, dim):
     return _unary_dim("fth_softmax_dim_tensor_contiguous_f64", np.float64, inp, meta, dim)
 
 
+def log_softmax_dim_tensor_contiguous_f32(inp, meta, dim):
+    """crates/ft-kernel-cpu/src/lib.rs:39298."""
+    return _unary_dim("fth_log_softmax_dim_tensor_contiguous_f32", np.float32, inp, meta, dim)
+
+
+def log_softmax_dim_tensor_contiguous_f64(inp, meta, dim):
+    """crates/ft-kernel-cpu/src/lib.rs:18504."""
+    return _unary_dim("fth_log_softmax_dim_tensor_contiguous_f64", np.float64, inp, meta, dim)
+
+
+def _cross_entropy(sfx, dtype, logits, target, dloss, batch, classes):
+    logits = _slice(logits, dtype)
+    target = np.ascontiguousarray(target, dtype=np.uint64).reshape(-1)
+    fn = getattr(_lib.load(), "fth_cross_entropy_%s_%s" % ("forward" if dloss is None else "backward", sfx))
+    if dloss is None:
+        out = np.empty(batch, dtype=dtype)
+        check(fn(_p(logits), logits.size, _p(target), target.size, batch, classes, _p(out), out.size))
+    else:
+        dloss = _slice(dloss, dtype)
+        out = np.empty(batch * classes, dtype=dtype)
+        check(fn(_p(logits), logits.size, _p(target), target.size, _p(dloss), dloss.size, batch, classes, _p(out), out.size))
+    return out
+
+
+def cross_entropy_forward_f32(logits, target, batch, classes):
+    """Per-row loss, crates/ft-kernel-cpu/src/lib.rs:6717."""
+    return _cross_entropy("f32", np.float32, logits, target, None, batch, classes)
+
+
+def cross_entropy_forward_f64(logits, target, batch, classes):
+    """crates/ft-kernel-cpu/src/lib.rs:6649."""
+    return _cross_entropy("f64", np.float64, logits, target, None, batch, classes)
+
+
+def cross_entropy_backward_f32(logits, target, dloss, batch, classes):
+    """dlogits, crates/ft-kernel-cpu/src/lib.rs:6745."""
+    return _cross_entropy("f32", np.float32, logits, target, dloss, batch, classes)
+
+
+def cross_entropy_backward_f64(logits, target, dloss, batch, classes):
+    """crates/ft-kernel-cpu/src/lib.rs:6679."""
+    return _cross_entropy("f64", np.float64, logits, target, dloss, batch, classes)
+
+
 def argmax_dim_tensor_contiguous_f32(inp, meta, dim):
     return _unary_dim("fth_argmax_dim_tensor_contiguous_f32", np.float32, inp, meta, dim)
 

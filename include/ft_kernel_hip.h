@@ -232,6 +232,23 @@ int32_t fth_dev_gemm_f32(const fth_gemm_desc *d, float alpha, const float *a, co
 int32_t fth_dev_gemm_f64(const fth_gemm_desc *d, double alpha, const double *a, const double *b, double *c,
                          const double *bias, const double *residual, fth_stream s);
 
+/* log-softmax over the middle dim of a contiguous [outer, reduce, inner] view (inner == 1: the last dim)
+ * (log_softmax_dim_tensor_contiguous_f32 / _f64, crates/ft-kernel-cpu/src/lib.rs:39298-39375, 18504-18590). */
+int32_t fth_dev_log_softmax_strided_f32(const float *x, float *y, int64_t outer, int64_t reduce, int64_t inner, fth_stream s);
+int32_t fth_dev_log_softmax_strided_f64(const double *x, double *y, int64_t outer, int64_t reduce, int64_t inner, fth_stream s);
+/* Fused softmax-cross-entropy over [batch, classes] logits with int64 class indices
+ * (cross_entropy_forward_f32 / _f64 :6717-6738, 6649-6671; cross_entropy_backward_f32 / _f64 :6745-6781, 6679-6712):
+ * loss[i] = lse(logits[i]) - logits[i][target[i]]; dlogits[i][c] = dloss[i] * (softmax(logits[i])[c] - [c == target[i]]).
+ * bad_index (may be NULL) receives the lowest row whose target is outside [0, classes), or -1; such rows are not written. */
+int32_t fth_dev_cross_entropy_forward_f32(const float *logits, const int64_t *target, int64_t batch, int64_t classes, float *loss,
+                                          int64_t *bad_index, fth_stream s);
+int32_t fth_dev_cross_entropy_forward_f64(const double *logits, const int64_t *target, int64_t batch, int64_t classes, double *loss,
+                                          int64_t *bad_index, fth_stream s);
+int32_t fth_dev_cross_entropy_backward_f32(const float *logits, const int64_t *target, const float *dloss, int64_t batch, int64_t classes,
+                                           float *dlogits, int64_t *bad_index, fth_stream s);
+int32_t fth_dev_cross_entropy_backward_f64(const double *logits, const int64_t *target, const double *dloss, int64_t batch, int64_t classes,
+                                           double *dlogits, int64_t *bad_index, fth_stream s);
+
 /* ---- backward kernels of the same ops (device pointers; caller-provided workspace) ----
  * Each entry point needs scratch memory for its fixed-order partial sums (and, for SDPA, for the
  * probability and score-gradient matrices the reference materialises per head): ask the matching
@@ -362,6 +379,21 @@ int32_t fth_rms_norm_forward_f32(const float *x, size_t x_len, const float *weig
                                  size_t norm_size, float eps, float *out, size_t out_cap);
 int32_t fth_rms_norm_forward_f64(const double *x, size_t x_len, const double *weight, size_t batch,
                                  size_t norm_size, double eps, double *out, size_t out_cap);
+/* log_softmax_dim_tensor_contiguous_f32 (:39298) / _f64 (:18504): the validation of softmax_dim_tensor_contiguous.
+ * cross_entropy_forward_f32 (:6717) / _f64 (:6649) -> loss [batch]; cross_entropy_backward_f32 (:6745) / _f64 (:6679)
+ * -> dlogits [batch*classes]. target holds class indices (the reference's &[usize]). */
+int32_t fth_log_softmax_dim_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta, size_t dim, float *out,
+                                                  size_t out_cap, size_t *out_len);
+int32_t fth_log_softmax_dim_tensor_contiguous_f64(const double *input, size_t input_len, const fth_meta *meta, size_t dim, double *out,
+                                                  size_t out_cap, size_t *out_len);
+int32_t fth_cross_entropy_forward_f32(const float *logits, size_t logits_len, const uint64_t *target, size_t target_len, size_t batch,
+                                      size_t classes, float *loss, size_t loss_cap);
+int32_t fth_cross_entropy_forward_f64(const double *logits, size_t logits_len, const uint64_t *target, size_t target_len, size_t batch,
+                                      size_t classes, double *loss, size_t loss_cap);
+int32_t fth_cross_entropy_backward_f32(const float *logits, size_t logits_len, const uint64_t *target, size_t target_len, const float *dloss,
+                                       size_t dloss_len, size_t batch, size_t classes, float *dlogits, size_t dlogits_cap);
+int32_t fth_cross_entropy_backward_f64(const double *logits, size_t logits_len, const uint64_t *target, size_t target_len, const double *dloss,
+                                       size_t dloss_len, size_t batch, size_t classes, double *dlogits, size_t dlogits_cap);
 /* Backward of the fused ops on host slices. Every output has its own capacity (in elements) and must hold its result:
  * layer_norm_backward_f32 (:6189) / _f64 (:6052) -> dx [batch*norm_size], dweight, dbias [norm_size];
  * rms_norm_backward_f32 (:6574) / _f64 (:6503) -> dx, dweight (weight == NULL: no dweight, pass NULL / 0);

@@ -15,7 +15,9 @@
 //     attention + brute force), permute;
 //     layer_norm / rms_norm / linear / sdpa backward: central differences of the pinned forward
 //     functions in f64, the reference's own test inputs (KC:43862-43911, 64200-64360) and the
-//     identities those tests assert (unit-dy shortcut, dbias = column sums).
+//     identities those tests assert (unit-dy shortcut, dbias = column sums);
+//     log_softmax: the reference's conformance fixtures (1e-10) and log(softmax); cross-entropy forward /
+//     backward: -log_softmax[target], central differences, rows of the gradient summing to zero.
 //   third-party arithmetic that is NOT in the reference tree:
 //     * GEMM: `matrixmultiply 0.3.11` (Cargo.lock:1420-1423; call sites KC:1645, KC:1673). Its
 //       f32 accumulation order is unspecified and the reference's own test shows it is not the
@@ -473,6 +475,73 @@ __attribute__((target("avx2,fma"))) void sgemm_blocked_avx2(int64_t m, int64_t n
 
 }  // namespace
 
+// log_softmax_dim_tensor_contiguous_f32 (KC:39298-39375), _f64 (KC:18504-18590): per lane,
+// max = fold(-inf, max); sum_exp = pairwise_sum(exp(x - max)); out = (x - max) - ln(sum_exp).
+inline float t_log(float x) { return logf(x); }
+inline double t_log(double x) { return log(x); }
+template <typename T> void log_softmax_impl(const T *x, T *y, int64_t outer, int64_t reduce, int64_t inner) {
+    if (outer <= 0 || reduce <= 0 || inner <= 0) return;
+#pragma omp parallel
+    {
+        std::vector<T> scratch((size_t)reduce), ex((size_t)reduce);
+#pragma omp for schedule(static) collapse(2)
+        for (int64_t o = 0; o < outer; ++o) {
+            for (int64_t c = 0; c < inner; ++c) {
+                const T *in = x + o * reduce * inner + c;
+                T *out = y + o * reduce * inner + c;
+                for (int64_t r = 0; r < reduce; ++r) scratch[r] = in[r * inner];
+                T m = -std::numeric_limits<T>::infinity();
+                for (int64_t r = 0; r < reduce; ++r) m = max_num(m, scratch[r]);
+                for (int64_t r = 0; r < reduce; ++r) ex[r] = t_exp(scratch[r] - m);
+                const T lse = t_log(pairwise_sum(ex.data(), (size_t)reduce));
+                for (int64_t r = 0; r < reduce; ++r) out[r * inner] = (scratch[r] - m) - lse;
+            }
+        }
+    }
+}
+
+// cross_entropy_forward_f32 / _f64 (KC:6717-6738, 6649-6671): strict `>` max scan, sequential sum of
+// exp(v - m), lse = m + ln(s), loss = lse - row[target]. Returns the first row with an invalid target, or -1.
+template <typename T> int64_t cross_entropy_forward_impl(const T *logits, const int64_t *target, int64_t batch, int64_t classes, T *loss) {
+    int64_t bad = -1;
+    for (int64_t i = 0; i < batch; ++i)
+        if (target[i] < 0 || target[i] >= classes) {
+            bad = i;
+            break;
+        }
+    if (bad >= 0) return bad;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < batch; ++i) {
+        const T *row = logits + i * classes;
+        T m = -std::numeric_limits<T>::infinity();
+        for (int64_t c = 0; c < classes; ++c)
+            if (row[c] > m) m = row[c];
+        T s = 0;
+        for (int64_t c = 0; c < classes; ++c) s += t_exp(row[c] - m);
+        loss[i] = (m + t_log(s)) - row[target[i]];
+    }
+    return -1;
+}
+
+// cross_entropy_backward_f32 / _f64 (KC:6745-6781, 6679-6712): dlogits[i][c] = dloss[i] * (exp(row[c] - lse) - [c == target[i]]).
+template <typename T>
+int64_t cross_entropy_backward_impl(const T *logits, const int64_t *target, const T *dloss, int64_t batch, int64_t classes, T *dlogits) {
+    for (int64_t i = 0; i < batch; ++i)
+        if (target[i] < 0 || target[i] >= classes) return i;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < batch; ++i) {
+        const T *row = logits + i * classes;
+        T m = -std::numeric_limits<T>::infinity();
+        for (int64_t c = 0; c < classes; ++c)
+            if (row[c] > m) m = row[c];
+        T s = 0;
+        for (int64_t c = 0; c < classes; ++c) s += t_exp(row[c] - m);
+        const T lse = m + t_log(s), g = dloss[i];
+        for (int64_t c = 0; c < classes; ++c) dlogits[i * classes + c] = g * (t_exp(row[c] - lse) - (c == target[i] ? T(1) : T(0)));
+    }
+    return -1;
+}
+
 // ------------------------------------------------------------------------------------------
 // Backward kernels of the same ops (the rows the forward path widens into next).
 
@@ -632,6 +701,27 @@ void sdpa_backward_impl(const T *q, const T *k, const T *v, const T *dout, int64
 }
 
 extern "C" {
+
+void fto_log_softmax_f32(const float *x, float *y, int64_t outer, int64_t reduce, int64_t inner) {
+    log_softmax_impl<float>(x, y, outer, reduce, inner);
+}
+void fto_log_softmax_f64(const double *x, double *y, int64_t outer, int64_t reduce, int64_t inner) {
+    log_softmax_impl<double>(x, y, outer, reduce, inner);
+}
+int64_t fto_cross_entropy_forward_f32(const float *logits, const int64_t *target, int64_t batch, int64_t classes, float *loss) {
+    return cross_entropy_forward_impl<float>(logits, target, batch, classes, loss);
+}
+int64_t fto_cross_entropy_forward_f64(const double *logits, const int64_t *target, int64_t batch, int64_t classes, double *loss) {
+    return cross_entropy_forward_impl<double>(logits, target, batch, classes, loss);
+}
+int64_t fto_cross_entropy_backward_f32(const float *logits, const int64_t *target, const float *dloss, int64_t batch, int64_t classes,
+                                       float *dlogits) {
+    return cross_entropy_backward_impl<float>(logits, target, dloss, batch, classes, dlogits);
+}
+int64_t fto_cross_entropy_backward_f64(const double *logits, const int64_t *target, const double *dloss, int64_t batch, int64_t classes,
+                                       double *dlogits) {
+    return cross_entropy_backward_impl<double>(logits, target, dloss, batch, classes, dlogits);
+}
 
 void fto_layer_norm_backward_f32(const float *dy, const float *x, const float *w, int64_t batch, int64_t n, float eps,
                                  float *dx, float *dw, float *db) {

@@ -204,6 +204,46 @@ def sdpa_forward(q, k, v, scale, causal):
     return out
 
 
+def log_softmax(x, dim: int = -1):
+    x = _c(x)
+    sfx, _ = _sfx(x.dtype)
+    dim = dim % x.ndim
+    outer = int(np.prod(x.shape[:dim], dtype=np.int64))
+    inner = int(np.prod(x.shape[dim + 1:], dtype=np.int64))
+    y = np.empty_like(x)
+    getattr(lib(), "fto_log_softmax_" + sfx)(_p(x), _p(y), _i64(outer), _i64(x.shape[dim]), _i64(inner))
+    return y
+
+
+def cross_entropy_forward(logits, target):
+    """Per-row loss lse(logits) - logits[target]; raises IndexError on a target outside [0, classes)."""
+    logits = _c(logits)
+    sfx, _ = _sfx(logits.dtype)
+    batch, classes = logits.shape
+    t = _c(np.asarray(target, dtype=np.int64))
+    loss = np.empty(batch, logits.dtype)
+    fn = getattr(lib(), "fto_cross_entropy_forward_" + sfx)
+    fn.restype = C.c_int64
+    bad = fn(_p(logits), _p(t), _i64(batch), _i64(classes), _p(loss))
+    if bad >= 0:
+        raise IndexError("target of row %d is out of range" % bad)
+    return loss
+
+
+def cross_entropy_backward(logits, target, dloss):
+    logits, dloss = _c(logits), _c(dloss)
+    sfx, _ = _sfx(logits.dtype)
+    batch, classes = logits.shape
+    t = _c(np.asarray(target, dtype=np.int64))
+    out = np.empty_like(logits)
+    fn = getattr(lib(), "fto_cross_entropy_backward_" + sfx)
+    fn.restype = C.c_int64
+    bad = fn(_p(logits), _p(t), _p(dloss), _i64(batch), _i64(classes), _p(out))
+    if bad >= 0:
+        raise IndexError("target of row %d is out of range" % bad)
+    return out
+
+
 def layer_norm_backward(dy, x, weight, eps):
     """Returns (dx, dweight, dbias) for y = layer_norm(x) * weight + bias over the last dim."""
     dy, x, weight = _c(dy), _c(x), _c(weight)

@@ -32,6 +32,9 @@ def test_conformance_fixtures(hip, vectors):
             elif c["op"] == "softmax":
                 fn = K.softmax_dim_tensor_contiguous_f64 if dt == np.float64 else K.softmax_dim_tensor_contiguous_f32
                 got = fn(_f(c["input"]), _m(c["shape"], dt), c["dim"])
+            elif c["op"] == "log_softmax":
+                fn = K.log_softmax_dim_tensor_contiguous_f64 if dt == np.float64 else K.log_softmax_dim_tensor_contiguous_f32
+                got = fn(_f(c["input"]), _m(c["shape"], dt), c["dim"])
             elif c["op"] == "add":
                 fn = K.add_tensor_contiguous_f64 if dt == np.float64 else K.add_tensor_contiguous_f32
                 got = fn(_f(c["lhs"]), _f(c["rhs"]), _m(c["shape"], dt), _m(c["shape"], dt))
@@ -41,6 +44,8 @@ def test_conformance_fixtures(hip, vectors):
             elif c["op"] == "index_select":
                 fn = K.index_select_tensor_contiguous_f64 if dt == np.float64 else K.index_select_tensor_contiguous_f32
                 got = fn(_f(c["input"]), _m(c["input_shape"], dt), c["dim"], _f(c["index"]))
+            else:
+                raise AssertionError("unhandled fixture op " + c["op"])
             assert got.dtype == dt and got.shape == exp.shape, c["name"]
             assert np.max(np.abs(got - exp)) <= tol + extra, (c["name"], dt)
 

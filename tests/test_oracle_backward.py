@@ -105,3 +105,36 @@ def test_sdpa_backward_is_the_gradient_of_the_forward(oracle, causal):
     f = np.float32
     dq32, dk32, dv32 = oracle.sdpa_backward(q.astype(f), k.astype(f), v.astype(f), dout.astype(f), f(scale), causal)
     assert np.allclose(dq32, dq, atol=2e-5) and np.allclose(dk32, dk_, atol=2e-5) and np.allclose(dv32, dv_, atol=2e-5)
+
+
+def test_log_softmax_reference_fixtures_and_identity(oracle, vectors):
+    cases = [c for c in vectors["conformance"] if c["op"] == "log_softmax"]
+    assert len(cases) == 2
+    for c in cases:
+        x = np.array(c["input"], np.float64).reshape(c["shape"])
+        got = oracle.log_softmax(x, c["dim"])
+        assert np.allclose(got.ravel(), c["expected_output"], rtol=0, atol=c["tolerance"])
+        assert np.allclose(oracle.log_softmax(x.astype(np.float32), c["dim"]).ravel(), c["expected_output"], atol=1e-6)
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((3, 7, 5)) * 4
+    for dim in (0, 1, 2):
+        assert np.allclose(oracle.log_softmax(x, dim), np.log(oracle.softmax(x, dim)), atol=1e-12)
+        assert np.allclose(np.exp(oracle.log_softmax(x, dim)).sum(dim), 1.0, atol=1e-12)
+
+
+def test_cross_entropy_is_minus_log_softmax_at_the_target_and_its_gradient(oracle):
+    rng = np.random.default_rng(10)
+    batch, classes = 6, 11
+    logits = rng.standard_normal((batch, classes)) * 3
+    target = rng.integers(0, classes, batch)
+    loss = oracle.cross_entropy_forward(logits, target)
+    assert np.allclose(loss, -oracle.log_softmax(logits, 1)[np.arange(batch), target], atol=1e-12)
+    dloss = rng.standard_normal(batch)
+    g = oracle.cross_entropy_backward(logits, target, dloss)
+    num = _num_grad(lambda t: oracle.cross_entropy_forward(t, target), logits.copy(), dloss)
+    assert np.allclose(g, num, atol=1e-7)
+    assert np.allclose(g.sum(1), 0, atol=1e-12)  # softmax sums to one, the one-hot too
+    l32 = oracle.cross_entropy_forward(logits.astype(np.float32), target)
+    assert np.allclose(l32, loss, atol=2e-6)
+    with pytest.raises(IndexError):
+        oracle.cross_entropy_forward(logits, np.full(batch, classes))

@@ -29,6 +29,8 @@ def test_conformance_fixtures(oracle, vectors):
             got = oracle.gelu(_f(c["input"]))
         elif c["op"] == "softmax":
             got = oracle.softmax(_f(c["input"]).reshape(c["shape"]), c["dim"]).ravel()
+        elif c["op"] == "log_softmax":
+            got = oracle.log_softmax(_f(c["input"]).reshape(c["shape"]), c["dim"]).ravel()
         elif c["op"] == "add":
             got = oracle.add(_f(c["lhs"]), _f(c["rhs"]))
         elif c["op"] == "matmul":
@@ -44,7 +46,7 @@ def test_conformance_fixtures(oracle, vectors):
         assert got.shape == exp.shape, c["name"]
         assert np.max(np.abs(got - exp)) <= tol, c["name"]
         seen.add(c["op"])
-    assert seen == {"gelu", "softmax", "add", "matmul", "index_select"}
+    assert seen == {"gelu", "softmax", "log_softmax", "add", "matmul", "index_select"}
 
 
 def test_in_source_known_answers(oracle, vectors):
