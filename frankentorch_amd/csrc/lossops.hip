@@ -5,11 +5,13 @@
 // cross_entropy_backward_f32 / _f64 (:6745-6781, 6679-6712).
 //
 // All three are HBM-bound row passes over [rows, classes] logits whose rows (50 257 floats for the
-// GPT-2 vocabulary) are neither a vector multiple nor aligned, so a 256-thread workgroup owns one
-// row and streams it with coalesced scalar loads; the second and third sweeps of a row hit L2.
-// Reductions are a fixed butterfly per wavefront and a fixed fold across the four wavefronts
-// (the reference scans a row sequentially; same values re-associated, inside the parity
-// tolerance), so results are bitwise repeatable. Class indices arrive as int64; an index outside
+// GPT-2 vocabulary) are neither a vector multiple nor aligned, so a workgroup owns one row and
+// moves it with coalesced dword accesses. Rows of up to 65 536 floats (32 768 doubles) are held in
+// registers across the max, sum and output steps (64, 256 or 1024 lanes by row length): the row is
+// read from HBM once and written once. Longer rows take the streaming kernels, which sweep the row
+// three times. Reductions are a fixed per-lane order, a fixed butterfly per wavefront and a fixed
+// fold across the wavefronts (the reference scans a row sequentially; same values re-associated,
+// inside the parity tolerance), so results are bitwise repeatable. Class indices arrive as int64; an index outside
 // [0, classes) (the reference would panic on the slice index) is reported through `bad_index` as
 // the lowest offending row, and that row's outputs are left unwritten.
 
@@ -37,17 +39,18 @@ template <typename T> __device__ __forceinline__ T max_num(T a, T b) {
 // the strict `>` scan of the cross-entropy kernels: a NaN never replaces the running maximum
 template <typename T> __device__ __forceinline__ T max_gt(T a, T b) { return b > a ? b : a; }
 
-template <typename T, class F> __device__ __forceinline__ T block_reduce(T v, F f, T *red, int &phase) {
+template <typename T, class F, int WAVES = kWaves> __device__ __forceinline__ T block_reduce(T v, F f, T *red, int &phase) {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) v = f(v, __shfl_xor(v, off, kWave));
-    T *buf = red + phase * kWaves;  // alternate halves: one barrier per reduction is enough
+    if (WAVES == 1) return v;
+    T *buf = red + phase * WAVES;  // alternate halves: one barrier per reduction is enough
     phase ^= 1;
     if (lane == 0) buf[wave] = v;
     __syncthreads();
     T s = buf[0];
 #pragma unroll
-    for (int w = 1; w < kWaves; ++w) s = f(s, buf[w]);
+    for (int w = 1; w < WAVES; ++w) s = f(s, buf[w]);
     return s;
 }
 struct SumOp {
@@ -146,6 +149,178 @@ __global__ __launch_bounds__(kThreads) void cross_entropy_backward_kernel(const 
     for (int64_t c = threadIdx.x; c < classes; c += kThreads) drow[c] = g * (t_exp<T>(row[c] - lse) - (c == t ? T(1) : T(0)));
 }
 
+// Keeps a workgroup-uniform pointer in scalar registers and stops the compiler from folding what is added to it
+// later into a per-lane offset.
+template <typename P> __device__ __forceinline__ P *uniform_ptr(P *p) {
+    asm volatile("" : "+s"(p));
+    return p;
+}
+
+// One row per workgroup, held in registers: lane t owns elements t, t + THREADS, ... (VPT of them).
+// MODE 0: log-softmax (max that skips NaN); 1: cross-entropy loss; 2: cross-entropy dlogits (strict `>` max).
+enum { kLogSoftmax = 0, kLossForward = 1, kLossBackward = 2 };
+
+// `lds_steps` further steps of the row (after the VPT register steps) live in dynamic LDS, filled by direct-to-LDS
+// loads: with 19 steps (76 KiB) there and at most 64 registers per lane, two 1024-lane workgroups share a compute unit
+// and one's loads overlap the other's arithmetic and stores. Each lane reads back only the LDS words its own loads
+// wrote, so a wait for the loads is enough and no barrier is needed. MINW: minimum wavefronts per SIMD (sets the
+// register budget).
+template <typename T, int VPT, int THREADS, int MODE, int MINW>
+__global__ __launch_bounds__(THREADS, MINW) void resident_rows_kernel(const T *__restrict__ x, const int64_t *__restrict__ target,
+                                                                     const T *__restrict__ dloss, int64_t cols, T *__restrict__ out,
+                                                                     int64_t *bad_index, int lds_steps) {
+    constexpr int WAVES = THREADS / kWave;
+    // Left free, the scheduler overlaps the exponentials of many elements and spills the row once the register budget
+    // is nearly all row data; there the per-element steps are kept in program order instead.
+    constexpr bool kPinOrder = THREADS == 1024 && VPT * (int)sizeof(T) * MINW > 384;
+    __shared__ T red[2 * WAVES];
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    T *lrow = reinterpret_cast<T *>(lds_raw) + threadIdx.x;  // this lane's word of LDS step 0
+    int phase = 0;
+    const int64_t i = blockIdx.x;
+    int64_t t = 0;
+    if (MODE != kLogSoftmax) {
+        t = target[i];
+        if (t < 0 || t >= cols) {  // uniform over the workgroup
+            note_bad(bad_index, i);
+            return;
+        }
+    }
+    const int tid = threadIdx.x;
+    // Lane slots are counted from the last 64-element boundary at or before the row's first output element (first
+    // input element for the loss, which writes no row), so every wavefront store covers whole, aligned 256-byte
+    // (fp64: 512-byte) pieces: rows of an odd length start at arbitrary element offsets, and partial-line
+    // writes from different wavefronts cost far more HBM time than they carry. Slot j holds element j - lead;
+    // slots below `lead` (only in step 0) and from `n` on are empty.
+    const T *row_out = (MODE == kLossForward ? x : out) + i * cols;
+    const int lead = (int)((reinterpret_cast<uintptr_t>(row_out) / sizeof(T)) % kWave);
+    const T *xr = x + i * cols - lead;   // slot 0 of the row
+    const int n = (int)cols + lead;      // one past the last occupied slot
+    const int n_lds = n - VPT * THREADS;  // occupied slots that live in LDS (<= 0: none)
+    if constexpr (sizeof(T) == 4) {
+        // oldest in the load queue, so the compiler's own counted waits for the register loads below stay exact
+        const unsigned wave = __builtin_amdgcn_readfirstlane((unsigned)(tid / kWave));
+        const unsigned wave_base = __builtin_amdgcn_readfirstlane((unsigned)reinterpret_cast<uintptr_t>(lds_raw)) + wave * (kWave * 4u);
+        const unsigned lane_off = (unsigned)(tid & (kWave - 1)) * 4u;
+        for (int k = 0; k < lds_steps; ++k) {
+            const T *pk = xr + (VPT + k) * THREADS + wave * kWave;  // scalar: the wavefront's 64 slots of step VPT + k
+            if (tid < n_lds - k * THREADS)
+                asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" ::"v"(lane_off), "s"(pk),
+                             "s"(wave_base + (unsigned)k * (THREADS * 4u))
+                             : "memory", "m0");
+        }
+    }
+    // Step k touches slots [k * THREADS, (k + 1) * THREADS): a scalar base per step plus the one per-lane offset
+    // `tid`, so no per-element address or bounds predicate stays live in a vector register between the passes.
+    T v[VPT];
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        const T *pk = uniform_ptr(xr + k * THREADS);
+        v[k] = (tid < n - k * THREADS && (k > 0 || tid >= lead)) ? pk[tid] : T(-__builtin_inf());
+    }
+    T m = T(-__builtin_inf());
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) m = MODE == kLogSoftmax ? max_num(m, v[k]) : max_gt(m, v[k]);  // the padding never wins
+    if (lds_steps > 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    for (int k = 0; k < lds_steps; ++k)
+        if (tid < n_lds - k * THREADS) m = MODE == kLogSoftmax ? max_num(m, lrow[k * THREADS]) : max_gt(m, lrow[k * THREADS]);
+    if (MODE == kLogSoftmax)
+        m = block_reduce<T, MaxNumOp, WAVES>(m, MaxNumOp{}, red, phase);
+    else
+        m = block_reduce<T, MaxGtOp, WAVES>(m, MaxGtOp{}, red, phase);
+    // The -inf padding adds exp(-inf - m) = +0 for a finite or +inf maximum and NaN for a -inf one, where the sum of
+    // the real elements is NaN already, so the sum over the registers needs no bounds test.
+    T s = T(0);
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        s += t_exp<T>(v[k] - m);
+        if (kPinOrder) __builtin_amdgcn_sched_barrier(0);
+    }
+    for (int k = 0; k < lds_steps; ++k)
+        if (tid < n_lds - k * THREADS) s += t_exp<T>(lrow[k * THREADS] - m);
+    s = block_reduce<T, SumOp, WAVES>(s, SumOp{}, red, phase);
+    if (MODE == kLogSoftmax) {
+        const T lse = t_log<T>(s);
+        T *yr = out + i * cols - lead;
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) {
+            T *pk = uniform_ptr(yr + k * THREADS);
+            if (tid < n - k * THREADS && (k > 0 || tid >= lead)) __builtin_nontemporal_store((v[k] - m) - lse, pk + tid);
+            if (kPinOrder) __builtin_amdgcn_sched_barrier(0);
+        }
+        for (int k = 0; k < lds_steps; ++k)
+            if (tid < n_lds - k * THREADS) __builtin_nontemporal_store((lrow[k * THREADS] - m) - lse, yr + (VPT + k) * THREADS + tid);
+    } else if (MODE == kLossForward) {
+        if (tid == 0) out[i] = (m + t_log<T>(s)) - x[i * cols + t];
+    } else {
+        const T lse = m + t_log<T>(s), g = dloss[i];
+        T *dr = out + i * cols - lead;
+        const int tt = (int)t + lead;  // the target's slot
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) {
+            T *pk = uniform_ptr(dr + k * THREADS);
+            if (tid < n - k * THREADS && (k > 0 || tid >= lead))
+                __builtin_nontemporal_store(g * (t_exp<T>(v[k] - lse) - (tid == tt - k * THREADS ? T(1) : T(0))), pk + tid);
+            if (kPinOrder) __builtin_amdgcn_sched_barrier(0);
+        }
+        for (int k = 0; k < lds_steps; ++k)
+            if (tid < n_lds - k * THREADS)
+                __builtin_nontemporal_store(g * (t_exp<T>(lrow[k * THREADS] - lse) - (tid == tt - (VPT + k) * THREADS ? T(1) : T(0))),
+                                            dr + (VPT + k) * THREADS + tid);
+    }
+}
+
+// Launches the register-resident kernel if the row fits; returns false if it does not (the caller streams).
+template <typename T, int MODE>
+bool launch_resident(const T *x, const int64_t *target, const T *dloss, int64_t rows, int64_t cols, T *out, int64_t *bad_index,
+                     hipStream_t st) {
+    constexpr int kMaxVpt = sizeof(T) == 4 ? 64 : 32;
+    const int64_t slots = cols + (kWave - 1);  // the row plus the longest alignment lead
+    if (slots > 1024LL * kMaxVpt) return false;
+    const int64_t steps = fth::ceil_div(slots, (int64_t)1024);
+    if constexpr (sizeof(T) == 4) {
+        // fp32 rows of 25..51 steps of 1024: up to 19 steps in LDS, the rest (8..32 steps) in registers, two workgroups
+        // per compute unit. Longer rows keep the whole row in registers at one workgroup per compute unit.
+        constexpr int64_t kLdsSteps = 19;
+        if (steps > 24 && steps <= 32 + kLdsSteps) {
+            const int64_t need = steps - kLdsSteps;
+#define FTH_HYBRID(VPT)                                                                                                         \
+    if (need <= (VPT)) {                                                                                                       \
+        const int lds_steps = (int)(steps - (VPT));                                                                            \
+        resident_rows_kernel<T, VPT, 1024, MODE, 8><<<dim3((unsigned)rows), dim3(1024), (size_t)lds_steps * 4096, st>>>(       \
+            x, target, dloss, cols, out, bad_index, lds_steps);                                                                \
+        return true;                                                                                                           \
+    }
+            FTH_HYBRID(8)
+            FTH_HYBRID(16)
+            FTH_HYBRID(24)
+            FTH_HYBRID(32)
+#undef FTH_HYBRID
+        }
+    }
+#define FTH_RESIDENT(THREADS, VPT)                                                                                                  \
+    if (slots <= (int64_t)(THREADS) * (VPT)) {                                                                                     \
+        if constexpr ((VPT) <= kMaxVpt)                                                                                            \
+            resident_rows_kernel<T, VPT, THREADS, MODE, 1><<<dim3((unsigned)rows), dim3(THREADS), 0, st>>>(x, target, dloss, cols, \
+                                                                                                            out, bad_index, 0);    \
+        return true;                                                                                                               \
+    }
+    FTH_RESIDENT(64, 4)
+    FTH_RESIDENT(64, 16)
+    FTH_RESIDENT(256, 8)
+    FTH_RESIDENT(256, 16)
+    FTH_RESIDENT(256, 32)
+    FTH_RESIDENT(1024, 16)
+    FTH_RESIDENT(1024, 24)
+    FTH_RESIDENT(1024, 32)
+    FTH_RESIDENT(1024, 40)
+    FTH_RESIDENT(1024, 48)
+    FTH_RESIDENT(1024, 56)
+    FTH_RESIDENT(1024, 64)
+#undef FTH_RESIDENT
+    return false;
+}
+
 __global__ void set_bad_index_kernel(int64_t *bad_index) { *bad_index = 0x7FFFFFFFFFFFFFFFLL; }
 __global__ void finish_bad_index_kernel(int64_t *bad_index) {
     if (*bad_index == 0x7FFFFFFFFFFFFFFFLL) *bad_index = -1;
@@ -159,7 +334,8 @@ template <typename T> int32_t log_softmax_entry(const T *x, T *y, int64_t outer,
     hipStream_t st = fth::resolve_stream(s);
     if (inner == 1) {
         FTH_ARG(outer <= 2147483647LL, "log_softmax: too many rows for one launch");
-        log_softmax_rows_kernel<T><<<dim3((unsigned)outer), dim3(kThreads), 0, st>>>(x, y, reduce);
+        if (!launch_resident<T, kLogSoftmax>(x, nullptr, nullptr, outer, reduce, y, nullptr, st))
+            log_softmax_rows_kernel<T><<<dim3((unsigned)outer), dim3(kThreads), 0, st>>>(x, y, reduce);
     } else {
         int64_t lanes;
         FTH_ARG(!__builtin_mul_overflow(outer, inner, &lanes) && fth::ceil_div(lanes, kThreads) <= 2147483647LL,
@@ -183,10 +359,13 @@ int32_t cross_entropy_entry(bool backward, const T *logits, const int64_t *targe
     if (batch > 0) {
         FTH_ARG(logits && target && out && (!backward || dloss), "cross_entropy: NULL operand");
         FTH_ARG(batch <= 2147483647LL, "cross_entropy: too many rows for one launch");
-        if (backward)
-            cross_entropy_backward_kernel<T><<<dim3((unsigned)batch), dim3(kThreads), 0, st>>>(logits, target, dloss, classes, out, bad_index);
-        else
-            cross_entropy_forward_kernel<T><<<dim3((unsigned)batch), dim3(kThreads), 0, st>>>(logits, target, classes, out, bad_index);
+        if (backward) {
+            if (!launch_resident<T, kLossBackward>(logits, target, dloss, batch, classes, out, bad_index, st))
+                cross_entropy_backward_kernel<T><<<dim3((unsigned)batch), dim3(kThreads), 0, st>>>(logits, target, dloss, classes, out, bad_index);
+        } else {
+            if (!launch_resident<T, kLossForward>(logits, target, nullptr, batch, classes, out, bad_index, st))
+                cross_entropy_forward_kernel<T><<<dim3((unsigned)batch), dim3(kThreads), 0, st>>>(logits, target, classes, out, bad_index);
+        }
         FTH_CHECK_LAUNCH("cross_entropy");
     }
     if (bad_index) {

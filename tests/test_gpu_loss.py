@@ -12,8 +12,9 @@ from frankentorch_amd.device import DeviceBuffer
 
 pytestmark = pytest.mark.gpu
 
-# ragged, unaligned, shorter than a workgroup, one element, the GPT-2 vocabulary
-ROW_SHAPES = [(7, 5), (64, 256), (33, 1000), (3, 1), (1, 50257), (19, 50257), (130, 1026), (5, 4099)]
+# ragged, unaligned, shorter than a workgroup, one element, the GPT-2 vocabulary, the longest register-resident rows
+# (fp32 65536, fp64 32768) and rows beyond them (the streaming kernels)
+ROW_SHAPES = [(7, 5), (64, 256), (33, 1000), (3, 1), (1, 50257), (19, 50257), (130, 1026), (5, 4099), (6, 16384), (3, 32768), (2, 65536), (2, 70001)]
 
 
 def _tol(dtype):
