@@ -48,9 +48,17 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def event_time_ms(device, launch, iters):
+WARM_SECONDS = 0.05  # untimed launches before each timed region: the GPU's clocks take tens of ms of load to settle
+
+
+def event_time_ms(device, launch, iters, warm_s=WARM_SECONDS):
     """Average duration of `launch` over `iters` back-to-back launches, by HIP events recorded on
-    the stream the kernels run on (the library stream)."""
+    the stream the kernels run on (the library stream), after `warm_s` of untimed launches of the same call."""
+    t_end = time.perf_counter() + warm_s
+    while time.perf_counter() < t_end:
+        for _ in range(4):
+            launch()
+        device.synchronize()
     e0, e1 = device.Event(), device.Event()
     e0.record()
     for _ in range(iters):
@@ -257,6 +265,30 @@ def bench_sdpa(device, synth, steps, with_cpu):
         res["cpu"] = {"value": round(flop * nh / (B * H) / best / 1e12, 4), "unit": "TFLOP/s", "cores": O.threads(), "kind": "port",
                       "sample": "%d of the %d heads, best of %d" % (nh, B * H, reps)}
         log("[sdpa] cpu baseline %.4f TFLOP/s (causal count) on %d threads" % (res["cpu"]["value"], O.threads()))
+    del dq, dk, dv, do
+    # grouped-query attention with an additive mask: 32 query heads on 8 K/V heads, the same S and D, a dense soft
+    # mask (every key visible), so the two products run over the full [S, S] rectangle and every mask value is read
+    Bg, Hq, Hkv = 2, 32, 8
+    qg = synth.normal(3, "Qg", (Bg, Hq, S, D), 0.0, s)
+    kg, vg = (synth.normal(3, t, (Bg, Hkv, S, D), 0.0, s) for t in ("Kg", "Vg"))
+    mask = synth.normal(3, "mask", (S, S), 0.0, 0.5)
+    bq, bk, bv, bm = (DeviceBuffer.from_host(t) for t in (qg, kg, vg, mask))
+    bo = DeviceBuffer(qg.shape)
+    gdesc = device.sdpa_desc_gqa(Bg, Hq, Hkv, S, S, D, D, False)
+    gfn = lambda: device.sdpa_forward_masked(gdesc, s, bq, bk, bv, bm, 0, bo)
+    for _ in range(2):
+        gfn()
+    device.synchronize()
+    gms = event_time_ms(device, gfn, max(5, steps // 2))
+    gflop = Bg * Hq * 4 * D * S * S
+    gtf = gflop / (gms * 1e-3) / 1e12
+    log("[sdpa] masked GQA B2 Hq32 Hkv8 S2048 D128  %.3f ms  %.2f TFLOP/s  %.1f%% of MFMA peak" % (gms, gtf, 100 * gtf / FP32_MFMA_PEAK_TF))
+    res["masked_gqa"] = {"ms": round(gms, 4), "TFLOP/s": round(gtf, 2), "frac": round(gtf / FP32_MFMA_PEAK_TF, 4), "flop": gflop,
+                         "workload": "B2, 32 query heads on 8 K/V heads, S2048 D128 fp32, shared additive [S,S] mask, no hidden keys"}
+    if with_cpu:
+        best, reps = cpu_time(lambda: O.sdpa_forward_masked_gqa(qg[:1, :16], kg[:1, :4], vg[:1, :4], np.float32(s), mask), 4.0, min_reps=1)
+        res["masked_gqa"]["cpu"] = {"value": round(gflop * 16 / (Bg * Hq) / best / 1e12, 4), "unit": "TFLOP/s", "cores": O.threads(),
+                                    "kind": "port", "sample": "16 of the 64 query heads, best of %d" % reps}
     return res
 
 
@@ -439,8 +471,8 @@ def bench_gpt2(device, synth, steps):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--cases", default="all", help="comma list of: gemm,sdpa,block,gpt2,backward (row ops always run); 'none' for row ops only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()

@@ -66,7 +66,7 @@ class SdpaDesc(C.Structure):
             "v_batch_stride", "v_head_stride", "v_row_stride",
             "o_batch_stride", "o_head_stride", "o_row_stride",
         )
-    ] + [("causal", C.c_int32), ("reserved", C.c_int32)]
+    ] + [("causal", C.c_int32), ("kv_group", C.c_int32)]
 
 
 class LayerWeights(C.Structure):

@@ -173,6 +173,9 @@ template <> struct Dev<float> {
         return fth_dev_gemm_f32(d, al, a, b, c, bias, nullptr, nullptr);
     }
     static int32_t softmax(const float *x, float *y, int64_t o, int64_t r, int64_t i) { return fth_dev_softmax_strided_f32(x, y, o, r, i, nullptr); }
+    static int32_t sdpa_masked(const fth_sdpa_desc *d, float sc, const float *q, const float *k, const float *v, const float *m, int64_t ms, float *o) {
+        return fth_dev_sdpa_forward_masked_f32(d, sc, q, k, v, m, ms, o, nullptr);
+    }
     static int32_t log_softmax(const float *x, float *y, int64_t o, int64_t r, int64_t i) { return fth_dev_log_softmax_strided_f32(x, y, o, r, i, nullptr); }
     static int32_t ce_fwd(const float *l, const int64_t *t, int64_t b, int64_t c, float *o, int64_t *bad) { return fth_dev_cross_entropy_forward_f32(l, t, b, c, o, bad, nullptr); }
     static int32_t ce_bwd(const float *l, const int64_t *t, const float *g, int64_t b, int64_t c, float *o, int64_t *bad) { return fth_dev_cross_entropy_backward_f32(l, t, g, b, c, o, bad, nullptr); }
@@ -190,6 +193,9 @@ template <> struct Dev<double> {
         return fth_dev_gemm_f64(d, al, a, b, c, bias, nullptr, nullptr);
     }
     static int32_t softmax(const double *x, double *y, int64_t o, int64_t r, int64_t i) { return fth_dev_softmax_strided_f64(x, y, o, r, i, nullptr); }
+    static int32_t sdpa_masked(const fth_sdpa_desc *d, double sc, const double *q, const double *k, const double *v, const double *m, int64_t ms, double *o) {
+        return fth_dev_sdpa_forward_masked_f64(d, sc, q, k, v, m, ms, o, nullptr);
+    }
     static int32_t log_softmax(const double *x, double *y, int64_t o, int64_t r, int64_t i) { return fth_dev_log_softmax_strided_f64(x, y, o, r, i, nullptr); }
     static int32_t ce_fwd(const double *l, const int64_t *t, int64_t b, int64_t c, double *o, int64_t *bad) { return fth_dev_cross_entropy_forward_f64(l, t, b, c, o, bad, nullptr); }
     static int32_t ce_bwd(const double *l, const int64_t *t, const double *g, int64_t b, int64_t c, double *o, int64_t *bad) { return fth_dev_cross_entropy_backward_f64(l, t, g, b, c, o, bad, nullptr); }
@@ -570,6 +576,49 @@ int32_t sdpa_impl(const T *q, size_t q_len, const T *k, size_t k_len, const T *v
     fth_sdpa_desc d;
     fth_sdpa_desc_contiguous(&d, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k, (int64_t)d_v, causal ? 1 : 0);
     if (int32_t rc = Dev<T>::sdpa(&d, scale, dq, dk, dv, dout)) return rc;
+    return fetch(out, dout, (size_t)on);
+}
+
+// sdpa_forward_masked_gqa_f64 (crates/ft-kernel-cpu/src/lib.rs:4777-4850) and, with h_q == h_kv, sdpa_forward_masked_f64
+// (:4661-4741): q [batch, h_q, seq_q, d_k], k / v [batch, h_kv, seq_k, d], additive mask with mask_bh_stride 0 (shared
+// [seq_q, seq_k]) or seq_q * seq_k (one per batch * h_q). The reference indexes the mask slice and panics when it is
+// short; that is InvalidArgument here.
+template <typename T>
+int32_t sdpa_masked_impl(const T *q, size_t q_len, const T *k, size_t k_len, const T *v, size_t v_len, size_t batch, size_t h_q,
+                         size_t h_kv, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, T scale, const T *mask, size_t mask_len,
+                         size_t mask_bh_stride, T *out, size_t out_cap) {
+    FTH_ARG(h_kv > 0 && h_q % h_kv == 0, "sdpa_masked_gqa: h_kv (%zu) must divide h_q (%zu)", h_kv, h_q);
+    uint64_t num_bh, num_kv, qn, kn, vn, on, mn, t;
+    FTH_ARG(checked_mul(batch, h_q, &num_bh) && checked_mul(batch, h_kv, &num_kv) && checked_mul(num_bh, seq_q, &t) &&
+                checked_mul(t, d_k, &qn) && checked_mul(t, d_v, &on) && checked_mul(num_kv, seq_k, &t) && checked_mul(t, d_k, &kn) &&
+                checked_mul(t, d_v, &vn) && checked_mul(seq_q, seq_k, &mn),
+            "sdpa_masked: shape product overflows");
+    if (int32_t rc = check_out(out, out_cap, (size_t)on)) return rc;
+    if (on == 0) return FTH_OK;
+    FTH_ARG(q_len >= qn && k_len >= kn && v_len >= vn, "sdpa_masked: q/k/v slice shorter than its shape");
+    FTH_ARG(mask_bh_stride == 0 || mask_bh_stride >= mn, "sdpa_masked: mask_bh_stride %zu is neither 0 nor >= seq_q * seq_k", mask_bh_stride);
+    uint64_t mask_need;
+    FTH_ARG(checked_mul(num_bh - 1, mask_bh_stride, &mask_need) && !__builtin_add_overflow(mask_need, mn, &mask_need) && mask_len >= mask_need,
+            "sdpa_masked: mask slice (%zu) shorter than the %llu elements the shape reads", mask_len, (unsigned long long)mask_need);
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *dq, *dk, *dv, *dm = nullptr, *dout;
+    if (int32_t rc = stage_in(sc, q, (size_t)qn, &dq)) return rc;
+    if (int32_t rc = stage_in(sc, k, (size_t)kn, &dk)) return rc;
+    if (int32_t rc = stage_in(sc, v, (size_t)vn, &dv)) return rc;
+    if (mask_need > 0)
+        if (int32_t rc = stage_in(sc, mask, (size_t)mask_need, &dm)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)on, &dout)) return rc;
+    fth_sdpa_desc d;
+    fth_sdpa_desc_contiguous(&d, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k, (int64_t)d_v, 0);
+    d.heads = (int64_t)h_q;
+    d.kv_group = (int32_t)(h_q / h_kv);
+    FTH_ARG(h_q / h_kv <= 2147483647ull, "sdpa_masked_gqa: group too large");
+    d.q_batch_stride = (int64_t)(h_q * seq_q * d_k); d.q_head_stride = (int64_t)(seq_q * d_k);
+    d.k_batch_stride = (int64_t)(h_kv * seq_k * d_k); d.k_head_stride = (int64_t)(seq_k * d_k);
+    d.v_batch_stride = (int64_t)(h_kv * seq_k * d_v); d.v_head_stride = (int64_t)(seq_k * d_v);
+    d.o_batch_stride = (int64_t)(h_q * seq_q * d_v); d.o_head_stride = (int64_t)(seq_q * d_v);
+    if (int32_t rc = Dev<T>::sdpa_masked(&d, scale, dq, dk, dv, dm, (int64_t)mask_bh_stride, dout)) return rc;
     return fetch(out, dout, (size_t)on);
 }
 
@@ -987,6 +1036,27 @@ int32_t fth_cross_entropy_backward_f32(const float *logits, size_t logits_len, c
 int32_t fth_cross_entropy_backward_f64(const double *logits, size_t logits_len, const uint64_t *target, size_t target_len, const double *dloss,
                                        size_t dloss_len, size_t batch, size_t classes, double *dlogits, size_t dlogits_cap) {
     return cross_entropy_impl<double>(true, logits, logits_len, target, target_len, dloss, dloss_len, batch, classes, dlogits, dlogits_cap);
+}
+
+int32_t fth_sdpa_forward_masked_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len, size_t num_bh,
+                                    size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, float scale, const float *mask, size_t mask_len,
+                                    size_t mask_bh_stride, float *out, size_t out_cap) {
+    return sdpa_masked_impl<float>(q, q_len, k, k_len, v, v_len, num_bh, 1, 1, seq_q, seq_k, d_k, d_v, scale, mask, mask_len, mask_bh_stride, out, out_cap);
+}
+int32_t fth_sdpa_forward_masked_f64(const double *q, size_t q_len, const double *k, size_t k_len, const double *v, size_t v_len, size_t num_bh,
+                                    size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, double scale, const double *mask, size_t mask_len,
+                                    size_t mask_bh_stride, double *out, size_t out_cap) {
+    return sdpa_masked_impl<double>(q, q_len, k, k_len, v, v_len, num_bh, 1, 1, seq_q, seq_k, d_k, d_v, scale, mask, mask_len, mask_bh_stride, out, out_cap);
+}
+int32_t fth_sdpa_forward_masked_gqa_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len, size_t batch,
+                                        size_t h_q, size_t h_kv, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, float scale,
+                                        const float *mask, size_t mask_len, size_t mask_bh_stride, float *out, size_t out_cap) {
+    return sdpa_masked_impl<float>(q, q_len, k, k_len, v, v_len, batch, h_q, h_kv, seq_q, seq_k, d_k, d_v, scale, mask, mask_len, mask_bh_stride, out, out_cap);
+}
+int32_t fth_sdpa_forward_masked_gqa_f64(const double *q, size_t q_len, const double *k, size_t k_len, const double *v, size_t v_len, size_t batch,
+                                        size_t h_q, size_t h_kv, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, double scale,
+                                        const double *mask, size_t mask_len, size_t mask_bh_stride, double *out, size_t out_cap) {
+    return sdpa_masked_impl<double>(q, q_len, k, k_len, v, v_len, batch, h_q, h_kv, seq_q, seq_k, d_k, d_v, scale, mask, mask_len, mask_bh_stride, out, out_cap);
 }
 
 }  // extern "C"

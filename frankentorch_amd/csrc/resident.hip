@@ -267,7 +267,7 @@ struct Stack {
             a.q_head_stride = a.k_head_stride = a.v_head_stride = hd;
             a.q_row_stride = a.k_row_stride = a.v_row_stride = 3 * d;
             a.o_batch_stride = seq * d; a.o_head_stride = hd; a.o_row_stride = d;
-            a.causal = causal; a.reserved = 0;
+            a.causal = causal; a.kv_group = 0;
             if ((rc = fth_dev_sdpa_forward_f32(&a, scale, ws.qkv, ws.qkv + d, ws.qkv + 2 * d, ws.ctx, s))) return rc;
             g = linear_desc(T, d, d, FTH_EPI_BIAS | FTH_EPI_RESIDUAL);
             if ((rc = fth_dev_gemm_f32(&g, 1.f, ws.ctx, L.wo, ws.xa, L.bo, x, s))) return rc;
@@ -495,7 +495,7 @@ int32_t fth_batch_mha(fth_batch *b, const fth_tensor *q, const fth_tensor *k, co
     a.q_head_stride = a.k_head_stride = a.v_head_stride = hd;
     a.q_row_stride = a.k_row_stride = a.v_row_stride = d;
     a.o_batch_stride = sq * d; a.o_head_stride = hd; a.o_row_stride = d;
-    a.causal = causal ? 1 : 0; a.reserved = 0;
+    a.causal = causal ? 1 : 0; a.kv_group = 0;
     const float scale = (float)(1.0 / std::sqrt((double)hd));
     return finish_op(fth_dev_sdpa_forward_f32(&a, scale, q->data, k->data, v->data, t->data, nullptr), t, out);
 }

@@ -49,6 +49,10 @@ struct SdpaArgs {
     fth_sdpa_desc d;
     double scale;
     int q_blocks;
+    const void *mask;        // additive [seq_q, seq_k] rows (row pitch seq_k), or NULL
+    int64_t mask_bh_stride;  // 0: one mask for every (batch, head); else elements between consecutive bh
+    int64_t group;           // query heads per K/V head (grouped-query attention), >= 1
+    int mask_vec;            // mask rows can be read as aligned float4 (seq_k % 4 == 0, 16-byte aligned base and bh stride)
 };
 
 // exp(x - m) for x <= m as 2^((x - m) * log2 e) on the hardware exp2 unit: subtract, multiply,
@@ -90,7 +94,9 @@ __device__ __forceinline__ float f4_get(const float4 &v, int e) { return e == 0 
 // time over 64 banks); logical vector q of tile row r is therefore stored in slot q ^ (r & 15), the
 // permutation being applied on the global side by choosing which vector each lane fetches. Rows
 // past seq_k are clamped to the last row (their scores are masked, their weights are zero).
-template <int D, int NW, bool PAIR, int BC, bool DIRECT>
+// MASK: an additive mask row is read for every (query, key) score, mask[bh * mask_bh_stride + qi * seq_k + key]
+// (sdpa_forward_masked_f64, crates/ft-kernel-cpu/src/lib.rs:4661-4741): score * scale + mask, then the same softmax.
+template <int D, int NW, bool PAIR, int BC, bool DIRECT, bool MASK>
 __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p) {
     constexpr int kBC = BC;
     constexpr int KS = BC / 32;        // 32-key sub-tiles per tile
@@ -119,23 +125,26 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
     int64_t bh;
     int unit;
     {
-        // Units are issued heaviest first across ALL heads (unit index is the slow digit), and
-        // when the head count allows it a head always lands on the same XCD.
+        // Units are issued heaviest first across ALL heads (unit index is the slow digit), and when the head count
+        // allows it a K/V head, with every query head that reads it, always lands on the same XCD (one L2).
         const int64_t pid = blockIdx.x;
-        if (d.num_bh % kXcds == 0) {
+        const int64_t g = p.group, kv_heads = d.num_bh / g;
+        if (kv_heads % kXcds == 0) {
             const int64_t xcd = pid % kXcds, w = pid / kXcds, per = d.num_bh / kXcds;
             unit = (int)(w / per);
-            bh = (w % per) * kXcds + xcd;
+            const int64_t idx = w % per;
+            bh = ((idx / g) * kXcds + xcd) * g + idx % g;
         } else {
             unit = (int)(pid / d.num_bh);
             bh = pid % d.num_bh;
         }
     }
-    const int64_t b = bh / d.heads, h = bh % d.heads;
+    const int64_t b = bh / d.heads, h = bh % d.heads, hk = h / p.group;  // query head h reads K/V head h / group
     const float *Q = static_cast<const float *>(p.q) + b * d.q_batch_stride + h * d.q_head_stride;
-    const float *K = static_cast<const float *>(p.k) + b * d.k_batch_stride + h * d.k_head_stride;
-    const float *Vg = static_cast<const float *>(p.v) + b * d.v_batch_stride + h * d.v_head_stride;
+    const float *K = static_cast<const float *>(p.k) + b * d.k_batch_stride + hk * d.k_head_stride;
+    const float *Vg = static_cast<const float *>(p.v) + b * d.v_batch_stride + hk * d.v_head_stride;
     float *O = static_cast<float *>(p.out) + b * d.o_batch_stride + h * d.o_head_stride;
+    const float *Mk = MASK ? static_cast<const float *>(p.mask) + bh * p.mask_bh_stride : nullptr;
     const float scale = (float)p.scale;
     const float c2 = scale * 1.44269502162933349609375f;  // scale * log2(e)
 
@@ -246,6 +255,33 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
             if (kt + 1 < num_kt) issue_tile(kt + 1, buf ^ 1);
             // A wavefront whose every query precedes this tile's first key has nothing to add.
             const bool wave_active = !d.causal || key0 <= wave_last_q;
+            // ---- the tile's mask values, requested before the score MFMAs that hide their latency:
+            //      lane (query qi) element r of sub-tile j is key key0 + 32 j + 8 (r / 4) + 4 half + r % 4 ----
+            Acc16 mk[MASK ? KS : 1];
+            if constexpr (MASK) {
+                if (wave_active) {
+                    const float *mrow = Mk + (int64_t)(q_live ? qi : 0) * seq_k_i;
+#pragma unroll
+                    for (int j = 0; j < KS; ++j)
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            const int key = key0 + 32 * j + 8 * g + 4 * half;
+                            float4 mv = make_float4(0.f, 0.f, 0.f, 0.f);
+                            if (p.mask_vec) {  // seq_k % 4 == 0: a group of four keys never straddles the row end
+                                if (key < seq_k_i) mv = *reinterpret_cast<const float4 *>(mrow + key);
+                            } else {
+                                if (key + 0 < seq_k_i) mv.x = mrow[key + 0];
+                                if (key + 1 < seq_k_i) mv.y = mrow[key + 1];
+                                if (key + 2 < seq_k_i) mv.z = mrow[key + 2];
+                                if (key + 3 < seq_k_i) mv.w = mrow[key + 3];
+                            }
+                            mk[j][4 * g + 0] = mv.x;
+                            mk[j][4 * g + 1] = mv.y;
+                            mk[j][4 * g + 2] = mv.z;
+                            mk[j][4 * g + 3] = mv.w;
+                        }
+                }
+            }
             // ---- S^T = K_tile . Q^T, one 32-key sub-tile per accumulator ----
             Acc16 s[KS];
             if (wave_active) {
@@ -277,7 +313,7 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
                 // ---- scale, mask, online softmax (lane-local query) ----
                 const bool need_mask = (d.causal && key0 + kBC - 1 > q_wave0) || (key0 + kBC > seq_k_i);
                 float mt = -__builtin_inff(), m_new, alpha, psum = 0.f;
-                if (scale > 0.f) {
+                if (!MASK && scale > 0.f) {
                     // Positive scale (every real caller): the row max is taken on the raw scores (scaling
                     // by a positive constant keeps the order), and scale * log2(e) is folded into one FMA
                     // per score, 2^(s * c2 - m) with the running max m kept in those log2 units.
@@ -311,6 +347,7 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
 #pragma unroll
                         for (int r = 0; r < 16; ++r) {
                             float x = s[j][r] * scale;
+                            if constexpr (MASK) x += mk[j][r];
                             if (need_mask) {
                                 const int key = key0 + 32 * j + 8 * (r >> 2) + 4 * half + (r & 3);
                                 if ((d.causal && key > qi) || key >= seq_k_i) x = -__builtin_inff();
@@ -320,12 +357,16 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
                         }
                     mt = fmaxf(mt, __shfl_xor(mt, 32, kWave));
                     m_new = fmaxf(m_run, mt);
-                    alpha = exp_diff(m_run, m_new);
+                    // A mask can hide every key seen so far (m_new still -inf): the weights are then 0 and the state
+                    // stays empty, instead of the NaN that exp(-inf - -inf) would carry into later tiles. A row with
+                    // no visible key at all ends as 0 / 0 = NaN, which is what the reference returns for it.
+                    const float m_ref = (MASK && m_new == -__builtin_inff()) ? 0.f : m_new;
+                    alpha = exp_diff(m_run, m_ref);
 #pragma unroll
                     for (int j = 0; j < KS; ++j)
 #pragma unroll
                         for (int r = 0; r < 16; ++r) {
-                            const float e = exp_diff(s[j][r], m_new);
+                            const float e = exp_diff(s[j][r], m_ref);
                             s[j][r] = e;
                             psum += e;
                         }
@@ -393,10 +434,11 @@ __global__ __launch_bounds__(64) void sdpa_generic_kernel(const SdpaArgs p) {
     const int lane = threadIdx.x;
     const int64_t row = blockIdx.x;
     const int64_t bh = row / d.seq_q, qi = row % d.seq_q;
-    const int64_t b = bh / d.heads, h = bh % d.heads;
+    const int64_t b = bh / d.heads, h = bh % d.heads, hk = h / p.group;
     const T *Q = static_cast<const T *>(p.q) + b * d.q_batch_stride + h * d.q_head_stride + qi * d.q_row_stride;
-    const T *K = static_cast<const T *>(p.k) + b * d.k_batch_stride + h * d.k_head_stride;
-    const T *V = static_cast<const T *>(p.v) + b * d.v_batch_stride + h * d.v_head_stride;
+    const T *K = static_cast<const T *>(p.k) + b * d.k_batch_stride + hk * d.k_head_stride;
+    const T *V = static_cast<const T *>(p.v) + b * d.v_batch_stride + hk * d.v_head_stride;
+    const T *mrow = p.mask ? static_cast<const T *>(p.mask) + bh * p.mask_bh_stride + qi * d.seq_k : nullptr;
     T *O = static_cast<T *>(p.out) + b * d.o_batch_stride + h * d.o_head_stride + qi * d.o_row_stride;
     const T scale = (T)p.scale;
     for (int64_t c = lane; c < d.d_k; c += 64) qs[c] = Q[c];
@@ -416,13 +458,15 @@ __global__ __launch_bounds__(64) void sdpa_generic_kernel(const SdpaArgs p) {
             T dot = T(0);
             for (int64_t c = 0; c < d.d_k; ++c) dot += qs[c] * kr[c];
             sc = dot * scale;
+            if (mrow) sc += mrow[key];
         }
         T mt = sc;
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) mt = t_max(mt, __shfl_xor(mt, off, 64));
         const T m_new = t_max(m_run, mt);
-        const T alpha = t_exp(m_run - m_new);
-        const T pj = (key < limit) ? t_exp(sc - m_new) : T(0);
+        const T m_ref = (mrow && m_new == ninf) ? T(0) : m_new;  // every key so far hidden by the mask: empty state, not NaN
+        const T alpha = t_exp(m_run - m_ref);
+        const T pj = (key < limit) ? t_exp(sc - m_ref) : T(0);
         T ps = pj;
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) ps += __shfl_xor(ps, off, 64);
@@ -448,11 +492,11 @@ __global__ __launch_bounds__(64) void sdpa_generic_kernel(const SdpaArgs p) {
     }
 }
 
-template <int D, int NW, bool PAIR> int32_t launch_mfma_cfg(SdpaArgs &a, hipStream_t st) {
+template <int D, int NW, bool PAIR, bool MASK> int32_t launch_mfma_cfg(SdpaArgs &a, hipStream_t st) {
     constexpr int BC = (D <= 64 && (NW == 4 || D <= 32)) ? 64 : 32;  // 64-key tiles where two workgroups still fit a CU
     constexpr bool DIRECT = D >= 64 && FTH_SDPA_DIRECT;
     constexpr size_t smem = DIRECT ? (size_t)2 * BC * 2 * D * sizeof(float) : (size_t)2 * BC * ((D + 4) + (D + 8)) * sizeof(float);
-    auto kern = sdpa_mfma_kernel<D, NW, PAIR, BC, DIRECT>;
+    auto kern = sdpa_mfma_kernel<D, NW, PAIR, BC, DIRECT, MASK>;
     static bool attr_set = false;
     if (!attr_set) {
         FTH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -484,24 +528,35 @@ template <int D> int32_t launch_mfma(SdpaArgs &a, hipStream_t st) {
         wide = D >= 128 || (forced & 1);
         pair = a.d.causal != 0 && (forced & 2);
     }
-    if (pair) return wide ? launch_mfma_cfg<D, 4, true>(a, st) : launch_mfma_cfg<D, 2, true>(a, st);
-    return wide ? launch_mfma_cfg<D, 4, false>(a, st) : launch_mfma_cfg<D, 2, false>(a, st);
+    if (a.mask) return wide ? launch_mfma_cfg<D, 4, false, true>(a, st) : launch_mfma_cfg<D, 2, false, true>(a, st);
+    if (pair) return wide ? launch_mfma_cfg<D, 4, true, false>(a, st) : launch_mfma_cfg<D, 2, true, false>(a, st);
+    return wide ? launch_mfma_cfg<D, 4, false, false>(a, st) : launch_mfma_cfg<D, 2, false, false>(a, st);
 }
 
 template <typename T>
-int32_t sdpa_entry(const fth_sdpa_desc *d, double scale, const T *q, const T *k, const T *v, T *out, fth_stream s) {
+int32_t sdpa_entry(const fth_sdpa_desc *d, double scale, const T *q, const T *k, const T *v, T *out, fth_stream s,
+                   const T *mask = nullptr, int64_t mask_bh_stride = 0, bool masked = false) {
     FTH_REQUIRE_DEVICE();
     FTH_ARG(d != nullptr, "sdpa: desc is NULL");
     FTH_ARG(d->num_bh >= 0 && d->seq_q >= 0 && d->seq_k >= 0 && d->d_k >= 0 && d->d_v >= 0, "sdpa: negative extent");
     FTH_ARG(d->heads >= 1 && d->num_bh % d->heads == 0, "sdpa: heads (%lld) must divide num_bh (%lld)",
             (long long)d->heads, (long long)d->num_bh);
+    const int64_t group = d->kv_group > 1 ? d->kv_group : 1;
+    FTH_ARG(d->kv_group >= 0 && d->heads % group == 0, "sdpa: kv_group (%d) must divide heads (%lld)", (int)d->kv_group, (long long)d->heads);
+    FTH_ARG(!masked || mask_bh_stride == 0 || mask_bh_stride >= d->seq_q * d->seq_k, "sdpa: mask_bh_stride %lld is neither 0 nor >= seq_q * seq_k",
+            (long long)mask_bh_stride);
     if (d->num_bh == 0 || d->seq_q == 0 || d->d_v == 0) return FTH_OK;
     FTH_ARG(q && k && v && out, "sdpa: NULL operand");
+    FTH_ARG(!masked || mask || d->seq_k == 0, "sdpa: NULL mask");
     FTH_ARG(d->seq_q < 2147483647LL - 256 && d->seq_k < 2147483647LL - 256, "sdpa: sequence too long");
     hipStream_t st = fth::resolve_stream(s);
     SdpaArgs a;
     a.q = q; a.k = k; a.v = v; a.out = out; a.d = *d; a.scale = scale;
     a.q_blocks = 0;  // set by the launcher of the chosen variant
+    a.mask = masked ? mask : nullptr;
+    a.mask_bh_stride = mask_bh_stride;
+    a.group = group;
+    a.mask_vec = (d->seq_k % 4 == 0 && mask_bh_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(mask) & 15u) == 0) ? 1 : 0;
     auto al16 = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; };
     auto m4 = [](int64_t x) { return x % 4 == 0; };
     if constexpr (std::is_same<T, float>::value) {
@@ -542,7 +597,7 @@ void fth_sdpa_desc_contiguous(fth_sdpa_desc *d, int64_t num_bh, int64_t seq_q, i
     d->v_batch_stride = seq_k * d_v; d->v_head_stride = 0; d->v_row_stride = d_v;
     d->o_batch_stride = seq_q * d_v; d->o_head_stride = 0; d->o_row_stride = d_v;
     d->causal = causal;
-    d->reserved = 0;
+    d->kv_group = 0;
 }
 
 int32_t fth_dev_sdpa_forward_f32(const fth_sdpa_desc *d, float scale, const float *q, const float *k, const float *v,
@@ -553,6 +608,16 @@ int32_t fth_dev_sdpa_forward_f32(const fth_sdpa_desc *d, float scale, const floa
 int32_t fth_dev_sdpa_forward_f64(const fth_sdpa_desc *d, double scale, const double *q, const double *k,
                                  const double *v, double *out, fth_stream s) {
     return sdpa_entry<double>(d, scale, q, k, v, out, s);
+}
+
+int32_t fth_dev_sdpa_forward_masked_f32(const fth_sdpa_desc *d, float scale, const float *q, const float *k, const float *v,
+                                        const float *mask, int64_t mask_bh_stride, float *out, fth_stream s) {
+    return sdpa_entry<float>(d, (double)scale, q, k, v, out, s, mask, mask_bh_stride, true);
+}
+
+int32_t fth_dev_sdpa_forward_masked_f64(const fth_sdpa_desc *d, double scale, const double *q, const double *k, const double *v,
+                                        const double *mask, int64_t mask_bh_stride, double *out, fth_stream s) {
+    return sdpa_entry<double>(d, scale, q, k, v, out, s, mask, mask_bh_stride, true);
 }
 
 }  // extern "C"

@@ -279,5 +279,24 @@ def sdpa_forward(desc, scale, q, k, v, out, stream=None):
                                                                   _ptr(v), _ptr(out), stream))
 
 
+def sdpa_desc_gqa(batch, h_q, h_kv, seq_q, seq_k, d_k, d_v, causal=False) -> _lib.SdpaDesc:
+    """Contiguous q [batch, h_q, seq_q, d_k] and k / v [batch, h_kv, seq_k, d]: query head h reads K/V head h // (h_q // h_kv)."""
+    if h_kv <= 0 or h_q % h_kv:
+        raise ValueError("h_kv must divide h_q")
+    d = sdpa_desc_contiguous(batch * h_q, seq_q, seq_k, d_k, d_v, causal)
+    d.heads, d.kv_group = h_q, h_q // h_kv
+    d.q_batch_stride, d.q_head_stride = h_q * seq_q * d_k, seq_q * d_k
+    d.k_batch_stride, d.k_head_stride = h_kv * seq_k * d_k, seq_k * d_k
+    d.v_batch_stride, d.v_head_stride = h_kv * seq_k * d_v, seq_k * d_v
+    d.o_batch_stride, d.o_head_stride = h_q * seq_q * d_v, seq_q * d_v
+    return d
+
+
+def sdpa_forward_masked(desc, scale, q, k, v, mask, mask_bh_stride, out, stream=None):
+    """softmax(scale * q k^T + mask) v; mask_bh_stride 0 shares one [seq_q, seq_k] mask, seq_q * seq_k reads one per head."""
+    check(getattr(_lib.load(), "fth_dev_sdpa_forward_masked_" + _sfx(q))(C.byref(desc), _real(q, scale), _ptr(q), _ptr(k), _ptr(v),
+                                                                         _ptr(mask), mask_bh_stride, _ptr(out), stream))
+
+
 def default_scale(head_dim: int) -> float:
     return 1.0 / math.sqrt(head_dim)

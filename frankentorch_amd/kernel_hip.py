@@ -336,6 +336,42 @@ def _sdpa(name, dtype, q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal):
     return out
 
 
+def _sdpa_masked(sfx, dtype, q, k, v, batch, h_q, h_kv, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride):
+    q, k, v, mask = _slice(q, dtype), _slice(k, dtype), _slice(v, dtype), _slice(mask, dtype)
+    out = np.empty(batch * h_q * seq_q * d_v, dtype=dtype)
+    check(getattr(_lib.load(), "fth_sdpa_forward_masked_gqa_" + sfx)(_p(q), q.size, _p(k), k.size, _p(v), v.size, batch, h_q, h_kv, seq_q,
+                                                                     seq_k, d_k, d_v, scale, _p(mask), mask.size, mask_bh_stride,
+                                                                     _p(out), out.size))
+    return out
+
+
+def sdpa_forward_masked_f64(q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride):
+    """crates/ft-kernel-cpu/src/lib.rs:4661."""
+    q, k, v, mask = _slice(q, np.float64), _slice(k, np.float64), _slice(v, np.float64), _slice(mask, np.float64)
+    out = np.empty(num_bh * seq_q * d_v, dtype=np.float64)
+    check(_lib.load().fth_sdpa_forward_masked_f64(_p(q), q.size, _p(k), k.size, _p(v), v.size, num_bh, seq_q, seq_k, d_k, d_v, scale,
+                                                  _p(mask), mask.size, mask_bh_stride, _p(out), out.size))
+    return out
+
+
+def sdpa_forward_masked_f32(q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride):
+    """The f32 twin of sdpa_forward_masked_f64 (the reference has the f64 form only)."""
+    q, k, v, mask = _slice(q, np.float32), _slice(k, np.float32), _slice(v, np.float32), _slice(mask, np.float32)
+    out = np.empty(num_bh * seq_q * d_v, dtype=np.float32)
+    check(_lib.load().fth_sdpa_forward_masked_f32(_p(q), q.size, _p(k), k.size, _p(v), v.size, num_bh, seq_q, seq_k, d_k, d_v, scale,
+                                                  _p(mask), mask.size, mask_bh_stride, _p(out), out.size))
+    return out
+
+
+def sdpa_forward_masked_gqa_f64(q, k, v, batch, h_q, h_kv, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride):
+    """crates/ft-kernel-cpu/src/lib.rs:4777."""
+    return _sdpa_masked("f64", np.float64, q, k, v, batch, h_q, h_kv, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride)
+
+
+def sdpa_forward_masked_gqa_f32(q, k, v, batch, h_q, h_kv, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride):
+    return _sdpa_masked("f32", np.float32, q, k, v, batch, h_q, h_kv, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride)
+
+
 def sdpa_forward_f32(q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal):
     return _sdpa("fth_sdpa_forward_f32", np.float32, q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal)
 

@@ -306,7 +306,8 @@ typedef struct fth_sdpa_desc {
     int64_t v_batch_stride, v_head_stride, v_row_stride;
     int64_t o_batch_stride, o_head_stride, o_row_stride;
     int32_t causal;
-    int32_t reserved;
+    int32_t kv_group; /* grouped-query attention: query heads per K/V head (query head h reads K/V head h / kv_group
+                         through k_head_stride / v_head_stride); 0 or 1: one K/V head per query head */
 } fth_sdpa_desc;
 /* Fills the strides for contiguous [num_bh, seq, d] operands. */
 void fth_sdpa_desc_contiguous(fth_sdpa_desc *d, int64_t num_bh, int64_t seq_q, int64_t seq_k,
@@ -315,6 +316,16 @@ int32_t fth_dev_sdpa_forward_f32(const fth_sdpa_desc *d, float scale, const floa
                                  const float *v, float *out, fth_stream s);
 int32_t fth_dev_sdpa_forward_f64(const fth_sdpa_desc *d, double scale, const double *q, const double *k,
                                  const double *v, double *out, fth_stream s);
+/* The same with an additive mask: score * scale + mask[bh * mask_bh_stride + qi * seq_k + key] before the softmax
+ * (sdpa_forward_masked_f64, crates/ft-kernel-cpu/src/lib.rs:4661-4741; with kv_group > 1 in the descriptor it is
+ * sdpa_forward_masked_gqa_f64, :4777-4850; the reference has the f64 forms only). mask_bh_stride is 0 for one
+ * [seq_q, seq_k] mask shared by every (batch, head), else the distance between the masks of consecutive bh
+ * (seq_q * seq_k for a packed [num_bh, seq_q, seq_k] mask). -inf hides a key; a row whose every key is hidden is NaN,
+ * as in the reference. */
+int32_t fth_dev_sdpa_forward_masked_f32(const fth_sdpa_desc *d, float scale, const float *q, const float *k, const float *v,
+                                        const float *mask, int64_t mask_bh_stride, float *out, fth_stream s);
+int32_t fth_dev_sdpa_forward_masked_f64(const fth_sdpa_desc *d, double scale, const double *q, const double *k, const double *v,
+                                        const double *mask, int64_t mask_bh_stride, double *out, fth_stream s);
 
 /* ------------------------------------------------------------------------------------------ */
 /* Tier A: host slices in, host buffer out (the ft_kernel_cpu surface)                        */
@@ -379,6 +390,22 @@ int32_t fth_rms_norm_forward_f32(const float *x, size_t x_len, const float *weig
                                  size_t norm_size, float eps, float *out, size_t out_cap);
 int32_t fth_rms_norm_forward_f64(const double *x, size_t x_len, const double *weight, size_t batch,
                                  size_t norm_size, double eps, double *out, size_t out_cap);
+/* sdpa_forward_masked_f64 (:4661-4741) and sdpa_forward_masked_gqa_f64 (:4777-4850), plus f32 twins the reference
+ * does not have yet: q [num_bh | batch, h_q][seq_q, d_k], k / v [num_bh | batch, h_kv][seq_k, d]; additive mask with
+ * mask_bh_stride 0 (one [seq_q, seq_k] for every head) or seq_q * seq_k (one per query head). A mask slice shorter than
+ * the shape reads (a slice-index panic in the reference) and h_q % h_kv != 0 are InvalidArgument. */
+int32_t fth_sdpa_forward_masked_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len, size_t num_bh,
+                                    size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, float scale, const float *mask, size_t mask_len,
+                                    size_t mask_bh_stride, float *out, size_t out_cap);
+int32_t fth_sdpa_forward_masked_f64(const double *q, size_t q_len, const double *k, size_t k_len, const double *v, size_t v_len, size_t num_bh,
+                                    size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, double scale, const double *mask, size_t mask_len,
+                                    size_t mask_bh_stride, double *out, size_t out_cap);
+int32_t fth_sdpa_forward_masked_gqa_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len, size_t batch,
+                                        size_t h_q, size_t h_kv, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, float scale,
+                                        const float *mask, size_t mask_len, size_t mask_bh_stride, float *out, size_t out_cap);
+int32_t fth_sdpa_forward_masked_gqa_f64(const double *q, size_t q_len, const double *k, size_t k_len, const double *v, size_t v_len, size_t batch,
+                                        size_t h_q, size_t h_kv, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, double scale,
+                                        const double *mask, size_t mask_len, size_t mask_bh_stride, double *out, size_t out_cap);
 /* log_softmax_dim_tensor_contiguous_f32 (:39298) / _f64 (:18504): the validation of softmax_dim_tensor_contiguous.
  * cross_entropy_forward_f32 (:6717) / _f64 (:6649) -> loss [batch]; cross_entropy_backward_f32 (:6745) / _f64 (:6679)
  * -> dlogits [batch*classes]. target holds class indices (the reference's &[usize]). */

@@ -328,6 +328,61 @@ void sdpa_impl(const T *q, const T *k, const T *v, int64_t num_bh, int64_t seq_q
     }
 }
 
+// sdpa_forward_masked_gqa_f64 (KC:4777-4850); sdpa_forward_masked_f64 (KC:4661-4741) is the h_q == h_kv case. q is
+// [batch, h_q, seq_q, d_k]; k / v are [batch, h_kv, seq_k, d_*]; query head hq reads K/V head hq / (h_q / h_kv).
+// scores = (q . k^T) * scale + mask over ALL seq_k keys (the additive mask carries any causality as -inf); max by a
+// strict `>` scan; e = exp(s - m); s /= sum; out = p . v. mask_bh_stride is 0 (one [seq_q, seq_k] mask for every head)
+// or seq_q * seq_k (one per batch*h_q). The reference has the f64 form only; the f32 instantiation is the same steps.
+template <typename T>
+void sdpa_masked_gqa_impl(const T *q, const T *k, const T *v, int64_t batch, int64_t h_q, int64_t h_kv, int64_t seq_q, int64_t seq_k,
+                          int64_t d_k, int64_t d_v, T scale, const T *mask, int64_t mask_bh_stride, T *out) {
+    const int64_t num_bh = batch * h_q;
+    if (num_bh <= 0 || seq_q <= 0 || d_v <= 0 || h_kv <= 0) return;
+    const int64_t group = h_q / h_kv;
+    using Wide = typename std::conditional<sizeof(T) == 4, double, long double>::type;
+#pragma omp parallel
+    {
+        std::vector<T> sc((size_t)std::max<int64_t>(seq_k, 1));
+        std::vector<Wide> acc((size_t)d_v);
+#pragma omp for schedule(dynamic, 8) collapse(2)
+        for (int64_t bh = 0; bh < num_bh; ++bh) {
+            for (int64_t qi = 0; qi < seq_q; ++qi) {
+                const int64_t b = bh / h_q, kv_head = (bh % h_q) / group;  // KC:4812-4813
+                const T *qr = q + (bh * seq_q + qi) * d_k;
+                const T *kh = k + (b * h_kv + kv_head) * seq_k * d_k;
+                const T *vh = v + (b * h_kv + kv_head) * seq_k * d_v;
+                const T *mrow = mask + bh * mask_bh_stride + qi * seq_k;
+                for (int64_t j = 0; j < seq_k; ++j) {  // dgemm_bt, KC:4823
+                    Wide dot = 0;
+                    const T *kr = kh + j * d_k;
+                    for (int64_t c = 0; c < d_k; ++c) dot += (Wide)qr[c] * (Wide)kr[c];
+                    sc[j] = (T)dot;
+                }
+                T m = -std::numeric_limits<T>::infinity();
+                for (int64_t j = 0; j < seq_k; ++j) {  // KC:4829-4834
+                    sc[j] = sc[j] * scale + mrow[j];
+                    if (sc[j] > m) m = sc[j];
+                }
+                T sum = 0;
+                for (int64_t j = 0; j < seq_k; ++j) {
+                    T e = t_exp(sc[j] - m);
+                    sc[j] = e;
+                    sum += e;
+                }
+                for (int64_t j = 0; j < seq_k; ++j) sc[j] /= sum;
+                std::fill(acc.begin(), acc.end(), (Wide)0);
+                for (int64_t j = 0; j < seq_k; ++j) {  // dgemm, KC:4846
+                    const Wide pj = (Wide)sc[j];
+                    const T *vr = vh + j * d_v;
+                    for (int64_t c = 0; c < d_v; ++c) acc[c] += pj * (Wide)vr[c];
+                }
+                T *o = out + (bh * seq_q + qi) * d_v;
+                for (int64_t c = 0; c < d_v; ++c) o[c] = (T)acc[c];
+            }
+        }
+    }
+}
+
 // normalize_strict_index_value (KC:20058-20090).
 inline int64_t strict_index(double v, int64_t dim_size) {
     if (!std::isfinite(v)) return -1;
@@ -882,6 +937,16 @@ void fto_linear_f64(const double *x, const double *w, const double *bias, int64_
 void fto_sdpa_forward_f32(const float *q, const float *k, const float *v, int64_t num_bh, int64_t seq_q,
                           int64_t seq_k, int64_t d_k, int64_t d_v, float scale, int causal, float *out) {
     sdpa_impl<float>(q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, out);
+}
+void fto_sdpa_forward_masked_gqa_f32(const float *q, const float *k, const float *v, int64_t batch, int64_t h_q, int64_t h_kv,
+                                     int64_t seq_q, int64_t seq_k, int64_t d_k, int64_t d_v, float scale, const float *mask,
+                                     int64_t mask_bh_stride, float *out) {
+    sdpa_masked_gqa_impl<float>(q, k, v, batch, h_q, h_kv, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride, out);
+}
+void fto_sdpa_forward_masked_gqa_f64(const double *q, const double *k, const double *v, int64_t batch, int64_t h_q, int64_t h_kv,
+                                     int64_t seq_q, int64_t seq_k, int64_t d_k, int64_t d_v, double scale, const double *mask,
+                                     int64_t mask_bh_stride, double *out) {
+    sdpa_masked_gqa_impl<double>(q, k, v, batch, h_q, h_kv, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride, out);
 }
 void fto_sdpa_forward_f64(const double *q, const double *k, const double *v, int64_t num_bh, int64_t seq_q,
                           int64_t seq_k, int64_t d_k, int64_t d_v, double scale, int causal, double *out) {

@@ -204,6 +204,29 @@ def sdpa_forward(q, k, v, scale, causal):
     return out
 
 
+def sdpa_forward_masked_gqa(q, k, v, scale, mask):
+    """q [batch, h_q, seq_q, d_k]; k, v [batch, h_kv, seq_k, d]; additive mask [seq_q, seq_k] (shared) or
+    [batch * h_q, seq_q, seq_k] (crates/ft-kernel-cpu/src/lib.rs:4777-4850)."""
+    q, k, v, mask = _c(q), _c(k), _c(v), _c(np.asarray(mask, dtype=q.dtype))
+    sfx, ct = _sfx(q.dtype)
+    batch, h_q, seq_q, d_k = q.shape
+    h_kv, seq_k = k.shape[1], k.shape[2]
+    d_v = v.shape[3]
+    assert h_q % h_kv == 0 and mask.shape[-2:] == (seq_q, seq_k)
+    stride = 0 if mask.ndim == 2 else seq_q * seq_k
+    assert mask.ndim == 2 or mask.shape[0] == batch * h_q
+    out = np.zeros((batch, h_q, seq_q, d_v), dtype=q.dtype)
+    getattr(lib(), "fto_sdpa_forward_masked_gqa_" + sfx)(_p(q), _p(k), _p(v), _i64(batch), _i64(h_q), _i64(h_kv), _i64(seq_q),
+                                                         _i64(seq_k), _i64(d_k), _i64(d_v), ct(scale), _p(mask), _i64(stride), _p(out))
+    return out
+
+
+def sdpa_forward_masked(q, k, v, scale, mask):
+    """q, k, v [num_bh, seq, d]: the h_q == h_kv case (crates/ft-kernel-cpu/src/lib.rs:4661-4741)."""
+    q, k, v = _c(q), _c(k), _c(v)
+    return sdpa_forward_masked_gqa(q[None], k[None], v[None], scale, mask)[0]
+
+
 def log_softmax(x, dim: int = -1):
     x = _c(x)
     sfx, _ = _sfx(x.dtype)

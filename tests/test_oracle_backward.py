@@ -138,3 +138,48 @@ def test_cross_entropy_is_minus_log_softmax_at_the_target_and_its_gradient(oracl
     assert np.allclose(l32, loss, atol=2e-6)
     with pytest.raises(IndexError):
         oracle.cross_entropy_forward(logits, np.full(batch, classes))
+
+
+def _reference_gqa_inputs():
+    """The inputs of sdpa_masked_gqa_f64_matches_expand_then_masked_bit_exact (crates/ft-kernel-cpu/src/lib.rs:45160-45183)."""
+    batch, h_q, h_kv, seq_q, seq_k, d_k, d_v = 2, 8, 2, 40, 40, 16, 16
+    i = lambda n: np.arange(n, dtype=np.float64)
+    q = (np.sin(i(batch * h_q * seq_q * d_k) * 0.017 + 0.3) * 0.2).reshape(batch, h_q, seq_q, d_k)
+    k = (np.sin(i(batch * h_kv * seq_k * d_k) * 0.013 + 1.1) * 0.2).reshape(batch, h_kv, seq_k, d_k)
+    v = (np.cos(i(batch * h_kv * seq_k * d_v) * 0.011 + 2.2) * 0.2).reshape(batch, h_kv, seq_k, d_v)
+    mask2d = np.where(np.arange(seq_q * seq_k) % 3 == 0, -0.5, 0.0).reshape(seq_q, seq_k)
+    mask3d = np.where(np.arange(batch * h_q * seq_q * seq_k) % 5 == 0, -0.7, 0.0).reshape(batch * h_q, seq_q, seq_k)
+    return q, k, v, mask2d, mask3d, 1.0 / np.sqrt(d_k)
+
+
+def test_masked_gqa_sdpa_restatement_is_pinned(oracle):
+    q, k, v, mask2d, mask3d, scale = _reference_gqa_inputs()
+    batch, h_q, seq_q, d_k = q.shape
+    h_kv, seq_k = k.shape[1], k.shape[2]
+    group = h_q // h_kv
+    k_rep, v_rep = np.repeat(k, group, axis=1), np.repeat(v, group, axis=1)  # head hq reads kv head hq // group
+    for mask in (mask2d, mask3d):
+        grouped = oracle.sdpa_forward_masked_gqa(q, k, v, scale, mask)
+        # the reference's own assertion: bit-exact with expand-then-masked
+        expanded = oracle.sdpa_forward_masked(q.reshape(batch * h_q, seq_q, d_k), k_rep.reshape(batch * h_q, seq_k, d_k),
+                                              v_rep.reshape(batch * h_q, seq_k, -1), scale, mask)
+        assert np.array_equal(grouped.reshape(expanded.shape).view(np.uint64), expanded.view(np.uint64))
+        # independent of the restatement: softmax(scale * q k^T + mask) v in numpy
+        s = np.einsum("bhqd,bhkd->bhqk", q, k_rep) * scale + mask.reshape((-1, h_q, seq_q, seq_k) if mask.ndim == 3 else (1, 1, seq_q, seq_k))
+        p = np.exp(s - s.max(-1, keepdims=True))
+        p /= p.sum(-1, keepdims=True)
+        assert np.allclose(grouped, np.einsum("bhqk,bhkd->bhqd", p, v_rep), rtol=0, atol=1e-14)
+    # a zero mask is the unmasked kernel, a -inf upper triangle the causal one (both pinned by the reference's fixtures)
+    qf, kf, vf = (t.reshape(batch * h_q, seq_q, -1) for t in (q, k_rep, v_rep))
+    zero = np.zeros((seq_q, seq_k))
+    assert np.allclose(oracle.sdpa_forward_masked(qf, kf, vf, scale, zero), oracle.sdpa_forward(qf, kf, vf, scale, False), atol=1e-15)
+    tri = np.where(np.arange(seq_k)[None, :] > np.arange(seq_q)[:, None], -np.inf, 0.0)
+    assert np.allclose(oracle.sdpa_forward_masked(qf, kf, vf, scale, tri), oracle.sdpa_forward(qf, kf, vf, scale, True), atol=1e-15)
+    # a fully masked row is NaN, as exp(-inf - -inf) makes it in the reference
+    tri[3, :] = -np.inf
+    out = oracle.sdpa_forward_masked(qf, kf, vf, scale, tri)
+    assert np.all(np.isnan(out[:, 3, :])) and not np.any(np.isnan(np.delete(out, 3, axis=1)))
+    # f32 instantiation agrees to f32 rounding
+    f = np.float32
+    o32 = oracle.sdpa_forward_masked_gqa(q.astype(f), k.astype(f), v.astype(f), f(scale), mask2d.astype(f))
+    assert np.allclose(o32, oracle.sdpa_forward_masked_gqa(q, k, v, scale, mask2d), atol=2e-6)
