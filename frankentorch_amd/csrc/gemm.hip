@@ -86,6 +86,12 @@ template <> struct Mfma<float> {
     __device__ __forceinline__ static V zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
     __device__ __forceinline__ static V make(const float *e) { return make_float4(e[0], e[1], e[2], e[3]); }
     __device__ __forceinline__ static float gelu(float x) { return (0.5f * x) * (1.0f + erff(x * 0.70710678118654752440f)); }
+    // tanh-form GELU as x * sigmoid(2u), u = sqrt(2/pi) (x + 0.044715 x^3): 0.5 (1 + tanh u) = 1 / (1 + e^-2u). One
+    // hardware exp2 and one division; e^-2u overflowing to inf gives x / inf = -0 where the tanh form gives -0 too.
+    __device__ __forceinline__ static float gelu_tanh(float x) {
+        const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+        return x / (1.0f + __builtin_amdgcn_exp2f(u * -2.8853900817779268f));  // -2 log2(e)
+    }
 };
 template <> struct Mfma<double> {
     static constexpr int MT = 16;
@@ -103,6 +109,9 @@ template <> struct Mfma<double> {
     __device__ __forceinline__ static V zero() { return make_double2(0.0, 0.0); }
     __device__ __forceinline__ static V make(const double *e) { return make_double2(e[0], e[1]); }
     __device__ __forceinline__ static double gelu(double x) { return (0.5 * x) * (1.0 + erf(x * 0.70710678118654752440)); }
+    __device__ __forceinline__ static double gelu_tanh(double x) {
+        return 0.5 * x * (1.0 + tanh(0.79788456080286535588 * (x + 0.044715 * x * x * x)));
+    }
 };
 
 template <typename T> struct GemmArgs {
@@ -302,6 +311,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_kernel(const GemmArg
     // residual, which is the order the unfused reference ops would apply them.
     const bool has_bias = (p.epilogue & FTH_EPI_BIAS) != 0;
     const bool has_gelu = (p.epilogue & FTH_EPI_GELU) != 0;
+    const bool has_gelu_tanh = (p.epilogue & FTH_EPI_GELU_TANH) != 0;
     const bool has_res = (p.epilogue & FTH_EPI_RESIDUAL) != 0;
     auto epilogue = [&]() {
 #pragma unroll
@@ -319,6 +329,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_kernel(const GemmArg
                         if (p.use_alpha) v = p.alpha * v;
                         if (has_bias) v = v + bv;
                         if (has_gelu) v = M::gelu(v);
+                        if (has_gelu_tanh) v = M::gelu_tanh(v);
                         if (has_res) v = v + p.residual[batch * p.stride_c + row * p.ldc + col];
                         C[row * p.ldc + col] = v;
                     }
@@ -492,6 +503,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
     const int epi = EPI >= 0 ? EPI : p.epilogue;
     const bool has_bias = (epi & FTH_EPI_BIAS) != 0;
     const bool has_gelu = (epi & FTH_EPI_GELU) != 0;
+    const bool has_gelu_tanh = (epi & FTH_EPI_GELU_TANH) != 0;
     const bool has_res = (epi & FTH_EPI_RESIDUAL) != 0;
     const bool use_alpha = EPI >= 0 ? false : p.use_alpha != 0;
 
@@ -668,6 +680,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
         if (use_alpha) v = p.alpha * v;
         if (has_bias) v = v + bv;
         if (has_gelu) v = M::gelu(v);
+        if (has_gelu_tanh) v = M::gelu_tanh(v);
         if (has_res) v = v + rv;
         return v;
     };
@@ -906,6 +919,7 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemm_fixup_kernel(const GemmArg
     T *C = p.c + batch * p.stride_c;
     const bool has_bias = (p.epilogue & FTH_EPI_BIAS) != 0;
     const bool has_gelu = (p.epilogue & FTH_EPI_GELU) != 0;
+    const bool has_gelu_tanh = (p.epilogue & FTH_EPI_GELU_TANH) != 0;
     const bool has_res = (p.epilogue & FTH_EPI_RESIDUAL) != 0;
 #pragma unroll
     for (int u = 0; u < PV; ++u) {
@@ -918,6 +932,7 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemm_fixup_kernel(const GemmArg
             if (p.use_alpha) v = p.alpha * v;
             if (has_bias) v = v + p.bias[col];
             if (has_gelu) v = M::gelu(v);
+            if (has_gelu_tanh) v = M::gelu_tanh(v);
             if (has_res) v = v + p.residual[batch * p.stride_c + row * p.ldc + col];
             C[row * p.ldc + col] = v;
         }
@@ -935,6 +950,7 @@ __global__ __launch_bounds__(256) void gemm_k0_kernel(const GemmArgs<T> p) {
     if (p.use_alpha) v = p.alpha * v;
     if (p.epilogue & FTH_EPI_BIAS) v = v + p.bias[col];
     if (p.epilogue & FTH_EPI_GELU) v = M::gelu(v);
+    if (p.epilogue & FTH_EPI_GELU_TANH) v = M::gelu_tanh(v);
     if (p.epilogue & FTH_EPI_RESIDUAL) v = v + p.residual[batch * p.stride_c + row * p.ldc + col];
     p.c[batch * p.stride_c + row * p.ldc + col] = v;
 }
@@ -1032,7 +1048,7 @@ int32_t launch_direct_epi(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
 }
 
 // SPECIALIZE: pick a kernel with the epilogue flags compiled in for the combinations the
-// transformer block uses (none, bias, bias+GELU, bias+residual; alpha = 1).
+// transformer block uses (none, bias, bias+GELU in either form, bias+residual; alpha = 1).
 template <typename T, int BM, int BN, int WM, int WN, int MINW, bool TRANS_B, bool SPECIALIZE>
 int32_t launch_direct(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     if constexpr (SPECIALIZE) {
@@ -1042,6 +1058,8 @@ int32_t launch_direct(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
                 case FTH_EPI_BIAS: return launch_direct_epi<T, BM, BN, WM, WN, MINW, false, TRANS_B, FTH_EPI_BIAS>(p, batch, st);
                 case FTH_EPI_BIAS | FTH_EPI_GELU:
                     return launch_direct_epi<T, BM, BN, WM, WN, MINW, false, TRANS_B, FTH_EPI_BIAS | FTH_EPI_GELU>(p, batch, st);
+                case FTH_EPI_BIAS | FTH_EPI_GELU_TANH:
+                    return launch_direct_epi<T, BM, BN, WM, WN, MINW, false, TRANS_B, FTH_EPI_BIAS | FTH_EPI_GELU_TANH>(p, batch, st);
                 case FTH_EPI_BIAS | FTH_EPI_RESIDUAL:
                     return launch_direct_epi<T, BM, BN, WM, WN, MINW, false, TRANS_B, FTH_EPI_BIAS | FTH_EPI_RESIDUAL>(p, batch, st);
                 default: break;
@@ -1163,7 +1181,8 @@ int32_t gemm_entry(const fth_gemm_desc *d, T alpha, const T *a, const T *b, T *c
     FTH_ARG(!(d->trans_a && d->trans_b), "gemm: trans_a together with trans_b is not supported");
     FTH_ARG(!(d->epilogue & FTH_EPI_BIAS) || bias, "gemm: bias epilogue without a bias pointer");
     FTH_ARG(!(d->epilogue & FTH_EPI_RESIDUAL) || residual, "gemm: residual epilogue without a residual pointer");
-    FTH_ARG((d->epilogue & ~(FTH_EPI_BIAS | FTH_EPI_GELU | FTH_EPI_RESIDUAL)) == 0, "gemm: unknown epilogue bits");
+    FTH_ARG((d->epilogue & ~(FTH_EPI_BIAS | FTH_EPI_GELU | FTH_EPI_RESIDUAL | FTH_EPI_GELU_TANH)) == 0, "gemm: unknown epilogue bits");
+    FTH_ARG((d->epilogue & (FTH_EPI_GELU | FTH_EPI_GELU_TANH)) != (FTH_EPI_GELU | FTH_EPI_GELU_TANH), "gemm: both GELU forms requested");
     hipStream_t st = fth::resolve_stream(s);
     GemmArgs<T> p;
     p.a = a; p.b = b; p.c = c; p.bias = bias; p.residual = residual;

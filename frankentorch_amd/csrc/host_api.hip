@@ -182,6 +182,7 @@ template <> struct Dev<float> {
     static int32_t layer_norm(const float *x, const float *w, const float *b, float *y, int64_t n, int64_t c, float e) { return fth_dev_layer_norm_f32(x, w, b, y, n, c, e, nullptr); }
     static int32_t rms_norm(const float *x, const float *w, float *y, int64_t n, int64_t c, float e) { return fth_dev_rms_norm_f32(x, w, y, n, c, e, nullptr); }
     static int32_t gelu(const float *x, float *y, int64_t n) { return fth_dev_gelu_f32(x, y, n, nullptr); }
+    static int32_t gelu_tanh(const float *x, float *y, int64_t n) { return fth_dev_gelu_tanh_f32(x, y, n, nullptr); }
     static int32_t add(const float *a, const float *b, float *y, int64_t n) { return fth_dev_add_f32(a, b, y, n, nullptr); }
     static int32_t sdpa(const fth_sdpa_desc *d, float s, const float *q, const float *k, const float *v, float *o) { return fth_dev_sdpa_forward_f32(d, s, q, k, v, o, nullptr); }
     static int32_t index_select(const float *x, int64_t o, int64_t ds, int64_t in, const double *idx, int64_t n, float *out) { return fth_dev_index_select_f32(x, o, ds, in, idx, n, out, nullptr, nullptr); }
@@ -202,6 +203,7 @@ template <> struct Dev<double> {
     static int32_t layer_norm(const double *x, const double *w, const double *b, double *y, int64_t n, int64_t c, double e) { return fth_dev_layer_norm_f64(x, w, b, y, n, c, e, nullptr); }
     static int32_t rms_norm(const double *x, const double *w, double *y, int64_t n, int64_t c, double e) { return fth_dev_rms_norm_f64(x, w, y, n, c, e, nullptr); }
     static int32_t gelu(const double *x, double *y, int64_t n) { return fth_dev_gelu_f64(x, y, n, nullptr); }
+    static int32_t gelu_tanh(const double *x, double *y, int64_t n) { return fth_dev_gelu_tanh_f64(x, y, n, nullptr); }
     static int32_t add(const double *a, const double *b, double *y, int64_t n) { return fth_dev_add_f64(a, b, y, n, nullptr); }
     static int32_t sdpa(const fth_sdpa_desc *d, double s, const double *q, const double *k, const double *v, double *o) { return fth_dev_sdpa_forward_f64(d, s, q, k, v, o, nullptr); }
     static int32_t index_select(const double *x, int64_t o, int64_t ds, int64_t in, const double *idx, int64_t n, double *out) { return fth_dev_index_select_f64(x, o, ds, in, idx, n, out, nullptr, nullptr); }
@@ -509,7 +511,7 @@ int32_t rms_norm_impl(const T *x, size_t x_len, const T *w, size_t batch, size_t
 // gelu_tensor_contiguous (unary_contiguous_f32 via define_unary_f32!, crates/ft-kernel-cpu/src/
 // lib.rs:37051-37064, 37123-37127)
 template <typename T>
-int32_t gelu_impl(const T *input, size_t input_len, const fth_meta *meta, T *out, size_t out_cap, size_t *out_len) {
+int32_t gelu_impl(const T *input, size_t input_len, const fth_meta *meta, T *out, size_t out_cap, size_t *out_len, bool tanh_form = false) {
     FTH_ARG(meta_ok(meta), "gelu: bad meta");
     if (out_len) *out_len = 0;
     if (int32_t rc = ensure_unary(input_len, meta)) return rc;
@@ -523,7 +525,7 @@ int32_t gelu_impl(const T *input, size_t input_len, const fth_meta *meta, T *out
     T *dx, *dy;
     if (int32_t rc = stage_in(sc, input + meta->storage_offset, (size_t)numel, &dx)) return rc;
     if (int32_t rc = stage_out(sc, (size_t)numel, &dy)) return rc;
-    if (int32_t rc = Dev<T>::gelu(dx, dy, (int64_t)numel)) return rc;
+    if (int32_t rc = tanh_form ? Dev<T>::gelu_tanh(dx, dy, (int64_t)numel) : Dev<T>::gelu(dx, dy, (int64_t)numel)) return rc;
     return fetch(out, dy, (size_t)numel);
 }
 
@@ -930,6 +932,14 @@ int32_t fth_rms_norm_forward_f64(const double *x, size_t x_len, const double *w,
 int32_t fth_gelu_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta, float *out,
                                        size_t out_cap, size_t *out_len) {
     return gelu_impl<float>(input, input_len, meta, out, out_cap, out_len);
+}
+int32_t fth_gelu_tanh_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta, float *out, size_t out_cap,
+                                            size_t *out_len) {
+    return gelu_impl<float>(input, input_len, meta, out, out_cap, out_len, true);
+}
+int32_t fth_gelu_tanh_tensor_contiguous_f64(const double *input, size_t input_len, const fth_meta *meta, double *out, size_t out_cap,
+                                            size_t *out_len) {
+    return gelu_impl<double>(input, input_len, meta, out, out_cap, out_len, true);
 }
 int32_t fth_gelu_tensor_contiguous_f64(const double *input, size_t input_len, const fth_meta *meta, double *out,
                                        size_t out_cap, size_t *out_len) {

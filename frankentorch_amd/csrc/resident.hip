@@ -181,6 +181,7 @@ struct Stack {
     int64_t d_model = 0, n_heads = 0, d_ff = 0;
     float eps = 1e-5f;
     int causal = 1;
+    int gelu_epilogue = FTH_EPI_GELU;  // FTH_EPI_GELU (erf form) or FTH_EPI_GELU_TANH
     std::vector<LayerDev> layers;
     std::vector<void *> owned;  // every device block this stack allocated
     Workspace ws;
@@ -272,7 +273,7 @@ struct Stack {
             g = linear_desc(T, d, d, FTH_EPI_BIAS | FTH_EPI_RESIDUAL);
             if ((rc = fth_dev_gemm_f32(&g, 1.f, ws.ctx, L.wo, ws.xa, L.bo, x, s))) return rc;
             if ((rc = fth_dev_layer_norm_f32(ws.xa, L.ln2_w, L.ln2_b, ws.h, T, d, eps, s))) return rc;
-            g = linear_desc(T, d_ff, d, FTH_EPI_BIAS | FTH_EPI_GELU);
+            g = linear_desc(T, d_ff, d, FTH_EPI_BIAS | gelu_epilogue);
             if ((rc = fth_dev_gemm_f32(&g, 1.f, ws.h, L.w1, ws.ff, L.b1, nullptr, s))) return rc;
             float *dst = (last && final_out) ? final_out : ws.xb;
             g = linear_desc(T, d, d_ff, FTH_EPI_BIAS | FTH_EPI_RESIDUAL);
@@ -452,6 +453,14 @@ int32_t fth_batch_rmsnorm(fth_batch *b, const fth_tensor *x, const fth_tensor *g
     return finish_op(fth_dev_rms_norm_f32(x->data, gamma ? gamma->data : nullptr, t->data, x->rows, x->cols, eps, nullptr), t, out);
 }
 
+int32_t fth_batch_gelu_tanh(fth_batch *b, const fth_tensor *x, fth_tensor **out) {
+    FTH_BATCH_PROLOGUE("batch_gelu_tanh");
+    FTH_ARG(x != nullptr, "batch_gelu_tanh: NULL operand");
+    fth_tensor *t;
+    if (int32_t rc = tensor_new(x->rows, x->cols, &t)) return rc;
+    return finish_op(fth_dev_gelu_tanh_f32(x->data, t->data, x->rows * x->cols, nullptr), t, out);
+}
+
 int32_t fth_batch_gelu(fth_batch *b, const fth_tensor *x, fth_tensor **out) {
     FTH_BATCH_PROLOGUE("batch_gelu");
     FTH_ARG(x != nullptr, "batch_gelu: NULL operand");
@@ -596,6 +605,15 @@ int32_t fth_encoder_forward_graph(fth_encoder *e, const float *x_dev, int64_t ba
     return FTH_OK;
 }
 
+int32_t fth_encoder_set_activation(fth_encoder *e, int32_t activation) {
+    FTH_ARG(e != nullptr, "encoder_set_activation: encoder is NULL");
+    FTH_ARG(activation == FTH_ACT_GELU_ERF || activation == FTH_ACT_GELU_TANH, "encoder_set_activation: unknown activation %d", activation);
+    std::lock_guard<std::mutex> lock(e->stack.mu);
+    FTH_ARG(e->graphs.empty(), "encoder_set_activation: a captured graph already holds the old activation");
+    e->stack.gelu_epilogue = activation == FTH_ACT_GELU_TANH ? FTH_EPI_GELU_TANH : FTH_EPI_GELU;
+    return FTH_OK;
+}
+
 // ---- GPT-2-shaped decoder --------------------------------------------------------------------
 int32_t fth_gpt2_new(int64_t vocab, int64_t max_pos, int64_t d_model, int64_t n_heads, int64_t d_ff, float ln_eps,
                      const float *wte, const float *wpe, const fth_layer_weights *layers, int64_t n_layers,
@@ -629,6 +647,14 @@ int32_t fth_gpt2_new(int64_t vocab, int64_t max_pos, int64_t d_model, int64_t n_
         return rc;
     }
     *out = g;
+    return FTH_OK;
+}
+
+int32_t fth_gpt2_set_activation(fth_gpt2 *g, int32_t activation) {
+    FTH_ARG(g != nullptr, "gpt2_set_activation: model is NULL");
+    FTH_ARG(activation == FTH_ACT_GELU_ERF || activation == FTH_ACT_GELU_TANH, "gpt2_set_activation: unknown activation %d", activation);
+    std::lock_guard<std::mutex> lock(g->stack.mu);
+    g->stack.gelu_epilogue = activation == FTH_ACT_GELU_TANH ? FTH_EPI_GELU_TANH : FTH_EPI_GELU;
     return FTH_OK;
 }
 

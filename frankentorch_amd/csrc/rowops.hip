@@ -104,6 +104,16 @@ __device__ __forceinline__ float dev_gelu(float x) {
 __device__ __forceinline__ double dev_gelu(double x) {
     return (0.5 * x) * (1.0 + erf(x * 0.70710678118654752440));
 }
+// tanh-form GELU, 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))): the `gelu` kernel of the reference's fused GPU module
+// (crates/ft-kernel-metal/src/fused.rs:301-313, with its |x| >= 10 clamp) and GELU::tanh() (crates/ft-nn/src/lib.rs:1924-1957).
+__device__ __forceinline__ float dev_gelu_tanh(float x) {
+    if (x >= 10.0f) return x;
+    if (x <= -10.0f) return 0.0f;
+    return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+}
+__device__ __forceinline__ double dev_gelu_tanh(double x) {
+    return 0.5 * x * (1.0 + tanh(0.79788456080286535588 * (x + 0.044715 * x * x * x)));
+}
 template <typename T> __device__ __forceinline__ T neg_inf();
 template <> __device__ __forceinline__ float neg_inf<float>() { return -__builtin_inff(); }
 template <> __device__ __forceinline__ double neg_inf<double>() { return -__builtin_inf(); }
@@ -451,7 +461,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_stream_kernel(const T *__restr
 // Elementwise: GELU, add. Each thread owns UNR 128-bit vectors a block-stride apart, loads them
 // all before the first use, and a scalar tail covers what is left.
 // ---------------------------------------------------------------------------------------------
-enum class Ew { Gelu, Add };
+enum class Ew { Gelu, Add, GeluTanh };
 constexpr int kUnr = 4;
 
 template <typename T, Ew OP>
@@ -479,6 +489,7 @@ __global__ __launch_bounds__(kBlock) void elementwise_vec_kernel(const T *__rest
 #pragma unroll
             for (int j = 0; j < R::EPV; ++j) {
                 if constexpr (OP == Ew::Gelu) ea[j] = dev_gelu(ea[j]);
+                else if constexpr (OP == Ew::GeluTanh) ea[j] = dev_gelu_tanh(ea[j]);
                 else ea[j] = ea[j] + eb[j];
             }
             stream_store(reinterpret_cast<V *>(y) + v, R::pack(ea));
@@ -492,6 +503,7 @@ __global__ __launch_bounds__(kBlock) void elementwise_scalar_kernel(const T *__r
     const int64_t i = begin + (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
     if constexpr (OP == Ew::Gelu) y[i] = dev_gelu(a[i]);
+    else if constexpr (OP == Ew::GeluTanh) y[i] = dev_gelu_tanh(a[i]);
     else y[i] = a[i] + b[i];
 }
 
@@ -698,11 +710,11 @@ int32_t launch_elementwise(const T *a, const T *b, T *y, int64_t n, fth_stream s
     FTH_REQUIRE_DEVICE();
     FTH_ARG(n >= 0, "elementwise: negative length");
     if (n == 0) return FTH_OK;
-    FTH_ARG(a && y && (OP == Ew::Gelu || b), "elementwise: NULL operand");
+    FTH_ARG(a && y && (OP != Ew::Add || b), "elementwise: NULL operand");
     hipStream_t st = fth::resolve_stream(s);
     constexpr int EPV = Vec128<T>::n;
     int64_t done = 0;
-    if (aligned16(a) && aligned16(y) && (OP == Ew::Gelu || aligned16(b))) {
+    if (aligned16(a) && aligned16(y) && (OP != Ew::Add || aligned16(b))) {
         int64_t nvec = n / EPV;
         if (nvec > 0) {
             int64_t grid = fth::ceil_div(nvec, kBlock * kUnr);
@@ -782,6 +794,12 @@ int32_t fth_dev_gelu_f32(const float *x, float *y, int64_t n, fth_stream s) {
 }
 int32_t fth_dev_gelu_f64(const double *x, double *y, int64_t n, fth_stream s) {
     return launch_elementwise<double, Ew::Gelu>(x, nullptr, y, n, s);
+}
+int32_t fth_dev_gelu_tanh_f32(const float *x, float *y, int64_t n, fth_stream s) {
+    return launch_elementwise<float, Ew::GeluTanh>(x, nullptr, y, n, s);
+}
+int32_t fth_dev_gelu_tanh_f64(const double *x, double *y, int64_t n, fth_stream s) {
+    return launch_elementwise<double, Ew::GeluTanh>(x, nullptr, y, n, s);
 }
 int32_t fth_dev_add_f32(const float *a, const float *b, float *y, int64_t n, fth_stream s) {
     return launch_elementwise<float, Ew::Add>(a, b, y, n, s);

@@ -12,7 +12,8 @@ import numpy as np
 from . import _lib
 from .core import check
 
-EPI_NONE, EPI_BIAS, EPI_GELU, EPI_RESIDUAL = 0, 1, 2, 4
+EPI_NONE, EPI_BIAS, EPI_GELU, EPI_RESIDUAL, EPI_GELU_TANH = 0, 1, 2, 4, 8
+ACT_GELU_ERF, ACT_GELU_TANH = 0, 1
 
 
 def is_available() -> bool:
@@ -165,6 +166,10 @@ def rms_norm(x, weight, y, batch, norm_size, eps, stream=None):
 
 def gelu(x, y, n, stream=None):
     check(getattr(_lib.load(), "fth_dev_gelu_" + _sfx(x))(_ptr(x), _ptr(y), n, stream))
+
+
+def gelu_tanh(x, y, n, stream=None):
+    check(getattr(_lib.load(), "fth_dev_gelu_tanh_" + _sfx(x))(_ptr(x), _ptr(y), n, stream))
 
 
 def add(a, b, y, n, stream=None):

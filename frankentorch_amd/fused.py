@@ -97,6 +97,9 @@ class Batch:
     def gelu(self, x) -> HipTensor:
         return self._op(_lib.load().fth_batch_gelu, _h(x))
 
+    def gelu_tanh(self, x) -> HipTensor:
+        return self._op(_lib.load().fth_batch_gelu_tanh, _h(x))
+
     def add(self, a, b) -> HipTensor:
         return self._op(_lib.load().fth_batch_add, _h(a), _h(b))
 
@@ -135,13 +138,16 @@ class EncoderHip:
     """Pre-LN transformer stack with resident weights (EncoderGpu, fused.rs:1024-1190)."""
 
     def __init__(self, d_model: int, n_heads: int, d_ff: int, layers: Sequence[dict], ln_eps: float = 1e-5,
-                 causal: bool = True):
+                 causal: bool = True, gelu_tanh: bool = False):
+        """gelu_tanh: the tanh form the Metal encoder computes (fused.rs:301-313) in place of ft-kernel-cpu's erf form."""
         self.d_model, self.n_heads, self.d_ff = d_model, n_heads, d_ff
         arr, keep = _pack_layers(layers)
         h = C.c_void_p()
         check(_lib.load().fth_encoder_new(d_model, n_heads, d_ff, ln_eps, 1 if causal else 0, arr, len(layers), C.byref(h)))
         self._e = h.value
         del keep
+        if gelu_tanh:
+            check(_lib.load().fth_encoder_set_activation(self._e, 1))
 
     def forward(self, x, batch: int, seq: int) -> np.ndarray:
         """Host in, host out."""
@@ -165,7 +171,8 @@ class EncoderHip:
 class Gpt2Hip:
     """GPT-2-shaped decoder: learned positions, pre-LN causal blocks, final LN, tied LM head."""
 
-    def __init__(self, wte, wpe, layers: Sequence[dict], lnf_w, lnf_b, n_heads: int, ln_eps: float = 1e-5):
+    def __init__(self, wte, wpe, layers: Sequence[dict], lnf_w, lnf_b, n_heads: int, ln_eps: float = 1e-5,
+                 gelu_tanh: bool = False):
         wte = np.ascontiguousarray(wte, dtype=np.float32)
         wpe = np.ascontiguousarray(wpe, dtype=np.float32)
         self.vocab, self.d_model = wte.shape
@@ -180,6 +187,8 @@ class Gpt2Hip:
                                        None if lb is None else lb.ctypes.data, C.byref(h)))
         self._g = h.value
         del keep
+        if gelu_tanh:  # GPT-2 checkpoints were trained with the tanh form
+            check(_lib.load().fth_gpt2_set_activation(self._g, 1))
 
     def forward_dev(self, ids: DeviceBuffer, batch: int, seq: int, logits: Optional[DeviceBuffer],
                     argmax: Optional[DeviceBuffer], stream=None) -> None:

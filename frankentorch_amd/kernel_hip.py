@@ -200,6 +200,15 @@ def gelu_tensor_contiguous_f64(inp, meta):
     return _gelu("fth_gelu_tensor_contiguous_f64", np.float64, inp, meta)
 
 
+def gelu_tanh_tensor_contiguous_f32(inp, meta):
+    """0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))), GELU::tanh() (crates/ft-nn/src/lib.rs:1949-1957)."""
+    return _gelu("fth_gelu_tanh_tensor_contiguous_f32", np.float32, inp, meta)
+
+
+def gelu_tanh_tensor_contiguous_f64(inp, meta):
+    return _gelu("fth_gelu_tanh_tensor_contiguous_f64", np.float64, inp, meta)
+
+
 def _index_select(name, dtype, inp, meta: TensorMeta, dim, indices):
     inp = _slice(inp, dtype)
     idx = _slice(indices, np.float64)

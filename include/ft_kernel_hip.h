@@ -164,6 +164,11 @@ int32_t fth_dev_rms_norm_f64(const double *x, const double *weight, double *y, i
 /* gelu_tensor_contiguous_f32 (crates/ft-kernel-cpu/src/lib.rs:37123-37127, 36966-36969): erf form. */
 int32_t fth_dev_gelu_f32(const float *x, float *y, int64_t n, fth_stream s);
 int32_t fth_dev_gelu_f64(const double *x, double *y, int64_t n, fth_stream s);
+/* tanh-form GELU 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))): the `gelu` kernel of the reference's fused GPU module
+ * (crates/ft-kernel-metal/src/fused.rs:301-313; f32 keeps its |x| >= 10 clamp) and GELU::tanh()
+ * (crates/ft-nn/src/lib.rs:1924-1957, golden values :21985-22004). */
+int32_t fth_dev_gelu_tanh_f32(const float *x, float *y, int64_t n, fth_stream s);
+int32_t fth_dev_gelu_tanh_f64(const double *x, double *y, int64_t n, fth_stream s);
 /* add_tensor_contiguous_f32 (crates/ft-kernel-cpu/src/lib.rs:36870-36877): exact IEEE l + r. */
 int32_t fth_dev_add_f32(const float *a, const float *b, float *y, int64_t n, fth_stream s);
 int32_t fth_dev_add_f64(const double *a, const double *b, double *y, int64_t n, fth_stream s);
@@ -214,9 +219,10 @@ int32_t fth_dev_permute_0213_f64(const double *src, double *dst, int64_t d0, int
  * Epilogue, applied to the rounded product in this order (each its own rounding):
  *   FTH_EPI_BIAS      + bias[n]             (linear_tensor_f32, :17336-17351)
  *   FTH_EPI_GELU      gelu_erf(.)           (:36966-36969)
+ *   FTH_EPI_GELU_TANH gelu_tanh(.) in place of gelu_erf (crates/ft-kernel-metal/src/fused.rs:301-313; not with FTH_EPI_GELU)
  *   FTH_EPI_RESIDUAL  + residual[m, n]      (row pitch ldc; add_tensor_contiguous_f32)
  * k == 0 writes zeros (or the epilogue of zero); m == 0 or n == 0 returns at once. */
-enum { FTH_EPI_NONE = 0, FTH_EPI_BIAS = 1, FTH_EPI_GELU = 2, FTH_EPI_RESIDUAL = 4 };
+enum { FTH_EPI_NONE = 0, FTH_EPI_BIAS = 1, FTH_EPI_GELU = 2, FTH_EPI_RESIDUAL = 4, FTH_EPI_GELU_TANH = 8 };
 typedef struct fth_gemm_desc {
     int64_t m, n, k;
     int64_t lda, ldb, ldc;
@@ -451,6 +457,11 @@ int32_t fth_sdpa_backward_f64(const double *q, size_t q_len, const double *k, si
 /* gelu_tensor_contiguous_f32 (:37123) / _f64 (:3657); add_tensor_contiguous_f32 (:36870) / _f64 */
 int32_t fth_gelu_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta,
                                        float *out, size_t out_cap, size_t *out_len);
+/* The tanh form through the same validation (session op tensor_gelu_tanh behind GELU::tanh(), crates/ft-nn/src/lib.rs:1949-1957). */
+int32_t fth_gelu_tanh_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta, float *out, size_t out_cap,
+                                            size_t *out_len);
+int32_t fth_gelu_tanh_tensor_contiguous_f64(const double *input, size_t input_len, const fth_meta *meta, double *out, size_t out_cap,
+                                            size_t *out_len);
 int32_t fth_gelu_tensor_contiguous_f64(const double *input, size_t input_len, const fth_meta *meta,
                                        double *out, size_t out_cap, size_t *out_len);
 int32_t fth_add_tensor_contiguous_f32(const float *lhs, size_t lhs_len, const float *rhs, size_t rhs_len,
@@ -509,7 +520,8 @@ int32_t fth_batch_linear(fth_batch *b, const fth_tensor *a, const fth_tensor *w,
 int32_t fth_batch_matmul(fth_batch *b, const fth_tensor *a, const fth_tensor *rhs, fth_tensor **out);
 int32_t fth_batch_layernorm(fth_batch *b, const fth_tensor *x, const fth_tensor *gamma, const fth_tensor *beta, float eps, fth_tensor **out);
 int32_t fth_batch_rmsnorm(fth_batch *b, const fth_tensor *x, const fth_tensor *gamma, float eps, fth_tensor **out);
-int32_t fth_batch_gelu(fth_batch *b, const fth_tensor *x, fth_tensor **out);
+int32_t fth_batch_gelu(fth_batch *b, const fth_tensor *x, fth_tensor **out);      /* erf form, the ft-kernel-cpu arithmetic */
+int32_t fth_batch_gelu_tanh(fth_batch *b, const fth_tensor *x, fth_tensor **out); /* tanh form, Batch::gelu's own (fused.rs:301-313, 814-825) */
 int32_t fth_batch_add(fth_batch *b, const fth_tensor *x, const fth_tensor *y, fth_tensor **out);
 int32_t fth_batch_softmax(fth_batch *b, const fth_tensor *x, fth_tensor **out);
 /* Multi-head attention over [seq, d_model] q/k/v with n_heads heads (Batch::mha, :861-925);
@@ -537,6 +549,11 @@ typedef struct fth_encoder fth_encoder;
 int32_t fth_encoder_new(int64_t d_model, int64_t n_heads, int64_t d_ff, float ln_eps, int32_t causal,
                         const fth_layer_weights *layers, int64_t n_layers, fth_encoder **out);
 int32_t fth_encoder_free(fth_encoder *e);
+/* Feed-forward activation of the blocks: the erf form of ft-kernel-cpu (default) or the tanh form the reference's
+ * Metal encoder computes (crates/ft-kernel-metal/src/fused.rs:301-313) and GPT-2 checkpoints were trained with.
+ * Refused once a graph of this encoder has been captured. */
+enum { FTH_ACT_GELU_ERF = 0, FTH_ACT_GELU_TANH = 1 };
+int32_t fth_encoder_set_activation(fth_encoder *e, int32_t activation);
 /* Host in / host out (EncoderGpu::forward, :1136-1146). */
 int32_t fth_encoder_forward(fth_encoder *e, const float *input, int64_t batch, int64_t seq, float *out, size_t out_cap);
 /* Resident in / resident out on stream `s`; no synchronisation. `x` [batch*seq, d_model]. */
@@ -550,6 +567,7 @@ int32_t fth_gpt2_new(int64_t vocab, int64_t max_pos, int64_t d_model, int64_t n_
                      const float *wte, const float *wpe, const fth_layer_weights *layers, int64_t n_layers,
                      const float *lnf_w, const float *lnf_b, fth_gpt2 **out);
 int32_t fth_gpt2_free(fth_gpt2 *g);
+int32_t fth_gpt2_set_activation(fth_gpt2 *g, int32_t activation); /* FTH_ACT_GELU_ERF (default) | FTH_ACT_GELU_TANH */
 /* ids: device f64 token-id values [batch*seq] (indices are float-valued tensors in the reference,
  * crates/ft-nn/examples/bert_rerank_spike.rs:61-63). logits_dev [batch*seq, vocab] and
  * argmax_dev [batch*seq] (f32 index values) may each be NULL to skip that output; when logits_dev

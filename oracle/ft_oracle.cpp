@@ -192,6 +192,15 @@ template <typename T> void rms_norm_impl(const T *x, const T *w, T *y, int64_t b
 // gelu_value_f32 (KC:36966-36969); f64 form KC:1924-1929.
 inline float gelu_value(float x) { return 0.5f * x * (1.0f + t_erf(x * 0.70710678118654752440f)); }
 inline double gelu_value(double x) { return 0.5 * x * (1.0 + t_erf(x * 0.70710678118654752440)); }
+// tanh-form GELU: the `gelu` kernel of the fused GPU module (crates/ft-kernel-metal/src/fused.rs:301-313, f32, with its
+// |x| >= 10 clamp; the CPU check of that kernel at :1256-1259 uses the same expression) and GELU::tanh()
+// (crates/ft-nn/src/lib.rs:1924-1957; four golden values at :21985-22004).
+inline float gelu_tanh_value(float x) {
+    if (x >= 10.0f) return x;
+    if (x <= -10.0f) return 0.0f;
+    return 0.5f * x * (1.0f + std::tanh(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+}
+inline double gelu_tanh_value(double x) { return 0.5 * x * (1.0 + std::tanh(0.79788456080286535588 * (x + 0.044715 * x * x * x))); }
 
 // GEMM truth for f32: accumulate in f64 (each product of two f32 is exact in f64), round once.
 // b_kn is [k, n] row-major with pitch ldb.
@@ -451,7 +460,7 @@ struct LayerW {
 // 14709-14744): x = x + MHA(LN1(x)); x = x + W2.gelu(W1.LN2(x)); MHA as
 // MultiheadAttention::forward_qkv_masked (crates/ft-nn/src/lib.rs:5088-5198), scale 1/sqrt(hd).
 void encoder_layer_impl(const LayerW &w, float *x, int64_t batch, int64_t seq, int64_t d_model, int64_t heads,
-                        int64_t d_ff, float eps, int causal) {
+                        int64_t d_ff, float eps, int causal, int gelu_tanh = 0) {
     const int64_t tokens = batch * seq, hd = d_model / heads;
     std::vector<float> h((size_t)tokens * d_model), qv(h.size()), kv(h.size()), vv(h.size());
     std::vector<float> qh(h.size()), kh(h.size()), vh(h.size()), ctx(h.size()), merged(h.size()), proj(h.size());
@@ -470,7 +479,7 @@ void encoder_layer_impl(const LayerW &w, float *x, int64_t batch, int64_t seq, i
     layer_norm_impl<float>(x, nullptr, w.ln2_w, w.ln2_b, h.data(), tokens, d_model, eps);
     std::vector<float> f1((size_t)tokens * d_ff);
     linear_impl<float>(h.data(), w.w1, w.b1, tokens, d_model, d_ff, f1.data());
-    for (size_t i = 0; i < f1.size(); ++i) f1[i] = gelu_value(f1[i]);
+    for (size_t i = 0; i < f1.size(); ++i) f1[i] = gelu_tanh ? gelu_tanh_value(f1[i]) : gelu_value(f1[i]);
     linear_impl<float>(f1.data(), w.w2, w.b2, tokens, d_ff, d_model, proj.data());
     for (size_t i = 0; i < proj.size(); ++i) x[i] = x[i] + proj[i];
 }
@@ -840,6 +849,14 @@ void fto_gelu_f32(const float *x, float *y, int64_t n) {
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < n; ++i) y[i] = gelu_value(x[i]);
 }
+void fto_gelu_tanh_f32(const float *x, float *y, int64_t n) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i) y[i] = gelu_tanh_value(x[i]);
+}
+void fto_gelu_tanh_f64(const double *x, double *y, int64_t n) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i) y[i] = gelu_tanh_value(x[i]);
+}
 void fto_gelu_f64(const double *x, double *y, int64_t n) {
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < n; ++i) y[i] = gelu_value(x[i]);
@@ -978,6 +995,12 @@ void fto_encoder_layer_f32(const float *const *w, float *x, int64_t batch, int64
                            int64_t heads, int64_t d_ff, float eps, int causal) {
     LayerW lw = {w[0], w[1], w[2], w[3], w[4], w[5], w[6], w[7], w[8], w[9], w[10], w[11], w[12], w[13], w[14], w[15]};
     encoder_layer_impl(lw, x, batch, seq, d_model, heads, d_ff, eps, causal);
+}
+// The same block with the tanh-form GELU (what the Metal encoder computes, fused.rs:301-313).
+void fto_encoder_layer_gelu_tanh_f32(const float *const *w, float *x, int64_t batch, int64_t seq, int64_t d_model,
+                                     int64_t heads, int64_t d_ff, float eps, int causal) {
+    LayerW lw = {w[0], w[1], w[2], w[3], w[4], w[5], w[6], w[7], w[8], w[9], w[10], w[11], w[12], w[13], w[14], w[15]};
+    encoder_layer_impl(lw, x, batch, seq, d_model, heads, d_ff, eps, causal, 1);
 }
 
 // GPT-2-shaped forward: x = wte[ids] + wpe[pos] (Embedding::forward, crates/ft-nn/src/lib.rs:

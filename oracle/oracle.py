@@ -112,6 +112,14 @@ def gelu(x):
     return y
 
 
+def gelu_tanh(x):
+    x = _c(x)
+    sfx, _ = _sfx(x.dtype)
+    y = np.empty_like(x)
+    getattr(lib(), "fto_gelu_tanh_" + sfx)(_p(x), _p(y), _i64(x.size))
+    return y
+
+
 def add(a, b):
     a = _c(a)
     b = _c(b)
@@ -359,14 +367,14 @@ def _layer_ptrs(layers):
     return arr, keep
 
 
-def encoder_layer(layer, x, batch, seq, heads, eps, causal):
+def encoder_layer(layer, x, batch, seq, heads, eps, causal, gelu_tanh=False):
     """One pre-LN block on x [batch*seq, d_model]; returns a new array."""
     x = np.array(x, dtype=np.float32, order="C", copy=True)
     d_model = x.shape[-1]
     d_ff = layer["w1"].shape[0]
     arr, keep = _layer_ptrs([layer])
-    lib().fto_encoder_layer_f32(arr, _p(x), _i64(batch), _i64(seq), _i64(d_model), _i64(heads), _i64(d_ff),
-                                C.c_float(eps), C.c_int(1 if causal else 0))
+    fn = lib().fto_encoder_layer_gelu_tanh_f32 if gelu_tanh else lib().fto_encoder_layer_f32
+    fn(arr, _p(x), _i64(batch), _i64(seq), _i64(d_model), _i64(heads), _i64(d_ff), C.c_float(eps), C.c_int(1 if causal else 0))
     del keep
     return x
 

@@ -84,6 +84,9 @@ IN_SOURCE = [
      "input": [1, 2, 3, 4], "shape": [2, 2], "dim": 0, "index": [1.0e300]},
     {"name": "index_select_negative_index", "source": "KC:57866-57875", "op": "index_select_error", "dtype": "f64",
      "input": [1, 2, 3, 4, 5, 6], "shape": [3, 2], "dim": 0, "index": [-1.0]},
+    {"name": "gelu_tanh_module_matches_torch", "source": "crates/ft-nn/src/lib.rs:21985-22004", "op": "gelu_tanh", "dtype": "f64",
+     "input": [-1.0, 0.5, 1.0, 2.0],
+     "expected_output": [-0.15880800939172324, 0.34571400982514394, 0.8411919906082768, 1.954597694087775], "abs_tol": 1e-9},
     {"name": "matmul_unit_vector_dot_k10001", "source": "KC:53274-53310", "op": "matmul_unit_dot", "dtype": "f64",
      "k": 10001, "expected": 1.0, "abs_tol": 1e-14},
 ]

@@ -183,3 +183,21 @@ def test_masked_gqa_sdpa_restatement_is_pinned(oracle):
     f = np.float32
     o32 = oracle.sdpa_forward_masked_gqa(q.astype(f), k.astype(f), v.astype(f), f(scale), mask2d.astype(f))
     assert np.allclose(o32, oracle.sdpa_forward_masked_gqa(q, k, v, scale, mask2d), atol=2e-6)
+
+
+def test_gelu_tanh_restatement_is_pinned(oracle, vectors):
+    c = {v["name"]: v for v in vectors["in_source"]}["gelu_tanh_module_matches_torch"]
+    x = np.array(c["input"], np.float64)
+    assert np.max(np.abs(oracle.gelu_tanh(x) - np.array(c["expected_output"]))) <= c["abs_tol"]
+    assert np.max(np.abs(oracle.gelu_tanh(x.astype(np.float32)) - np.array(c["expected_output"]))) <= 2e-7
+    # a library routine for the rest of the range: torch's CPU kernel of the same approximation
+    import torch
+
+    xs = np.linspace(-12.0, 12.0, 4801)
+    want = torch.nn.functional.gelu(torch.from_numpy(xs), approximate="tanh").numpy()
+    assert np.max(np.abs(oracle.gelu_tanh(xs) - want)) <= 1e-14
+    want32 = torch.nn.functional.gelu(torch.from_numpy(xs.astype(np.float32)), approximate="tanh").numpy()
+    assert np.max(np.abs(oracle.gelu_tanh(xs.astype(np.float32)) - want32)) <= 1e-6
+    # equals x * sigmoid(2u), the form the GEMM epilogue computes
+    u = 0.7978845608028654 * (xs + 0.044715 * xs ** 3)
+    assert np.max(np.abs(oracle.gelu_tanh(xs) - xs / (1.0 + np.exp(-2.0 * u)))) <= 1e-14
