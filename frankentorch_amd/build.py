@@ -26,6 +26,7 @@ HIP_SOURCES = [
     "sdpa.hip",
     "backward.hip",
     "lossops.hip",
+    "ingest.hip",
     "host_api.hip",
     "resident.hip",
 ]

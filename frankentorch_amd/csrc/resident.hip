@@ -21,6 +21,7 @@
 #include <map>
 #include <mutex>
 #include <new>
+#include <string>
 #include <tuple>
 #include <unordered_map>
 #include <vector>
@@ -647,6 +648,130 @@ int32_t fth_gpt2_new(int64_t vocab, int64_t max_pos, int64_t d_model, int64_t n_
         return rc;
     }
     *out = g;
+    return FTH_OK;
+}
+
+// ---- GPT-2 from a safetensors checkpoint -------------------------------------------------------
+namespace {
+
+struct CheckpointReader {
+    const fth_safetensors *f;
+    Stack &st;
+    std::string prefix;
+
+    bool has(const std::string &name) const {
+        fth_safetensors_tensor info;
+        const std::string full = prefix + name;
+        for (int64_t i = 0, n = fth_safetensors_count(f); i < n; ++i)
+            if (full == fth_safetensors_name(f, i)) return fth_safetensors_info(f, full.c_str(), &info) == FTH_OK;
+        return false;
+    }
+    int32_t shape(const std::string &name, int ndim, uint64_t *dims) const {
+        fth_safetensors_tensor info;
+        const std::string full = prefix + name;
+        if (!has(name)) return fth::set_error(FTH_ERR_CORRUPT, "checkpoint has no tensor '%s'", full.c_str());
+        if (int32_t rc = fth_safetensors_info(f, full.c_str(), &info)) return rc;
+        if (info.ndim != ndim) return fth::set_error(FTH_ERR_CORRUPT, "checkpoint tensor '%s' has %d dimensions, expected %d", full.c_str(), info.ndim, ndim);
+        for (int i = 0; i < ndim; ++i) dims[i] = info.shape[i];
+        return FTH_OK;
+    }
+    // Reads `name` (shape [d0] or [d0, d1] as stored) into a new device block owned by the stack.
+    int32_t load(const std::string &name, uint64_t d0, uint64_t d1, bool transpose, float **dev) {
+        uint64_t dims[2] = {0, 0};
+        const int ndim = d1 ? 2 : 1;
+        if (int32_t rc = shape(name, ndim, dims)) return rc;
+        if (dims[0] != d0 || (ndim == 2 && dims[1] != d1))
+            return fth::set_error(FTH_ERR_CORRUPT, "checkpoint tensor '%s%s' is [%llu, %llu], expected [%llu, %llu]", prefix.c_str(), name.c_str(),
+                                  (unsigned long long)dims[0], (unsigned long long)dims[1], (unsigned long long)d0, (unsigned long long)d1);
+        const size_t n = (size_t)(d0 * (d1 ? d1 : 1));
+        void *p = nullptr;
+        if (int32_t rc = fth::pool_alloc(&p, n * sizeof(float))) return rc;
+        st.owned.push_back(p);
+        *dev = static_cast<float *>(p);
+        return fth_safetensors_read_f32_dev(f, (prefix + name).c_str(), transpose ? 1 : 0, *dev, n, nullptr);
+    }
+};
+
+}  // namespace
+
+int32_t fth_gpt2_from_safetensors(const fth_safetensors *f, int64_t n_heads, float ln_eps, int32_t activation, fth_gpt2 **out) {
+    FTH_ARG(out != nullptr, "gpt2_from_safetensors: out is NULL");
+    *out = nullptr;
+    FTH_ARG(f != nullptr, "gpt2_from_safetensors: file is NULL");
+    FTH_ARG(activation == FTH_ACT_GELU_ERF || activation == FTH_ACT_GELU_TANH, "gpt2_from_safetensors: unknown activation %d", activation);
+    FTH_REQUIRE_DEVICE();
+    fth_gpt2 *g = new (std::nothrow) fth_gpt2();
+    if (!g) return fth::set_error(FTH_ERR_KERNEL, "gpt2_from_safetensors: host allocation failed");
+    Stack &st = g->stack;
+    CheckpointReader rd{f, st, ""};
+    if (!rd.has("wte.weight")) rd.prefix = "transformer.";
+    uint64_t e[2], pdim[2], fc[2];
+    int32_t rc = rd.shape("wte.weight", 2, e);
+    if (!rc) rc = rd.shape("wpe.weight", 2, pdim);
+    int64_t n_layers = 0;
+    while (!rc && rd.has("h." + std::to_string(n_layers) + ".ln_1.weight")) ++n_layers;
+    const uint64_t d = e[1];
+    uint64_t d_ff = d;
+    if (!rc && n_layers > 0) {
+        rc = rd.shape("h.0.mlp.c_fc.weight", 2, fc);
+        d_ff = fc[1];
+    }
+    if (!rc && pdim[1] != d) rc = fth::set_error(FTH_ERR_CORRUPT, "checkpoint: wpe.weight width %llu differs from wte.weight width %llu",
+                                                 (unsigned long long)pdim[1], (unsigned long long)d);
+    if (!rc) rc = check_dims((int64_t)d, n_heads, (int64_t)d_ff, n_layers);
+    if (!rc) {
+        st.d_model = (int64_t)d; st.n_heads = n_heads; st.d_ff = (int64_t)d_ff; st.eps = ln_eps; st.causal = 1;
+        st.gelu_epilogue = activation == FTH_ACT_GELU_TANH ? FTH_EPI_GELU_TANH : FTH_EPI_GELU;
+        g->vocab = (int64_t)e[0]; g->max_pos = (int64_t)pdim[0];
+        rc = rd.load("wte.weight", e[0], d, false, &g->wte);
+    }
+    if (!rc) rc = rd.load("wpe.weight", pdim[0], d, false, &g->wpe);
+    if (!rc) rc = rd.load("ln_f.weight", d, 0, false, &g->lnf_w);
+    if (!rc) rc = rd.load("ln_f.bias", d, 0, false, &g->lnf_b);
+    for (int64_t i = 0; !rc && i < n_layers; ++i) {
+        const std::string h = "h." + std::to_string(i) + ".";
+        LayerDev L = {};
+        // Conv1D weights are stored [in, out]; the linear kernels read [out, in], so c_attn.weight^T is the packed
+        // [3d, d] query / key / value matrix as it stands.
+        rc = rd.load(h + "ln_1.weight", d, 0, false, &L.ln1_w);
+        if (!rc) rc = rd.load(h + "ln_1.bias", d, 0, false, &L.ln1_b);
+        if (!rc) rc = rd.load(h + "attn.c_attn.weight", d, 3 * d, true, &L.wqkv);
+        if (!rc) rc = rd.load(h + "attn.c_attn.bias", 3 * d, 0, false, &L.bqkv);
+        if (!rc) rc = rd.load(h + "attn.c_proj.weight", d, d, true, &L.wo);
+        if (!rc) rc = rd.load(h + "attn.c_proj.bias", d, 0, false, &L.bo);
+        if (!rc) rc = rd.load(h + "ln_2.weight", d, 0, false, &L.ln2_w);
+        if (!rc) rc = rd.load(h + "ln_2.bias", d, 0, false, &L.ln2_b);
+        if (!rc) rc = rd.load(h + "mlp.c_fc.weight", d, d_ff, true, &L.w1);
+        if (!rc) rc = rd.load(h + "mlp.c_fc.bias", d_ff, 0, false, &L.b1);
+        if (!rc) rc = rd.load(h + "mlp.c_proj.weight", d_ff, d, true, &L.w2);
+        if (!rc) rc = rd.load(h + "mlp.c_proj.bias", d, 0, false, &L.b2);
+        if (!rc) st.layers.push_back(L);
+    }
+    if (!rc) {
+        void *p = nullptr;
+        rc = fth::pool_alloc(&p, sizeof(int64_t));
+        if (!rc) {
+            st.owned.push_back(p);
+            g->bad = static_cast<int64_t *>(p);
+        }
+    }
+    if (rc) {
+        delete g;
+        return rc;
+    }
+    *out = g;
+    return FTH_OK;
+}
+
+int32_t fth_gpt2_dims(const fth_gpt2 *g, int64_t *vocab, int64_t *max_pos, int64_t *d_model, int64_t *n_heads, int64_t *d_ff,
+                      int64_t *n_layers) {
+    FTH_ARG(g != nullptr, "gpt2_dims: model is NULL");
+    if (vocab) *vocab = g->vocab;
+    if (max_pos) *max_pos = g->max_pos;
+    if (d_model) *d_model = g->stack.d_model;
+    if (n_heads) *n_heads = g->stack.n_heads;
+    if (d_ff) *d_ff = g->stack.d_ff;
+    if (n_layers) *n_layers = (int64_t)g->stack.layers.size();
     return FTH_OK;
 }
 

@@ -94,6 +94,8 @@ const char *fth_status_name(int32_t code) {
         case FTH_ERR_STREAM: return "CommandBuffer";
         case FTH_ERR_INVALID_ARGUMENT: return "InvalidArgument";
         case FTH_ERR_OUTPUT_TOO_SMALL: return "OutputTooSmall";
+        case FTH_ERR_CORRUPT: return "Corrupt";
+        case FTH_ERR_IO: return "Io";
         default: return "Unknown";
     }
 }

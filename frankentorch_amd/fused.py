@@ -190,6 +190,22 @@ class Gpt2Hip:
         if gelu_tanh:  # GPT-2 checkpoints were trained with the tanh form
             check(_lib.load().fth_gpt2_set_activation(self._g, 1))
 
+    @classmethod
+    def from_safetensors(cls, source, n_heads: int, ln_eps: float = 1e-5, gelu_tanh: bool = True) -> "Gpt2Hip":
+        """A GPT-2 checkpoint (path, bytes or an open serialize.SafeTensorsFile) straight into resident buffers: Conv1D
+        weights are transposed and F16 / BF16 / F64 tensors converted on the GPU while loading."""
+        from .serialize import SafeTensorsFile
+
+        f = source if isinstance(source, SafeTensorsFile) else SafeTensorsFile(source)
+        h = C.c_void_p()
+        check(_lib.load().fth_gpt2_from_safetensors(f._h, n_heads, ln_eps, 1 if gelu_tanh else 0, C.byref(h)))
+        self = cls.__new__(cls)
+        self._g = h.value
+        dims = [C.c_int64() for _ in range(6)]
+        check(_lib.load().fth_gpt2_dims(self._g, *[C.byref(d) for d in dims]))
+        self.vocab, self.max_pos, self.d_model, self.n_heads, self.d_ff, self.n_layers = (d.value for d in dims)
+        return self
+
     def forward_dev(self, ids: DeviceBuffer, batch: int, seq: int, logits: Optional[DeviceBuffer],
                     argmax: Optional[DeviceBuffer], stream=None) -> None:
         check(_lib.load().fth_gpt2_forward_dev(self._g, ids.ptr, batch, seq, None if logits is None else logits.ptr,

@@ -59,13 +59,16 @@ enum {
     FTH_ERR_BUFFER_TOO_LARGE = 103,    /* Error::BufferTooLarge         */
     FTH_ERR_STREAM = 104,              /* Error::CommandBuffer(state)   */
     FTH_ERR_INVALID_ARGUMENT = 105,    /* reference would panic         */
-    FTH_ERR_OUTPUT_TOO_SMALL = 106     /* caller's out buffer < result  */
+    FTH_ERR_OUTPUT_TOO_SMALL = 106,    /* caller's out buffer < result  */
+    FTH_ERR_CORRUPT = 107,             /* TensorIOError::Corrupt{reason} (crates/ft-serialize) */
+    FTH_ERR_IO = 108                   /* TensorIOError::Io{path, source}                     */
 };
 
 /* DType / Device tags: crates/ft-core/src/lib.rs:23-35 and :176-179, plus the HIP device id the
  * backend adds to `Device`. Only F64 and F32 are computed here (crates/ft-dispatch/src/lib.rs:
  * 4123-4308 narrows F16/BF16 above the kernels). */
-enum { FTH_DTYPE_F64 = 0, FTH_DTYPE_F32 = 1 };
+enum { FTH_DTYPE_F64 = 0, FTH_DTYPE_F32 = 1, FTH_DTYPE_F16 = 2, FTH_DTYPE_BF16 = 3 }; /* the kernels compute in the first two;
+                                                                                       the other two are storage types of a weight file */
 enum { FTH_DEVICE_CPU = 0, FTH_DEVICE_CUDA = 1, FTH_DEVICE_HIP = 2 };
 
 #define FTH_MAX_DIMS 8
@@ -561,11 +564,59 @@ int32_t fth_encoder_forward_dev(fth_encoder *e, const float *x_dev, int64_t batc
 /* Captures forward_dev for (batch, seq) into a HIP graph and replays it: one launch per forward. */
 int32_t fth_encoder_forward_graph(fth_encoder *e, const float *x_dev, int64_t batch, int64_t seq, float *out_dev, fth_stream s);
 
+/* ------------------------------------------------------------------------------------------ */
+/* Weight ingestion: safetensors -> resident buffers                                           */
+/* ------------------------------------------------------------------------------------------ */
+/* load_safetensors (crates/ft-serialize/src/lib.rs:2170-2176), load_safetensors_from_bytes (:2179-2241) and
+ * load_safetensors_metadata (:2274-2286), for a caller whose tensors live on the GPU. open / open_bytes validate the
+ * whole container (the checks of safetensors 0.8.0's SafeTensors::deserialize, then the loader's own: only F64 / F32 /
+ * F16 / BF16 tensors, each of exactly numel * width bytes) and fail with FTH_ERR_CORRUPT where the reference returns
+ * TensorIOError::Corrupt, FTH_ERR_IO where it returns TensorIOError::Io. The file is memory-mapped; `open_bytes` borrows
+ * `data`, which must outlive the handle. Tensors are listed in name order (the reference's BTreeMap). */
+typedef struct fth_safetensors fth_safetensors;
+typedef struct fth_safetensors_tensor {
+    int32_t dtype; /* FTH_DTYPE_* as stored in the file */
+    int32_t ndim;
+    uint64_t shape[FTH_MAX_DIMS];
+    uint64_t numel;
+    uint64_t byte_len;
+} fth_safetensors_tensor;
+int32_t fth_safetensors_open(const char *path, fth_safetensors **out);
+int32_t fth_safetensors_open_bytes(const void *data, size_t len, fth_safetensors **out);
+int32_t fth_safetensors_close(fth_safetensors *f);
+int64_t fth_safetensors_count(const fth_safetensors *f);
+const char *fth_safetensors_name(const fth_safetensors *f, int64_t index); /* NULL past the end */
+int32_t fth_safetensors_info(const fth_safetensors *f, const char *name, fth_safetensors_tensor *info);
+/* The tensor's little-endian bytes as stored (what the reference decodes into a DenseTensor), into host memory. */
+int32_t fth_safetensors_read(const fth_safetensors *f, const char *name, void *dst, size_t dst_bytes);
+/* The tensor into device memory as f32 / f64, whatever its stored type (F16 / BF16 / F32 widen exactly; F64 -> f32
+ * rounds to nearest), optionally transposed when it is a matrix ([rows, cols] in the file -> [cols, rows] in dst; GPT-2
+ * checkpoints store their projections [in, out], the linear kernels read [out, in]). The bytes go through pinned staging
+ * buffers with asynchronous copies and are converted / transposed on the GPU. Synchronises `s` before returning. */
+int32_t fth_safetensors_read_f32_dev(const fth_safetensors *f, const char *name, int32_t transpose_2d, float *dst_dev, size_t dst_elems,
+                                     fth_stream s);
+int32_t fth_safetensors_read_f64_dev(const fth_safetensors *f, const char *name, int32_t transpose_2d, double *dst_dev, size_t dst_elems,
+                                     fth_stream s);
+/* The "__metadata__" string map: number of entries (-1 if the file has none) and lookup (NULL if absent). */
+int32_t fth_safetensors_metadata_count(const fth_safetensors *f);
+const char *fth_safetensors_metadata(const fth_safetensors *f, const char *key);
+
 /* GPT-2-shaped decoder: learned positions, pre-LN blocks, final LN, LM head tied to wte. */
 typedef struct fth_gpt2 fth_gpt2;
 int32_t fth_gpt2_new(int64_t vocab, int64_t max_pos, int64_t d_model, int64_t n_heads, int64_t d_ff, float ln_eps,
                      const float *wte, const float *wpe, const fth_layer_weights *layers, int64_t n_layers,
                      const float *lnf_w, const float *lnf_b, fth_gpt2 **out);
+/* The same model with its weights read from a GPT-2 checkpoint in safetensors form, straight into resident buffers:
+ * "wte.weight" [vocab, d], "wpe.weight" [max_pos, d], per layer i "h.i.ln_1.{weight,bias}", "h.i.attn.c_attn.{weight [d, 3d],
+ * bias}", "h.i.attn.c_proj.{weight [d, d], bias}", "h.i.ln_2.{weight,bias}", "h.i.mlp.c_fc.{weight [d, d_ff], bias}",
+ * "h.i.mlp.c_proj.{weight [d_ff, d], bias}", "ln_f.{weight,bias}", each optionally under a "transformer." prefix. The
+ * projection matrices are stored [in, out] and are transposed on the GPU while loading; F16 / BF16 / F64 tensors are
+ * converted to f32 there. Shapes are taken from the file; other tensors in it (attention mask buffers) are ignored.
+ * A missing or mis-shaped tensor is FTH_ERR_CORRUPT. activation: FTH_ACT_GELU_TANH is what GPT-2 was trained with. */
+int32_t fth_gpt2_from_safetensors(const fth_safetensors *f, int64_t n_heads, float ln_eps, int32_t activation, fth_gpt2 **out);
+/* vocab, max_pos, d_model, n_heads, d_ff, n_layers of a model (any pointer may be NULL). */
+int32_t fth_gpt2_dims(const fth_gpt2 *g, int64_t *vocab, int64_t *max_pos, int64_t *d_model, int64_t *n_heads, int64_t *d_ff,
+                      int64_t *n_layers);
 int32_t fth_gpt2_free(fth_gpt2 *g);
 int32_t fth_gpt2_set_activation(fth_gpt2 *g, int32_t activation); /* FTH_ACT_GELU_ERF (default) | FTH_ACT_GELU_TANH */
 /* ids: device f64 token-id values [batch*seq] (indices are float-valued tensors in the reference,

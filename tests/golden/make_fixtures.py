@@ -5,6 +5,7 @@ Sources (read as text / JSON from the reference checkout; nothing is imported or
   * crates/ft-conformance/fixtures/*.json          conformance cases (copied case by case)
   * artifacts/optimization/golden_outputs/*.txt    golden output text files (numbers parsed out)
   * artifacts/perf/frankentorch-kgs4.54/pass1_golden_gemm_bt.digest_lines   f64 GEMM checksums
+  * fuzz/corpus/ft_serialize_safetensors/*         seed containers of the safetensors fuzz target (hex)
   * in-source #[test] literals of crates/ft-kernel-cpu/src/lib.rs, transcribed by hand below with
     their line numbers (the literal input vectors and the asserted outputs)
 
@@ -164,10 +165,18 @@ def golden_texts():
     return out
 
 
+def safetensors_corpus():
+    """The seed inputs of the reference's safetensors fuzz target (fuzz/corpus/ft_serialize_safetensors/*, which its unit
+    test fuzz_corpus_safetensors_does_not_panic reads): small binary containers, kept as hex strings."""
+    d = os.path.join(REF, "fuzz", "corpus", "ft_serialize_safetensors")
+    return [{"name": n, "hex": open(os.path.join(d, n), "rb").read().hex()} for n in sorted(os.listdir(d))]
+
+
 def main():
     if not os.path.isdir(REF):
         sys.exit("reference checkout not found at %s" % REF)
-    doc = {"conformance": conformance_cases(), "in_source": IN_SOURCE, "golden_text": golden_texts()}
+    doc = {"conformance": conformance_cases(), "in_source": IN_SOURCE, "golden_text": golden_texts(),
+           "safetensors_corpus": safetensors_corpus()}
     with open(OUT, "w") as f:
         json.dump(doc, f, indent=1, sort_keys=True)
         f.write("\n")
