@@ -77,6 +77,7 @@ class LayerWeights(C.Structure):
 
 
 _SCALARS = {
+    "int8_t": C.c_int8,
     "int32_t": C.c_int32,
     "int64_t": C.c_int64,
     "uint64_t": C.c_uint64,

@@ -27,6 +27,7 @@ HIP_SOURCES = [
     "backward.hip",
     "lossops.hip",
     "ingest.hip",
+    "int8ops.hip",
     "host_api.hip",
     "resident.hip",
 ]

@@ -722,6 +722,55 @@ int32_t cross_entropy_impl(bool backward, const T *logits, size_t logits_len, co
     return fetch(out, dout, n_out);
 }
 
+// quantize_per_output_channel_i8 / quantize_rows_i8 (crates/ft-kernel-cpu/src/lib.rs:37836-37905): the two functions
+// are the same arithmetic on the rows of a matrix.
+int32_t quantize_i8_impl(const float *w, size_t w_len, size_t rows, size_t cols, int8_t *q, size_t q_cap, float *scales, size_t scales_cap) {
+    uint64_t total;
+    FTH_ARG(checked_mul(rows, cols, &total), "quantize_i8: rows * cols overflows");
+    FTH_ARG(w_len == total, "quantize_i8: slice length %zu must equal rows * cols = %llu", w_len, (unsigned long long)total);
+    if (int32_t rc = check_out(q, q_cap, (size_t)total)) return rc;
+    if (int32_t rc = check_out(scales, scales_cap, rows)) return rc;
+    if (rows == 0) return FTH_OK;
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    float *dw = nullptr, *ds = nullptr;
+    int8_t *dq = nullptr;
+    if (int32_t rc = stage_in(sc, w, (size_t)total, &dw)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)total, &dq)) return rc;
+    if (int32_t rc = stage_out(sc, rows, &ds)) return rc;
+    if (int32_t rc = fth_dev_quantize_rows_i8(dw, (int64_t)rows, (int64_t)cols, dq, ds, nullptr)) return rc;
+    if (int32_t rc = fetch(q, dq, (size_t)total)) return rc;
+    return fetch(scales, ds, rows);
+}
+
+// linear_int8_dynamic_f32 (crates/ft-kernel-cpu/src/lib.rs:37966-38060)
+int32_t linear_int8_impl(const float *x, size_t x_len, size_t m, size_t k, const int8_t *w_i8, size_t w_len, const float *w_scales,
+                         size_t w_scales_len, size_t n, const float *bias, size_t bias_len, float *out, size_t out_cap) {
+    uint64_t xn, wn, on;
+    FTH_ARG(checked_mul(m, k, &xn) && checked_mul(n, k, &wn) && checked_mul(m, n, &on), "linear_int8: shape product overflows");
+    FTH_ARG(x_len == xn, "x length must equal m*k");
+    FTH_ARG(w_len == wn, "w_i8 length must equal n*k");
+    FTH_ARG(w_scales_len == n, "w_scales length must equal n");
+    FTH_ARG(bias == nullptr || bias_len == n, "bias length must equal n");
+    if (int32_t rc = check_out(out, out_cap, (size_t)on)) return rc;
+    if (on == 0) return FTH_OK;
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    float *dx = nullptr, *dws = nullptr, *db = nullptr, *dout = nullptr;
+    int8_t *dw = nullptr;
+    void *ws = nullptr;
+    if (int32_t rc = stage_in(sc, x, (size_t)xn, &dx)) return rc;
+    if (int32_t rc = stage_in(sc, w_i8, (size_t)wn, &dw)) return rc;
+    if (int32_t rc = stage_in(sc, w_scales, n, &dws)) return rc;
+    if (bias)
+        if (int32_t rc = stage_in(sc, bias, n, &db)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)on, &dout)) return rc;
+    const size_t ws_bytes = fth_dev_linear_int8_workspace_bytes((int64_t)m, (int64_t)k);
+    if (int32_t rc = sc.get(&ws, ws_bytes)) return rc;
+    if (int32_t rc = fth_dev_linear_int8_dynamic_f32(dx, (int64_t)m, (int64_t)k, dw, dws, (int64_t)n, db, dout, ws, ws_bytes, nullptr)) return rc;
+    return fetch(out, dout, (size_t)on);
+}
+
 // ---- backward entry points on host slices ----
 // Several outputs per call, each with its own capacity; every output the call produces must fit.
 template <typename T> int32_t fetch_no_sync(T *host, const T *dev, size_t n) {
@@ -1067,6 +1116,18 @@ int32_t fth_sdpa_forward_masked_gqa_f64(const double *q, size_t q_len, const dou
                                         size_t h_q, size_t h_kv, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, double scale,
                                         const double *mask, size_t mask_len, size_t mask_bh_stride, double *out, size_t out_cap) {
     return sdpa_masked_impl<double>(q, q_len, k, k_len, v, v_len, batch, h_q, h_kv, seq_q, seq_k, d_k, d_v, scale, mask, mask_len, mask_bh_stride, out, out_cap);
+}
+
+int32_t fth_quantize_per_output_channel_i8(const float *w, size_t w_len, size_t rows, size_t cols, int8_t *q, size_t q_cap, float *scales,
+                                           size_t scales_cap) {
+    return quantize_i8_impl(w, w_len, rows, cols, q, q_cap, scales, scales_cap);
+}
+int32_t fth_quantize_rows_i8(const float *x, size_t x_len, size_t rows, size_t cols, int8_t *q, size_t q_cap, float *scales, size_t scales_cap) {
+    return quantize_i8_impl(x, x_len, rows, cols, q, q_cap, scales, scales_cap);
+}
+int32_t fth_linear_int8_dynamic_f32(const float *x, size_t x_len, size_t m, size_t k, const int8_t *w_i8, size_t w_len, const float *w_scales,
+                                    size_t w_scales_len, size_t n, const float *bias, size_t bias_len, float *out, size_t out_cap) {
+    return linear_int8_impl(x, x_len, m, k, w_i8, w_len, w_scales, w_scales_len, n, bias, bias_len, out, out_cap);
 }
 
 }  // extern "C"

@@ -303,5 +303,22 @@ def sdpa_forward_masked(desc, scale, q, k, v, mask, mask_bh_stride, out, stream=
                                                                          _ptr(mask), mask_bh_stride, _ptr(out), stream))
 
 
+def quantize_rows_i8(x, rows, cols, q, scales, stream=None):
+    """Per-row symmetric int8 (activations, or weights per output channel): q int8 [rows, cols], scales f32 [rows]."""
+    check(_lib.load().fth_dev_quantize_rows_i8(_ptr(x), rows, cols, _ptr(q), _ptr(scales), stream))
+
+
+def linear_int8_workspace_bytes(m, k) -> int:
+    return int(_lib.load().fth_dev_linear_int8_workspace_bytes(m, k))
+
+
+def linear_int8_dynamic(x, m, k, w_i8, w_scales, n, bias, out, workspace=None, stream=None):
+    """out [m, n] = dequant(quant_rows(x) . w_i8^T) + bias; returns the workspace buffer so callers can reuse it."""
+    workspace = _workspace(linear_int8_workspace_bytes(m, k), workspace)
+    check(_lib.load().fth_dev_linear_int8_dynamic_f32(_ptr(x), m, k, _ptr(w_i8), _ptr(w_scales), n, _ptr(bias), _ptr(out),
+                                                      _ptr(workspace), workspace.nbytes, stream))
+    return workspace
+
+
 def default_scale(head_dim: int) -> float:
     return 1.0 / math.sqrt(head_dim)

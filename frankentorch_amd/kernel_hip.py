@@ -345,6 +345,34 @@ def _sdpa(name, dtype, q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal):
     return out
 
 
+def _quantize_i8(name, w, rows, cols):
+    w = _slice(w, np.float32)
+    q, scales = np.empty(rows * cols, np.int8), np.empty(rows, np.float32)
+    check(getattr(_lib.load(), name)(_p(w), w.size, rows, cols, _p(q), q.size, _p(scales), scales.size))
+    return q, scales
+
+
+def quantize_per_output_channel_i8(w, out, in_):
+    """(w_i8, scales), crates/ft-kernel-cpu/src/lib.rs:37836."""
+    return _quantize_i8("fth_quantize_per_output_channel_i8", w, out, in_)
+
+
+def quantize_rows_i8(x, m, k):
+    """(x_i8, a_scales), crates/ft-kernel-cpu/src/lib.rs:37879."""
+    return _quantize_i8("fth_quantize_rows_i8", x, m, k)
+
+
+def linear_int8_dynamic_f32(x, m, k, w_i8, w_scales, n, bias=None):
+    """crates/ft-kernel-cpu/src/lib.rs:37966."""
+    x, w_scales = _slice(x, np.float32), _slice(w_scales, np.float32)
+    w_i8 = np.ascontiguousarray(w_i8, dtype=np.int8).reshape(-1)
+    bias = None if bias is None else _slice(bias, np.float32)
+    out = np.empty(m * n, np.float32)
+    check(_lib.load().fth_linear_int8_dynamic_f32(_p(x), x.size, m, k, _p(w_i8), w_i8.size, _p(w_scales), w_scales.size, n,
+                                                  _p(bias), 0 if bias is None else bias.size, _p(out), out.size))
+    return out
+
+
 def _sdpa_masked(sfx, dtype, q, k, v, batch, h_q, h_kv, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride):
     q, k, v, mask = _slice(q, dtype), _slice(k, dtype), _slice(v, dtype), _slice(mask, dtype)
     out = np.empty(batch * h_q * seq_q * d_v, dtype=dtype)

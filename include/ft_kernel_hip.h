@@ -258,6 +258,19 @@ int32_t fth_dev_cross_entropy_backward_f32(const float *logits, const int64_t *t
 int32_t fth_dev_cross_entropy_backward_f64(const double *logits, const int64_t *target, const double *dloss, int64_t batch, int64_t classes,
                                            double *dlogits, int64_t *bad_index, fth_stream s);
 
+/* Int8 dynamic-quantised linear (quantize_rows_i8, crates/ft-kernel-cpu/src/lib.rs:37879-37905; quantize_per_output_channel_i8
+ * :37836-37868, the same arithmetic on weight rows; linear_int8_dynamic_f32 :37966-38060). Quantisation is per row, symmetric:
+ * scale = max|row| / 127 (1 for an all-zero row), q = clamp(round_ties_even(v / scale), -127, 127). The product accumulates
+ * in int32 on the integer matrix cores and each output is (float)acc * a_scale[row] * w_scale[col] (+ bias[col]): bit-exact
+ * against the reference for any summation order. `fth_dev_linear_int8_dynamic_f32` quantises x into the workspace
+ * (fth_dev_linear_int8_workspace_bytes(m, k) bytes) and multiplies; `_prequantized_` takes activations quantised earlier. */
+int32_t fth_dev_quantize_rows_i8(const float *x, int64_t rows, int64_t cols, int8_t *q, float *scales, fth_stream s);
+size_t fth_dev_linear_int8_workspace_bytes(int64_t m, int64_t k);
+int32_t fth_dev_linear_int8_dynamic_f32(const float *x, int64_t m, int64_t k, const int8_t *w_i8, const float *w_scales, int64_t n,
+                                        const float *bias, float *out, void *workspace, size_t workspace_bytes, fth_stream s);
+int32_t fth_dev_linear_int8_prequantized_f32(const int8_t *x_i8, const float *a_scales, int64_t m, int64_t k, const int8_t *w_i8,
+                                             const float *w_scales, int64_t n, const float *bias, float *out, fth_stream s);
+
 /* ---- backward kernels of the same ops (device pointers; caller-provided workspace) ----
  * Each entry point needs scratch memory for its fixed-order partial sums (and, for SDPA, for the
  * probability and score-gradient matrices the reference materialises per head): ask the matching
@@ -399,6 +412,14 @@ int32_t fth_rms_norm_forward_f32(const float *x, size_t x_len, const float *weig
                                  size_t norm_size, float eps, float *out, size_t out_cap);
 int32_t fth_rms_norm_forward_f64(const double *x, size_t x_len, const double *weight, size_t batch,
                                  size_t norm_size, double eps, double *out, size_t out_cap);
+/* quantize_per_output_channel_i8 (:37836) / quantize_rows_i8 (:37879): w [rows, cols] -> q [rows * cols], scales [rows].
+ * linear_int8_dynamic_f32 (:37966): x [m, k] f32, w_i8 [n, k], w_scales [n], bias [n] or NULL -> out [m * n]. Slice lengths
+ * that the reference asserts (x_len == m*k, ...) are InvalidArgument when they differ. */
+int32_t fth_quantize_per_output_channel_i8(const float *w, size_t w_len, size_t rows, size_t cols, int8_t *q, size_t q_cap, float *scales,
+                                           size_t scales_cap);
+int32_t fth_quantize_rows_i8(const float *x, size_t x_len, size_t rows, size_t cols, int8_t *q, size_t q_cap, float *scales, size_t scales_cap);
+int32_t fth_linear_int8_dynamic_f32(const float *x, size_t x_len, size_t m, size_t k, const int8_t *w_i8, size_t w_len, const float *w_scales,
+                                    size_t w_scales_len, size_t n, const float *bias, size_t bias_len, float *out, size_t out_cap);
 /* sdpa_forward_masked_f64 (:4661-4741) and sdpa_forward_masked_gqa_f64 (:4777-4850), plus f32 twins the reference
  * does not have yet: q [num_bh | batch, h_q][seq_q, d_k], k / v [num_bh | batch, h_kv][seq_k, d]; additive mask with
  * mask_bh_stride 0 (one [seq_q, seq_k] for every head) or seq_q * seq_k (one per query head). A mask slice shorter than

@@ -392,6 +392,45 @@ void sdpa_masked_gqa_impl(const T *q, const T *k, const T *v, int64_t batch, int
     }
 }
 
+// quantize_rows_i8 (KC:37879-37905) and quantize_per_output_channel_i8 (KC:37836-37868): per row, amax = fold(0, max(acc, |v|))
+// (f32::max ignores a NaN operand), scale = amax > 0 ? amax / 127 : 1, q = clamp(round_ties_even(v / scale), -127, 127) as i8
+// (`as i8` turns NaN into 0).
+void quantize_rows_i8_impl(const float *x, int64_t rows, int64_t cols, int8_t *q, float *scales) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float *row = x + r * cols;
+        float amax = 0.0f;
+        for (int64_t i = 0; i < cols; ++i) amax = std::fmax(amax, std::fabs(row[i]));
+        const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
+        for (int64_t i = 0; i < cols; ++i) {
+            const float v = std::nearbyintf(row[i] / scale);  // default rounding mode: ties to even
+            q[r * cols + i] = (v != v) ? (int8_t)0 : (int8_t)std::fmin(std::fmax(v, -127.0f), 127.0f);
+        }
+        scales[r] = scale;
+    }
+}
+
+// linear_int8_dynamic_f32 (KC:37966-38060): quantise x per row, i32 dot products (dot_i8, KC:38282-38313), then
+// y = acc as f32 * a_scale * w_scale (+ bias), the three float operations in that order.
+void linear_int8_dynamic_impl(const float *x, int64_t m, int64_t k, const int8_t *w_i8, const float *w_scales, int64_t n, const float *bias,
+                              float *out) {
+    std::vector<int8_t> xq((size_t)(m * k));
+    std::vector<float> a_scales((size_t)m);
+    quantize_rows_i8_impl(x, m, k, xq.data(), a_scales.data());
+#pragma omp parallel for schedule(static)
+    for (int64_t s = 0; s < m; ++s) {
+        const int8_t *xr = xq.data() + s * k;
+        for (int64_t o = 0; o < n; ++o) {
+            const int8_t *wr = w_i8 + o * k;
+            int32_t acc = 0;
+            for (int64_t i = 0; i < k; ++i) acc += (int32_t)xr[i] * (int32_t)wr[i];
+            float y = (float)acc * a_scales[s] * w_scales[o];
+            if (bias) y += bias[o];
+            out[s * n + o] = y;
+        }
+    }
+}
+
 // normalize_strict_index_value (KC:20058-20090).
 inline int64_t strict_index(double v, int64_t dim_size) {
     if (!std::isfinite(v)) return -1;
@@ -954,6 +993,11 @@ void fto_linear_f64(const double *x, const double *w, const double *bias, int64_
 void fto_sdpa_forward_f32(const float *q, const float *k, const float *v, int64_t num_bh, int64_t seq_q,
                           int64_t seq_k, int64_t d_k, int64_t d_v, float scale, int causal, float *out) {
     sdpa_impl<float>(q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, out);
+}
+void fto_quantize_rows_i8(const float *x, int64_t rows, int64_t cols, int8_t *q, float *scales) { quantize_rows_i8_impl(x, rows, cols, q, scales); }
+void fto_linear_int8_dynamic_f32(const float *x, int64_t m, int64_t k, const int8_t *w_i8, const float *w_scales, int64_t n, const float *bias,
+                                 float *out) {
+    linear_int8_dynamic_impl(x, m, k, w_i8, w_scales, n, bias, out);
 }
 void fto_sdpa_forward_masked_gqa_f32(const float *q, const float *k, const float *v, int64_t batch, int64_t h_q, int64_t h_kv,
                                      int64_t seq_q, int64_t seq_k, int64_t d_k, int64_t d_v, float scale, const float *mask,

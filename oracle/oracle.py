@@ -235,6 +235,24 @@ def sdpa_forward_masked(q, k, v, scale, mask):
     return sdpa_forward_masked_gqa(q[None], k[None], v[None], scale, mask)[0]
 
 
+def quantize_rows_i8(x):
+    """Per-row symmetric int8 of a [rows, cols] f32 matrix -> (q int8, scales f32); also quantize_per_output_channel_i8."""
+    x = _c(x, np.float32)
+    rows, cols = x.shape
+    q, scales = np.empty((rows, cols), np.int8), np.empty(rows, np.float32)
+    lib().fto_quantize_rows_i8(_p(x), _i64(rows), _i64(cols), _p(q), _p(scales))
+    return q, scales
+
+
+def linear_int8_dynamic(x, w_i8, w_scales, bias=None):
+    x, w_i8, w_scales = _c(x, np.float32), _c(w_i8, np.int8), _c(w_scales, np.float32)
+    m, k = x.shape
+    n = w_i8.shape[0]
+    out = np.empty((m, n), np.float32)
+    lib().fto_linear_int8_dynamic_f32(_p(x), _i64(m), _i64(k), _p(w_i8), _p(w_scales), _i64(n), _p(_c(bias, np.float32)), _p(out))
+    return out
+
+
 def log_softmax(x, dim: int = -1):
     x = _c(x)
     sfx, _ = _sfx(x.dtype)

@@ -201,3 +201,48 @@ def test_gelu_tanh_restatement_is_pinned(oracle, vectors):
     # equals x * sigmoid(2u), the form the GEMM epilogue computes
     u = 0.7978845608028654 * (xs + 0.044715 * xs ** 3)
     assert np.max(np.abs(oracle.gelu_tanh(xs) - xs / (1.0 + np.exp(-2.0 * u)))) <= 1e-14
+
+
+def _lcg_matrices(m, k, n):
+    """The generator of linear_int8_dynamic_matches_f32_reference (crates/ft-kernel-cpu/src/lib.rs:43650-43662)."""
+    state = [0x123456789ABCDEF0 ^ (m * 131 + k * 17 + n)]
+
+    def lcg():
+        state[0] = (state[0] * 6364136223846793005 + 1442695040888963407) % (1 << 64)
+        return np.float32(np.float32(state[0] >> 33) / np.float32(1 << 31)) - np.float32(1.0)
+
+    x = np.array([lcg() * np.float32(3.0) for _ in range(m * k)], np.float32).reshape(m, k)
+    w = np.array([lcg() * np.float32(0.5) for _ in range(n * k)], np.float32).reshape(n, k)
+    bias = np.array([lcg() for _ in range(n)], np.float32)
+    return x, w, bias
+
+
+def test_int8_dynamic_linear_restatement_is_pinned(oracle):
+    # int8_quantizers_round_signed_ties_to_even (:43721-43740): exact expected bytes and scale
+    ties = np.array([[-127.0, -2.5, -1.5, -0.5, 0.5, 1.5, 2.5, 127.0]], np.float32)
+    q, scales = oracle.quantize_rows_i8(ties)
+    assert q.tolist() == [[-127, -2, -2, 0, 0, 2, 2, 127]] and scales.tolist() == [1.0]
+    # an all-zero row keeps scale 1; NaN quantises to 0 and does not move the scale; the scale is amax / 127
+    q, scales = oracle.quantize_rows_i8(np.array([[0.0, 0.0, -0.0], [np.nan, 2.0, -4.0], [1e-3, 5e-4, 0.0]], np.float32))
+    assert scales[0] == 1.0 and q[0].tolist() == [0, 0, 0]
+    assert scales[1] == np.float32(4.0) / np.float32(127.0) and q[1].tolist() == [0, 64, -127]  # 63.5 rounds to the even 64
+    assert scales[2] == np.float32(1e-3) / np.float32(127.0) and q[2].tolist() == [127, 64, 0]
+    # linear_int8_dynamic_matches_f32_reference (:43645-43708): the reference's shapes, inputs and bounds
+    for m, k, n in ((8, 384, 384), (4, 384, 1536), (7, 200, 53)):
+        x, w, bias = _lcg_matrices(m, k, n)
+        w_i8, w_scales = oracle.quantize_rows_i8(w)
+        y = oracle.linear_int8_dynamic(x, w_i8, w_scales, bias).astype(np.float64)
+        ref = (x.astype(np.float64) @ w.astype(np.float64).T + bias).astype(np.float32).astype(np.float64)
+        cos = (ref * y).sum() / np.sqrt((ref * ref).sum() * (y * y).sum())
+        assert cos > 0.999 and np.abs(ref - y).max() / np.abs(ref).max() < 0.05
+        # independent of the restatement: the same integers through numpy
+        xq, a_scales = oracle.quantize_rows_i8(x)
+        acc = xq.astype(np.int64) @ w_i8.astype(np.int64).T
+        want = (acc.astype(np.float32) * a_scales[:, None]) * w_scales[None, :] + bias[None, :]
+        assert np.array_equal(oracle.linear_int8_dynamic(x, w_i8, w_scales, bias).view(np.uint32), want.astype(np.float32).view(np.uint32))
+    # linear_int8_dynamic_is_deterministic (:43710-43719)
+    m, k, n = 6, 384, 384
+    x = (((np.arange(m * k) % 17).astype(np.float32) - 8.0) * np.float32(0.1)).reshape(m, k)
+    w = (((np.arange(n * k) % 13).astype(np.float32) - 6.0) * np.float32(0.05)).reshape(n, k)
+    w_i8, w_scales = oracle.quantize_rows_i8(w)
+    assert np.array_equal(oracle.linear_int8_dynamic(x, w_i8, w_scales), oracle.linear_int8_dynamic(x, w_i8, w_scales))
