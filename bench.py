@@ -399,6 +399,32 @@ def bench_backward(device, synth, steps, with_cpu):
             best, reps = cpu_time(cpu_fn, 2.0)
             out[name]["cpu"] = {"value": round(nbytes * 64 / rows / best / 1e9, 2), "unit": "GB/s", "cores": O.threads(), "kind": "port",
                                 "sample": "64 of the 8192 rows, best of %d" % reps}
+    del lg, lo, dh, dwte
+    # int8 dynamic-quantised linear: quantise x per row, integer matrix-core product, dequantise (+ bias)
+    m8, k8, n8 = 8192, 4096, 4096
+    x8 = synth.normal(6, "x8", (m8, k8), 0.0, 3.0)
+    w8 = synth.normal(6, "w8", (n8, k8), 0.0, 0.5)
+    b8 = synth.normal(6, "b8", (n8,))
+    dx8, dw8f, db8 = DeviceBuffer.from_host(x8), DeviceBuffer.from_host(w8), DeviceBuffer.from_host(b8)
+    dwq, dws, dy8 = DeviceBuffer((n8, k8), np.int8), DeviceBuffer((n8,)), DeviceBuffer((m8, n8))
+    device.quantize_rows_i8(dw8f, n8, k8, dwq, dws)  # weights: once, outside the timed region
+    ws8 = device.linear_int8_dynamic(dx8, m8, k8, dwq, dws, n8, db8, dy8)
+    ms = timed(lambda: device.linear_int8_dynamic(dx8, m8, k8, dwq, dws, n8, db8, dy8, workspace=ws8))
+    dxq, dxs = DeviceBuffer((m8, k8), np.int8), DeviceBuffer((m8,))
+    ms_q = timed(lambda: device.quantize_rows_i8(dx8, m8, k8, dxq, dxs))
+    ops = 2 * m8 * n8 * k8
+    tops = ops / ((ms - ms_q) * 1e-3) / 1e12
+    qbytes = m8 * k8 * 5 + m8 * 4
+    out["linear_int8_dynamic"] = {"ms": round(ms, 4), "quantize_ms": round(ms_q, 4), "product_TOP/s": round(tops, 1), "frac": round(tops / 5000.0, 4),
+                                  "peak_TOP/s": 5000.0, "ops": ops, "quantize_GB/s": round(qbytes / (ms_q * 1e-3) / 1e9, 1),
+                                  "workload": "x fp32 [8192,4096] . int8 W[4096,4096]^T + bias; product rate = ops / (whole call - quantiser)"}
+    log("[backward] linear_int8_dynamic    %.4f ms (quantiser %.4f ms = %.0f GB/s); product %.0f TOP/s  %.1f%% of the 5.0 POP/s int8 peak"
+        % (ms, ms_q, qbytes / (ms_q * 1e-3) / 1e9, tops, 100 * tops / 5000.0))
+    if with_cpu:
+        wq_h, ws_h = O.quantize_rows_i8(w8[:512])
+        best, reps = cpu_time(lambda: O.linear_int8_dynamic(x8[:256], wq_h, ws_h, b8[:512]), 3.0, min_reps=1)
+        out["linear_int8_dynamic"]["cpu"] = {"value": round(2 * 256 * 512 * k8 / best / 1e12, 4), "unit": "TOP/s", "cores": O.threads(), "kind": "port",
+                                             "sample": "256 rows x 512 outputs of the 8192 x 4096, scalar i32 dot products, best of %d" % reps}
     return out
 
 

@@ -8,13 +8,17 @@
 // the order of the sum and every output equals the reference's bit for bit; the three float operations
 // of the dequantisation are kept apart (this file is built without contraction).
 //
-// Product kernel: v_mfma_i32_32x32x32_i8, 128 x 128 output tile per workgroup (2 x 2 wavefronts of
-// 64 x 64), K in steps of 64 bytes through double-buffered LDS filled by global_load_lds_dwordx4. Both
+// Product kernel: v_mfma_i32_32x32x32_i8, 256 x 256 output tile per workgroup (2 x 2 wavefronts of 128 x 128;
+// 128 x 128 tiles for problems with few tiles), K in steps of 64 bytes through a ring of four LDS stages filled by global_load_lds_dwordx4 (a
+// stage of this kernel is only 256 MFMA cycles per wavefront, far less than a memory round trip, so three
+// stages are kept in flight). Both
 // operands are k-contiguous ([m, k] activations, [n, k] weights), so a lane's fragment is 16 consecutive
 // bytes of one row. Rows are 64 bytes in LDS; 16-byte slot q of row r is stored at q ^ ((r >> 2) & 3),
 // which spreads any 16 consecutive rows of one slot over all 64 banks. Rows past m / n are clamped to the
 // last valid row on the load side and never stored. Shapes whose K is not a multiple of 64 or whose
 // operands are not 16-byte aligned take a plain one-thread-per-output kernel.
+
+#include <cstdlib>
 
 #include "common.hpp"
 
@@ -66,102 +70,190 @@ __device__ __forceinline__ void load_to_lds_16(const int8_t *src, unsigned lds_c
                  : "memory", "m0");
 }
 
-constexpr int kBM = 128, kBN = 128, kBK = 64;  // bytes of K per stage
-constexpr int kTileBytes = kBM * kBK;          // 8 KiB per operand per stage
+constexpr int kBK = 64;     // bytes of K per stage
+constexpr int kStages = 4;  // ring of LDS stages: three loads in flight under one stage of MFMAs
+constexpr int kGroup = 8;   // tiles are walked in kGroup x kGroup squares, one square at a time per XCD
 
-__global__ __launch_bounds__(256, 2) void i8_gemm_kernel(const I8Args p) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];  // [2][A 8 KiB | B 8 KiB]
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    // s_waitcnt with only the vector-memory counter set: low four bits [3:0], high two bits [15:14]
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
+// TW x TW MFMA tiles (32 x 32 each) per wavefront, 2 x 2 wavefronts: a 64 TW x 64 TW output tile per workgroup.
+// TW = 2 (128 x 128, two workgroups per compute unit) suits problems with few tiles; TW = 4 (256 x 256, one workgroup,
+// 256 accumulator registers per lane) halves both the L2 -> LDS traffic and the LDS reads per MFMA. The integer MFMA
+// retires 65 536 operations in 32 cycles, so an LDS-fed loop is bound by fragment reads: measured on this chip with no
+// global traffic at all, one 128-bit read per MFMA (TW = 2) sustains half of the matrix peak, one per two MFMAs (TW = 4)
+// four fifths.
+template <int TW>
+__global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8Args p) {
+    constexpr int BM = 64 * TW, BN = 64 * TW;
+    constexpr int A_BYTES = BM * kBK, STAGE = (BM + BN) * kBK;
+    constexpr int LD = BM / 64;        // load instructions per operand per wavefront per stage (16 rows each)
+    constexpr int LPS = 2 * LD;        // load instructions per stage per wavefront
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];  // [kStages][A | B]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;  // 2 x 2 wavefronts
-    // tiles walked so that the 8 workgroups of consecutive ids (one per XCD, round-robin) share tile rows
-    const int tile = blockIdx.x;
-    const int tile_m = tile / p.tiles_n, tile_n = tile % p.tiles_n;
-    const int64_t m0 = (int64_t)tile_m * kBM, n0 = (int64_t)tile_n * kBN;
+    // Workgroup ids go round-robin over the 8 XCDs. Each XCD takes a contiguous run of the tile sequence, and the
+    // sequence walks kGroup x kGroup squares of tiles, so the workgroups resident on one XCD at a time share a few
+    // row panels of A and of B through that XCD's L2.
+    int tile = blockIdx.x;
+    {
+        const int grid = (int)gridDim.x, per = grid / 8;
+        if (per > 0 && tile < per * 8) tile = (tile % 8) * per + tile / 8;
+    }
+    int tile_m, tile_n;
+    {
+        const int band = kGroup * p.tiles_n;  // tiles in a band of kGroup tile rows
+        const int b = tile / band, r = tile % band;
+        const int rows = (p.tiles_m - b * kGroup) < kGroup ? (p.tiles_m - b * kGroup) : kGroup;  // the last band may be short
+        const int sq = r / (rows * kGroup), rs = r % (rows * kGroup);
+        tile_m = b * kGroup + rs % rows;
+        tile_n = sq * kGroup + rs / rows;
+    }
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
 
-    // Loader: one wavefront instruction covers 16 rows x 64 bytes; a wavefront loads 32 rows of A and 32 of B
-    // per stage (2 + 2 instructions). Lane L -> row L / 4 of the 16, slot L % 4, fetched from the
-    // swizzled source slot so that the LDS image is already swizzled.
+    // Loader: one wavefront instruction covers 16 rows x 64 bytes; a wavefront loads BM / 4 rows of A and BN / 4 of B
+    // per stage. Lane L -> row L / 4 of the 16, slot L % 4, fetched from the swizzled source slot so that the LDS
+    // image is already swizzled.
     const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)reinterpret_cast<uintptr_t>(smem));
     const unsigned wave_u = __builtin_amdgcn_readfirstlane((unsigned)wave);
     const int lrow = lane >> 2, lslot = lane & 3;
-    const int8_t *a_src[2], *b_src[2];
+    const int8_t *a_src[LD], *b_src[LD];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int r = wave * 32 + i * 16 + lrow;  // row inside the tile
-        const int q = lslot ^ ((r >> 2) & 3);     // the logical slot that lives at physical slot lslot
+    for (int i = 0; i < LD; ++i) {
+        const int r = wave * (16 * LD) + i * 16 + lrow;  // row inside the tile
+        const int q = lslot ^ ((r >> 2) & 3);            // the logical slot that lives at physical slot lslot
         int64_t ar = m0 + r, br = n0 + r;
         ar = ar < p.m ? ar : p.m - 1;
         br = br < p.n ? br : p.n - 1;
         a_src[i] = p.a + ar * p.k + q * 16;
         b_src[i] = p.b + br * p.k + q * 16;
     }
-    auto issue = [&](int kt, int buf) __attribute__((always_inline)) {
-        const unsigned base = lds0 + (unsigned)buf * (2 * kTileBytes) + wave_u * 2048u;
+    auto issue = [&](int kt) __attribute__((always_inline)) {
+        const unsigned base = lds0 + (unsigned)(kt % kStages) * STAGE + wave_u * (LD * 1024u);
         const int64_t koff = (int64_t)kt * kBK;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < LD; ++i) {
             load_to_lds_16(a_src[i] + koff, base + i * 1024u);
-            load_to_lds_16(b_src[i] + koff, base + kTileBytes + i * 1024u);
+            load_to_lds_16(b_src[i] + koff, base + A_BYTES + i * 1024u);
         }
     };
 
-    V16i acc[2][2];
+    V16i acc[TW][TW];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TW; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TW; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
     const int num_kt = (int)(p.k / kBK);
-    issue(0, 0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    __syncthreads();
+#pragma unroll
+    for (int st = 0; st < kStages - 1; ++st)
+        if (st < num_kt) issue(st);
     // Fragment addresses: lane (row = lane % 32 of a 32-row MFMA tile, k group = lane / 32).
     const int frow = lane & 31, kg = lane >> 5;
-    for (int kt = 0; kt < num_kt; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < num_kt) issue(kt + 1, buf ^ 1);
-        const unsigned char *As = smem + buf * (2 * kTileBytes), *Bs = As + kTileBytes;
+    V4i af[2][TW], bf[2][TW];  // fragment registers of the two 32-byte K steps of a stage
+    auto fetch = [&](int kt, int ks) __attribute__((always_inline)) {
+        const unsigned char *As = smem + (kt % kStages) * STAGE, *Bs = As + A_BYTES;
+        const int q = ks * 2 + kg;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {  // two 32-byte K steps per stage
-            const int q = ks * 2 + kg;
-            V4i af[2], bf[2];
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const int ra = wm * 64 + i * 32 + frow, rb = wn * 64 + i * 32 + frow;
-                af[i] = *reinterpret_cast<const V4i *>(As + ra * kBK + ((q ^ ((ra >> 2) & 3)) << 4));
-                bf[i] = *reinterpret_cast<const V4i *>(Bs + rb * kBK + ((q ^ ((rb >> 2) & 3)) << 4));
-            }
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+        for (int i = 0; i < TW; ++i) {
+            const int ra = wm * (32 * TW) + i * 32 + frow, rb = wn * (32 * TW) + i * 32 + frow;
+            af[ks][i] = *reinterpret_cast<const V4i *>(As + ra * kBK + ((q ^ ((ra >> 2) & 3)) << 4));
+            bf[ks][i] = *reinterpret_cast<const V4i *>(Bs + rb * kBK + ((q ^ ((rb >> 2) & 3)) << 4));
         }
-        __builtin_amdgcn_s_waitcnt(0x0F70);
+    };
+    auto mma = [&](int ks) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < TW; ++i)
+#pragma unroll
+            for (int j = 0; j < TW; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks][i], bf[ks][j], acc[i][j], 0, 0, 0);
+    };
+    // Stage s has landed for everybody once each wavefront has waited for its own loads of s and passed a barrier.
+    auto land = [&](int s_) __attribute__((always_inline)) {
+        // loads of the stages after s_ stay in flight: LPS instructions each, at most kStages - 2 stages
+        const int younger = num_kt - 1 - s_;
+        if (younger >= kStages - 2) wait_vmcnt<(kStages - 2) * LPS>();
+        else if (younger == 1) wait_vmcnt<LPS>();
+        else wait_vmcnt<0>();
         __syncthreads();
+    };
+    land(0);
+    if (kStages - 1 < num_kt) issue(kStages - 1);
+    fetch(0, 0);
+    // Steady state, one stage per iteration: the fragments of a K step are read from LDS while the MFMAs of the step
+    // before it run, across the stage boundary as well, so neither the LDS latency nor the barrier wait is followed
+    // by an MFMA that needs what was just requested.
+    // The last stage is peeled off so that the loop body is straight-line code: with a conditional fetch the
+    // compiler's wait-count pass joins two paths in front of the second batch of MFMAs and makes it wait for the
+    // reads that were only just issued.
+    for (int kt = 0; kt + 1 < num_kt; ++kt) {
+        fetch(kt, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(0);
+        __builtin_amdgcn_sched_barrier(0);
+        land(kt + 1);  // also: every wavefront has finished reading stage kt, whose buffer takes stage kt + kStages
+        if (kt + kStages < num_kt) issue(kt + kStages);
+        fetch(kt + 1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(1);
+        __builtin_amdgcn_sched_barrier(0);
     }
+    fetch(num_kt - 1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    mma(0);
+    mma(1);
 
     // Dequantise and store: lane owns column n = lane % 32 of each MFMA tile, rows 8 (r / 4) + 4 (lane / 32) + r % 4.
+    // The row scales of the tile go through LDS (free by now): one coalesced load instead of 16 scattered loads per
+    // MFMA tile row.
+    __syncthreads();
+    float *row_scale = reinterpret_cast<float *>(smem);
+    for (int t = tid; t < BM; t += 256) row_scale[t] = (m0 + t < p.m) ? p.a_scales[m0 + t] : 0.0f;
+    __syncthreads();
+    const bool interior = m0 + BM <= p.m && n0 + BN <= p.n;  // no bounds tests on the common path
+    const int64_t ldc = p.n;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int64_t col = n0 + wn * 64 + j * 32 + frow;
-        if (col >= p.n) continue;
-        const float ws = p.b_scales[col];
-        const float bv = p.bias ? p.bias[col] : 0.0f;
+    for (int i = 0; i < TW; ++i) {
+        const int lrow0 = wm * (32 * TW) + i * 32 + 4 * kg;  // tile row of accumulator element 0
+        float as_[16];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int r = 0; r < 16; ++r) as_[r] = row_scale[lrow0 + 8 * (r >> 2) + (r & 3)];
+#pragma unroll
+        for (int j = 0; j < TW; ++j) {
+            const int64_t col = n0 + wn * (32 * TW) + j * 32 + frow;
+            if (!interior && col >= p.n) continue;
+            const float ws = p.b_scales[col];
+            const float bv = p.bias ? p.bias[col] : 0.0f;
+            float *c0 = p.c + (m0 + lrow0) * ldc + col;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int64_t row = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * kg + (r & 3);
-                if (row < p.m) {
-                    float y = (float)acc[i][j][r] * p.a_scales[row] * ws;
+                const int dr = 8 * (r >> 2) + (r & 3);
+                if (interior || m0 + lrow0 + dr < p.m) {
+                    float y = (float)acc[i][j][r] * as_[r] * ws;
                     if (p.bias) y += bv;
-                    p.c[row * p.n + col] = y;
+                    __builtin_nontemporal_store(y, c0 + dr * ldc);
                 }
             }
         }
     }
+}
+
+template <int TW> int32_t launch_i8_gemm(I8Args &p, hipStream_t st) {
+    constexpr int BM = 64 * TW;
+    constexpr size_t smem = (size_t)kStages * 2 * BM * kBK;  // 64 KiB (two workgroups per compute unit) or 128 KiB (one)
+    p.tiles_m = (int)fth::ceil_div(p.m, BM);
+    p.tiles_n = (int)fth::ceil_div(p.n, BM);
+    static bool attr_set = false;
+    if (!attr_set) {
+        FTH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(i8_gemm_kernel<TW>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_set = true;
+    }
+    i8_gemm_kernel<TW><<<dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(256), smem, st>>>(p);
+    FTH_CHECK_LAUNCH("i8_gemm");
+    return FTH_OK;
 }
 
 // Any shape and alignment: one thread per output element.
@@ -213,14 +305,18 @@ int32_t fth_dev_linear_int8_prequantized_f32(const int8_t *x_i8, const float *a_
     I8Args p;
     p.a = x_i8; p.b = w_i8; p.a_scales = a_scales; p.b_scales = w_scales; p.bias = bias; p.c = out;
     p.m = m; p.n = n; p.k = k;
-    p.tiles_m = (int)fth::ceil_div(m, kBM);
-    p.tiles_n = (int)fth::ceil_div(n, kBN);
+    p.tiles_m = p.tiles_n = 0;
     const bool aligned = ((reinterpret_cast<uintptr_t>(x_i8) | reinterpret_cast<uintptr_t>(w_i8)) & 15u) == 0;
-    const int64_t tiles = fth::ceil_div(m, kBM) * fth::ceil_div(n, kBN);
-    if (k >= kBK && k % kBK == 0 && aligned && tiles <= 2147483647LL) {
-        constexpr size_t smem = 2 * 2 * kTileBytes;
-        i8_gemm_kernel<<<dim3((unsigned)tiles), dim3(256), smem, st>>>(p);
-        FTH_CHECK_LAUNCH("i8_gemm");
+    const int64_t tiles128 = fth::ceil_div(m, 128) * fth::ceil_div(n, 128), tiles256 = fth::ceil_div(m, 256) * fth::ceil_div(n, 256);
+    if (k >= kBK && k % kBK == 0 && aligned && tiles128 <= 2147483647LL) {
+        // 256 x 256 tiles once they give every compute unit a workgroup; the choice depends on the shape only
+        const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
+        static const int forced = [] {
+            const char *e = std::getenv("FT_HIP_I8_TILE");  // tuning knob: 128 or 256; anything else = automatic
+            return e ? std::atoi(e) : 0;
+        }();
+        const bool big = forced == 256 || (forced != 128 && tiles256 >= cus);
+        if (int32_t rc = big ? launch_i8_gemm<4>(p, st) : launch_i8_gemm<2>(p, st)) return rc;
     } else {
         int64_t total;
         FTH_ARG(!__builtin_mul_overflow(m, n, &total) && fth::ceil_div(total, 256) <= 2147483647LL, "linear_int8: output too large for one launch");

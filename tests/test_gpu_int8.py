@@ -56,8 +56,10 @@ def _linear(hip, x, w_i8, w_scales, bias):
     return out.to_host()
 
 
-# the reference's three test shapes (k = 200 takes the plain kernel), matrix-core shapes with ragged m / n, K of one stage
-SHAPES = [(8, 384, 384), (4, 384, 1536), (7, 200, 53), (128, 64, 128), (130, 768, 300), (257, 1024, 129), (1, 64, 1), (512, 3072, 768)]
+# the reference's three test shapes (k = 200 takes the plain kernel), matrix-core shapes with ragged m / n, K of one stage,
+# and two shapes with enough 256 x 256 tiles for the large-tile kernel (ragged edges; K of one, two and five stages)
+SHAPES = [(8, 384, 384), (4, 384, 1536), (7, 200, 53), (128, 64, 128), (130, 768, 300), (257, 1024, 129), (1, 64, 1), (512, 3072, 768),
+          (4100, 128, 4100), (4096, 64, 4096), (8200, 320, 2050)]
 
 
 @pytest.mark.parametrize("m,k,n", SHAPES)
