@@ -492,6 +492,218 @@ __global__ __launch_bounds__(64) void sdpa_generic_kernel(const SdpaArgs p) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// fp64 on v_mfma_f64_16x16x4_f64 (sdpa_forward_f64, crates/ft-kernel-cpu/src/lib.rs:4572-4651, and the masked /
+// grouped-query forms :4661-4850). The same scheme as the fp32 kernel at the shape of the fp64 MFMA: a wavefront
+// owns 16 queries and a block of 4 wavefronts (64 queries) shares each tile of 16 keys through double-buffered LDS.
+//   S^T[key, query] = K_tile . Q^T    16 x 16 accumulator: lane (query = lane % 16, g = lane / 16) holds keys
+//                                     4 r + g, r = 0..3. The dot product over d_k is cut into four contiguous
+//                                     ranges, one per lane group g (any split of the k index works as long as both
+//                                     operands use it), so a lane's K and Q fragments are contiguous doubles:
+//                                     128-bit LDS reads, and Q stays in registers for the whole kernel. Two
+//                                     accumulators take alternate k steps, which halves the dependent MFMA chain.
+//   O^T[d, query] += V_tile^T . P^T   MFMA step r contracts over keys 4 r + g, which is exactly what accumulator
+//                                     element r of the lane holds: P is the B operand as it stands. Row i of
+//                                     d-tile e is d = 32 (e / 2) + 2 i + e % 2, so one 128-bit read of V feeds two
+//                                     d-tiles and a lane's outputs pair up into 16-byte stores.
+// Row max / sum: four in-lane values and two exchanges across the lane groups. exp is the library's double exp.
+// ---------------------------------------------------------------------------------------------
+using Acc4d = double __attribute__((ext_vector_type(4)));
+
+template <int D, bool MASK>
+__global__ __launch_bounds__(256, 2) void sdpa_mfma_f64_kernel(const SdpaArgs p) {
+    constexpr int BC = 16;           // keys per tile
+    constexpr int BQ = 64;           // queries per block
+    constexpr int P = D + 2;         // LDS row pitch in doubles: 16 bytes of padding keep the 16 key rows of a fragment read on distinct banks
+    constexpr int KT = BC * P;       // doubles per K (or V) tile
+    constexpr int DQ = D / 4;        // doubles of a row that one lane group contracts over
+    constexpr int NE = D / 16;       // d-tiles of the output
+    constexpr int NV = BC * (D / 2) / 256;  // 16-byte vectors per thread per tile
+    static_assert(BC * (D / 2) % 256 == 0 && NV >= 1, "tile must divide over the block");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    double *Ks = reinterpret_cast<double *>(smem_raw);  // [2][BC][P]
+    double *Vs = Ks + 2 * KT;                           // [2][BC][P]
+
+    const fth_sdpa_desc &d = p.d;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lq = lane & 15, g = lane >> 4;
+    const int64_t pid = blockIdx.x;
+    const int unit = (int)(pid / d.num_bh);  // heaviest (latest) query blocks first across all heads
+    const int64_t bh = pid % d.num_bh;
+    const int qb = p.q_blocks - 1 - unit;
+    const int64_t b = bh / d.heads, h = bh % d.heads, hk = h / p.group;
+    const double *Q = static_cast<const double *>(p.q) + b * d.q_batch_stride + h * d.q_head_stride;
+    const double *K = static_cast<const double *>(p.k) + b * d.k_batch_stride + hk * d.k_head_stride;
+    const double *Vg = static_cast<const double *>(p.v) + b * d.v_batch_stride + hk * d.v_head_stride;
+    double *O = static_cast<double *>(p.out) + b * d.o_batch_stride + h * d.o_head_stride;
+    const double *Mk = MASK ? static_cast<const double *>(p.mask) + bh * p.mask_bh_stride : nullptr;
+    const double scale = p.scale;
+    const int seq_q_i = (int)d.seq_q, seq_k_i = (int)d.seq_k;
+    const int q_blk0 = qb * BQ, q_wave0 = q_blk0 + wave * 16, qi = q_wave0 + lq;
+    const bool q_live = qi < seq_q_i;
+
+    // Q: lane holds Q[qi][g * DQ + t], t = 0..DQ-1 (contiguous)
+    double2 qr[DQ / 2];
+#pragma unroll
+    for (int t = 0; t < DQ / 2; ++t)
+        qr[t] = q_live ? *reinterpret_cast<const double2 *>(Q + (int64_t)qi * d.q_row_stride + g * DQ + 2 * t) : make_double2(0.0, 0.0);
+
+    int blk_last_q = q_blk0 + BQ - 1;
+    if (blk_last_q > seq_q_i - 1) blk_last_q = seq_q_i - 1;
+    int k_end = seq_k_i;
+    if (d.causal && blk_last_q + 1 < k_end) k_end = blk_last_q + 1;
+    const int num_kt = (k_end + BC - 1) / BC;
+    int wave_last_q = q_wave0 + 15;
+    if (wave_last_q > seq_q_i - 1) wave_last_q = seq_q_i - 1;
+
+    // Tile loader through registers: thread owns vector column ld_c of rows ld_row + i * RS.
+    constexpr int RS = 256 / (D / 2);
+    const int ld_row = tid / (D / 2), ld_c = tid % (D / 2);
+    double2 kst[NV], vst[NV];
+    auto load_tile = [&](int kt) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int row = kt * BC + ld_row + i * RS;
+            if (row < seq_k_i) {
+                kst[i] = *reinterpret_cast<const double2 *>(K + (int64_t)row * d.k_row_stride + 2 * ld_c);
+                vst[i] = *reinterpret_cast<const double2 *>(Vg + (int64_t)row * d.v_row_stride + 2 * ld_c);
+            } else {
+                kst[i] = make_double2(0.0, 0.0);
+                vst[i] = make_double2(0.0, 0.0);
+            }
+        }
+    };
+    auto store_tile = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            *reinterpret_cast<double2 *>(Ks + buf * KT + (ld_row + i * RS) * P + 2 * ld_c) = kst[i];
+            *reinterpret_cast<double2 *>(Vs + buf * KT + (ld_row + i * RS) * P + 2 * ld_c) = vst[i];
+        }
+    };
+
+    Acc4d o[NE];
+#pragma unroll
+    for (int e = 0; e < NE; ++e) o[e] = (Acc4d){0.0, 0.0, 0.0, 0.0};
+    const double ninf = -__builtin_inf();
+    double m_run = ninf, l_run = 0.0;
+
+    if (num_kt > 0) {
+        load_tile(0);
+        store_tile(0);
+    }
+    __syncthreads();
+    for (int kt = 0; kt < num_kt; ++kt) {
+        const int buf = kt & 1, key0 = kt * BC;
+        if (kt + 1 < num_kt) load_tile(kt + 1);  // in flight under this tile's matrix work
+        const bool wave_active = !d.causal || key0 <= wave_last_q;
+        if (wave_active) {
+            // ---- the lane's four mask values, requested ahead of the score MFMAs ----
+            double mk[4] = {0.0, 0.0, 0.0, 0.0};
+            if constexpr (MASK) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int key = key0 + 4 * r + g;
+                    if (q_live && key < seq_k_i) mk[r] = Mk[(int64_t)qi * seq_k_i + key];
+                }
+            }
+            // ---- S^T = K_tile . Q^T ----
+            Acc4d s0 = (Acc4d){0.0, 0.0, 0.0, 0.0}, s1 = s0;
+            const double *kp = Ks + buf * KT + lq * P + g * DQ;
+#pragma unroll
+            for (int t = 0; t < DQ / 2; ++t) {
+                const double2 kv = *reinterpret_cast<const double2 *>(kp + 2 * t);
+                s0 = __builtin_amdgcn_mfma_f64_16x16x4f64(kv.x, qr[t].x, s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f64_16x16x4f64(kv.y, qr[t].y, s1, 0, 0, 0);
+            }
+            // ---- scale, mask, online softmax (lane-local query; keys 4 r + g) ----
+            double x[4], mt = ninf;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = key0 + 4 * r + g;
+                double v = (s0[r] + s1[r]) * scale;
+                if constexpr (MASK) v += mk[r];
+                if ((d.causal && key > qi) || key >= seq_k_i) v = ninf;
+                x[r] = v;
+                mt = fmax(mt, v);
+            }
+            mt = fmax(mt, __shfl_xor(mt, 16, kWave));
+            mt = fmax(mt, __shfl_xor(mt, 32, kWave));
+            const double m_new = fmax(m_run, mt);
+            // Every key so far hidden (possible only under a mask): keep the state empty instead of carrying the NaN
+            // of exp(-inf - -inf) into later tiles; a row with no visible key at all ends as 0 / 0 = NaN, as in the reference.
+            const double m_ref = (m_new == ninf) ? 0.0 : m_new;
+            const double alpha = exp(m_run - m_ref);
+            Acc4d pr;
+            double psum = 0.0;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const double e = exp(x[r] - m_ref);
+                pr[r] = e;
+                psum += e;
+            }
+            psum += __shfl_xor(psum, 16, kWave);
+            psum += __shfl_xor(psum, 32, kWave);
+            l_run = l_run * alpha + psum;
+            m_run = m_new;
+            if (__any(alpha != 1.0)) {
+#pragma unroll
+                for (int e = 0; e < NE; ++e)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) o[e][r] *= alpha;
+            }
+            // ---- O^T += V_tile^T . P^T: step r contracts keys 4 r + g; d-tiles 2 e2 and 2 e2 + 1 share one read ----
+            const double *vp = Vs + buf * KT + g * P + 2 * lq;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+#pragma unroll
+                for (int e2 = 0; e2 < NE / 2; ++e2) {
+                    const double2 vv = *reinterpret_cast<const double2 *>(vp + (4 * r) * P + 32 * e2);
+                    o[2 * e2] = __builtin_amdgcn_mfma_f64_16x16x4f64(vv.x, pr[r], o[2 * e2], 0, 0, 0);
+                    o[2 * e2 + 1] = __builtin_amdgcn_mfma_f64_16x16x4f64(vv.y, pr[r], o[2 * e2 + 1], 0, 0, 0);
+                }
+            }
+        }
+        if (kt + 1 < num_kt) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- normalise and store: element r of d-tile e is d = 32 (e / 2) + 2 (4 r + g) + e % 2 of query qi ----
+    if (q_live) {
+        double *orow = O + (int64_t)qi * d.o_row_stride;
+#pragma unroll
+        for (int e2 = 0; e2 < NE / 2; ++e2)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const double a0 = (num_kt > 0) ? o[2 * e2][r] / l_run : 0.0, a1 = (num_kt > 0) ? o[2 * e2 + 1][r] / l_run : 0.0;
+                *reinterpret_cast<double2 *>(orow + 32 * e2 + 2 * (4 * r + g)) = make_double2(a0, a1);
+            }
+    }
+}
+
+template <int D> int32_t launch_mfma_f64(SdpaArgs &a, hipStream_t st) {
+    constexpr size_t smem = (size_t)2 * 2 * 16 * (D + 2) * sizeof(double);
+    a.q_blocks = (int)fth::ceil_div(a.d.seq_q, 64);
+    const int64_t grid = a.d.num_bh * a.q_blocks;
+    FTH_ARG(grid <= 2147483647LL, "sdpa: grid too large");
+    if (a.mask) {
+        static bool attr_set = false;
+        if (!attr_set) {
+            FTH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(sdpa_mfma_f64_kernel<D, true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+            attr_set = true;
+        }
+        sdpa_mfma_f64_kernel<D, true><<<dim3((unsigned)grid), dim3(256), smem, st>>>(a);
+    } else {
+        static bool attr_set = false;
+        if (!attr_set) {
+            FTH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(sdpa_mfma_f64_kernel<D, false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+            attr_set = true;
+        }
+        sdpa_mfma_f64_kernel<D, false><<<dim3((unsigned)grid), dim3(256), smem, st>>>(a);
+    }
+    FTH_CHECK_LAUNCH("sdpa_mfma_f64");
+    return FTH_OK;
+}
+
 template <int D, int NW, bool PAIR, bool MASK> int32_t launch_mfma_cfg(SdpaArgs &a, hipStream_t st) {
     constexpr int BC = (D <= 64 && (NW == 4 || D <= 32)) ? 64 : 32;  // 64-key tiles where two workgroups still fit a CU
     constexpr bool DIRECT = D >= 64 && FTH_SDPA_DIRECT;
@@ -569,6 +781,22 @@ int32_t sdpa_entry(const fth_sdpa_desc *d, double scale, const T *q, const T *k,
             if (d->d_k == 128) return launch_mfma<128>(a, st);
             if (d->d_k == 64) return launch_mfma<64>(a, st);
             if (d->d_k == 32) return launch_mfma<32>(a, st);
+        }
+    }
+    if constexpr (std::is_same<T, double>::value) {
+        auto m2 = [](int64_t x) { return x % 2 == 0; };
+        const bool strides_ok = m2(d->q_batch_stride) && m2(d->q_head_stride) && m2(d->q_row_stride) && m2(d->k_batch_stride) &&
+                                m2(d->k_head_stride) && m2(d->k_row_stride) && m2(d->v_batch_stride) && m2(d->v_head_stride) &&
+                                m2(d->v_row_stride) && m2(d->o_batch_stride) && m2(d->o_head_stride) && m2(d->o_row_stride) &&
+                                al16(q) && al16(k) && al16(v) && al16(out);
+        static const bool generic_only = [] {
+            const char *e = std::getenv("FT_HIP_SDPA_F64_GENERIC");  // tuning / testing knob: 1 keeps fp64 on the generic kernel
+            return e && std::atoi(e) != 0;
+        }();
+        if (strides_ok && d->d_k == d->d_v && d->seq_k > 0 && !generic_only) {
+            if (d->d_k == 128) return launch_mfma_f64<128>(a, st);
+            if (d->d_k == 64) return launch_mfma_f64<64>(a, st);
+            if (d->d_k == 32) return launch_mfma_f64<32>(a, st);
         }
     }
     FTH_ARG(d->d_v <= 64 * 8, "sdpa: d_v %lld exceeds the generic kernel's limit of 512", (long long)d->d_v);

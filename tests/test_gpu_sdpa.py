@@ -44,7 +44,12 @@ def test_sdpa_f32_matches_oracle(hip, oracle, bh, sq, sk, dk, dv, causal):
     assert rel_err(got, oracle.sdpa_forward(q, k, v, scale, causal)) <= TOL_GEMM_F32
 
 
-@pytest.mark.parametrize("bh,sq,sk,dk,dv,causal", [(2, 33, 33, 64, 64, True), (2, 20, 45, 16, 24, False), (1, 70, 70, 128, 128, True)])
+# matrix-core head sizes (32 / 64 / 128) with ragged tails, seq_q != seq_k, single rows and keys, several query blocks per head;
+# (16, 24) takes the generic kernel
+@pytest.mark.parametrize("bh,sq,sk,dk,dv,causal", [(2, 33, 33, 64, 64, True), (2, 20, 45, 16, 24, False), (1, 70, 70, 128, 128, True),
+                                                   (3, 100, 100, 32, 32, True), (2, 130, 77, 64, 64, False), (2, 77, 130, 128, 128, True),
+                                                   (1, 1, 1, 64, 64, True), (2, 1, 300, 32, 32, False), (2, 300, 1, 64, 64, True),
+                                                   (5, 257, 257, 128, 128, True), (4, 200, 200, 64, 64, False)])
 def test_sdpa_f64_matches_oracle(hip, oracle, bh, sq, sk, dk, dv, causal):
     q, k, v = _qkv(3, bh, sq, sk, dk, dv, np.float64)
     scale = 1.0 / math.sqrt(dk)
