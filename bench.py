@@ -266,6 +266,21 @@ def bench_sdpa(device, synth, steps, with_cpu):
                       "sample": "%d of the %d heads, best of %d" % (nh, B * H, reps)}
         log("[sdpa] cpu baseline %.4f TFLOP/s (causal count) on %d threads" % (res["cpu"]["value"], O.threads()))
     del dq, dk, dv, do
+    # the same causal problem in fp64 (the reference's own SDPA precision), on the fp64 matrix cores
+    q64, k64, v64 = (t.astype(np.float64) for t in (q, k, v))
+    eq, ek, ev = (DeviceBuffer.from_host(t) for t in (q64, k64, v64))
+    eo = DeviceBuffer(q64.shape, np.float64)
+    fn64 = lambda: device.sdpa_forward(desc, s, eq, ek, ev, eo)
+    ms64 = event_time_ms(device, fn64, max(5, steps // 4))
+    tf64 = flop / (ms64 * 1e-3) / 1e12
+    log("[sdpa] B4 H32 S2048 D128 causal fp64  %.3f ms  %.2f TFLOP/s (causal count)  %.1f%% of the fp64 MFMA peak" % (ms64, tf64, 100 * tf64 / FP64_MFMA_PEAK_TF))
+    res["fp64"] = {"ms": round(ms64, 4), "TFLOP/s": round(tf64, 2), "frac": round(tf64 / FP64_MFMA_PEAK_TF, 4), "flop": flop,
+                   "peak_TFLOP/s": FP64_MFMA_PEAK_TF, "workload": "B4 H32 S2048 D128 causal fp64"}
+    if with_cpu:
+        best, reps = cpu_time(lambda: O.sdpa_forward(q64[:nh], k64[:nh], v64[:nh], s, True), 4.0, min_reps=1)
+        res["fp64"]["cpu"] = {"value": round(flop * nh / (B * H) / best / 1e12, 4), "unit": "TFLOP/s", "cores": O.threads(), "kind": "port",
+                              "sample": "%d of the %d heads, best of %d" % (nh, B * H, reps)}
+    del eq, ek, ev, eo, q64, k64, v64
     # grouped-query attention with an additive mask: 32 query heads on 8 K/V heads, the same S and D, a dense soft
     # mask (every key visible), so the two products run over the full [S, S] rectangle and every mask value is read
     Bg, Hq, Hkv = 2, 32, 8

@@ -632,7 +632,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_f64_kernel(const SdpaArgs p)
             // Every key so far hidden (possible only under a mask): keep the state empty instead of carrying the NaN
             // of exp(-inf - -inf) into later tiles; a row with no visible key at all ends as 0 / 0 = NaN, as in the reference.
             const double m_ref = (m_new == ninf) ? 0.0 : m_new;
-            const double alpha = exp(m_run - m_ref);
+            // Once the running maximum has settled (after the first few tiles of most rows) no lane of the wavefront
+            // needs the rescale: skip its exp and the pass over the accumulators.
+            const bool rescale = __any(m_new != m_run);
+            const double alpha = rescale ? exp(m_run - m_ref) : 1.0;
             Acc4d pr;
             double psum = 0.0;
 #pragma unroll
@@ -645,7 +648,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_f64_kernel(const SdpaArgs p)
             psum += __shfl_xor(psum, 32, kWave);
             l_run = l_run * alpha + psum;
             m_run = m_new;
-            if (__any(alpha != 1.0)) {
+            if (rescale) {
 #pragma unroll
                 for (int e = 0; e < NE; ++e)
 #pragma unroll
