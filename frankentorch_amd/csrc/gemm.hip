@@ -939,6 +939,94 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemm_fixup_kernel(const GemmArg
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Small problems (the 128-token transformer block: 17 to 67 MFLOP per product): one launch, no fix-up pass.
+// A workgroup owns one 32 x 32 output tile and splits K across its NW wavefronts; each wavefront feeds the MFMA
+// straight from global memory (a 128-bit load along k is four MFMA steps; the operands are small and L2-resident, and
+// nothing in a workgroup would reuse an LDS copy), and the NW partial tiles are added through LDS in wavefront order,
+// so the sum order is fixed by the shape. The large-tile kernels need a second launch to combine split tiles, which at
+// this size costs as much as the product itself.
+// ---------------------------------------------------------------------------------------------
+template <int NW, bool TRANS_B>
+__global__ __launch_bounds__(64 * NW) void gemm_small_kernel(const GemmArgs<float> p) {
+    using M = Mfma<float>;
+    __shared__ float part[NW][32][33];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lrow = lane & 31, g = lane >> 5;
+    const int64_t batch = blockIdx.y;
+    const int tile_m = (int)(blockIdx.x / p.tiles_n), tile_n = (int)(blockIdx.x % p.tiles_n);
+    const int64_t m0 = (int64_t)tile_m * 32, n0 = (int64_t)tile_n * 32;
+    const float *A = p.a + batch * p.stride_a;
+    const float *B = p.b + batch * p.stride_b;
+    // this wavefront's K range: whole groups of 8 (one 128-bit load per lane group), contiguous, in wavefront order
+    const int groups = (int)(p.k / 8), per = (groups + NW - 1) / NW;
+    const int g0 = wave * per, g1 = (g0 + per < groups) ? g0 + per : groups;
+    int64_t ar = m0 + lrow, br = n0 + lrow;  // rows past the edge read the last valid row; they are never stored
+    ar = ar < p.m ? ar : p.m - 1;
+    br = br < p.n ? br : p.n - 1;
+    const float *ap = A + ar * p.lda + 4 * g;
+    const float *bp = TRANS_B ? B + br * p.ldb + 4 * g : B + (int64_t)(4 * g) * p.ldb + br;
+    typename M::Acc acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll 8
+    for (int t = g0; t < g1; ++t) {
+        const float4 av = *reinterpret_cast<const float4 *>(ap + 8 * t);
+        float4 bv;
+        if (TRANS_B) {
+            bv = *reinterpret_cast<const float4 *>(bp + 8 * t);
+        } else {
+            const float *bk = bp + (int64_t)(8 * t) * p.ldb;
+            bv = make_float4(bk[0], bk[p.ldb], bk[2 * p.ldb], bk[3 * p.ldb]);
+        }
+        acc = M::mma(av.x, bv.x, acc);
+        acc = M::mma(av.y, bv.y, acc);
+        acc = M::mma(av.z, bv.z, acc);
+        acc = M::mma(av.w, bv.w, acc);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) part[wave][M::acc_row(r, lane)][lrow] = acc[r];
+    __syncthreads();
+    const bool has_bias = (p.epilogue & FTH_EPI_BIAS) != 0, has_gelu = (p.epilogue & FTH_EPI_GELU) != 0;
+    const bool has_gelu_tanh = (p.epilogue & FTH_EPI_GELU_TANH) != 0, has_res = (p.epilogue & FTH_EPI_RESIDUAL) != 0;
+    float *C = p.c + batch * p.stride_c;
+#pragma unroll
+    for (int e = tid; e < 1024; e += 64 * NW) {
+        const int r = e >> 5, c = e & 31;
+        const int64_t row = m0 + r, col = n0 + c;
+        if (row < p.m && col < p.n) {
+            float v = part[0][r][c];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) v += part[w][r][c];
+            if (p.use_alpha) v = p.alpha * v;
+            if (has_bias) v = v + p.bias[col];
+            if (has_gelu) v = M::gelu(v);
+            if (has_gelu_tanh) v = M::gelu_tanh(v);
+            if (has_res) v = v + p.residual[batch * p.stride_c + row * p.ldc + col];
+            C[row * p.ldc + col] = v;
+        }
+    }
+}
+
+// True (and the kernel launched) when the problem is one of the small ones this kernel is for.
+template <bool TRANS_B> bool launch_small(GemmArgs<float> &p, int64_t batch, bool vec_a, bool vec_b, hipStream_t st, int32_t *rc) {
+    static const bool off = [] {
+        const char *e = std::getenv("FT_HIP_GEMM_SMALL");  // tuning knob: 0 sends small problems to the large-tile kernels
+        return e && std::atoi(e) == 0;
+    }();
+    const int64_t tiles = fth::ceil_div(p.m, 32) * fth::ceil_div(p.n, 32);
+    double flop = 2.0 * (double)p.m * (double)p.n * (double)p.k * (double)batch;
+    if (off || !vec_a || (TRANS_B && !vec_b) || p.k % 8 != 0 || p.k < 64 || flop > 4.0e8 || tiles > 2147483647LL || batch > 65535) return false;
+    p.tiles_m = (int)fth::ceil_div(p.m, 32);
+    p.tiles_n = (int)fth::ceil_div(p.n, 32);
+    const dim3 grid((unsigned)tiles, (unsigned)batch);
+    if (p.k <= 512) gemm_small_kernel<4, TRANS_B><<<grid, dim3(256), 0, st>>>(p);
+    else gemm_small_kernel<8, TRANS_B><<<grid, dim3(512), 0, st>>>(p);
+    hipError_t e = hipGetLastError();
+    *rc = e == hipSuccess ? FTH_OK : fth::hip_fail(e, "gemm_small");
+    return true;
+}
+
 // Epilogue-only kernel for k == 0 (the product is all zeros).
 template <typename T>
 __global__ __launch_bounds__(256) void gemm_k0_kernel(const GemmArgs<T> p) {
@@ -1206,6 +1294,11 @@ int32_t gemm_entry(const fth_gemm_desc *d, T alpha, const T *a, const T *b, T *c
     // 128-bit global loads along k need 16-byte aligned rows in every batch.
     bool vec = d->k % EPV == 0 && d->lda % EPV == 0 && al(a) && d->stride_a % EPV == 0;
     if (d->trans_b) vec = vec && d->ldb % EPV == 0 && al(b) && d->stride_b % EPV == 0;
+    if constexpr (std::is_same<T, float>::value) {
+        int32_t rc = FTH_OK;
+        const bool vec_bt = d->ldb % EPV == 0 && al(b) && d->stride_b % EPV == 0;
+        if (d->trans_b ? launch_small<true>(p, d->batch, vec, vec_bt, st, &rc) : launch_small<false>(p, d->batch, vec, true, st, &rc)) return rc;
+    }
     if (d->trans_b) {
         return vec ? launch_shape<T, true, true, false>(p, d->batch, st) : launch_shape<T, true, false, false>(p, d->batch, st);
     }
