@@ -53,6 +53,42 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const float *__restr
     for (int64_t i = threadIdx.x; i < k; i += 256) qr[i] = quantize_one(xr[i], scale);
 }
 
+// Rows of whole 128-bit vectors that fit the registers of a workgroup (k <= 1024 VPT): read once with 128-bit loads,
+// written as packed bytes (one 32-bit store per four values).
+template <int VPT>
+__global__ __launch_bounds__(256) void quantize_rows_vec_kernel(const float *__restrict__ x, int64_t k, int8_t *__restrict__ q,
+                                                               float *__restrict__ scales) {
+    __shared__ float red[4];
+    const int64_t row = blockIdx.x;
+    const float4 *xr = reinterpret_cast<const float4 *>(x + row * k);
+    const int nvec = (int)(k / 4);
+    float4 v[VPT];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = threadIdx.x + i * 256;
+        v[i] = c < nvec ? xr[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+        amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[i].x), fabsf(v[i].y)), fmaxf(fabsf(v[i].z), fabsf(v[i].w))));
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, kWave));
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
+    if (threadIdx.x == 0) scales[row] = scale;
+    uint32_t *qr = reinterpret_cast<uint32_t *>(q + row * k);
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = threadIdx.x + i * 256;
+        if (c < nvec) {
+            const uint32_t b0 = (uint8_t)quantize_one(v[i].x, scale), b1 = (uint8_t)quantize_one(v[i].y, scale);
+            const uint32_t b2 = (uint8_t)quantize_one(v[i].z, scale), b3 = (uint8_t)quantize_one(v[i].w, scale);
+            __builtin_nontemporal_store(b0 | (b1 << 8) | (b2 << 16) | (b3 << 24), qr + c);
+        }
+    }
+}
+
 // ---- the product -------------------------------------------------------------------------------------
 struct I8Args {
     const int8_t *a;  // [m, k] quantised activations
@@ -275,7 +311,13 @@ int32_t quantize_entry(const float *x, int64_t rows, int64_t cols, int8_t *q, fl
     if (rows == 0) return FTH_OK;
     FTH_ARG(scales && (cols == 0 || (x && q)), "quantize_i8: NULL operand");
     FTH_ARG(rows <= 2147483647LL, "quantize_i8: too many rows for one launch");
-    quantize_rows_kernel<<<dim3((unsigned)rows), dim3(256), 0, fth::resolve_stream(s)>>>(x, cols, q, scales);
+    hipStream_t st = fth::resolve_stream(s);
+    const bool vec = cols % 4 == 0 && cols > 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(q) & 3u) == 0;
+    if (vec && cols <= 1024) quantize_rows_vec_kernel<1><<<dim3((unsigned)rows), dim3(256), 0, st>>>(x, cols, q, scales);
+    else if (vec && cols <= 2048) quantize_rows_vec_kernel<2><<<dim3((unsigned)rows), dim3(256), 0, st>>>(x, cols, q, scales);
+    else if (vec && cols <= 4096) quantize_rows_vec_kernel<4><<<dim3((unsigned)rows), dim3(256), 0, st>>>(x, cols, q, scales);
+    else if (vec && cols <= 8192) quantize_rows_vec_kernel<8><<<dim3((unsigned)rows), dim3(256), 0, st>>>(x, cols, q, scales);
+    else quantize_rows_kernel<<<dim3((unsigned)rows), dim3(256), 0, st>>>(x, cols, q, scales);
     FTH_CHECK_LAUNCH("quantize_rows_i8");
     return FTH_OK;
 }

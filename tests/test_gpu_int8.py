@@ -23,7 +23,9 @@ def _quantize(hip, x):
     return dq.to_host(), ds.to_host()
 
 
-@pytest.mark.parametrize("rows,cols", [(1, 8), (7, 200), (64, 384), (33, 4099), (300, 768), (5, 1)])
+# vector kernel (cols a multiple of 4 up to 8192, every registers-per-thread variant), scalar kernel (ragged or longer rows)
+@pytest.mark.parametrize("rows,cols", [(1, 8), (7, 200), (64, 384), (33, 4099), (300, 768), (5, 1), (40, 1028), (9, 2048), (17, 4096), (6, 8192),
+                                       (3, 8196), (5, 12288)])
 def test_quantize_rows_is_exact(hip, oracle, rows, cols):
     x = synth.normal(41, "x", (rows, cols), 0.0, 2.0)
     x[0, 0] = 0.0
