@@ -351,13 +351,16 @@ int32_t fth_dev_linear_int8_prequantized_f32(const int8_t *x_i8, const float *a_
     const bool aligned = ((reinterpret_cast<uintptr_t>(x_i8) | reinterpret_cast<uintptr_t>(w_i8)) & 15u) == 0;
     const int64_t tiles128 = fth::ceil_div(m, 128) * fth::ceil_div(n, 128), tiles256 = fth::ceil_div(m, 256) * fth::ceil_div(n, 256);
     if (k >= kBK && k % kBK == 0 && aligned && tiles128 <= 2147483647LL) {
-        // 256 x 256 tiles once they give every compute unit a workgroup; the choice depends on the shape only
+        // 256 x 256 tiles once they give every compute unit a workgroup and the reduction is long enough to pay for their
+        // longer fill and drain (measured crossover between k = 4096 and k = 16384); the choice depends on the shape only.
+        // With real operands the sustained rate of either tile is set by the chip's power limit, not by the loop: the same
+        // launch runs 30% faster on all-zero operands than on operands spread over [-127, 127].
         const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
         static const int forced = [] {
             const char *e = std::getenv("FT_HIP_I8_TILE");  // tuning knob: 128 or 256; anything else = automatic
             return e ? std::atoi(e) : 0;
         }();
-        const bool big = forced == 256 || (forced != 128 && tiles256 >= cus);
+        const bool big = forced == 256 || (forced != 128 && tiles256 >= cus && k >= 8192);
         if (int32_t rc = big ? launch_i8_gemm<4>(p, st) : launch_i8_gemm<2>(p, st)) return rc;
     } else {
         int64_t total;
