@@ -374,14 +374,17 @@ def bench_backward(device, synth, steps, with_cpu):
     gq, gk, gv = DeviceBuffer(q.shape), DeviceBuffer(q.shape), DeviceBuffer(q.shape)
     ws3 = device.sdpa_backward(dq, dk, dv, ddo, B * H, S, S, D, D, sc, True, gq, gk, gv)
     ms = timed(lambda: device.sdpa_backward(dq, dk, dv, ddo, B * H, S, S, D, D, sc, True, gq, gk, gv, workspace=ws3), max(3, steps // 10))
-    flop = 5 * 2 * B * H * S * S * D
+    flop_full = 5 * 2 * B * H * S * S * D          # what the reference executes: five full [S,S] products per head
+    flop = 5 * 2 * B * H * (S * (S + 1) // 2) * D  # the causal count, as for the forward
     tf = flop / (ms * 1e-3) / 1e12
     out["sdpa_backward"] = {"ms": round(ms, 3), "TFLOP/s": round(tf, 2), "frac": round(tf / FP32_MFMA_PEAK_TF, 4), "flop": flop,
-                            "workload": "B4 H32 S2048 D128 causal fp32; flop = the reference's five full [S,S] products per head"}
+                            "reference_count_TFLOP/s": round(flop_full / (ms * 1e-3) / 1e12, 2),
+                            "workload": "B4 H32 S2048 D128 causal fp32; flop = five products over the causal half (4 D S(S+1)/2 x 2.5 per head); "
+                                        "reference_count = the reference's five full [S,S] products per head"}
     log("[backward] sdpa_backward        %.3f ms  %6.2f TFLOP/s  %.1f%% of MFMA peak" % (ms, tf, 100 * tf / FP32_MFMA_PEAK_TF))
     if with_cpu:
         best, reps = cpu_time(lambda: O.sdpa_backward(q[:1], k[:1], v[:1], do[:1], np.float32(sc), True), 3.0, min_reps=1)
-        out["sdpa_backward"]["cpu"] = {"value": round(flop / (B * H) / best / 1e12, 4), "unit": "TFLOP/s", "cores": O.threads(),
+        out["sdpa_backward"]["cpu"] = {"value": round(flop_full / (B * H) / best / 1e12, 4), "unit": "TFLOP/s (reference count)", "cores": O.threads(),
                                        "kind": "port", "sample": "1 of the 128 heads, wide-accumulation products, best of %d" % reps}
     del dq, dk, dv, ddo, gq, gk, gv, ws3
     # log-softmax and the fused cross-entropy on the forward's logits [8192, 50257] (made on the device by the LM-head product)

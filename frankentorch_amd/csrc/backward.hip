@@ -19,8 +19,11 @@
 // through the [k, m] operand path) and a column sum of dy. SDPA backward follows the reference's
 // own structure on the device: P = softmax(scale * Q.K^T) and dU are materialised per
 // (batch*head) in a caller-provided workspace (2 * num_bh * seq_q * seq_k elements), the five
-// products are batched MFMA GEMMs and the two row passes are HBM-bound row kernels.
+// products are batched MFMA GEMMs and the two row passes are HBM-bound row kernels. Long causal
+// square problems cut every product into blocks along the sequence and leave out what lies above
+// the block diagonal.
 
+#include <algorithm>
 #include <type_traits>
 
 #include "common.hpp"
@@ -588,12 +591,18 @@ __global__ __launch_bounds__(kThreads) void sdpa_softmax_backward_rows_kernel(co
     for (int64_t j = lane; j < seq_k; j += kWave) dr[j] = pr[j] * (dr[j] - dot);
 }
 
+// Columns of query row i that the block-causal products compute and read: whole key blocks up to the one holding i.
+__device__ __forceinline__ int sdpa_block_limit(int64_t i, int blk, int seq_k) {
+    const int64_t l = (i / blk + 1) * blk;
+    return (int)(l < seq_k ? l : seq_k);
+}
+
 // Register-resident forms of the two row passes for rows of up to 64 * VPL 16-byte vectors: the row is
 // read once (only its first `limit` entries matter for the softmax; the rest is written as zeros)
 // and written once. Same arithmetic as the streaming kernels above, lane-strided partial sums.
 template <typename T, int VPL>
 __global__ __launch_bounds__(kThreads) void sdpa_softmax_rows_vec_kernel(T *__restrict__ p, int64_t rows, int64_t seq_q, int seq_k,
-                                                                        T scale, int causal) {
+                                                                        T scale, int causal, int blk) {
     using V = typename Vec16<T>::type;
     constexpr int N = Vec16<T>::N;
     const int lane = threadIdx.x & (kWave - 1);
@@ -601,7 +610,8 @@ __global__ __launch_bounds__(kThreads) void sdpa_softmax_rows_vec_kernel(T *__re
     if (r >= rows) return;
     const int64_t i = r % seq_q;
     const int limit = causal ? (int)(i + 1 < seq_k ? i + 1 : seq_k) : seq_k;
-    const int nvec = seq_k / N;
+    // blk > 0: only the first (i / blk + 1) * blk columns of the row exist downstream (block-causal products)
+    const int nvec = (blk > 0 ? sdpa_block_limit(i, blk, seq_k) : seq_k) / N;
     V *row = reinterpret_cast<V *>(p + r * seq_k);
     T e[VPL][N];
     T m = -__builtin_inf();
@@ -654,13 +664,13 @@ __global__ __launch_bounds__(kThreads) void sdpa_softmax_rows_vec_kernel(T *__re
 
 template <typename T, int VPL>
 __global__ __launch_bounds__(kThreads) void sdpa_softmax_backward_rows_vec_kernel(const T *__restrict__ p, T *__restrict__ du, int64_t rows,
-                                                                                 int seq_k) {
+                                                                                 int64_t seq_q, int seq_k, int blk) {
     using V = typename Vec16<T>::type;
     constexpr int N = Vec16<T>::N;
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t r = (int64_t)blockIdx.x * kWaves + threadIdx.x / kWave;
     if (r >= rows) return;
-    const int nvec = seq_k / N;
+    const int nvec = (blk > 0 ? sdpa_block_limit(r % seq_q, blk, seq_k) : seq_k) / N;
     const V *pr = reinterpret_cast<const V *>(p + r * seq_k);
     V *dr = reinterpret_cast<V *>(du + r * seq_k);
     V pv[VPL], dv[VPL];
@@ -727,15 +737,40 @@ int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, i
     T *du = p + pe;
     const int64_t rows = num_bh * seq_q;
     FTH_ARG(fth::ceil_div(rows, kWaves) <= 2147483647LL, "sdpa backward: too many rows");
+    const int vpl = sdpa_row_vpl<T>(seq_k, p, du);
+    const dim3 row_grid((unsigned)fth::ceil_div(rows, kWaves));
+    // Causal square problems: the five products are cut into key / query blocks of `blk` rows so that nothing above the
+    // block diagonal is computed, stored or read (a little over half of the full work at eight blocks). Each block is one
+    // batched launch over all (batch, head) pairs; the choice depends on the shape only.
+    int64_t blk = 0;
+    if (causal && seq_q == seq_k && vpl > 0 && seq_k >= 512 && seq_k % 128 == 0 && d_k > 0 && d_v > 0) {
+        blk = (seq_k / 8 + 127) / 128 * 128;
+        if (blk < 128) blk = 128;
+    }
+    const int64_t nblk = blk > 0 ? fth::ceil_div(seq_q, blk) : 1;
+    auto strided = [&](int64_t m, int64_t n, int64_t kk, int ta, int tb, int64_t lda, int64_t ldb, int64_t ldc, int64_t sa, int64_t sb,
+                       int64_t sc) {
+        fth_gemm_desc d{};
+        d.m = m; d.n = n; d.k = kk;
+        d.lda = lda; d.ldb = ldb; d.ldc = ldc;
+        d.batch = num_bh;
+        d.stride_a = sa; d.stride_b = sb; d.stride_c = sc;
+        d.trans_a = ta; d.trans_b = tb;
+        return d;
+    };
     // P = Q . K^T  (scores; scaled inside the row pass)
-    if (d_k > 0) {
+    if (blk > 0) {
+        for (int64_t ib = 0; ib < nblk; ++ib) {
+            const int64_t i0 = ib * blk, i1 = std::min(seq_q, i0 + blk);
+            fth_gemm_desc d = strided(i1 - i0, i1, d_k, 0, 1, d_k, d_k, seq_k, seq_q * d_k, seq_k * d_k, seq_q * seq_k);
+            if (int32_t rc = dev_gemm<T>(&d, T(1), q + i0 * d_k, k, p + i0 * seq_k, fs)) return rc;
+        }
+    } else if (d_k > 0) {
         fth_gemm_desc d = make_desc(seq_q, seq_k, d_k, 0, 1, num_bh);
         if (int32_t rc = dev_gemm<T>(&d, T(1), q, k, p, fs)) return rc;
     } else {
         if (int32_t rc = zero_fill<T>(p, pe, st)) return rc;
     }
-    const int vpl = sdpa_row_vpl<T>(seq_k, p, du);
-    const dim3 row_grid((unsigned)fth::ceil_div(rows, kWaves));
 #define FTH_ROWS_VEC(KERN, ...)                                                         \
     switch (vpl) {                                                                      \
         case 1: KERN<T, 1><<<row_grid, dim3(kThreads), 0, st>>>(__VA_ARGS__); break;     \
@@ -745,31 +780,55 @@ int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, i
         default: KERN<T, 16><<<row_grid, dim3(kThreads), 0, st>>>(__VA_ARGS__); break;   \
     }
     if (vpl > 0) {
-        FTH_ROWS_VEC(sdpa_softmax_rows_vec_kernel, p, rows, seq_q, (int)seq_k, scale, causal)
+        FTH_ROWS_VEC(sdpa_softmax_rows_vec_kernel, p, rows, seq_q, (int)seq_k, scale, causal, (int)blk)
     } else {
         sdpa_softmax_rows_kernel<T><<<row_grid, dim3(kThreads), 0, st>>>(p, rows, seq_q, seq_k, scale, causal);
     }
     FTH_CHECK_LAUNCH("sdpa_backward_softmax");
     // dU = dOut . V^T
-    if (d_v > 0) {
+    if (blk > 0) {
+        for (int64_t ib = 0; ib < nblk; ++ib) {
+            const int64_t i0 = ib * blk, i1 = std::min(seq_q, i0 + blk);
+            fth_gemm_desc d = strided(i1 - i0, i1, d_v, 0, 1, d_v, d_v, seq_k, seq_q * d_v, seq_k * d_v, seq_q * seq_k);
+            if (int32_t rc = dev_gemm<T>(&d, T(1), dout + i0 * d_v, v, du + i0 * seq_k, fs)) return rc;
+        }
+    } else if (d_v > 0) {
         fth_gemm_desc d = make_desc(seq_q, seq_k, d_v, 0, 1, num_bh);
         if (int32_t rc = dev_gemm<T>(&d, T(1), dout, v, du, fs)) return rc;
     } else {
         if (int32_t rc = zero_fill<T>(du, pe, st)) return rc;
     }
-    // dV = P^T . dOut  (P read as the [k, m] operand) -- before dU is overwritten? dV does not use dU.
-    if (d_v > 0) {
+    // dV = P^T . dOut  (P read as the [k, m] operand); key block j only sees the queries from its first row on
+    if (blk > 0) {
+        for (int64_t jb = 0; jb < nblk; ++jb) {
+            const int64_t j0 = jb * blk, j1 = std::min(seq_k, j0 + blk);
+            fth_gemm_desc d = strided(j1 - j0, d_v, seq_q - j0, 1, 0, seq_k, d_v, d_v, seq_q * seq_k, seq_q * d_v, seq_k * d_v);
+            if (int32_t rc = dev_gemm<T>(&d, T(1), p + j0 * seq_k + j0, dout + j0 * d_v, dv + j0 * d_v, fs)) return rc;
+        }
+    } else if (d_v > 0) {
         fth_gemm_desc d = make_desc(seq_k, d_v, seq_q, 1, 0, num_bh);
         if (int32_t rc = dev_gemm<T>(&d, T(1), p, dout, dv, fs)) return rc;
     }
     if (vpl > 0) {
-        FTH_ROWS_VEC(sdpa_softmax_backward_rows_vec_kernel, p, du, rows, (int)seq_k)
+        FTH_ROWS_VEC(sdpa_softmax_backward_rows_vec_kernel, p, du, rows, seq_q, (int)seq_k, (int)blk)
     } else {
         sdpa_softmax_backward_rows_kernel<T><<<row_grid, dim3(kThreads), 0, st>>>(p, du, rows, seq_k);
     }
 #undef FTH_ROWS_VEC
     FTH_CHECK_LAUNCH("sdpa_backward_softmax_grad");
-    if (d_k > 0) {
+    if (blk > 0) {
+        // dQ = scale * dU . K over the keys up to the query block's end; dK = scale * dU^T . Q over the queries from the key block on
+        for (int64_t ib = 0; ib < nblk; ++ib) {
+            const int64_t i0 = ib * blk, i1 = std::min(seq_q, i0 + blk);
+            fth_gemm_desc d = strided(i1 - i0, d_k, i1, 0, 0, seq_k, d_k, d_k, seq_q * seq_k, seq_k * d_k, seq_q * d_k);
+            if (int32_t rc = dev_gemm<T>(&d, scale, du + i0 * seq_k, k, dq + i0 * d_k, fs)) return rc;
+        }
+        for (int64_t jb = 0; jb < nblk; ++jb) {
+            const int64_t j0 = jb * blk, j1 = std::min(seq_k, j0 + blk);
+            fth_gemm_desc d = strided(j1 - j0, d_k, seq_q - j0, 1, 0, seq_k, d_k, d_k, seq_q * seq_k, seq_q * d_k, seq_k * d_k);
+            if (int32_t rc = dev_gemm<T>(&d, scale, du + j0 * seq_k + j0, q + j0 * d_k, dk + j0 * d_k, fs)) return rc;
+        }
+    } else if (d_k > 0) {
         // dQ = scale * dU . K ; dK = scale * dU^T . Q
         fth_gemm_desc dqd = make_desc(seq_q, d_k, seq_k, 0, 0, num_bh);
         if (int32_t rc = dev_gemm<T>(&dqd, scale, du, k, dq, fs)) return rc;
