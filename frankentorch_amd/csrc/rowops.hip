@@ -817,5 +817,9 @@ int32_t fth_dev_bias_residual_add_f32(const float *x, const float *bias, const f
                                       int64_t rows, int64_t cols, fth_stream s) {
     return launch_bias<float, true>(x, bias, residual, y, rows, cols, s);
 }
+int32_t fth_dev_bias_residual_add_f64(const double *x, const double *bias, const double *residual, double *y,
+                                      int64_t rows, int64_t cols, fth_stream s) {
+    return launch_bias<double, true>(x, bias, residual, y, rows, cols, s);
+}
 
 }  // extern "C"

@@ -155,6 +155,8 @@ def layer_norm(x, weight, bias, y, batch, norm_size, eps, stream=None):
 
 
 def add_layer_norm(a, b, weight, bias, y, batch, norm_size, eps, stream=None):
+    if a.dtype != np.float32:
+        raise TypeError("add_layer_norm exists for float32 only (add_layer_norm_forward_f32 has no f64 twin)")
     check(_lib.load().fth_dev_add_layer_norm_f32(_ptr(a), _ptr(b), _ptr(weight), _ptr(bias), _ptr(y), batch, norm_size,
                                                  C.c_float(eps), stream))
 
@@ -181,7 +183,7 @@ def bias_add(x, bias, y, rows, cols, stream=None):
 
 
 def bias_residual_add(x, bias, residual, y, rows, cols, stream=None):
-    check(_lib.load().fth_dev_bias_residual_add_f32(_ptr(x), _ptr(bias), _ptr(residual), _ptr(y), rows, cols, stream))
+    check(getattr(_lib.load(), "fth_dev_bias_residual_add_" + _sfx(x))(_ptr(x), _ptr(bias), _ptr(residual), _ptr(y), rows, cols, stream))
 
 
 def index_select(inp, outer, dim_size, inner, indices, num_indices, out, bad_index=None, stream=None):

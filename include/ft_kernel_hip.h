@@ -184,6 +184,8 @@ int32_t fth_dev_bias_add_f64(const double *x, const double *bias, double *y, int
  * (crates/ft-kernel-cpu/src/lib.rs:17336-17351 then :36870-36877). */
 int32_t fth_dev_bias_residual_add_f32(const float *x, const float *bias, const float *residual, float *y,
                                       int64_t rows, int64_t cols, fth_stream s);
+int32_t fth_dev_bias_residual_add_f64(const double *x, const double *bias, const double *residual, double *y,
+                                      int64_t rows, int64_t cols, fth_stream s);
 
 /* index_select along dim 0 of a [table_rows, width] table: the embedding gather of
  * index_select_tensor_contiguous_f32 (crates/ft-kernel-cpu/src/lib.rs:40216-40253). Indices are
