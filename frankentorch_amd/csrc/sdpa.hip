@@ -313,34 +313,52 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
                 // ---- scale, mask, online softmax (lane-local query) ----
                 const bool need_mask = (d.causal && key0 + kBC - 1 > q_wave0) || (key0 + kBC > seq_k_i);
                 float mt = -__builtin_inff(), m_new, alpha, psum = 0.f;
-                if (!MASK && scale > 0.f) {
-                    // Positive scale (every real caller): the row max is taken on the raw scores (scaling
-                    // by a positive constant keeps the order), and scale * log2(e) is folded into one FMA
-                    // per score, 2^(s * c2 - m) with the running max m kept in those log2 units.
+                const float *vp = Vs + buf * VT + (4 * half) * VP + NDT * lq;
+                if constexpr (!MASK) {
+                    // Positive scale (the launcher sends unmasked calls with any other scale to the generic
+                    // kernel): the row max is taken on the raw scores (scaling by a positive constant keeps
+                    // the order), and scale * log2(e) is folded into one FMA per score, 2^(s * c2 - m) with
+                    // the running max m kept in those log2 units.
+                    if (need_mask) {  // wavefront-uniform; selects, no per-element branches
+#pragma unroll
+                        for (int j = 0; j < KS; ++j)
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) {
+                                const int key = key0 + 32 * j + 8 * (r >> 2) + 4 * half + (r & 3);
+                                const bool hidden = (d.causal && key > qi) | (key >= seq_k_i);
+                                s[j][r] = hidden ? -__builtin_inff() : s[j][r];
+                            }
+                    }
 #pragma unroll
                     for (int j = 0; j < KS; ++j)
 #pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            float x = s[j][r];
-                            if (need_mask) {
-                                const int key = key0 + 32 * j + 8 * (r >> 2) + 4 * half + (r & 3);
-                                if ((d.causal && key > qi) || key >= seq_k_i) x = -__builtin_inff();
-                            }
-                            s[j][r] = x;
-                            mt = fmaxf(mt, x);
-                        }
+                        for (int r = 0; r < 16; ++r) mt = fmaxf(mt, s[j][r]);
                     mt = fmaxf(mt, __shfl_xor(mt, 32, kWave));
                     m_new = fmaxf(m_run, mt * c2);
                     alpha = __builtin_amdgcn_exp2f(m_run - m_new);
                     const float neg_m = -m_new;
+                    if (__any(alpha != 1.0f)) {
+#pragma unroll
+                        for (int e = 0; e < NDT; ++e)
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) o[e][r] *= alpha;
+                    }
+                    // ---- O^T += V_tile^T . P^T with the exponentials in the same instruction stream: MFMA step r needs
+                    //      only weight r, so the exponential of weight r + 1 issues while the matrix unit works on step r ----
 #pragma unroll
                     for (int j = 0; j < KS; ++j)
 #pragma unroll
                         for (int r = 0; r < 16; ++r) {
                             const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][r], c2, neg_m));
-                            s[j][r] = e;
                             psum += e;
+                            const VV vv = *reinterpret_cast<const VV *>(vp + (32 * j + 8 * (r >> 2) + (r & 3)) * VP);
+#pragma unroll
+                            for (int ee = 0; ee < NDT; ++ee)
+                                o[ee] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(vv, ee), e, o[ee], 0, 0, 0);
                         }
+                    psum += __shfl_xor(psum, 32, kWave);
+                    l_run = l_run * alpha + psum;
+                    m_run = m_new;
                 } else {
 #pragma unroll
                     for (int j = 0; j < KS; ++j)
@@ -370,27 +388,26 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
                             s[j][r] = e;
                             psum += e;
                         }
-                }
-                psum += __shfl_xor(psum, 32, kWave);
-                l_run = l_run * alpha + psum;
-                m_run = m_new;
-                if (__any(alpha != 1.0f)) {
-#pragma unroll
-                    for (int e = 0; e < NDT; ++e)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) o[e][r] *= alpha;
-                }
-                // ---- O^T += V_tile^T . P^T ----
-                const float *vp = Vs + buf * VT + (4 * half) * VP + NDT * lq;
-#pragma unroll
-                for (int j = 0; j < KS; ++j)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const VV vv = *reinterpret_cast<const VV *>(vp + (32 * j + 8 * (r >> 2) + (r & 3)) * VP);
+                    psum += __shfl_xor(psum, 32, kWave);
+                    l_run = l_run * alpha + psum;
+                    m_run = m_new;
+                    if (__any(alpha != 1.0f)) {
 #pragma unroll
                         for (int e = 0; e < NDT; ++e)
-                            o[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(vv, e), s[j][r], o[e], 0, 0, 0);
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) o[e][r] *= alpha;
                     }
+                    // ---- O^T += V_tile^T . P^T ----
+#pragma unroll
+                    for (int j = 0; j < KS; ++j)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const VV vv = *reinterpret_cast<const VV *>(vp + (32 * j + 8 * (r >> 2) + (r & 3)) * VP);
+#pragma unroll
+                            for (int e = 0; e < NDT; ++e)
+                                o[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(vv, e), s[j][r], o[e], 0, 0, 0);
+                        }
+                }
             }
             if (kt + 1 < num_kt) store_tile(buf ^ 1);
             if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -780,7 +797,8 @@ int32_t sdpa_entry(const fth_sdpa_desc *d, double scale, const T *q, const T *k,
                                 m4(d->v_batch_stride) && m4(d->v_head_stride) && m4(d->v_row_stride) &&
                                 m4(d->o_batch_stride) && m4(d->o_head_stride) && m4(d->o_row_stride) &&
                                 al16(q) && al16(k) && al16(v) && al16(out);
-        if (strides_ok && d->d_k == d->d_v && d->seq_k > 0) {
+        // the unmasked MFMA kernels take the row maximum on the raw scores, which needs a positive scale
+        if (strides_ok && d->d_k == d->d_v && d->seq_k > 0 && (masked || scale > T(0))) {
             if (d->d_k == 128) return launch_mfma<128>(a, st);
             if (d->d_k == 64) return launch_mfma<64>(a, st);
             if (d->d_k == 32) return launch_mfma<32>(a, st);
