@@ -72,6 +72,21 @@ __device__ __forceinline__ void load_to_lds_16(const float *src, unsigned lds_ch
                  : "memory", "m0");
 }
 
+// The same with a scalar base and one unsigned 32-bit byte offset per lane: the offsets of a tile's chunks do not
+// change from tile to tile, so the per-tile address work is scalar.
+__device__ __forceinline__ void load_to_lds_16(const float *base, unsigned lane_off, unsigned lds_chunk) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base),
+                 "s"(__builtin_amdgcn_readfirstlane(lds_chunk))
+                 : "memory", "m0");
+}
+
+// x of lanes 0..31 and x of lanes 32..63, each broadcast to both halves (one v_permlane32_swap, no LDS round trip).
+__device__ __forceinline__ void both_halves(float x, float &lo, float &hi) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    lo = __uint_as_float(r[0]);
+    hi = __uint_as_float(r[1]);
+}
+
 template <int N> struct VecN;
 template <> struct VecN<1> { using type = float; };
 template <> struct VecN<2> { using type = float2; };
@@ -191,19 +206,40 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
         static_assert(!DIRECT || kBC % (RPC * NW) == 0, "tile rows must divide into chunks per wavefront");
         const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)reinterpret_cast<uintptr_t>(smem_raw));
         const unsigned wave_u = __builtin_amdgcn_readfirstlane((unsigned)wave);
+        // Per-lane byte offsets of this wavefront's chunks inside any full tile (row pitches up to 2^22 elements: launcher check).
+        unsigned k_off[DIRECT ? CPW : 1], v_off[DIRECT ? CPW : 1];
+        if constexpr (DIRECT) {
+#pragma unroll
+            for (int ci = 0; ci < CPW; ++ci) {
+                const int trow = (wave * CPW + ci) * RPC + lane / VPR;  // row inside the tile
+                const int slot = lane % VPR;
+                const int kq = (slot & ~15) | ((slot ^ trow) & 15);
+                k_off[ci] = (unsigned)trow * (unsigned)d.k_row_stride * 4u + 16u * (unsigned)kq;
+                v_off[ci] = (unsigned)trow * (unsigned)d.v_row_stride * 4u + 16u * (unsigned)slot;
+            }
+        }
         auto issue_tile = [&](int kt, int buf) __attribute__((always_inline)) {
             if constexpr (DIRECT) {
                 const int row_t0 = kt * kBC;
+                const float *kb = K + (int64_t)row_t0 * d.k_row_stride, *vb = Vg + (int64_t)row_t0 * d.v_row_stride;  // uniform
+                const unsigned kdst = lds0 + (unsigned)(buf * KT * 4) + wave_u * (CPW * 1024u);
+                const unsigned vdst = lds0 + (unsigned)((2 * KT + buf * VT) * 4) + wave_u * (CPW * 1024u);
+                if (row_t0 + kBC <= seq_k_i) {
 #pragma unroll
-                for (int ci = 0; ci < CPW; ++ci) {
-                    const int trow = (wave * CPW + ci) * RPC + lane / VPR;  // row inside the tile
-                    const int slot = lane % VPR;
-                    int grow = row_t0 + trow;
-                    grow = grow < seq_k_i ? grow : seq_k_i - 1;
-                    const int kq = (slot & ~15) | ((slot ^ trow) & 15);
-                    const unsigned chunk = (wave_u * CPW + ci) * 1024u;
-                    load_to_lds_16(K + (int64_t)grow * d.k_row_stride + 4 * kq, lds0 + (unsigned)(buf * KT * 4) + chunk);
-                    load_to_lds_16(Vg + (int64_t)grow * d.v_row_stride + 4 * slot, lds0 + (unsigned)((2 * KT + buf * VT) * 4) + chunk);
+                    for (int ci = 0; ci < CPW; ++ci) {
+                        load_to_lds_16(kb, k_off[ci], kdst + ci * 1024u);
+                        load_to_lds_16(vb, v_off[ci], vdst + ci * 1024u);
+                    }
+                } else {  // the last, partial tile: rows past the end re-read the last row (their scores are masked)
+#pragma unroll
+                    for (int ci = 0; ci < CPW; ++ci) {
+                        const int trow = (wave * CPW + ci) * RPC + lane / VPR;
+                        const int slot = lane % VPR;
+                        const int kq = (slot & ~15) | ((slot ^ trow) & 15);
+                        const int crow = row_t0 + trow < seq_k_i ? trow : seq_k_i - 1 - row_t0;
+                        load_to_lds_16(kb, (unsigned)crow * (unsigned)d.k_row_stride * 4u + 16u * (unsigned)kq, kdst + ci * 1024u);
+                        load_to_lds_16(vb, (unsigned)crow * (unsigned)d.v_row_stride * 4u + 16u * (unsigned)slot, vdst + ci * 1024u);
+                    }
                 }
             }
         };
@@ -248,8 +284,18 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
         if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): own tile parts have landed
         __syncthreads();
 
-        for (int kt = 0; kt < num_kt; ++kt) {
-            const int buf = kt & 1;
+        // Direct layout: fragment read t of K row lq is slot (2t) ^ lx; bits 1..3 of it take eight per-lane values, bit 4
+        // is 2t's own (lx < 16), so eight addresses plus immediates cover every read of every tile.
+        const int lx = half ^ (lq & 15);
+        const float *kfrag[DIRECT ? 8 : 1];
+        if constexpr (DIRECT) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) kfrag[u] = Ks + lq * KP + 4 * (((2 * u) ^ lx) & 15);
+        }
+        // One tile of the loop; the LDS buffer index is a compile-time constant (the loop below alternates two copies),
+        // so every LDS address of a tile is a per-lane base plus an immediate.
+        auto tile_step = [&](const int kt, auto buf_c) __attribute__((always_inline)) {
+            constexpr int buf = decltype(buf_c)::value;
             const int key0 = kt * kBC;
             // The other buffer was released by the barrier that ended the previous tile.
             if (kt + 1 < num_kt) issue_tile(kt + 1, buf ^ 1);
@@ -289,14 +335,14 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
                 for (int j = 0; j < KS; ++j)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) s[j][r] = 0.f;
-                const float *kp = Ks + buf * KT + lq * KP + (DIRECT ? 0 : 4 * half);
-                // direct layout: vector 2t + half of row lq sits in slot (2t + half) ^ (lq & 15) = 2t ^ lx
-                const int lx = half ^ (lq & 15);
+                const float *kp = Ks + buf * KT + lq * KP + 4 * half;  // staged layout
 #pragma unroll
                 for (int t = 0; t < D / 8; ++t) {
 #pragma unroll
                     for (int j = 0; j < KS; ++j) {
-                        const float4 kv = *reinterpret_cast<const float4 *>(kp + j * 32 * KP + (DIRECT ? 4 * ((2 * t) ^ lx) : 8 * t));
+                        // direct layout: vector 2t + half of row lq sits in slot (2t + half) ^ (lq & 15) = 2t ^ lx
+                        const float4 kv = DIRECT ? *reinterpret_cast<const float4 *>(kfrag[t & 7] + buf * KT + j * 32 * KP + 4 * ((2 * t) & 16))
+                                                 : *reinterpret_cast<const float4 *>(kp + j * 32 * KP + 8 * t);
                         s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.x, qr[t].x, s[j], 0, 0, 0);
                         s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.y, qr[t].y, s[j], 0, 0, 0);
                         s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.z, qr[t].z, s[j], 0, 0, 0);
@@ -333,7 +379,9 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
                     for (int j = 0; j < KS; ++j)
 #pragma unroll
                         for (int r = 0; r < 16; ++r) mt = fmaxf(mt, s[j][r]);
-                    mt = fmaxf(mt, __shfl_xor(mt, 32, kWave));
+                    float mlo, mhi;
+                    both_halves(mt, mlo, mhi);
+                    mt = fmaxf(mlo, mhi);
                     m_new = fmaxf(m_run, mt * c2);
                     alpha = __builtin_amdgcn_exp2f(m_run - m_new);
                     const float neg_m = -m_new;
@@ -356,8 +404,9 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
                             for (int ee = 0; ee < NDT; ++ee)
                                 o[ee] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(vv, ee), e, o[ee], 0, 0, 0);
                         }
-                    psum += __shfl_xor(psum, 32, kWave);
-                    l_run = l_run * alpha + psum;
+                    float plo, phi;
+                    both_halves(psum, plo, phi);
+                    l_run = l_run * alpha + (plo + phi);
                     m_run = m_new;
                 } else {
 #pragma unroll
@@ -412,6 +461,10 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
             if (kt + 1 < num_kt) store_tile(buf ^ 1);
             if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0x0F70);
             __syncthreads();
+        };
+        for (int kt = 0; kt < num_kt; kt += 2) {
+            tile_step(kt, std::integral_constant<int, 0>{});
+            if (kt + 1 < num_kt) tile_step(kt + 1, std::integral_constant<int, 1>{});
         }
 
         // ---- normalise and store: lane owns query qi, d = NDT * rho + e ----
@@ -796,7 +849,8 @@ int32_t sdpa_entry(const fth_sdpa_desc *d, double scale, const T *q, const T *k,
                                 m4(d->k_batch_stride) && m4(d->k_head_stride) && m4(d->k_row_stride) &&
                                 m4(d->v_batch_stride) && m4(d->v_head_stride) && m4(d->v_row_stride) &&
                                 m4(d->o_batch_stride) && m4(d->o_head_stride) && m4(d->o_row_stride) &&
-                                al16(q) && al16(k) && al16(v) && al16(out);
+                                al16(q) && al16(k) && al16(v) && al16(out) &&
+                                d->k_row_stride < (1 << 22) && d->v_row_stride < (1 << 22);  // a tile's lane offsets fit 32 bits
         // the unmasked MFMA kernels take the row maximum on the raw scores, which needs a positive scale
         if (strides_ok && d->d_k == d->d_v && d->seq_k > 0 && (masked || scale > T(0))) {
             if (d->d_k == 128) return launch_mfma<128>(a, st);
