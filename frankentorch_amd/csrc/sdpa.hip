@@ -415,47 +415,53 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
                         for (int r = 0; r < 16; ++r) {
                             float x = s[j][r] * scale;
                             if constexpr (MASK) x += mk[j][r];
-                            if (need_mask) {
-                                const int key = key0 + 32 * j + 8 * (r >> 2) + 4 * half + (r & 3);
-                                if ((d.causal && key > qi) || key >= seq_k_i) x = -__builtin_inff();
-                            }
                             s[j][r] = x;
-                            mt = fmaxf(mt, x);
                         }
-                    mt = fmaxf(mt, __shfl_xor(mt, 32, kWave));
+                    if (need_mask) {  // wavefront-uniform; selects, no per-element branches
+#pragma unroll
+                        for (int j = 0; j < KS; ++j)
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) {
+                                const int key = key0 + 32 * j + 8 * (r >> 2) + 4 * half + (r & 3);
+                                const bool hidden = (d.causal && key > qi) | (key >= seq_k_i);
+                                s[j][r] = hidden ? -__builtin_inff() : s[j][r];
+                            }
+                    }
+#pragma unroll
+                    for (int j = 0; j < KS; ++j)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) mt = fmaxf(mt, s[j][r]);
+                    float mlo, mhi;
+                    both_halves(mt, mlo, mhi);
+                    mt = fmaxf(mlo, mhi);
                     m_new = fmaxf(m_run, mt);
                     // A mask can hide every key seen so far (m_new still -inf): the weights are then 0 and the state
                     // stays empty, instead of the NaN that exp(-inf - -inf) would carry into later tiles. A row with
                     // no visible key at all ends as 0 / 0 = NaN, which is what the reference returns for it.
                     const float m_ref = (MASK && m_new == -__builtin_inff()) ? 0.f : m_new;
                     alpha = exp_diff(m_run, m_ref);
-#pragma unroll
-                    for (int j = 0; j < KS; ++j)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            const float e = exp_diff(s[j][r], m_ref);
-                            s[j][r] = e;
-                            psum += e;
-                        }
-                    psum += __shfl_xor(psum, 32, kWave);
-                    l_run = l_run * alpha + psum;
-                    m_run = m_new;
                     if (__any(alpha != 1.0f)) {
 #pragma unroll
                         for (int e = 0; e < NDT; ++e)
 #pragma unroll
                             for (int r = 0; r < 16; ++r) o[e][r] *= alpha;
                     }
-                    // ---- O^T += V_tile^T . P^T ----
+                    // ---- O^T += V_tile^T . P^T, exponentials inside the MFMA stream as above ----
 #pragma unroll
                     for (int j = 0; j < KS; ++j)
 #pragma unroll
                         for (int r = 0; r < 16; ++r) {
+                            const float e = exp_diff(s[j][r], m_ref);
+                            psum += e;
                             const VV vv = *reinterpret_cast<const VV *>(vp + (32 * j + 8 * (r >> 2) + (r & 3)) * VP);
 #pragma unroll
-                            for (int e = 0; e < NDT; ++e)
-                                o[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(vv, e), s[j][r], o[e], 0, 0, 0);
+                            for (int ee = 0; ee < NDT; ++ee)
+                                o[ee] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(vv, ee), e, o[ee], 0, 0, 0);
                         }
+                    float plo, phi;
+                    both_halves(psum, plo, phi);
+                    l_run = l_run * alpha + (plo + phi);
+                    m_run = m_new;
                 }
             }
             if (kt + 1 < num_kt) store_tile(buf ^ 1);
@@ -662,8 +668,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_f64_kernel(const SdpaArgs p)
         store_tile(0);
     }
     __syncthreads();
-    for (int kt = 0; kt < num_kt; ++kt) {
-        const int buf = kt & 1, key0 = kt * BC;
+    // One tile of the loop; the LDS buffer index is a compile-time constant (the loop below alternates two copies).
+    auto tile_step = [&](const int kt, auto buf_c) __attribute__((always_inline)) {
+        constexpr int buf = decltype(buf_c)::value;
+        const int key0 = kt * BC;
         if (kt + 1 < num_kt) load_tile(kt + 1);  // in flight under this tile's matrix work
         const bool wave_active = !d.causal || key0 <= wave_last_q;
         if (wave_active) {
@@ -692,7 +700,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_f64_kernel(const SdpaArgs p)
                 const int key = key0 + 4 * r + g;
                 double v = (s0[r] + s1[r]) * scale;
                 if constexpr (MASK) v += mk[r];
-                if ((d.causal && key > qi) || key >= seq_k_i) v = ninf;
+                const bool hidden = (d.causal && key > qi) | (key >= seq_k_i);
+                v = hidden ? ninf : v;
                 x[r] = v;
                 mt = fmax(mt, v);
             }
@@ -706,38 +715,48 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_f64_kernel(const SdpaArgs p)
             // needs the rescale: skip its exp and the pass over the accumulators.
             const bool rescale = __any(m_new != m_run);
             const double alpha = rescale ? exp(m_run - m_ref) : 1.0;
-            Acc4d pr;
-            double psum = 0.0;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const double e = exp(x[r] - m_ref);
-                pr[r] = e;
-                psum += e;
-            }
-            psum += __shfl_xor(psum, 16, kWave);
-            psum += __shfl_xor(psum, 32, kWave);
-            l_run = l_run * alpha + psum;
-            m_run = m_new;
             if (rescale) {
 #pragma unroll
                 for (int e = 0; e < NE; ++e)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) o[e][r] *= alpha;
             }
-            // ---- O^T += V_tile^T . P^T: step r contracts keys 4 r + g; d-tiles 2 e2 and 2 e2 + 1 share one read ----
+            // ---- O^T += V_tile^T . P^T: step r contracts keys 4 r + g; d-tiles 2 e2 and 2 e2 + 1 share one read.
+            //      Step r needs only weight r, so the exponential of weight r + 1 (some forty fp64 operations) is
+            //      spread between the MFMAs of step r. ----
             const double *vp = Vs + buf * KT + g * P + 2 * lq;
+            double psum = 0.0;
+            double e_cur = exp(x[0] - m_ref);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
+                const double e_r = e_cur;
+                psum += e_r;
+                if (r + 1 < 4) e_cur = exp(x[r + 1] - m_ref);
 #pragma unroll
                 for (int e2 = 0; e2 < NE / 2; ++e2) {
                     const double2 vv = *reinterpret_cast<const double2 *>(vp + (4 * r) * P + 32 * e2);
-                    o[2 * e2] = __builtin_amdgcn_mfma_f64_16x16x4f64(vv.x, pr[r], o[2 * e2], 0, 0, 0);
-                    o[2 * e2 + 1] = __builtin_amdgcn_mfma_f64_16x16x4f64(vv.y, pr[r], o[2 * e2 + 1], 0, 0, 0);
+                    o[2 * e2] = __builtin_amdgcn_mfma_f64_16x16x4f64(vv.x, e_r, o[2 * e2], 0, 0, 0);
+                    o[2 * e2 + 1] = __builtin_amdgcn_mfma_f64_16x16x4f64(vv.y, e_r, o[2 * e2 + 1], 0, 0, 0);
+                }
+                if (r + 1 < 4) {
+#pragma unroll
+                    for (int i = 0; i < NE; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA of step r ...
+                        __builtin_amdgcn_sched_group_barrier(0x002, 48 / NE, 0);  // ... then a share of the next exponential
+                    }
                 }
             }
+            psum += __shfl_xor(psum, 16, kWave);
+            psum += __shfl_xor(psum, 32, kWave);
+            l_run = l_run * alpha + psum;
+            m_run = m_new;
         }
         if (kt + 1 < num_kt) store_tile(buf ^ 1);
         __syncthreads();
+    };
+    for (int kt = 0; kt < num_kt; kt += 2) {
+        tile_step(kt, std::integral_constant<int, 0>{});
+        if (kt + 1 < num_kt) tile_step(kt + 1, std::integral_constant<int, 1>{});
     }
 
     // ---- normalise and store: element r of d-tile e is d = 32 (e / 2) + 2 (4 r + g) + e % 2 of query qi ----
