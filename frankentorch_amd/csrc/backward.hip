@@ -548,16 +548,21 @@ template <> __device__ __forceinline__ double dev_exp_t<double>(double v) { retu
 
 template <typename T>
 __global__ __launch_bounds__(kThreads) void sdpa_softmax_rows_kernel(T *__restrict__ p, int64_t rows, int64_t seq_q, int64_t seq_k,
-                                                                    T scale, int causal) {
+                                                                    T scale, int causal, const T *__restrict__ mask,
+                                                                    int64_t mask_bh_stride) {
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t r = (int64_t)blockIdx.x * kWaves + threadIdx.x / kWave;
     if (r >= rows) return;
     const int64_t i = r % seq_q;
     const int64_t limit = causal ? (i + 1 < seq_k ? i + 1 : seq_k) : seq_k;
     T *row = p + r * seq_k;
+    // additive mask row (sdpa_backward_masked_f64, :5466-5475): the score becomes s * scale + mask
+    const T *mrow = mask ? mask + (r / seq_q) * mask_bh_stride + i * seq_k : nullptr;
     T m = -__builtin_inf();
     for (int64_t j = lane; j < limit; j += kWave) {
-        const T v = row[j] * scale;
+        T v = row[j] * scale;
+        if (mrow) v = v + mrow[j];
+        row[j] = v;
         m = v > m ? v : m;
     }
 #pragma unroll
@@ -566,8 +571,8 @@ __global__ __launch_bounds__(kThreads) void sdpa_softmax_rows_kernel(T *__restri
         m = o > m ? o : m;
     }
     T sum = T(0);
-    for (int64_t j = lane; j < limit; j += kWave) {
-        const T e = dev_exp_t<T>(row[j] * scale - m);
+    for (int64_t j = lane; j < limit; j += kWave) {  // each lane re-reads only what it wrote above
+        const T e = dev_exp_t<T>(row[j] - m);
         row[j] = e;
         sum += e;
     }
@@ -602,7 +607,8 @@ __device__ __forceinline__ int sdpa_block_limit(int64_t i, int blk, int seq_k) {
 // and written once. Same arithmetic as the streaming kernels above, lane-strided partial sums.
 template <typename T, int VPL>
 __global__ __launch_bounds__(kThreads) void sdpa_softmax_rows_vec_kernel(T *__restrict__ p, int64_t rows, int64_t seq_q, int seq_k,
-                                                                        T scale, int causal, int blk) {
+                                                                        T scale, int causal, int blk, const T *__restrict__ mask,
+                                                                        int64_t mask_bh_stride) {
     using V = typename Vec16<T>::type;
     constexpr int N = Vec16<T>::N;
     const int lane = threadIdx.x & (kWave - 1);
@@ -613,6 +619,8 @@ __global__ __launch_bounds__(kThreads) void sdpa_softmax_rows_vec_kernel(T *__re
     // blk > 0: only the first (i / blk + 1) * blk columns of the row exist downstream (block-causal products)
     const int nvec = (blk > 0 ? sdpa_block_limit(i, blk, seq_k) : seq_k) / N;
     V *row = reinterpret_cast<V *>(p + r * seq_k);
+    // additive mask row, 16-byte aligned like the score row (the launcher checks)
+    const V *mrow = mask ? reinterpret_cast<const V *>(mask + (r / seq_q) * mask_bh_stride + i * seq_k) : nullptr;
     T e[VPL][N];
     T m = -__builtin_inf();
 #pragma unroll
@@ -620,9 +628,12 @@ __global__ __launch_bounds__(kThreads) void sdpa_softmax_rows_vec_kernel(T *__re
         const int v = lane + u * kWave;
         if (v < nvec && v * N < limit) {
             const V x = row[v];
+            V mv;
+            if (mrow) mv = mrow[v];
 #pragma unroll
             for (int c = 0; c < N; ++c) {
                 e[u][c] = vget(x, c) * scale;
+                if (mrow) e[u][c] = e[u][c] + vget(mv, c);
                 if (v * N + c < limit) m = e[u][c] > m ? e[u][c] : m;
             }
         } else {
@@ -714,7 +725,7 @@ template <typename T> size_t sdpa_backward_workspace(int64_t num_bh, int64_t seq
 template <typename T>
 int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, int64_t num_bh, int64_t seq_q, int64_t seq_k,
                             int64_t d_k, int64_t d_v, T scale, int causal, T *dq, T *dk, T *dv, void *workspace,
-                            size_t workspace_bytes, fth_stream s) {
+                            size_t workspace_bytes, fth_stream s, const T *mask = nullptr, int64_t mask_bh_stride = 0) {
     FTH_REQUIRE_DEVICE();
     FTH_ARG(num_bh >= 0 && seq_q >= 0 && seq_k >= 0 && d_k >= 0 && d_v >= 0, "sdpa backward: negative extent");
     hipStream_t st = fth::resolve_stream(s);
@@ -737,7 +748,8 @@ int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, i
     T *du = p + pe;
     const int64_t rows = num_bh * seq_q;
     FTH_ARG(fth::ceil_div(rows, kWaves) <= 2147483647LL, "sdpa backward: too many rows");
-    const int vpl = sdpa_row_vpl<T>(seq_k, p, du);
+    int vpl = sdpa_row_vpl<T>(seq_k, p, du);
+    if (mask && ((reinterpret_cast<uintptr_t>(mask) & 15u) != 0 || mask_bh_stride % Vec16<T>::N != 0)) vpl = 0;  // unaligned mask rows
     const dim3 row_grid((unsigned)fth::ceil_div(rows, kWaves));
     // Causal square problems: the five products are cut into key / query blocks of `blk` rows so that nothing above the
     // block diagonal is computed, stored or read (a little over half of the full work at eight blocks). Each block is one
@@ -780,9 +792,9 @@ int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, i
         default: KERN<T, 16><<<row_grid, dim3(kThreads), 0, st>>>(__VA_ARGS__); break;   \
     }
     if (vpl > 0) {
-        FTH_ROWS_VEC(sdpa_softmax_rows_vec_kernel, p, rows, seq_q, (int)seq_k, scale, causal, (int)blk)
+        FTH_ROWS_VEC(sdpa_softmax_rows_vec_kernel, p, rows, seq_q, (int)seq_k, scale, causal, (int)blk, mask, mask_bh_stride)
     } else {
-        sdpa_softmax_rows_kernel<T><<<row_grid, dim3(kThreads), 0, st>>>(p, rows, seq_q, seq_k, scale, causal);
+        sdpa_softmax_rows_kernel<T><<<row_grid, dim3(kThreads), 0, st>>>(p, rows, seq_q, seq_k, scale, causal, mask, mask_bh_stride);
     }
     FTH_CHECK_LAUNCH("sdpa_backward_softmax");
     // dU = dOut . V^T
@@ -893,6 +905,24 @@ int32_t fth_dev_sdpa_backward_f64(const double *q, const double *k, const double
                                   int64_t seq_k, int64_t d_k, int64_t d_v, double scale, int32_t causal, double *dq, double *dk,
                                   double *dv, void *workspace, size_t workspace_bytes, fth_stream s) {
     return sdpa_backward_entry<double>(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dk, dv, workspace, workspace_bytes, s);
+}
+int32_t fth_dev_sdpa_backward_masked_f32(const float *q, const float *k, const float *v, const float *dout, int64_t num_bh, int64_t seq_q,
+                                         int64_t seq_k, int64_t d_k, int64_t d_v, float scale, const float *mask, int64_t mask_bh_stride,
+                                         float *dq, float *dk, float *dv, void *workspace, size_t workspace_bytes, fth_stream s) {
+    FTH_ARG(mask != nullptr || num_bh == 0 || seq_q == 0 || seq_k == 0, "sdpa backward: NULL mask");
+    FTH_ARG(mask_bh_stride == 0 || mask_bh_stride >= seq_q * seq_k, "sdpa backward: mask_bh_stride %lld is neither 0 nor >= seq_q * seq_k",
+            (long long)mask_bh_stride);
+    return sdpa_backward_entry<float>(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, 0, dq, dk, dv, workspace, workspace_bytes, s, mask,
+                                      mask_bh_stride);
+}
+int32_t fth_dev_sdpa_backward_masked_f64(const double *q, const double *k, const double *v, const double *dout, int64_t num_bh, int64_t seq_q,
+                                         int64_t seq_k, int64_t d_k, int64_t d_v, double scale, const double *mask, int64_t mask_bh_stride,
+                                         double *dq, double *dk, double *dv, void *workspace, size_t workspace_bytes, fth_stream s) {
+    FTH_ARG(mask != nullptr || num_bh == 0 || seq_q == 0 || seq_k == 0, "sdpa backward: NULL mask");
+    FTH_ARG(mask_bh_stride == 0 || mask_bh_stride >= seq_q * seq_k, "sdpa backward: mask_bh_stride %lld is neither 0 nor >= seq_q * seq_k",
+            (long long)mask_bh_stride);
+    return sdpa_backward_entry<double>(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, 0, dq, dk, dv, workspace, workspace_bytes, s, mask,
+                                       mask_bh_stride);
 }
 
 }  // extern "C"

@@ -863,11 +863,12 @@ int32_t linear_backward_impl(const T *dy, size_t dy_len, const T *x, size_t x_le
     return fetch(dx, ddx, (size_t)n_x);
 }
 
-// sdpa_backward (crates/ft-kernel-cpu/src/lib.rs:5539-5650 / 5300-5414)
+// sdpa_backward (crates/ft-kernel-cpu/src/lib.rs:5539-5650 / 5300-5414) and sdpa_backward_masked (:5423-5530, `masked`)
 template <typename T>
 int32_t sdpa_backward_impl(const T *q, size_t q_len, const T *k, size_t k_len, const T *v, size_t v_len, const T *dout, size_t do_len,
                            size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, T scale, int32_t causal, T *dq,
-                           size_t dq_cap, T *dk, size_t dk_cap, T *dv, size_t dv_cap) {
+                           size_t dq_cap, T *dk, size_t dk_cap, T *dv, size_t dv_cap, bool masked = false, const T *mask = nullptr,
+                           size_t mask_len = 0, size_t mask_bh_stride = 0) {
     uint64_t nq, nk, nv, no, t;
     FTH_ARG(checked_mul(num_bh, seq_q, &t) && checked_mul(t, d_k, &nq) && checked_mul(t, d_v, &no) && checked_mul(num_bh, seq_k, &t) &&
                 checked_mul(t, d_k, &nk) && checked_mul(t, d_v, &nv),
@@ -876,11 +877,23 @@ int32_t sdpa_backward_impl(const T *q, size_t q_len, const T *k, size_t k_len, c
     if (int32_t rc = check_out(dk, dk_cap, (size_t)nk)) return rc;
     if (int32_t rc = check_out(dv, dv_cap, (size_t)nv)) return rc;
     FTH_ARG(q_len >= nq && k_len >= nk && v_len >= nv && do_len >= no, "sdpa backward: input slice shorter than its shape");
+    uint64_t nm = 0;
+    if (masked && num_bh > 0 && seq_q > 0 && seq_k > 0) {
+        uint64_t plane, span;
+        FTH_ARG(checked_mul(seq_q, seq_k, &plane) && checked_mul(num_bh - 1, mask_bh_stride, &span) && span + plane >= span,
+                "sdpa backward: mask extents overflow");
+        nm = span + plane;
+        FTH_ARG(mask_bh_stride == 0 || mask_bh_stride >= plane, "sdpa backward: mask_bh_stride %zu is neither 0 nor >= seq_q * seq_k",
+                mask_bh_stride);
+        FTH_ARG(mask != nullptr && mask_len >= nm, "sdpa backward: mask slice shorter than (num_bh - 1) * mask_bh_stride + seq_q * seq_k");
+    }
     if (nq == 0 && nk == 0 && nv == 0) return FTH_OK;
     FTH_REQUIRE_DEVICE();
     fth::Scratch sc;
-    T *dqi = nullptr, *dki = nullptr, *dvi = nullptr, *ddo = nullptr, *gq = nullptr, *gk = nullptr, *gv = nullptr;
+    T *dqi = nullptr, *dki = nullptr, *dvi = nullptr, *ddo = nullptr, *gq = nullptr, *gk = nullptr, *gv = nullptr, *dmask = nullptr;
     void *ws = nullptr;
+    if (nm > 0)
+        if (int32_t rc = stage_in(sc, mask, (size_t)nm, &dmask)) return rc;
     if (int32_t rc = stage_in(sc, q, (size_t)nq, &dqi)) return rc;
     if (int32_t rc = stage_in(sc, k, (size_t)nk, &dki)) return rc;
     if (int32_t rc = stage_in(sc, v, (size_t)nv, &dvi)) return rc;
@@ -891,12 +904,17 @@ int32_t sdpa_backward_impl(const T *q, size_t q_len, const T *k, size_t k_len, c
     const size_t wsb = fth_dev_sdpa_backward_workspace_bytes((int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, Dev<T>::dtype);
     if (int32_t rc = sc.get(&ws, wsb)) return rc;
     int32_t rc;
-    if constexpr (std::is_same<T, float>::value)
-        rc = fth_dev_sdpa_backward_f32(dqi, dki, dvi, ddo, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k, (int64_t)d_v, scale,
-                                       causal, gq, gk, gv, ws, wsb, nullptr);
-    else
-        rc = fth_dev_sdpa_backward_f64(dqi, dki, dvi, ddo, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k, (int64_t)d_v, scale,
-                                       causal, gq, gk, gv, ws, wsb, nullptr);
+    if constexpr (std::is_same<T, float>::value) {
+        rc = masked ? fth_dev_sdpa_backward_masked_f32(dqi, dki, dvi, ddo, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k,
+                                                       (int64_t)d_v, scale, dmask, (int64_t)mask_bh_stride, gq, gk, gv, ws, wsb, nullptr)
+                    : fth_dev_sdpa_backward_f32(dqi, dki, dvi, ddo, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k,
+                                                (int64_t)d_v, scale, causal, gq, gk, gv, ws, wsb, nullptr);
+    } else {
+        rc = masked ? fth_dev_sdpa_backward_masked_f64(dqi, dki, dvi, ddo, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k,
+                                                       (int64_t)d_v, scale, dmask, (int64_t)mask_bh_stride, gq, gk, gv, ws, wsb, nullptr)
+                    : fth_dev_sdpa_backward_f64(dqi, dki, dvi, ddo, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k,
+                                                (int64_t)d_v, scale, causal, gq, gk, gv, ws, wsb, nullptr);
+    }
     if (rc) return rc;
     if (int32_t r2 = fetch_no_sync(dk, gk, (size_t)nk)) return r2;
     if (int32_t r2 = fetch_no_sync(dv, gv, (size_t)nv)) return r2;
@@ -1070,6 +1088,20 @@ int32_t fth_sdpa_backward_f64(const double *q, size_t q_len, const double *k, si
                               int32_t causal, double *dq, size_t dq_cap, double *dk, size_t dk_cap, double *dv, size_t dv_cap) {
     return sdpa_backward_impl<double>(q, q_len, k, k_len, v, v_len, dout, dout_len, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dq_cap,
                                       dk, dk_cap, dv, dv_cap);
+}
+int32_t fth_sdpa_backward_masked_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len, const float *dout,
+                                     size_t dout_len, size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, float scale,
+                                     const float *mask, size_t mask_len, size_t mask_bh_stride, float *dq, size_t dq_cap, float *dk,
+                                     size_t dk_cap, float *dv, size_t dv_cap) {
+    return sdpa_backward_impl<float>(q, q_len, k, k_len, v, v_len, dout, dout_len, num_bh, seq_q, seq_k, d_k, d_v, scale, 0, dq, dq_cap, dk,
+                                     dk_cap, dv, dv_cap, true, mask, mask_len, mask_bh_stride);
+}
+int32_t fth_sdpa_backward_masked_f64(const double *q, size_t q_len, const double *k, size_t k_len, const double *v, size_t v_len, const double *dout,
+                                     size_t dout_len, size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, double scale,
+                                     const double *mask, size_t mask_len, size_t mask_bh_stride, double *dq, size_t dq_cap, double *dk,
+                                     size_t dk_cap, double *dv, size_t dv_cap) {
+    return sdpa_backward_impl<double>(q, q_len, k, k_len, v, v_len, dout, dout_len, num_bh, seq_q, seq_k, d_k, d_v, scale, 0, dq, dq_cap, dk,
+                                      dk_cap, dv, dv_cap, true, mask, mask_len, mask_bh_stride);
 }
 
 int32_t fth_log_softmax_dim_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta, size_t dim, float *out,

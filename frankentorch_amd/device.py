@@ -275,6 +275,16 @@ def sdpa_backward(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, 
     return ws
 
 
+def sdpa_backward_masked(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride, dq, dk, dv, workspace=None,
+                         stream=None):
+    """sdpa_backward_masked_f64 and its f32 twin: P = softmax(scale * Q.K^T + mask); mask_bh_stride 0 shares one [seq_q, seq_k] mask."""
+    ws = _workspace(_lib.load().fth_dev_sdpa_backward_workspace_bytes(num_bh, seq_q, seq_k, _dtype_code(q)), workspace)
+    check(getattr(_lib.load(), "fth_dev_sdpa_backward_masked_" + _sfx(q))(_ptr(q), _ptr(k), _ptr(v), _ptr(dout), num_bh, seq_q, seq_k, d_k,
+                                                                          d_v, _real(q, scale), _ptr(mask), mask_bh_stride, _ptr(dq),
+                                                                          _ptr(dk), _ptr(dv), ws.ptr, ws.nbytes, stream))
+    return ws
+
+
 def sdpa_desc_contiguous(num_bh, seq_q, seq_k, d_k, d_v, causal) -> _lib.SdpaDesc:
     d = _lib.SdpaDesc()
     _lib.load().fth_sdpa_desc_contiguous(C.byref(d), num_bh, seq_q, seq_k, d_k, d_v, 1 if causal else 0)

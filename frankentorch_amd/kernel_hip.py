@@ -337,6 +337,27 @@ def sdpa_backward_f64(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, caus
     return _sdpa_backward("f64", np.float64, q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal)
 
 
+def _sdpa_backward_masked(sfx, dtype, q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride):
+    q, k, v, dout, mask = _slice(q, dtype), _slice(k, dtype), _slice(v, dtype), _slice(dout, dtype), _slice(mask, dtype)
+    dq = np.empty(num_bh * seq_q * d_k, dtype=dtype)
+    dk = np.empty(num_bh * seq_k * d_k, dtype=dtype)
+    dv = np.empty(num_bh * seq_k * d_v, dtype=dtype)
+    check(getattr(_lib.load(), "fth_sdpa_backward_masked_" + sfx)(_p(q), q.size, _p(k), k.size, _p(v), v.size, _p(dout), dout.size, num_bh,
+                                                                  seq_q, seq_k, d_k, d_v, scale, _p(mask), mask.size, mask_bh_stride, _p(dq),
+                                                                  dq.size, _p(dk), dk.size, _p(dv), dv.size))
+    return dq, dk, dv
+
+
+def sdpa_backward_masked_f64(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride):
+    """(dq, dk, dv) with P = softmax(scale * Q.K^T + mask), crates/ft-kernel-cpu/src/lib.rs:5423."""
+    return _sdpa_backward_masked("f64", np.float64, q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride)
+
+
+def sdpa_backward_masked_f32(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride):
+    """The f32 twin of sdpa_backward_masked_f64 (the reference has the masked backward in f64 only)."""
+    return _sdpa_backward_masked("f32", np.float32, q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride)
+
+
 def _sdpa(name, dtype, q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal):
     q, k, v = _slice(q, dtype), _slice(k, dtype), _slice(v, dtype)
     out = np.empty(num_bh * seq_q * d_v, dtype=dtype)

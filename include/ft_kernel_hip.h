@@ -313,6 +313,15 @@ int32_t fth_dev_sdpa_backward_f32(const float *q, const float *k, const float *v
 int32_t fth_dev_sdpa_backward_f64(const double *q, const double *k, const double *v, const double *dout, int64_t num_bh, int64_t seq_q,
                                   int64_t seq_k, int64_t d_k, int64_t d_v, double scale, int32_t causal, double *dq, double *dk,
                                   double *dv, void *workspace, size_t workspace_bytes, fth_stream s);
+/* sdpa_backward_masked_f64 (:5423-5530; the same formulas in f32): the recomputed P is softmax(scale * Q.K^T + mask) per row,
+ * mask [seq_q, seq_k] rows shared by every (batch, head) when mask_bh_stride == 0, else mask_bh_stride elements apart
+ * (>= seq_q * seq_k); the mask is a constant (no gradient). Same workspace as the unmasked form. */
+int32_t fth_dev_sdpa_backward_masked_f32(const float *q, const float *k, const float *v, const float *dout, int64_t num_bh, int64_t seq_q,
+                                         int64_t seq_k, int64_t d_k, int64_t d_v, float scale, const float *mask, int64_t mask_bh_stride,
+                                         float *dq, float *dk, float *dv, void *workspace, size_t workspace_bytes, fth_stream s);
+int32_t fth_dev_sdpa_backward_masked_f64(const double *q, const double *k, const double *v, const double *dout, int64_t num_bh, int64_t seq_q,
+                                         int64_t seq_k, int64_t d_k, int64_t d_v, double scale, const double *mask, int64_t mask_bh_stride,
+                                         double *dq, double *dk, double *dv, void *workspace, size_t workspace_bytes, fth_stream s);
 
 /* Fused scaled-dot-product attention forward, q [num_bh, seq_q, d_k], k [num_bh, seq_k, d_k],
  * v [num_bh, seq_k, d_v] -> out [num_bh, seq_q, d_v]; causal limit = min(qi + 1, seq_k)
@@ -480,6 +489,15 @@ int32_t fth_sdpa_backward_f32(const float *q, size_t q_len, const float *k, size
 int32_t fth_sdpa_backward_f64(const double *q, size_t q_len, const double *k, size_t k_len, const double *v, size_t v_len, const double *dout,
                               size_t dout_len, size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, double scale,
                               int32_t causal, double *dq, size_t dq_cap, double *dk, size_t dk_cap, double *dv, size_t dv_cap);
+/* sdpa_backward_masked_f64 (:5423) and its f32 twin: mask slice of (num_bh - 1) * mask_bh_stride + seq_q * seq_k elements. */
+int32_t fth_sdpa_backward_masked_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len, const float *dout,
+                                     size_t dout_len, size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, float scale,
+                                     const float *mask, size_t mask_len, size_t mask_bh_stride, float *dq, size_t dq_cap, float *dk,
+                                     size_t dk_cap, float *dv, size_t dv_cap);
+int32_t fth_sdpa_backward_masked_f64(const double *q, size_t q_len, const double *k, size_t k_len, const double *v, size_t v_len, const double *dout,
+                                     size_t dout_len, size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, double scale,
+                                     const double *mask, size_t mask_len, size_t mask_bh_stride, double *dq, size_t dq_cap, double *dk,
+                                     size_t dk_cap, double *dv, size_t dv_cap);
 /* gelu_tensor_contiguous_f32 (:37123) / _f64 (:3657); add_tensor_contiguous_f32 (:36870) / _f64 */
 int32_t fth_gelu_tensor_contiguous_f32(const float *input, size_t input_len, const fth_meta *meta,
                                        float *out, size_t out_cap, size_t *out_len);

@@ -760,9 +760,12 @@ void linear_backward_impl(const T *dy, const T *x, const T *w, int64_t batch, in
 // sum, divide, zero tail), dU = dOut.V^T, dot_i = sum_j P_ij dU_ij, dU_ij = P_ij (dU_ij - dot_i),
 // dV = P^T.dOut, dQ = scale * dU.K, dK = scale * dU^T.Q. The products are the wide-accumulation
 // truth; the alpha of the scaled products is applied to the rounded product.
+// sdpa_backward_masked_f64 (KC:5423-5530) is the same with the score s * scale + mask[bh * mask_bh_stride + i * seq_k + j]
+// (KC:5466-5475) and no causal limit; `mask` non-NULL selects it.
 template <typename T>
 void sdpa_backward_impl(const T *q, const T *k, const T *v, const T *dout, int64_t num_bh, int64_t seq_q, int64_t seq_k,
-                        int64_t d_k, int64_t d_v, T scale, int causal, T *dq, T *dk, T *dv) {
+                        int64_t d_k, int64_t d_v, T scale, int causal, T *dq, T *dk, T *dv, const T *mask = nullptr,
+                        int64_t mask_bh_stride = 0) {
     std::vector<T> p((size_t)std::max<int64_t>(seq_q * seq_k, 1)), du((size_t)std::max<int64_t>(seq_q * seq_k, 1));
     for (int64_t bh = 0; bh < num_bh; ++bh) {
         const T *qh = q + bh * seq_q * d_k, *kh = k + bh * seq_k * d_k, *vh = v + bh * seq_k * d_v;
@@ -773,8 +776,9 @@ void sdpa_backward_impl(const T *q, const T *k, const T *v, const T *dout, int64
             const int64_t limit = causal ? std::min<int64_t>(i + 1, seq_k) : seq_k;
             T *row = p.data() + i * seq_k;
             T m = -std::numeric_limits<T>::infinity();
+            const T *mrow = mask ? mask + bh * mask_bh_stride + i * seq_k : nullptr;
             for (int64_t j = 0; j < limit; ++j) {
-                row[j] *= scale;
+                row[j] = mrow ? row[j] * scale + mrow[j] : row[j] * scale;
                 if (row[j] > m) m = row[j];
             }
             T sum = 0;
@@ -853,6 +857,16 @@ void fto_linear_backward_f64(const double *dy, const double *x, const double *w,
 void fto_sdpa_backward_f32(const float *q, const float *k, const float *v, const float *dout, int64_t num_bh, int64_t seq_q,
                            int64_t seq_k, int64_t d_k, int64_t d_v, float scale, int causal, float *dq, float *dk, float *dv) {
     sdpa_backward_impl<float>(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dk, dv);
+}
+void fto_sdpa_backward_masked_f32(const float *q, const float *k, const float *v, const float *dout, int64_t num_bh, int64_t seq_q,
+                                  int64_t seq_k, int64_t d_k, int64_t d_v, float scale, const float *mask, int64_t mask_bh_stride, float *dq,
+                                  float *dk, float *dv) {
+    sdpa_backward_impl<float>(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, 0, dq, dk, dv, mask, mask_bh_stride);
+}
+void fto_sdpa_backward_masked_f64(const double *q, const double *k, const double *v, const double *dout, int64_t num_bh, int64_t seq_q,
+                                  int64_t seq_k, int64_t d_k, int64_t d_v, double scale, const double *mask, int64_t mask_bh_stride,
+                                  double *dq, double *dk, double *dv) {
+    sdpa_backward_impl<double>(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, 0, dq, dk, dv, mask, mask_bh_stride);
 }
 void fto_sdpa_backward_f64(const double *q, const double *k, const double *v, const double *dout, int64_t num_bh,
                            int64_t seq_q, int64_t seq_k, int64_t d_k, int64_t d_v, double scale, int causal, double *dq,

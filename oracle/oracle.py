@@ -338,6 +338,21 @@ def sdpa_backward(q, k, v, dout, scale, causal):
     return dq, dk, dv
 
 
+def sdpa_backward_masked(q, k, v, dout, scale, mask, mask_bh_stride=None):
+    """(dq, dk, dv) for out = sdpa_forward_masked(q, k, v, scale, mask); mask [seq_q, seq_k] shared (stride 0) or [num_bh, seq_q, seq_k]."""
+    q, k, v, dout = _c(q), _c(k), _c(v), _c(dout)
+    mask = _c(np.asarray(mask, dtype=q.dtype))
+    sfx, ct = _sfx(q.dtype)
+    num_bh, seq_q, d_k = q.shape
+    seq_k, d_v = k.shape[1], v.shape[2]
+    if mask_bh_stride is None:
+        mask_bh_stride = 0 if mask.ndim == 2 else seq_q * seq_k
+    dq, dk, dv = np.zeros_like(q), np.zeros_like(k), np.zeros_like(v)
+    getattr(lib(), "fto_sdpa_backward_masked_" + sfx)(_p(q), _p(k), _p(v), _p(dout), _i64(num_bh), _i64(seq_q), _i64(seq_k), _i64(d_k),
+                                                      _i64(d_v), ct(scale), _p(mask), _i64(mask_bh_stride), _p(dq), _p(dk), _p(dv))
+    return dq, dk, dv
+
+
 def index_select(x, dim, indices):
     """Returns (out, bad): bad is the position of the first invalid index, or -1."""
     x = _c(x)

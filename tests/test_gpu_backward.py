@@ -112,6 +112,71 @@ def test_sdpa_backward(hip, oracle, bh, sq, sk, dk, dv, causal, dtype):
         assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
 
 
+@pytest.mark.parametrize("bh,sq,sk,dk,dv", [(2, 64, 64, 64, 64), (3, 100, 70, 32, 48), (1, 5, 6, 4, 3), (2, 33, 203, 16, 16), (2, 512, 384, 128, 128)])
+@pytest.mark.parametrize("shared", [True, False])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_sdpa_backward_masked(hip, oracle, bh, sq, sk, dk, dv, shared, dtype):
+    """sdpa_backward_masked_f64 (crates/ft-kernel-cpu/src/lib.rs:5423-5530) and its f32 twin: soft additive masks with hidden keys,
+    one mask for all heads or one per head; seq_k = 203 and the one-element offset below take the unvectorised row pass."""
+    tol = TOL_GEMM_F32 if dtype == np.float32 else TOL_F64
+    s = 1.0 / math.sqrt(dk)
+    q = synth.normal(24, "q", (bh, sq, dk), dtype=dtype)
+    k = synth.normal(24, "k", (bh, sk, dk), dtype=dtype)
+    v = synth.normal(24, "v", (bh, sk, dv), dtype=dtype)
+    do = synth.normal(24, "do", (bh, sq, dv), dtype=dtype)
+    mshape = (sq, sk) if shared else (bh, sq, sk)
+    mask = synth.normal(24, "mask", mshape, dtype=dtype)
+    mask = np.where(synth.uniform(24, "hide", mshape, 0, 1) < 0.25, -np.inf, mask).astype(dtype)
+    mask[..., 0] = 0  # every row keeps one key
+    ref = oracle.sdpa_backward_masked(q, k, v, do, dtype(s), mask)
+    dq_, dk_, dv_, ddo, dmask = _up(q, k, v, do, mask)
+    gq, gk, gv = DeviceBuffer(q.shape, dtype), DeviceBuffer(k.shape, dtype), DeviceBuffer(v.shape, dtype)
+    stride = 0 if shared else sq * sk
+    hip.sdpa_backward_masked(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, s, dmask, stride, gq, gk, gv)
+    got = (gq.to_host(), gk.to_host(), gv.to_host())
+    for g, r in zip(got, ref):
+        assert rel_err(g, r) <= tol * 2
+    hip.sdpa_backward_masked(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, s, dmask, stride, gq, gk, gv)
+    for a, b in zip(got, (gq.to_host(), gk.to_host(), gv.to_host())):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+    if shared:  # a mask that starts one element into its buffer: unaligned rows
+        pad = DeviceBuffer.from_host(np.concatenate([np.zeros(1, dtype), mask.ravel()]))
+        hip.sdpa_backward_masked(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, s, pad.view(1), 0, gq, gk, gv)
+        for g, r in zip((gq.to_host(), gk.to_host(), gv.to_host()), ref):
+            assert rel_err(g, r) <= tol * 2
+
+
+def test_sdpa_backward_masked_reduces_to_the_unmasked_and_causal_forms(hip):
+    bh, sq, sk, dk, dv = 2, 96, 96, 32, 32
+    q, k, v, do = (synth.normal(25, t, (bh, sq, dk)) for t in ("q", "k", "v", "do"))
+    dq_, dk_, dv_, ddo = _up(q, k, v, do)
+    outs = []
+    for mask, causal in ((np.zeros((sq, sk), np.float32), False), (np.where(np.arange(sk)[None, :] <= np.arange(sq)[:, None], 0.0, -np.inf).astype(np.float32), True)):
+        gq, gk, gv = DeviceBuffer(q.shape), DeviceBuffer(k.shape), DeviceBuffer(v.shape)
+        hq, hk, hv = DeviceBuffer(q.shape), DeviceBuffer(k.shape), DeviceBuffer(v.shape)
+        hip.sdpa_backward_masked(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, 0.2, DeviceBuffer.from_host(mask), 0, gq, gk, gv)
+        hip.sdpa_backward(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, 0.2, causal, hq, hk, hv)
+        for a, b in zip((gq, gk, gv), (hq, hk, hv)):
+            assert rel_err(a.to_host(), b.to_host()) <= TOL_GEMM_F32
+
+
+def test_host_slice_sdpa_backward_masked_and_its_errors(oracle):
+    from frankentorch_amd import kernel_hip as K
+    from frankentorch_amd.core import HipError, KernelError
+
+    bh, sq, sk, dk, dv = 2, 17, 23, 16, 8
+    q, k, v = synth.normal(26, "q", (bh, sq, dk), dtype=np.float64), synth.normal(26, "k", (bh, sk, dk), dtype=np.float64), synth.normal(26, "v", (bh, sk, dv), dtype=np.float64)
+    do = synth.normal(26, "do", (bh, sq, dv), dtype=np.float64)
+    mask = synth.normal(26, "m", (bh, sq, sk), dtype=np.float64)
+    got = K.sdpa_backward_masked_f64(q.ravel(), k.ravel(), v.ravel(), do.ravel(), bh, sq, sk, dk, dv, 0.25, mask.ravel(), sq * sk)
+    for g, r in zip(got, oracle.sdpa_backward_masked(q, k, v, do, 0.25, mask)):
+        assert rel_err(g, r.ravel()) <= 2 * TOL_F64
+    with pytest.raises((KernelError, HipError)):  # a mask slice shorter than num_bh planes
+        K.sdpa_backward_masked_f64(q.ravel(), k.ravel(), v.ravel(), do.ravel(), bh, sq, sk, dk, dv, 0.25, mask.ravel()[:-1], sq * sk)
+    with pytest.raises((KernelError, HipError)):  # a per-head stride smaller than one plane
+        K.sdpa_backward_masked_f64(q.ravel(), k.ravel(), v.ravel(), do.ravel(), bh, sq, sk, dk, dv, 0.25, mask.ravel(), 5)
+
+
 def test_norm_backward_at_the_row_op_benchmark_shape(hip, oracle):
     """fp32 [8192, 4096]: sampled rows against the checker, column sums against an f64 numpy sum, and the
     property that dx rows of LayerNorm sum to zero."""

@@ -107,6 +107,44 @@ def test_sdpa_backward_is_the_gradient_of_the_forward(oracle, causal):
     assert np.allclose(dq32, dq, atol=2e-5) and np.allclose(dk32, dk_, atol=2e-5) and np.allclose(dv32, dv_, atol=2e-5)
 
 
+@pytest.mark.parametrize("shared", [True, False])
+def test_sdpa_backward_masked_is_the_gradient_of_the_masked_forward(oracle, shared):
+    """sdpa_backward_masked_f64 (crates/ft-kernel-cpu/src/lib.rs:5423-5530) has no test of its own in the reference: it is pinned by
+    central differences of the pinned masked forward, by its reduction to the unmasked and causal backward for a zero and a
+    -inf-triangle mask, and by an einsum restatement of the textbook formulas."""
+    rng = np.random.default_rng(18)
+    bh, sq, sk, dk, dv = 3, 5, 6, 4, 3
+    q, k, v = rng.standard_normal((bh, sq, dk)), rng.standard_normal((bh, sk, dk)), rng.standard_normal((bh, sk, dv))
+    dout = rng.standard_normal((bh, sq, dv))
+    scale = 0.41
+    mask = rng.standard_normal((sq, sk) if shared else (bh, sq, sk))
+    mask[..., 1, 2] = -np.inf  # a hidden key in a row that keeps others
+    dq, dk_, dv_ = oracle.sdpa_backward_masked(q, k, v, dout, scale, mask)
+    assert np.allclose(dq, _num_grad(lambda t: oracle.sdpa_forward_masked(t, k, v, scale, mask), q.copy(), dout), atol=1e-7)
+    assert np.allclose(dk_, _num_grad(lambda t: oracle.sdpa_forward_masked(q, t, v, scale, mask), k.copy(), dout), atol=1e-7)
+    assert np.allclose(dv_, _num_grad(lambda t: oracle.sdpa_forward_masked(q, k, t, scale, mask), v.copy(), dout), atol=1e-7)
+    # einsum restatement
+    m3 = np.broadcast_to(mask, (bh, sq, sk))
+    sc = np.einsum("bqd,bkd->bqk", q, k) * scale + m3
+    p = np.exp(sc - sc.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    dp = np.einsum("bqd,bkd->bqk", dout, v)
+    du = p * (dp - (p * dp).sum(-1, keepdims=True))
+    assert np.allclose(dq, scale * np.einsum("bqk,bkd->bqd", du, k), atol=1e-12)
+    assert np.allclose(dk_, scale * np.einsum("bqk,bqd->bkd", du, q), atol=1e-12)
+    assert np.allclose(dv_, np.einsum("bqk,bqd->bkd", p, dout), atol=1e-12)
+    # zero mask = unmasked; -inf above the diagonal = causal
+    for got, ref in zip(oracle.sdpa_backward_masked(q, k, v, dout, scale, np.zeros((sq, sk))), oracle.sdpa_backward(q, k, v, dout, scale, False)):
+        assert np.array_equal(got, ref)
+    tri = np.where(np.arange(sk)[None, :] <= np.arange(sq)[:, None], 0.0, -np.inf)
+    for got, ref in zip(oracle.sdpa_backward_masked(q, k, v, dout, scale, tri), oracle.sdpa_backward(q, k, v, dout, scale, True)):
+        assert np.allclose(got, ref, atol=1e-14)
+    f = np.float32
+    g32 = oracle.sdpa_backward_masked(q.astype(f), k.astype(f), v.astype(f), dout.astype(f), f(scale), mask.astype(f))
+    for a, b in zip(g32, (dq, dk_, dv_)):
+        assert np.allclose(a, b, atol=2e-5)
+
+
 def test_log_softmax_reference_fixtures_and_identity(oracle, vectors):
     cases = [c for c in vectors["conformance"] if c["op"] == "log_softmax"]
     assert len(cases) == 2
