@@ -375,17 +375,18 @@ __global__ __launch_bounds__(kThreads) void col_final_kernel(const T *__restrict
 }
 
 // Zero fill as a kernel (memset nodes are avoided so that callers can capture these entry points).
-template <typename T> __global__ __launch_bounds__(kThreads) void zero_kernel(T *dst, int64_t n) {
+template <typename T> __global__ __launch_bounds__(kThreads) void fill_kernel(T *dst, int64_t n, T value) {
     const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-    if (i < n) dst[i] = T(0);
+    if (i < n) dst[i] = value;
 }
-template <typename T> int32_t zero_fill(T *dst, int64_t n, hipStream_t st) {
+template <typename T> int32_t value_fill(T *dst, int64_t n, T value, hipStream_t st) {
     if (n <= 0) return FTH_OK;
-    FTH_ARG(fth::ceil_div(n, kThreads) <= 2147483647LL, "zero fill: extent too large");
-    zero_kernel<T><<<dim3((unsigned)fth::ceil_div(n, kThreads)), dim3(kThreads), 0, st>>>(dst, n);
-    FTH_CHECK_LAUNCH("zero_fill");
+    FTH_ARG(fth::ceil_div(n, kThreads) <= 2147483647LL, "fill: extent too large");
+    fill_kernel<T><<<dim3((unsigned)fth::ceil_div(n, kThreads)), dim3(kThreads), 0, st>>>(dst, n, value);
+    FTH_CHECK_LAUNCH("fill");
     return FTH_OK;
 }
+template <typename T> int32_t zero_fill(T *dst, int64_t n, hipStream_t st) { return value_fill<T>(dst, n, T(0), st); }
 
 inline int pick_rows_per_block(int64_t rows) {
     // enough workgroups to fill the chip several times over, at most 64 rows each
@@ -725,7 +726,8 @@ template <typename T> size_t sdpa_backward_workspace(int64_t num_bh, int64_t seq
 template <typename T>
 int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, int64_t num_bh, int64_t seq_q, int64_t seq_k,
                             int64_t d_k, int64_t d_v, T scale, int causal, T *dq, T *dk, T *dv, void *workspace,
-                            size_t workspace_bytes, fth_stream s, const T *mask = nullptr, int64_t mask_bh_stride = 0) {
+                            size_t workspace_bytes, fth_stream s, const T *mask = nullptr, int64_t mask_bh_stride = 0,
+                            bool unit_dout = false) {
     FTH_REQUIRE_DEVICE();
     FTH_ARG(num_bh >= 0 && seq_q >= 0 && seq_k >= 0 && d_k >= 0 && d_v >= 0, "sdpa backward: negative extent");
     hipStream_t st = fth::resolve_stream(s);
@@ -738,14 +740,24 @@ int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, i
         if (dv && num_bh * seq_k * d_v > 0) if (int32_t rc = zero_fill<T>(dv, num_bh * seq_k * d_v, st)) return rc;
         return FTH_OK;
     }
-    FTH_ARG(q && k && v && dout && dq && dk && dv, "sdpa backward: NULL operand");
+    FTH_ARG(q && k && v && (dout || unit_dout) && dq && dk && dv, "sdpa backward: NULL operand");
     int64_t pe;
     FTH_ARG(!__builtin_mul_overflow(num_bh, seq_q, &pe) && !__builtin_mul_overflow(pe, seq_k, &pe) && pe < ((int64_t)1 << 40),
             "sdpa backward: score matrix too large");
-    FTH_ARG(workspace != nullptr && workspace_bytes >= sdpa_backward_workspace<T>(num_bh, seq_q, seq_k),
-            "sdpa backward: workspace of %zu bytes needed, %zu given", sdpa_backward_workspace<T>(num_bh, seq_q, seq_k), workspace_bytes);
+    const size_t ws_need = sdpa_backward_workspace<T>(num_bh, seq_q, seq_k) + (unit_dout ? (size_t)(seq_q * d_v + 4) * sizeof(T) : 0);
+    FTH_ARG(workspace != nullptr && workspace_bytes >= ws_need, "sdpa backward: workspace of %zu bytes needed, %zu given", ws_need,
+            workspace_bytes);
     T *p = static_cast<T *>(workspace);
     T *du = p + pe;
+    // dOut = ones (sdpa_backward_f32_unit_dout, :5662-5770): one [seq_q, d_v] plane of ones shared by every (batch, head)
+    // through a zero batch stride stands in for the gradient; nothing of size num_bh is materialised.
+    int64_t dout_bs = seq_q * d_v;
+    if (unit_dout) {
+        T *ones = p + ((2 * pe + 64 + 3) & ~(int64_t)3);  // keeps the 16-byte alignment of the workspace base
+        if (int32_t rc = value_fill<T>(ones, seq_q * d_v, T(1), st)) return rc;
+        dout = ones;
+        dout_bs = 0;
+    }
     const int64_t rows = num_bh * seq_q;
     FTH_ARG(fth::ceil_div(rows, kWaves) <= 2147483647LL, "sdpa backward: too many rows");
     int vpl = sdpa_row_vpl<T>(seq_k, p, du);
@@ -801,11 +813,12 @@ int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, i
     if (blk > 0) {
         for (int64_t ib = 0; ib < nblk; ++ib) {
             const int64_t i0 = ib * blk, i1 = std::min(seq_q, i0 + blk);
-            fth_gemm_desc d = strided(i1 - i0, i1, d_v, 0, 1, d_v, d_v, seq_k, seq_q * d_v, seq_k * d_v, seq_q * seq_k);
+            fth_gemm_desc d = strided(i1 - i0, i1, d_v, 0, 1, d_v, d_v, seq_k, dout_bs, seq_k * d_v, seq_q * seq_k);
             if (int32_t rc = dev_gemm<T>(&d, T(1), dout + i0 * d_v, v, du + i0 * seq_k, fs)) return rc;
         }
     } else if (d_v > 0) {
         fth_gemm_desc d = make_desc(seq_q, seq_k, d_v, 0, 1, num_bh);
+        d.stride_a = dout_bs;
         if (int32_t rc = dev_gemm<T>(&d, T(1), dout, v, du, fs)) return rc;
     } else {
         if (int32_t rc = zero_fill<T>(du, pe, st)) return rc;
@@ -814,11 +827,12 @@ int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, i
     if (blk > 0) {
         for (int64_t jb = 0; jb < nblk; ++jb) {
             const int64_t j0 = jb * blk, j1 = std::min(seq_k, j0 + blk);
-            fth_gemm_desc d = strided(j1 - j0, d_v, seq_q - j0, 1, 0, seq_k, d_v, d_v, seq_q * seq_k, seq_q * d_v, seq_k * d_v);
+            fth_gemm_desc d = strided(j1 - j0, d_v, seq_q - j0, 1, 0, seq_k, d_v, d_v, seq_q * seq_k, dout_bs, seq_k * d_v);
             if (int32_t rc = dev_gemm<T>(&d, T(1), p + j0 * seq_k + j0, dout + j0 * d_v, dv + j0 * d_v, fs)) return rc;
         }
     } else if (d_v > 0) {
         fth_gemm_desc d = make_desc(seq_k, d_v, seq_q, 1, 0, num_bh);
+        d.stride_b = dout_bs;
         if (int32_t rc = dev_gemm<T>(&d, T(1), p, dout, dv, fs)) return rc;
     }
     if (vpl > 0) {
@@ -905,6 +919,23 @@ int32_t fth_dev_sdpa_backward_f64(const double *q, const double *k, const double
                                   int64_t seq_k, int64_t d_k, int64_t d_v, double scale, int32_t causal, double *dq, double *dk,
                                   double *dv, void *workspace, size_t workspace_bytes, fth_stream s) {
     return sdpa_backward_entry<double>(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dk, dv, workspace, workspace_bytes, s);
+}
+size_t fth_dev_sdpa_backward_unit_dout_workspace_bytes(int64_t num_bh, int64_t seq_q, int64_t seq_k, int64_t d_v, int32_t dtype) {
+    if (num_bh < 0 || seq_q < 0 || seq_k < 0 || d_v < 0) return 0;
+    const size_t el = dtype == FTH_DTYPE_F64 ? sizeof(double) : sizeof(float);
+    return fth_dev_sdpa_backward_workspace_bytes(num_bh, seq_q, seq_k, dtype) + (size_t)(seq_q * d_v + 4) * el;
+}
+int32_t fth_dev_sdpa_backward_unit_dout_f32(const float *q, const float *k, const float *v, int64_t num_bh, int64_t seq_q, int64_t seq_k,
+                                            int64_t d_k, int64_t d_v, float scale, int32_t causal, float *dq, float *dk, float *dv,
+                                            void *workspace, size_t workspace_bytes, fth_stream s) {
+    return sdpa_backward_entry<float>(q, k, v, nullptr, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dk, dv, workspace, workspace_bytes, s,
+                                      nullptr, 0, true);
+}
+int32_t fth_dev_sdpa_backward_unit_dout_f64(const double *q, const double *k, const double *v, int64_t num_bh, int64_t seq_q, int64_t seq_k,
+                                            int64_t d_k, int64_t d_v, double scale, int32_t causal, double *dq, double *dk, double *dv,
+                                            void *workspace, size_t workspace_bytes, fth_stream s) {
+    return sdpa_backward_entry<double>(q, k, v, nullptr, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dk, dv, workspace, workspace_bytes, s,
+                                       nullptr, 0, true);
 }
 int32_t fth_dev_sdpa_backward_masked_f32(const float *q, const float *k, const float *v, const float *dout, int64_t num_bh, int64_t seq_q,
                                          int64_t seq_k, int64_t d_k, int64_t d_v, float scale, const float *mask, int64_t mask_bh_stride,

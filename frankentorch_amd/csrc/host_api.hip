@@ -868,7 +868,7 @@ template <typename T>
 int32_t sdpa_backward_impl(const T *q, size_t q_len, const T *k, size_t k_len, const T *v, size_t v_len, const T *dout, size_t do_len,
                            size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, T scale, int32_t causal, T *dq,
                            size_t dq_cap, T *dk, size_t dk_cap, T *dv, size_t dv_cap, bool masked = false, const T *mask = nullptr,
-                           size_t mask_len = 0, size_t mask_bh_stride = 0) {
+                           size_t mask_len = 0, size_t mask_bh_stride = 0, bool unit_dout = false) {
     uint64_t nq, nk, nv, no, t;
     FTH_ARG(checked_mul(num_bh, seq_q, &t) && checked_mul(t, d_k, &nq) && checked_mul(t, d_v, &no) && checked_mul(num_bh, seq_k, &t) &&
                 checked_mul(t, d_k, &nk) && checked_mul(t, d_v, &nv),
@@ -876,7 +876,7 @@ int32_t sdpa_backward_impl(const T *q, size_t q_len, const T *k, size_t k_len, c
     if (int32_t rc = check_out(dq, dq_cap, (size_t)nq)) return rc;
     if (int32_t rc = check_out(dk, dk_cap, (size_t)nk)) return rc;
     if (int32_t rc = check_out(dv, dv_cap, (size_t)nv)) return rc;
-    FTH_ARG(q_len >= nq && k_len >= nk && v_len >= nv && do_len >= no, "sdpa backward: input slice shorter than its shape");
+    FTH_ARG(q_len >= nq && k_len >= nk && v_len >= nv && (unit_dout || do_len >= no), "sdpa backward: input slice shorter than its shape");
     uint64_t nm = 0;
     if (masked && num_bh > 0 && seq_q > 0 && seq_k > 0) {
         uint64_t plane, span;
@@ -897,20 +897,27 @@ int32_t sdpa_backward_impl(const T *q, size_t q_len, const T *k, size_t k_len, c
     if (int32_t rc = stage_in(sc, q, (size_t)nq, &dqi)) return rc;
     if (int32_t rc = stage_in(sc, k, (size_t)nk, &dki)) return rc;
     if (int32_t rc = stage_in(sc, v, (size_t)nv, &dvi)) return rc;
-    if (int32_t rc = stage_in(sc, dout, (size_t)no, &ddo)) return rc;
+    if (!unit_dout)
+        if (int32_t rc = stage_in(sc, dout, (size_t)no, &ddo)) return rc;
     if (int32_t rc = stage_out(sc, (size_t)nq, &gq)) return rc;
     if (int32_t rc = stage_out(sc, (size_t)nk, &gk)) return rc;
     if (int32_t rc = stage_out(sc, (size_t)nv, &gv)) return rc;
-    const size_t wsb = fth_dev_sdpa_backward_workspace_bytes((int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, Dev<T>::dtype);
+    const size_t wsb = unit_dout ? fth_dev_sdpa_backward_unit_dout_workspace_bytes((int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k,
+                                                                                   (int64_t)d_v, Dev<T>::dtype)
+                                 : fth_dev_sdpa_backward_workspace_bytes((int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, Dev<T>::dtype);
     if (int32_t rc = sc.get(&ws, wsb)) return rc;
     int32_t rc;
     if constexpr (std::is_same<T, float>::value) {
-        rc = masked ? fth_dev_sdpa_backward_masked_f32(dqi, dki, dvi, ddo, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k,
+        rc = unit_dout ? fth_dev_sdpa_backward_unit_dout_f32(dqi, dki, dvi, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k,
+                                                             (int64_t)d_v, scale, causal, gq, gk, gv, ws, wsb, nullptr)
+             : masked ? fth_dev_sdpa_backward_masked_f32(dqi, dki, dvi, ddo, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k,
                                                        (int64_t)d_v, scale, dmask, (int64_t)mask_bh_stride, gq, gk, gv, ws, wsb, nullptr)
                     : fth_dev_sdpa_backward_f32(dqi, dki, dvi, ddo, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k,
                                                 (int64_t)d_v, scale, causal, gq, gk, gv, ws, wsb, nullptr);
     } else {
-        rc = masked ? fth_dev_sdpa_backward_masked_f64(dqi, dki, dvi, ddo, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k,
+        rc = unit_dout ? fth_dev_sdpa_backward_unit_dout_f64(dqi, dki, dvi, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k,
+                                                             (int64_t)d_v, scale, causal, gq, gk, gv, ws, wsb, nullptr)
+             : masked ? fth_dev_sdpa_backward_masked_f64(dqi, dki, dvi, ddo, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k,
                                                        (int64_t)d_v, scale, dmask, (int64_t)mask_bh_stride, gq, gk, gv, ws, wsb, nullptr)
                     : fth_dev_sdpa_backward_f64(dqi, dki, dvi, ddo, (int64_t)num_bh, (int64_t)seq_q, (int64_t)seq_k, (int64_t)d_k,
                                                 (int64_t)d_v, scale, causal, gq, gk, gv, ws, wsb, nullptr);
@@ -1088,6 +1095,12 @@ int32_t fth_sdpa_backward_f64(const double *q, size_t q_len, const double *k, si
                               int32_t causal, double *dq, size_t dq_cap, double *dk, size_t dk_cap, double *dv, size_t dv_cap) {
     return sdpa_backward_impl<double>(q, q_len, k, k_len, v, v_len, dout, dout_len, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dq_cap,
                                       dk, dk_cap, dv, dv_cap);
+}
+int32_t fth_sdpa_backward_f32_unit_dout(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len, size_t num_bh,
+                                        size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, float scale, int32_t causal, float *dq,
+                                        size_t dq_cap, float *dk, size_t dk_cap, float *dv, size_t dv_cap) {
+    return sdpa_backward_impl<float>(q, q_len, k, k_len, v, v_len, nullptr, 0, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dq_cap, dk,
+                                     dk_cap, dv, dv_cap, false, nullptr, 0, 0, true);
 }
 int32_t fth_sdpa_backward_masked_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len, const float *dout,
                                      size_t dout_len, size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, float scale,

@@ -275,6 +275,15 @@ def sdpa_backward(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, 
     return ws
 
 
+def sdpa_backward_unit_dout(q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dk, dv, workspace=None, stream=None):
+    """sdpa_backward_f32_unit_dout (and an f64 twin): the backward for dout = ones, which is not passed."""
+    ws = _workspace(_lib.load().fth_dev_sdpa_backward_unit_dout_workspace_bytes(num_bh, seq_q, seq_k, d_v, _dtype_code(q)), workspace)
+    check(getattr(_lib.load(), "fth_dev_sdpa_backward_unit_dout_" + _sfx(q))(_ptr(q), _ptr(k), _ptr(v), num_bh, seq_q, seq_k, d_k, d_v,
+                                                                             _real(q, scale), 1 if causal else 0, _ptr(dq), _ptr(dk),
+                                                                             _ptr(dv), ws.ptr, ws.nbytes, stream))
+    return ws
+
+
 def sdpa_backward_masked(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride, dq, dk, dv, workspace=None,
                          stream=None):
     """sdpa_backward_masked_f64 and its f32 twin: P = softmax(scale * Q.K^T + mask); mask_bh_stride 0 shares one [seq_q, seq_k] mask."""

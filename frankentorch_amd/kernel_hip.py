@@ -337,6 +337,17 @@ def sdpa_backward_f64(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, caus
     return _sdpa_backward("f64", np.float64, q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal)
 
 
+def sdpa_backward_f32_unit_dout(q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal):
+    """(dq, dk, dv) for dout = ones([num_bh, seq_q, d_v]) without that tensor, crates/ft-kernel-cpu/src/lib.rs:5662."""
+    q, k, v = _slice(q, np.float32), _slice(k, np.float32), _slice(v, np.float32)
+    dq = np.empty(num_bh * seq_q * d_k, dtype=np.float32)
+    dk = np.empty(num_bh * seq_k * d_k, dtype=np.float32)
+    dv = np.empty(num_bh * seq_k * d_v, dtype=np.float32)
+    check(_lib.load().fth_sdpa_backward_f32_unit_dout(_p(q), q.size, _p(k), k.size, _p(v), v.size, num_bh, seq_q, seq_k, d_k, d_v, scale,
+                                                      1 if causal else 0, _p(dq), dq.size, _p(dk), dk.size, _p(dv), dv.size))
+    return dq, dk, dv
+
+
 def _sdpa_backward_masked(sfx, dtype, q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, mask, mask_bh_stride):
     q, k, v, dout, mask = _slice(q, dtype), _slice(k, dtype), _slice(v, dtype), _slice(dout, dtype), _slice(mask, dtype)
     dq = np.empty(num_bh * seq_q * d_k, dtype=dtype)

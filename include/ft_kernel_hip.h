@@ -313,6 +313,15 @@ int32_t fth_dev_sdpa_backward_f32(const float *q, const float *k, const float *v
 int32_t fth_dev_sdpa_backward_f64(const double *q, const double *k, const double *v, const double *dout, int64_t num_bh, int64_t seq_q,
                                   int64_t seq_k, int64_t d_k, int64_t d_v, double scale, int32_t causal, double *dq, double *dk,
                                   double *dv, void *workspace, size_t workspace_bytes, fth_stream s);
+/* sdpa_backward_f32_unit_dout (:5662-5770) and an f64 twin: the backward for dOut = ones([num_bh, seq_q, d_v]) without that
+ * tensor (one shared [seq_q, d_v] plane of ones lives in the workspace, which is this much larger than the general form's). */
+size_t fth_dev_sdpa_backward_unit_dout_workspace_bytes(int64_t num_bh, int64_t seq_q, int64_t seq_k, int64_t d_v, int32_t dtype);
+int32_t fth_dev_sdpa_backward_unit_dout_f32(const float *q, const float *k, const float *v, int64_t num_bh, int64_t seq_q, int64_t seq_k,
+                                            int64_t d_k, int64_t d_v, float scale, int32_t causal, float *dq, float *dk, float *dv,
+                                            void *workspace, size_t workspace_bytes, fth_stream s);
+int32_t fth_dev_sdpa_backward_unit_dout_f64(const double *q, const double *k, const double *v, int64_t num_bh, int64_t seq_q, int64_t seq_k,
+                                            int64_t d_k, int64_t d_v, double scale, int32_t causal, double *dq, double *dk, double *dv,
+                                            void *workspace, size_t workspace_bytes, fth_stream s);
 /* sdpa_backward_masked_f64 (:5423-5530; the same formulas in f32): the recomputed P is softmax(scale * Q.K^T + mask) per row,
  * mask [seq_q, seq_k] rows shared by every (batch, head) when mask_bh_stride == 0, else mask_bh_stride elements apart
  * (>= seq_q * seq_k); the mask is a constant (no gradient). Same workspace as the unmasked form. */
@@ -489,6 +498,10 @@ int32_t fth_sdpa_backward_f32(const float *q, size_t q_len, const float *k, size
 int32_t fth_sdpa_backward_f64(const double *q, size_t q_len, const double *k, size_t k_len, const double *v, size_t v_len, const double *dout,
                               size_t dout_len, size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, double scale,
                               int32_t causal, double *dq, size_t dq_cap, double *dk, size_t dk_cap, double *dv, size_t dv_cap);
+/* sdpa_backward_f32_unit_dout (:5662): dOut = ones, not passed. */
+int32_t fth_sdpa_backward_f32_unit_dout(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len, size_t num_bh,
+                                        size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, float scale, int32_t causal, float *dq,
+                                        size_t dq_cap, float *dk, size_t dk_cap, float *dv, size_t dv_cap);
 /* sdpa_backward_masked_f64 (:5423) and its f32 twin: mask slice of (num_bh - 1) * mask_bh_stride + seq_q * seq_k elements. */
 int32_t fth_sdpa_backward_masked_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len, const float *dout,
                                      size_t dout_len, size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v, float scale,

@@ -807,6 +807,60 @@ void sdpa_backward_impl(const T *q, const T *k, const T *v, const T *dout, int64
     }
 }
 
+// sdpa_backward_f32_unit_dout (KC:5662-5770): dOut = ones without materialising it. dP_ij = sum_l V_jl (sequential), the
+// dot and dU rows from it, dV_jl = sum_i P_ij for every l (accumulated row by row), dQ / dK as in the general form.
+template <typename T>
+void sdpa_backward_unit_dout_impl(const T *q, const T *k, const T *v, int64_t num_bh, int64_t seq_q, int64_t seq_k, int64_t d_k, int64_t d_v,
+                                  T scale, int causal, T *dq, T *dk, T *dv) {
+    std::vector<T> p((size_t)std::max<int64_t>(seq_q * seq_k, 1)), du((size_t)std::max<int64_t>(seq_q * seq_k, 1));
+    std::vector<T> vrs((size_t)std::max<int64_t>(seq_k, 1)), pcs((size_t)std::max<int64_t>(seq_k, 1));
+    for (int64_t bh = 0; bh < num_bh; ++bh) {
+        const T *qh = q + bh * seq_q * d_k, *kh = k + bh * seq_k * d_k, *vh = v + bh * seq_k * d_v;
+        T *dqh = dq + bh * seq_q * d_k, *dkh = dk + bh * seq_k * d_k, *dvh = dv + bh * seq_k * d_v;
+        if (seq_q > 0 && seq_k > 0) gemm_any(1, seq_q, seq_k, d_k, qh, d_k, kh, d_k, p.data(), seq_k);
+        for (int64_t i = 0; i < seq_q; ++i) {
+            const int64_t limit = causal ? std::min<int64_t>(i + 1, seq_k) : seq_k;
+            T *row = p.data() + i * seq_k;
+            T m = -std::numeric_limits<T>::infinity();
+            for (int64_t j = 0; j < limit; ++j) {
+                row[j] *= scale;
+                if (row[j] > m) m = row[j];
+            }
+            T sum = 0;
+            for (int64_t j = 0; j < limit; ++j) {
+                const T e = std::exp(row[j] - m);
+                row[j] = e;
+                sum += e;
+            }
+            for (int64_t j = 0; j < limit; ++j) row[j] /= sum;
+            for (int64_t j = limit; j < seq_k; ++j) row[j] = 0;
+        }
+        for (int64_t j = 0; j < seq_k; ++j) {
+            T sum = 0;
+            for (int64_t l = 0; l < d_v; ++l) sum += vh[j * d_v + l];
+            vrs[j] = sum;
+            pcs[j] = 0;
+        }
+        for (int64_t i = 0; i < seq_q; ++i) {
+            const T *pr = p.data() + i * seq_k;
+            T *dr = du.data() + i * seq_k;
+            T dot = 0;
+            for (int64_t j = 0; j < seq_k; ++j) dot += pr[j] * vrs[j];
+            for (int64_t j = 0; j < seq_k; ++j) {
+                dr[j] = pr[j] * (vrs[j] - dot);
+                pcs[j] += pr[j];
+            }
+        }
+        for (int64_t j = 0; j < seq_k; ++j)
+            for (int64_t l = 0; l < d_v; ++l) dvh[j * d_v + l] = pcs[j];
+        if (seq_q > 0 && d_k > 0) {
+            gemm_any(0, seq_q, d_k, seq_k, du.data(), seq_k, kh, d_k, dqh, d_k);
+            for (int64_t i = 0; i < seq_q * d_k; ++i) dqh[i] = scale * dqh[i];
+        }
+        gemm_tb_any<T>(seq_k, d_k, seq_q, scale, du.data(), qh, dkh);
+    }
+}
+
 extern "C" {
 
 void fto_log_softmax_f32(const float *x, float *y, int64_t outer, int64_t reduce, int64_t inner) {
@@ -857,6 +911,14 @@ void fto_linear_backward_f64(const double *dy, const double *x, const double *w,
 void fto_sdpa_backward_f32(const float *q, const float *k, const float *v, const float *dout, int64_t num_bh, int64_t seq_q,
                            int64_t seq_k, int64_t d_k, int64_t d_v, float scale, int causal, float *dq, float *dk, float *dv) {
     sdpa_backward_impl<float>(q, k, v, dout, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dk, dv);
+}
+void fto_sdpa_backward_unit_dout_f32(const float *q, const float *k, const float *v, int64_t num_bh, int64_t seq_q, int64_t seq_k, int64_t d_k,
+                                     int64_t d_v, float scale, int causal, float *dq, float *dk, float *dv) {
+    sdpa_backward_unit_dout_impl<float>(q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dk, dv);
+}
+void fto_sdpa_backward_unit_dout_f64(const double *q, const double *k, const double *v, int64_t num_bh, int64_t seq_q, int64_t seq_k, int64_t d_k,
+                                     int64_t d_v, double scale, int causal, double *dq, double *dk, double *dv) {
+    sdpa_backward_unit_dout_impl<double>(q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal, dq, dk, dv);
 }
 void fto_sdpa_backward_masked_f32(const float *q, const float *k, const float *v, const float *dout, int64_t num_bh, int64_t seq_q,
                                   int64_t seq_k, int64_t d_k, int64_t d_v, float scale, const float *mask, int64_t mask_bh_stride, float *dq,

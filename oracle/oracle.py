@@ -338,6 +338,18 @@ def sdpa_backward(q, k, v, dout, scale, causal):
     return dq, dk, dv
 
 
+def sdpa_backward_unit_dout(q, k, v, scale, causal):
+    """(dq, dk, dv) for dout = ones, without that tensor (crates/ft-kernel-cpu/src/lib.rs:5662-5770)."""
+    q, k, v = _c(q), _c(k), _c(v)
+    sfx, ct = _sfx(q.dtype)
+    num_bh, seq_q, d_k = q.shape
+    seq_k, d_v = k.shape[1], v.shape[2]
+    dq, dk, dv = np.zeros_like(q), np.zeros_like(k), np.zeros_like(v)
+    getattr(lib(), "fto_sdpa_backward_unit_dout_" + sfx)(_p(q), _p(k), _p(v), _i64(num_bh), _i64(seq_q), _i64(seq_k), _i64(d_k), _i64(d_v),
+                                                         ct(scale), C.c_int(1 if causal else 0), _p(dq), _p(dk), _p(dv))
+    return dq, dk, dv
+
+
 def sdpa_backward_masked(q, k, v, dout, scale, mask, mask_bh_stride=None):
     """(dq, dk, dv) for out = sdpa_forward_masked(q, k, v, scale, mask); mask [seq_q, seq_k] shared (stride 0) or [num_bh, seq_q, seq_k]."""
     q, k, v, dout = _c(q), _c(k), _c(v), _c(dout)

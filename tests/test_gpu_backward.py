@@ -146,6 +146,29 @@ def test_sdpa_backward_masked(hip, oracle, bh, sq, sk, dk, dv, shared, dtype):
             assert rel_err(g, r) <= tol * 2
 
 
+@pytest.mark.parametrize("bh,sq,sk,dk,dv", [(2, 5, 6, 4, 3), (3, 100, 70, 32, 48), (2, 640, 640, 64, 64)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_sdpa_backward_unit_dout(hip, oracle, bh, sq, sk, dk, dv, causal, dtype):
+    """sdpa_backward_f32_unit_dout (crates/ft-kernel-cpu/src/lib.rs:5662-5770): against the checker's restatement and against the
+    general backward given a materialised ones tensor (the reference's own test, :45119-45155); 640 takes the block-causal path."""
+    tol = TOL_GEMM_F32 if dtype == np.float32 else TOL_F64
+    s = 1.0 / math.sqrt(dk)
+    q, k, v = (synth.normal(27, t, shp, dtype=dtype) for t, shp in (("q", (bh, sq, dk)), ("k", (bh, sk, dk)), ("v", (bh, sk, dv))))
+    ref = oracle.sdpa_backward_unit_dout(q, k, v, dtype(s), causal)
+    dq_, dk_, dv_ = _up(q, k, v)
+    gq, gk, gv = DeviceBuffer(q.shape, dtype), DeviceBuffer(k.shape, dtype), DeviceBuffer(v.shape, dtype)
+    hip.sdpa_backward_unit_dout(dq_, dk_, dv_, bh, sq, sk, dk, dv, s, causal, gq, gk, gv)
+    got = (gq.to_host(), gk.to_host(), gv.to_host())
+    for g, r in zip(got, ref):
+        assert rel_err(g, r) <= tol * 2
+    assert np.all(got[2] == got[2][:, :, :1])  # every value lane of a key gets the same gradient, bit for bit
+    hq, hk, hv = DeviceBuffer(q.shape, dtype), DeviceBuffer(k.shape, dtype), DeviceBuffer(v.shape, dtype)
+    hip.sdpa_backward(dq_, dk_, dv_, DeviceBuffer.from_host(np.ones((bh, sq, dv), dtype)), bh, sq, sk, dk, dv, s, causal, hq, hk, hv)
+    for a, b in zip(got, (hq.to_host(), hk.to_host(), hv.to_host())):
+        assert rel_err(a, b) <= tol
+
+
 def test_sdpa_backward_masked_reduces_to_the_unmasked_and_causal_forms(hip):
     bh, sq, sk, dk, dv = 2, 96, 96, 32, 32
     q, k, v, do = (synth.normal(25, t, (bh, sq, dk)) for t in ("q", "k", "v", "do"))
@@ -171,6 +194,10 @@ def test_host_slice_sdpa_backward_masked_and_its_errors(oracle):
     got = K.sdpa_backward_masked_f64(q.ravel(), k.ravel(), v.ravel(), do.ravel(), bh, sq, sk, dk, dv, 0.25, mask.ravel(), sq * sk)
     for g, r in zip(got, oracle.sdpa_backward_masked(q, k, v, do, 0.25, mask)):
         assert rel_err(g, r.ravel()) <= 2 * TOL_F64
+    got = K.sdpa_backward_f32_unit_dout(q.astype(np.float32).ravel(), k.astype(np.float32).ravel(), v.astype(np.float32).ravel(), bh, sq, sk, dk,
+                                        dv, 0.25, True)
+    for g, r in zip(got, oracle.sdpa_backward_unit_dout(q.astype(np.float32), k.astype(np.float32), v.astype(np.float32), np.float32(0.25), True)):
+        assert rel_err(g, r.ravel()) <= 2 * TOL_GEMM_F32
     with pytest.raises((KernelError, HipError)):  # a mask slice shorter than num_bh planes
         K.sdpa_backward_masked_f64(q.ravel(), k.ravel(), v.ravel(), do.ravel(), bh, sq, sk, dk, dv, 0.25, mask.ravel()[:-1], sq * sk)
     with pytest.raises((KernelError, HipError)):  # a per-head stride smaller than one plane

@@ -107,6 +107,27 @@ def test_sdpa_backward_is_the_gradient_of_the_forward(oracle, causal):
     assert np.allclose(dq32, dq, atol=2e-5) and np.allclose(dk32, dk_, atol=2e-5) and np.allclose(dv32, dv_, atol=2e-5)
 
 
+def test_sdpa_backward_unit_dout_matches_dense_ones_on_the_reference_inputs(oracle):
+    """The reference's own test (crates/ft-kernel-cpu/src/lib.rs:45119-45155): its inputs, its bound 2e-4 + 2e-4 |want|."""
+    num_bh, seq_q, seq_k, d_k, d_v = 2, 5, 6, 4, 3
+    f = np.float32
+    q = (((np.arange(num_bh * seq_q * d_k) % 11).astype(f) - f(5.0)) * f(0.07)).reshape(num_bh, seq_q, d_k)
+    k = (((np.arange(num_bh * seq_k * d_k) % 13).astype(f) - f(6.0)) * f(0.05)).reshape(num_bh, seq_k, d_k)
+    v = (((np.arange(num_bh * seq_k * d_v) % 7).astype(f) - f(3.0)) * f(0.09)).reshape(num_bh, seq_k, d_v)
+    scale = f(1.0) / np.sqrt(f(d_k))
+    for causal in (False, True):
+        want = oracle.sdpa_backward(q, k, v, np.ones((num_bh, seq_q, d_v), f), scale, causal)
+        got = oracle.sdpa_backward_unit_dout(q, k, v, scale, causal)
+        for a, b in zip(got, want):
+            assert np.all(np.abs(a - b) <= 2.0e-4 + 2.0e-4 * np.abs(b))
+            assert np.allclose(a, b, atol=2e-6)  # in fact far closer
+        # every value lane of a key gets the same gradient
+        assert np.all(got[2] == got[2][:, :, :1])
+    q64, k64, v64 = q.astype(np.float64), k.astype(np.float64), v.astype(np.float64)
+    for a, b in zip(oracle.sdpa_backward_unit_dout(q64, k64, v64, 0.5, True), oracle.sdpa_backward(q64, k64, v64, np.ones((num_bh, seq_q, d_v)), 0.5, True)):
+        assert np.allclose(a, b, atol=1e-14)
+
+
 @pytest.mark.parametrize("shared", [True, False])
 def test_sdpa_backward_masked_is_the_gradient_of_the_masked_forward(oracle, shared):
     """sdpa_backward_masked_f64 (crates/ft-kernel-cpu/src/lib.rs:5423-5530) has no test of its own in the reference: it is pinned by
