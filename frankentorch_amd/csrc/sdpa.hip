@@ -815,6 +815,155 @@ template <int D, int NW, bool PAIR, bool MASK> int32_t launch_mfma_cfg(SdpaArgs 
     return FTH_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Small problems (the 128-token block: 4 heads x 128 queries): too few query blocks to fill the chip, so the time is a
+// chain of latencies. A workgroup owns 32 queries and splits the KEYS over its four wavefronts (wavefront w takes the
+// 32-key tiles w, w + 4, ...), each feeding the MFMAs straight from global memory (the operands are L2-resident; no LDS
+// staging, no barrier in the loop), and the four partial (max, sum, output) states are merged through LDS in wavefront
+// order. Same zero-shuffle S^T / P^T scheme and the same arithmetic per tile as sdpa_mfma_kernel.
+template <int D>
+__global__ __launch_bounds__(256) void sdpa_small_kernel(const SdpaArgs p) {
+    constexpr int NDT = D / 32;
+    constexpr int OP = D + 1;  // LDS row pitch of a partial output (odd: the 32 query rows land on distinct banks)
+    using VV = typename VecN<NDT>::type;
+    __shared__ float Os[4][32][OP];
+    __shared__ float ms[4][32], ls[4][32];
+    const fth_sdpa_desc &d = p.d;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lq = lane & 31, half = lane >> 5;
+    const int64_t pid = blockIdx.x;
+    const int qb = (int)(pid % p.q_blocks);
+    const int64_t bh = pid / p.q_blocks;
+    const int64_t b = bh / d.heads, h = bh % d.heads, hk = h / p.group;
+    const float *Q = static_cast<const float *>(p.q) + b * d.q_batch_stride + h * d.q_head_stride;
+    const float *K = static_cast<const float *>(p.k) + b * d.k_batch_stride + hk * d.k_head_stride;
+    const float *Vg = static_cast<const float *>(p.v) + b * d.v_batch_stride + hk * d.v_head_stride;
+    float *O = static_cast<float *>(p.out) + b * d.o_batch_stride + h * d.o_head_stride;
+    const float c2 = (float)p.scale * 1.44269502162933349609375f;  // scale * log2(e); scale > 0 (launcher check)
+    const int seq_q_i = (int)d.seq_q, seq_k_i = (int)d.seq_k;
+    const int q0 = qb * 32, qi = q0 + lq;
+    const bool q_live = qi < seq_q_i;
+
+    float4 qr[D / 8];
+#pragma unroll
+    for (int t = 0; t < D / 8; ++t)
+        qr[t] = q_live ? *reinterpret_cast<const float4 *>(Q + (int64_t)qi * d.q_row_stride + 8 * t + 4 * half) : make_float4(0.f, 0.f, 0.f, 0.f);
+
+    int last_q = q0 + 31;
+    if (last_q > seq_q_i - 1) last_q = seq_q_i - 1;
+    int k_end = seq_k_i;
+    if (d.causal && last_q + 1 < k_end) k_end = last_q + 1;
+    const int num_kt = (k_end + 31) / 32;
+
+    Acc16 o[NDT];
+#pragma unroll
+    for (int e = 0; e < NDT; ++e)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[e][r] = 0.f;
+    float m_run = -__builtin_inff(), l_run = 0.f;
+
+    for (int kt = wave; kt < num_kt; kt += 4) {
+        const int key0 = kt * 32;
+        int krow = key0 + lq;
+        krow = krow < seq_k_i ? krow : seq_k_i - 1;  // rows past the end repeat the last one; their scores are masked
+        const float *kp = K + (int64_t)krow * d.k_row_stride + 4 * half;
+        Acc16 s;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+        for (int t = 0; t < D / 8; ++t) {
+            const float4 kv = *reinterpret_cast<const float4 *>(kp + 8 * t);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.x, qr[t].x, s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.y, qr[t].y, s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.z, qr[t].z, s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.w, qr[t].w, s, 0, 0, 0);
+        }
+        // V fragments of the tile, requested before the softmax that hides their latency
+        VV vv[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            int vrow = key0 + 8 * (r >> 2) + (r & 3) + 4 * half;
+            vrow = vrow < seq_k_i ? vrow : seq_k_i - 1;
+            vv[r] = *reinterpret_cast<const VV *>(Vg + (int64_t)vrow * d.v_row_stride + NDT * lq);
+        }
+        float mt = -__builtin_inff();
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int key = key0 + 8 * (r >> 2) + 4 * half + (r & 3);
+            const bool hidden = (d.causal && key > qi) | (key >= seq_k_i);
+            s[r] = hidden ? -__builtin_inff() : s[r];
+            mt = fmaxf(mt, s[r]);
+        }
+        float mlo, mhi;
+        both_halves(mt, mlo, mhi);
+        mt = fmaxf(mlo, mhi);
+        const float m_new = fmaxf(m_run, mt * c2);
+        // a wavefront's tiles can all lie past a query's causal limit (m_new still -inf): keep its state empty
+        const float m_ref = (m_new == -__builtin_inff()) ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+            for (int e = 0; e < NDT; ++e)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o[e][r] *= alpha;
+        }
+        float psum = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], c2, -m_ref));
+            psum += e;
+#pragma unroll
+            for (int ee = 0; ee < NDT; ++ee) o[ee] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(vv[r], ee), e, o[ee], 0, 0, 0);
+        }
+        float plo, phi;
+        both_halves(psum, plo, phi);
+        l_run = l_run * alpha + (plo + phi);
+        m_run = m_new;
+    }
+
+    // ---- merge the four partial states in wavefront order ----
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int rho = 8 * (r >> 2) + 4 * half + (r & 3);
+#pragma unroll
+        for (int e = 0; e < NDT; ++e) Os[wave][lq][NDT * rho + e] = o[e][r];
+    }
+    if (half == 0) {
+        ms[wave][lq] = m_run;
+        ls[wave][lq] = l_run;
+    }
+    __syncthreads();
+    const int qf = tid & 31, dc = tid >> 5;  // query and one of eight d-chunks
+    float m = ms[0][qf];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) m = fmaxf(m, ms[w][qf]);
+    float wgt[4], l = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        wgt[w] = (ms[w][qf] == -__builtin_inff()) ? 0.f : __builtin_amdgcn_exp2f(ms[w][qf] - m);
+        l += ls[w][qf] * wgt[w];
+    }
+    if (q0 + qf < seq_q_i) {
+        float *orow = O + (int64_t)(q0 + qf) * d.o_row_stride;
+#pragma unroll
+        for (int i = 0; i < D / 8; ++i) {
+            const int dd = dc * (D / 8) + i;
+            float acc = 0.f;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) acc += Os[w][qf][dd] * wgt[w];
+            orow[dd] = acc / l;
+        }
+    }
+}
+
+template <int D> int32_t launch_small_sdpa(SdpaArgs &a, hipStream_t st) {
+    a.q_blocks = (int)fth::ceil_div(a.d.seq_q, 32);
+    const int64_t grid = a.d.num_bh * a.q_blocks;
+    sdpa_small_kernel<D><<<dim3((unsigned)grid), dim3(256), 0, st>>>(a);
+    FTH_CHECK_LAUNCH("sdpa_small");
+    return FTH_OK;
+}
+
 // Blocks of 128 queries (4 wavefronts) are used whenever they still give every other CU a
 // workgroup; shorter problems fall back to blocks of 64 queries. Workgroups are issued heaviest
 // first, which balances causal problems well enough that pairing a long with a short query
@@ -872,6 +1021,16 @@ int32_t sdpa_entry(const fth_sdpa_desc *d, double scale, const T *q, const T *k,
                                 d->k_row_stride < (1 << 22) && d->v_row_stride < (1 << 22);  // a tile's lane offsets fit 32 bits
         // the unmasked MFMA kernels take the row maximum on the raw scores, which needs a positive scale
         if (strides_ok && d->d_k == d->d_v && d->seq_k > 0 && (masked || scale > T(0))) {
+            // Too few 32-query blocks to give every compute unit one: the key-split kernel (one launch, no LDS staging)
+            static const bool small_off = [] {
+                const char *e = std::getenv("FT_HIP_SDPA_SMALL");  // tuning knob: 0 disables the small-problem kernel
+                return e && std::atoi(e) == 0;
+            }();
+            const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
+            if (!masked && !small_off && d->num_bh * fth::ceil_div(d->seq_q, 32) <= cus && d->seq_k <= 4096) {
+                if (d->d_k == 64) return launch_small_sdpa<64>(a, st);  // (128: the merge buffers would exceed 64 KiB of LDS)
+                if (d->d_k == 32) return launch_small_sdpa<32>(a, st);
+            }
             if (d->d_k == 128) return launch_mfma<128>(a, st);
             if (d->d_k == 64) return launch_mfma<64>(a, st);
             if (d->d_k == 32) return launch_mfma<32>(a, st);

@@ -89,7 +89,7 @@ def test_sdpa_forward_and_backward_random_shapes(hip, seed):
     rng = np.random.default_rng(seed)
     for _ in range(40):
         dt = np.float32 if rng.random() < 0.6 else np.float64
-        bh = int(rng.integers(1, 7))
+        bh = int(rng.integers(1, 7)) if rng.random() < 0.6 else int(rng.integers(20, 60))  # few / many query blocks: both fp32 kernels
         sq = dims(rng, 1, 600)
         sk = sq if rng.random() < 0.6 else dims(rng, 1, 600)
         dk = int(rng.choice([32, 64, 128, 16, 40, 8, 96]))

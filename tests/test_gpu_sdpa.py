@@ -33,7 +33,10 @@ def _run(hip, q, k, v, scale, causal):
 # and head sizes that take the generic kernel (48, d_k != d_v)
 CASES = [(2, 64, 64, 64, 64, True), (3, 100, 100, 128, 128, True), (2, 130, 77, 64, 64, False), (2, 77, 130, 32, 32, True),
          (2, 129, 129, 128, 128, False), (1, 1, 1, 64, 64, True), (2, 1, 300, 128, 128, False), (2, 300, 1, 64, 64, True),
-         (8, 256, 256, 128, 128, True), (2, 50, 50, 48, 48, True), (2, 40, 33, 16, 24, False), (4, 128, 128, 64, 64, True)]
+         (8, 256, 256, 128, 128, True), (2, 50, 50, 48, 48, True), (2, 40, 33, 16, 24, False), (4, 128, 128, 64, 64, True),
+         # head sizes 32 / 64 with more than one 32-query block per compute unit take the tiled kernel, fewer the key-split one
+         (70, 130, 77, 64, 64, False), (100, 77, 130, 32, 32, True), (72, 129, 129, 64, 64, True), (3, 65, 300, 64, 64, True),
+         (2, 31, 1000, 32, 32, False), (1, 128, 4000, 64, 64, True), (5, 64, 64, 32, 32, True)]
 
 
 @pytest.mark.parametrize("bh,sq,sk,dk,dv,causal", CASES)
