@@ -1008,6 +1008,70 @@ __global__ __launch_bounds__(64 * NW) void gemm_small_kernel(const GemmArgs<floa
     }
 }
 
+// The same for long reductions (k >= 512) with 16 x 16 output tiles (v_mfma_f32_16x16x4_f32): four times the workgroups, and
+// a wavefront load covers 64 contiguous bytes of each of 16 rows instead of 32 bytes of each of 32. With 32 x 32 tiles a
+// [128, 256] x k = 1024 product kept only 32 compute units busy and each spent its time moving 256 KiB of operands through its
+// one vector memory pipe.
+template <int NW, bool TRANS_B>
+__global__ __launch_bounds__(64 * NW) void gemm_small16_kernel(const GemmArgs<float> p) {
+    using M = Mfma<float>;
+    typedef float Acc4 __attribute__((ext_vector_type(4)));
+    __shared__ float part[NW][16][17];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lrow = lane & 15, g = lane >> 4;
+    const int64_t batch = blockIdx.y;
+    const int tile_m = (int)(blockIdx.x / p.tiles_n), tile_n = (int)(blockIdx.x % p.tiles_n);
+    const int64_t m0 = (int64_t)tile_m * 16, n0 = (int64_t)tile_n * 16;
+    const float *A = p.a + batch * p.stride_a;
+    const float *B = p.b + batch * p.stride_b;
+    // this wavefront's K range: whole groups of 16 (one 128-bit load per lane group), contiguous, in wavefront order
+    const int groups = (int)(p.k / 16), per = (groups + NW - 1) / NW;
+    const int g0 = wave * per, g1 = (g0 + per < groups) ? g0 + per : groups;
+    int64_t ar = m0 + lrow, br = n0 + lrow;  // rows past the edge read the last valid row; they are never stored
+    ar = ar < p.m ? ar : p.m - 1;
+    br = br < p.n ? br : p.n - 1;
+    const float *ap = A + ar * p.lda + 4 * g;
+    const float *bp = TRANS_B ? B + br * p.ldb + 4 * g : B + (int64_t)(4 * g) * p.ldb + br;
+    Acc4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
+    for (int t = g0; t < g1; ++t) {
+        const float4 av = *reinterpret_cast<const float4 *>(ap + 16 * t);
+        float4 bv;
+        if (TRANS_B) {
+            bv = *reinterpret_cast<const float4 *>(bp + 16 * t);
+        } else {
+            const float *bk = bp + (int64_t)(16 * t) * p.ldb;
+            bv = make_float4(bk[0], bk[p.ldb], bk[2 * p.ldb], bk[3 * p.ldb]);
+        }
+        // step i contracts k = 16 t + 4 g + i over the four lane groups
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, bv.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, bv.y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, bv.z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, bv.w, acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) part[wave][4 * g + r][lrow] = acc[r];  // accumulator element r: row 4 (lane / 16) + r, column lane % 16
+    __syncthreads();
+    const bool has_bias = (p.epilogue & FTH_EPI_BIAS) != 0, has_gelu = (p.epilogue & FTH_EPI_GELU) != 0;
+    const bool has_gelu_tanh = (p.epilogue & FTH_EPI_GELU_TANH) != 0, has_res = (p.epilogue & FTH_EPI_RESIDUAL) != 0;
+    float *C = p.c + batch * p.stride_c;
+    if (tid < 256) {
+        const int r = tid >> 4, c = tid & 15;
+        const int64_t row = m0 + r, col = n0 + c;
+        if (row < p.m && col < p.n) {
+            float v = part[0][r][c];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) v += part[w][r][c];
+            if (p.use_alpha) v = p.alpha * v;
+            if (has_bias) v = v + p.bias[col];
+            if (has_gelu) v = M::gelu(v);
+            if (has_gelu_tanh) v = M::gelu_tanh(v);
+            if (has_res) v = v + p.residual[batch * p.stride_c + row * p.ldc + col];
+            C[row * p.ldc + col] = v;
+        }
+    }
+}
+
 // True (and the kernel launched) when the problem is one of the small ones this kernel is for.
 template <bool TRANS_B> bool launch_small(GemmArgs<float> &p, int64_t batch, bool vec_a, bool vec_b, hipStream_t st, int32_t *rc) {
     static const bool off = [] {
@@ -1020,8 +1084,18 @@ template <bool TRANS_B> bool launch_small(GemmArgs<float> &p, int64_t batch, boo
     p.tiles_m = (int)fth::ceil_div(p.m, 32);
     p.tiles_n = (int)fth::ceil_div(p.n, 32);
     const dim3 grid((unsigned)tiles, (unsigned)batch);
-    if (p.k <= 512) gemm_small_kernel<4, TRANS_B><<<grid, dim3(256), 0, st>>>(p);
-    else gemm_small_kernel<8, TRANS_B><<<grid, dim3(512), 0, st>>>(p);
+    const int64_t tiles16 = fth::ceil_div(p.m, 16) * fth::ceil_div(p.n, 16);
+    if (p.k < 512) {
+        gemm_small_kernel<4, TRANS_B><<<grid, dim3(256), 0, st>>>(p);
+    } else if (p.k % 16 == 0 && tiles16 * batch <= 4096) {  // long reduction, few tiles: 16 x 16 tiles on four times the compute units
+        p.tiles_m = (int)fth::ceil_div(p.m, 16);
+        p.tiles_n = (int)fth::ceil_div(p.n, 16);
+        gemm_small16_kernel<8, TRANS_B><<<dim3((unsigned)tiles16, (unsigned)batch), dim3(512), 0, st>>>(p);
+    } else if (p.k <= 512) {
+        gemm_small_kernel<4, TRANS_B><<<grid, dim3(256), 0, st>>>(p);
+    } else {
+        gemm_small_kernel<8, TRANS_B><<<grid, dim3(512), 0, st>>>(p);
+    }
     hipError_t e = hipGetLastError();
     *rc = e == hipSuccess ? FTH_OK : fth::hip_fail(e, "gemm_small");
     return true;
