@@ -131,24 +131,46 @@ template <typename T> __device__ __forceinline__ Cand<T> cand_shfl_xor(const Can
     return r;
 }
 
-// Last-dim argmax: one block per row, lanes stride the row (coalesced dword loads; rows such as
-// 50 257 floats are only 4-byte aligned, so no wider load is assumed).
+// Last-dim argmax: one block per row. Rows such as 50 257 floats start at arbitrary 4-byte offsets, so a row is read as a
+// scalar head up to the first 16-byte boundary, 128-bit vectors, and a scalar tail. Every lane feeds its candidates in
+// increasing index order (head < body < tail, and a lane's vectors ascend), which is what "first strict maximum" needs.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void argmax_lastdim_kernel(const T *__restrict__ x, int64_t rows, int64_t cols,
                                                                 T *__restrict__ out) {
+    constexpr int EPV = 16 / (int)sizeof(T);
+    using V = typename std::conditional<sizeof(T) == 4, float4, double2>::type;
     __shared__ Cand<T> smem[kBlock / kWave];
     const T *xr = x + (int64_t)blockIdx.x * cols;
     Cand<T> c = cand_init<T>();
+    int64_t lead = (int64_t)(((16u - (unsigned)(reinterpret_cast<uintptr_t>(xr) & 15u)) & 15u) / sizeof(T));
+    if (lead > cols) lead = cols;
+    if ((int64_t)threadIdx.x < lead) cand_feed(c, xr[threadIdx.x], (int64_t)threadIdx.x);
+    const int64_t nvec = (cols - lead) / EPV;
+    const V *xv = reinterpret_cast<const V *>(xr + lead);
+    auto feed_vec = [&](const V &v, int64_t vi) __attribute__((always_inline)) {
+        const int64_t i0 = lead + vi * EPV;
+        if constexpr (sizeof(T) == 4) {
+            cand_feed(c, (T)v.x, i0);
+            cand_feed(c, (T)v.y, i0 + 1);
+            cand_feed(c, (T)v.z, i0 + 2);
+            cand_feed(c, (T)v.w, i0 + 3);
+        } else {
+            cand_feed(c, (T)v.x, i0);
+            cand_feed(c, (T)v.y, i0 + 1);
+        }
+    };
     int64_t j = threadIdx.x;
-    // Four independent loads in flight per lane.
-    for (; j + 3 * kBlock < cols; j += 4 * kBlock) {
-        T v0 = xr[j], v1 = xr[j + kBlock], v2 = xr[j + 2 * kBlock], v3 = xr[j + 3 * kBlock];
-        cand_feed(c, v0, j);
-        cand_feed(c, v1, j + kBlock);
-        cand_feed(c, v2, j + 2 * kBlock);
-        cand_feed(c, v3, j + 3 * kBlock);
+    // Eight independent 128-bit loads in flight per lane.
+    for (; j + 7 * kBlock < nvec; j += 8 * kBlock) {
+        V v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = xv[j + u * kBlock];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) feed_vec(v[u], j + u * kBlock);
     }
-    for (; j < cols; j += kBlock) cand_feed(c, xr[j], j);
+    for (; j < nvec; j += kBlock) feed_vec(xv[j], j);
+    const int64_t t0 = lead + nvec * EPV + threadIdx.x;
+    if (t0 < cols) cand_feed(c, xr[t0], t0);
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) c = cand_merge(c, cand_shfl_xor(c, off));
     if ((threadIdx.x & (kWave - 1)) == 0) smem[threadIdx.x / kWave] = c;

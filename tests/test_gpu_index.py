@@ -29,6 +29,26 @@ def test_argmax_semantics_ties_nan_and_all_neg_inf(hip, oracle, dtype):
     assert got[3] == 100 and got[4] == 0 and got[5] == 7 and got[6] == 50256 and got[7] == 0 and got[8] == 12 and got[9] == 5
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("cols", [1, 2, 3, 4, 5, 7, 9, 33, 1027, 4099])
+def test_argmax_last_dim_short_and_unaligned_rows_with_ties(hip, oracle, cols, dtype):
+    """Rows whose scalar head, vector body and scalar tail are empty or a few elements long, every starting alignment
+    (odd row length, plus a base one element into the buffer), heavy ties and NaNs: first maximum / first NaN must win."""
+    rows = 37
+    x = np.round(synth.normal(9, "am3", (rows, cols)) * 1.5).astype(dtype)
+    if cols > 4:
+        x[5, cols // 2] = np.nan
+        x[6, cols - 1] = np.nan
+        x[7, 0] = np.nan
+    pad = np.concatenate([np.zeros(1, dtype), x.ravel()])
+    dpad = DeviceBuffer.from_host(pad)
+    dy = DeviceBuffer((rows,), dtype)
+    hip.argmax(dpad.view(1), rows, cols, 1, dy)
+    assert np.array_equal(dy.to_host(), oracle.argmax(x, 1))
+    hip.argmax(DeviceBuffer.from_host(x), rows, cols, 1, dy)
+    assert np.array_equal(dy.to_host(), oracle.argmax(x, 1))
+
+
 @pytest.mark.parametrize("shape,dim", [((5, 17, 9), 1), ((64, 3), 0), ((2, 300, 4), 1), ((1, 7), 1), ((3, 1, 5), 1)])
 def test_argmax_any_dim(hip, oracle, shape, dim):
     x = np.round(synth.normal(8, "am2", shape) * 2)  # many ties
