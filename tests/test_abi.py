@@ -124,6 +124,27 @@ def test_add_and_addmm_shape_rules():
     assert e.kind == "InvalidDimension" and e.dim == 2 and e.ndim == 2
 
 
+def test_fused_entry_points_check_slice_lengths_before_any_device_call():
+    """The reference's fused kernels panic on short slices (plain indexing); the C ABI reports InvalidArgument instead, and does
+    so before it needs a device, for the forward, backward, masked and loss forms alike."""
+    bh, sq, sk, dk, dv = 2, 5, 6, 4, 3
+    q, k, v = np.zeros(bh * sq * dk), np.zeros(bh * sk * dk), np.zeros(bh * sk * dv)
+    do, mask = np.zeros(bh * sq * dv), np.zeros(bh * sq * sk)
+    for call in (
+        lambda: K.sdpa_forward_f64(q[:-1], k, v, bh, sq, sk, dk, dv, 0.5, True),
+        lambda: K.sdpa_backward_f64(q, k, v, do[:-1], bh, sq, sk, dk, dv, 0.5, False),
+        lambda: K.sdpa_backward_masked_f64(q, k, v, do, bh, sq, sk, dk, dv, 0.5, mask[:-1], sq * sk),  # mask shorter than num_bh planes
+        lambda: K.sdpa_backward_masked_f64(q, k, v, do, bh, sq, sk, dk, dv, 0.5, mask, 7),             # stride smaller than a plane
+        lambda: K.sdpa_forward_masked_f64(q, k, v, bh, sq, sk, dk, dv, 0.5, mask[:-1], sq * sk),
+        lambda: K.sdpa_backward_f32_unit_dout(q.astype(np.float32), k.astype(np.float32)[:-1], v.astype(np.float32), bh, sq, sk, dk, dv, 0.5, True),
+        lambda: K.cross_entropy_forward_f64(np.zeros(11), np.zeros(3, np.int64), 3, 4),
+        lambda: K.layer_norm_backward_f64(np.zeros(11), np.zeros(12), None, 3, 4, 1e-5),
+    ):
+        with pytest.raises((core.KernelError, core.HipError)) as ei:
+            call()
+        assert ei.value.kind != "Unavailable", "the length check must come before the device check"
+
+
 def test_empty_results_need_no_device():
     f32 = lambda s: TensorMeta.from_shape(s, DType.F32)
     z = np.zeros(0, np.float32)
