@@ -18,6 +18,14 @@
 //     identities those tests assert (unit-dy shortcut, dbias = column sums);
 //     log_softmax: the reference's conformance fixtures (1e-10) and log(softmax); cross-entropy forward /
 //     backward: -log_softmax[target], central differences, rows of the gradient summing to zero.
+//     masked / grouped-query sdpa: the reference's expand-then-masked identity on its own inputs (KC:45159-45218), an einsum
+//     restatement, reduction to the pinned unmasked and causal forms; masked sdpa backward (KC:5423): central differences of
+//     the pinned masked forward, the same reductions, an einsum restatement; unit-dOut sdpa backward (KC:5662): the
+//     reference's own test against dense ones on its inputs and bound (KC:45119-45155);
+//     tanh gelu: ft-nn's golden values and torch's CPU kernel; int8 quantisers and linear: the reference's tie vector and
+//     scale (KC:43721-43740), its accuracy bounds on its LCG inputs (KC:43645-43708), an independent integer product.
+//   parity unpinned: none of the functions in this file (what the checkout cannot pin -- session RNG dependent golden files,
+//     kernel routing inside the missing ft-api crate, matrixmultiply's bit digests -- is not restated here).
 //   third-party arithmetic that is NOT in the reference tree:
 //     * GEMM: `matrixmultiply 0.3.11` (Cargo.lock:1420-1423; call sites KC:1645, KC:1673). Its
 //       f32 accumulation order is unspecified and the reference's own test shows it is not the
