@@ -446,6 +446,43 @@ def bench_backward(device, synth, steps, with_cpu):
     return out
 
 
+def bench_index(device, synth, steps):
+    """The integer-exact kernels at the config-5 shapes: fused token + position embedding gather, head split (perm [0,2,1,3]) and
+    the argmax over the logits. Algorithmic bytes = every input element the kernel must read once + every output element once."""
+    from frankentorch_amd.device import DeviceBuffer
+    import numpy as np
+
+    out = {}
+    vocab, width, batch, seq, heads = 50257, 768, 8, 1024, 12
+    tokens = batch * seq
+    iters = max(10, steps // 4)
+    wte = DeviceBuffer.from_host(synth.normal(4, "wte", (vocab, width)) * np.float32(0.02))
+    wpe = DeviceBuffer.from_host(synth.normal(4, "wpe", (seq, width)) * np.float32(0.02))
+    ids = DeviceBuffer.from_host(synth.token_ids(4, "ids", (tokens,), vocab))
+    emb = DeviceBuffer((tokens, width))
+    ms = event_time_ms(device, lambda: device.embedding_add(wte, vocab, wpe, seq, ids, tokens, seq, width, emb), iters)
+    nbytes = tokens * 8 + 2 * tokens * width * 4 + seq * width * 4  # ids, gathered rows + output, the position table once
+    out["embedding_add"] = {"ms": round(ms, 5), "GB/s": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                            "bytes": nbytes, "workload": "wte[50257,768] + wpe[1024,768] gather for 8192 ids (50 MB per launch: back-to-back launches run out of the 256 MB last-level cache, so this is not an HBM rate)"}
+    log("[index] embedding_add   %.4f ms  %7.1f GB/s" % (ms, nbytes / ms / 1e6))
+    src, dst = DeviceBuffer((batch, seq, heads, width // heads)), DeviceBuffer((batch, heads, seq, width // heads))
+    ms = event_time_ms(device, lambda: device.permute_0213(emb, dst, batch, seq, heads, width // heads), iters)
+    nbytes = 2 * tokens * width * 4
+    out["permute_0213"] = {"ms": round(ms, 5), "GB/s": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                           "bytes": nbytes, "workload": "[8,1024,12,64] -> [8,12,1024,64] fp32 (50 MB per launch: served by the last-level cache when repeated; the block path never runs it)"}
+    log("[index] permute_0213    %.4f ms  %7.1f GB/s" % (ms, nbytes / ms / 1e6))
+    del src
+    logits = DeviceBuffer((tokens, vocab))
+    device.gemm(device.gemm_desc(tokens, vocab, width, trans_b=True), emb, wte, logits)
+    am = DeviceBuffer((tokens,))
+    ms = event_time_ms(device, lambda: device.argmax(logits, tokens, vocab, 1, am), iters)
+    nbytes = tokens * vocab * 4 + tokens * 4
+    out["argmax"] = {"ms": round(ms, 5), "GB/s": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                     "bytes": nbytes, "workload": "argmax over the last dim of fp32 logits [8192,50257] (read-only stream)"}
+    log("[index] argmax          %.4f ms  %7.1f GB/s  %.1f%% of HBM peak" % (ms, nbytes / ms / 1e6, 100 * nbytes / ms / 1e6 / HBM_PEAK_GBS))
+    return out
+
+
 def make_layer(synth, seed, li, d, f):
     n = lambda tag, *s: synth.normal(seed, "L%d.%s" % (li, tag), s, 0.0, 0.02)
     one, zero = (lambda m: np.ones(m, np.float32)), (lambda m: np.zeros(m, np.float32))
@@ -553,7 +590,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--cases", default="all", help="comma list of: gemm,sdpa,block,gpt2,backward (row ops always run); 'none' for row ops only")
+    ap.add_argument("--cases", default="all", help="comma list of: gemm,sdpa,block,gpt2,backward,index (row ops always run); 'none' for row ops only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -566,7 +603,7 @@ def main():
     info = device.device_info()
     log("[device] %s, %d CUs, %.0f GiB HBM, engine %d MHz" % (info["arch"], info["compute_units"], info["hbm_bytes"] / 2 ** 30,
                                                                info["engine_clock_khz"] // 1000))
-    cases = {"gemm", "sdpa", "block", "gpt2", "backward"} if args.cases == "all" else set(c for c in args.cases.split(",") if c and c != "none")
+    cases = {"gemm", "sdpa", "block", "gpt2", "backward", "index"} if args.cases == "all" else set(c for c in args.cases.split(",") if c and c != "none")
 
     value, ms_per_step, roof, per_kernel, cpu = bench_rowops(device, synth, args.steps, args.warmup, not args.no_cpu)
     extra = {"row_ops": per_kernel}
@@ -580,6 +617,8 @@ def main():
         extra["gpt2_forward"] = bench_gpt2(device, synth, args.steps)
     if "backward" in cases:
         extra["backward"] = bench_backward(device, synth, args.steps, not args.no_cpu)
+    if "index" in cases:
+        extra["index"] = bench_index(device, synth, args.steps)
 
     line = {
         "metric": "row-op GB/s (fp32, 1 MI355X)",
