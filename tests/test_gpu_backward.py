@@ -88,7 +88,7 @@ def test_linear_backward_reference_test_inputs(hip, oracle):
 
 
 # The last four shapes are square and long enough for the causal form to take the block-causal products
-# (blocks of 128, 128, 128 and 256 rows; the last one ends in a partial block).
+# (blocks of 256 rows; 640 and 1152 end in a partial block).
 @pytest.mark.parametrize("bh,sq,sk,dk,dv", [(2, 64, 64, 64, 64), (3, 100, 70, 32, 48), (4, 128, 128, 128, 128), (1, 5, 6, 4, 3), (2, 33, 200, 16, 16),
                                             (2, 512, 512, 64, 64), (1, 640, 640, 32, 48), (3, 1024, 1024, 64, 64), (2, 1152, 1152, 128, 128)])
 @pytest.mark.parametrize("causal", [False, True])
