@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 
 
 def rel(a, b):
-    a = np.asarray(a)
+    a = np.asarray(a).ravel()
     d = np.max(np.abs(a.astype(np.float64) - np.asarray(b).ravel())) if a.size else 0.0
     return d / max(1.0, np.max(np.abs(b)) if np.asarray(b).size else 1.0)
 
@@ -85,3 +85,52 @@ def test_host_slice_entry_points_random_shapes_and_offsets(hip, seed):
         Y, _ = store(rng, shape, off2, dt)
         got = getattr(K, "add_tensor_contiguous_" + sfx)(X, Y, mt, meta(shape, off2, dt))
         assert np.array_equal(np.asarray(got), (xs + Y[off2:off2 + xs.size].reshape(shape)).ravel())
+
+
+@pytest.mark.parametrize("seed", [61])
+def test_resident_batch_ops_random_shapes(hip, seed):
+    """The stream-ordered batch of resident tensors (the ft_kernel_metal::fused surface): random shapes through a chain
+    x -> LayerNorm -> linear(+bias) -> GELU -> linear -> add -> softmax, and multi-head attention over [batch * seq, d_model] rows
+    with random head counts, against float64 numpy restatements."""
+    from frankentorch_amd.fused import Batch, HipTensor
+
+    rng = np.random.default_rng(seed)
+    for _ in range(25):
+        m, d, f = int(rng.integers(1, 200)), int(rng.choice([8, 24, 64, 100, 256])), int(rng.choice([16, 40, 128, 300]))
+        print("batch chain", dict(m=m, d=d, f=f), flush=True)
+        x = rng.normal(size=(m, d)).astype(np.float32)
+        g, be = rng.uniform(0.5, 1.5, d).astype(np.float32), rng.normal(size=d).astype(np.float32)
+        w1, b1 = (rng.normal(size=(f, d)) * 0.2).astype(np.float32), rng.normal(size=f).astype(np.float32)
+        w2 = (rng.normal(size=(d, f)) * 0.2).astype(np.float32)
+        bt = Batch()
+        tx = HipTensor.upload(x)
+        h = bt.layernorm(tx, HipTensor.upload(g, 1, d), HipTensor.upload(be, 1, d), 1e-5)
+        h = bt.gelu(bt.matmul_bias(h, HipTensor.upload(w1), HipTensor.upload(b1, 1, f)))
+        y = bt.softmax(bt.add(bt.matmul_bias(h, HipTensor.upload(w2)), tx))
+        bt.finish()
+        x64 = x.astype(np.float64)
+        r = (x64 - x64.mean(1, keepdims=True)) / np.sqrt(x64.var(1, keepdims=True) + 1e-5) * g + be
+        r = r @ w1.T.astype(np.float64) + b1
+        r = 0.5 * r * (1 + erf(r / math.sqrt(2)))
+        r = r @ w2.T.astype(np.float64) + x64
+        e = np.exp(r - r.max(1, keepdims=True))
+        assert rel(y.download(), e / e.sum(1, keepdims=True)) <= 4e-5
+
+        heads = int(rng.choice([1, 2, 4]))
+        hd = int(rng.choice([16, 32, 64]))
+        batch, seq = int(rng.integers(1, 4)), int(rng.integers(1, 150))
+        causal = bool(rng.random() < 0.5)
+        print("batch mha", dict(heads=heads, hd=hd, batch=batch, seq=seq, causal=causal), flush=True)
+        dm = heads * hd
+        q, k, v = (rng.normal(size=(batch * seq, dm)).astype(np.float32) for _ in range(3))
+        bt = Batch()
+        o = bt.mha(HipTensor.upload(q), HipTensor.upload(k), HipTensor.upload(v), heads, batch, causal)
+        bt.finish()
+        split = lambda t: t.astype(np.float64).reshape(batch, seq, heads, hd).transpose(0, 2, 1, 3)
+        sc = np.einsum("bhqd,bhkd->bhqk", split(q), split(k)) / math.sqrt(hd)
+        if causal:
+            sc = np.where(np.arange(seq)[None, None, None, :] <= np.arange(seq)[None, None, :, None], sc, -np.inf)
+        p = np.exp(sc - sc.max(-1, keepdims=True))
+        p /= p.sum(-1, keepdims=True)
+        ref = np.einsum("bhqk,bhkd->bhqd", p, split(v)).transpose(0, 2, 1, 3).reshape(batch * seq, dm)
+        assert rel(o.download(), ref) <= 2e-5
