@@ -194,3 +194,51 @@ def test_int8_linear_random_shapes_bit_exact(hip, seed):
         hip.linear_int8_dynamic(DeviceBuffer.from_host(x), m, k, DeviceBuffer.from_host(wq), DeviceBuffer.from_host(ws), n,
                                 DeviceBuffer.from_host(bias), out)
         assert np.array_equal(out.to_host().view(np.uint32), ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("seed", [71])
+def test_small_problem_kernels_random_shapes(hip, seed):
+    """The latency-oriented kernels: key-split attention (few query blocks, up to 4096 keys, head size 32 / 64) and the
+    16 x 16-tile GEMM for reductions of 512 and more, NT and NN, batched, with every epilogue."""
+    rng = np.random.default_rng(seed)
+    for _ in range(40):
+        bh, sq = int(rng.integers(1, 5)), int(rng.integers(1, 300))
+        sk = int(rng.integers(1, 4097)) if rng.random() < 0.5 else sq
+        dk, causal = int(rng.choice([32, 64])), bool(rng.random() < 0.5)
+        print("sdpa_small", dict(bh=bh, sq=sq, sk=sk, d=dk, causal=causal), flush=True)
+        q, k, v = (rng.normal(size=(bh, n, dk)).astype(np.float32) for n in (sq, sk, sk))
+        s = 1 / math.sqrt(dk)
+        sc = np.einsum("bqd,bkd->bqk", q.astype(np.float64), k.astype(np.float64)) * s
+        if causal:
+            sc = np.where(np.arange(sk)[None, None, :] <= np.arange(sq)[None, :, None], sc, -np.inf)
+        p = np.exp(sc - sc.max(-1, keepdims=True))
+        p /= p.sum(-1, keepdims=True)
+        o = DeviceBuffer((bh, sq, dk))
+        hip.sdpa_forward(D.sdpa_desc_contiguous(bh, sq, sk, dk, dk, causal), s, DeviceBuffer.from_host(q), DeviceBuffer.from_host(k),
+                         DeviceBuffer.from_host(v), o)
+        assert rel(o.to_host(), np.einsum("bqk,bkd->bqd", p, v.astype(np.float64))) <= 2e-5
+    for _ in range(60):
+        m, n, k = int(rng.integers(1, 300)), int(rng.integers(1, 300)), int(rng.integers(32, 257)) * 16
+        tb = bool(rng.random() < 0.6)
+        if not tb:
+            n = max(4, n // 4 * 4)
+        if 2.0 * m * n * k > 4e8:
+            continue
+        batch, epi = int(rng.choice([1, 1, 2, 5])), int(rng.choice([0, 1, 3, 5, 9]))
+        print("gemm_small16", dict(m=m, n=n, k=k, tb=tb, batch=batch, epi=epi), flush=True)
+        A = rng.uniform(-1, 1, (batch, m, k)).astype(np.float32)
+        B = rng.uniform(-1, 1, (batch, n, k) if tb else (batch, k, n)).astype(np.float32)
+        bias, res = rng.uniform(-1, 1, n).astype(np.float32), rng.uniform(-1, 1, (batch, m, n)).astype(np.float32)
+        c = DeviceBuffer((batch, m, n))
+        hip.gemm(D.gemm_desc(m, n, k, trans_b=tb, batch=batch, epilogue=epi), DeviceBuffer.from_host(A), DeviceBuffer.from_host(B), c,
+                 bias=DeviceBuffer.from_host(bias) if epi & 1 else None, residual=DeviceBuffer.from_host(res) if epi & 4 else None)
+        r = A.astype(np.float64) @ (np.swapaxes(B, 1, 2) if tb else B).astype(np.float64)
+        if epi & 1:
+            r = r + bias
+        if epi & 2:
+            r = 0.5 * r * (1 + erf(r / math.sqrt(2)))
+        if epi & 8:
+            r = 0.5 * r * (1 + np.tanh(math.sqrt(2 / math.pi) * (r + 0.044715 * r**3)))
+        if epi & 4:
+            r = r + res
+        assert rel(c.to_host(), r) <= 2e-5 * max(1.0, math.sqrt(k) / 4)
