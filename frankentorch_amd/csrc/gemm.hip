@@ -1123,19 +1123,30 @@ struct StreamWorkspace {
     size_t partial_bytes = 0;
 };
 // slot 0: split-tile accumulators; slot 1: transposed copy of a [k, m] A operand.
+//
+// A block that a larger request outgrows is retired, never handed back to the shared pool: kernels
+// queued on the stream may still be using it, the pool serves every stream and thread (so "ordered
+// on the same stream" would not protect the next owner), and a captured HIP graph keeps the address
+// it was recorded with for as long as its executable lives. Requests up to 512 MiB grow
+// geometrically, so the retired blocks of a stream add up to less than its current one.
 int32_t get_workspace(hipStream_t st, size_t partial_bytes, void **partials, int slot = 0) {
     static std::mutex mu;
     static std::map<std::pair<hipStream_t, int>, StreamWorkspace> *table = new std::map<std::pair<hipStream_t, int>, StreamWorkspace>();
+    static std::vector<void *> *retired = new std::vector<void *>();
     std::lock_guard<std::mutex> lock(mu);
     StreamWorkspace &w = (*table)[std::make_pair(st, slot)];
     if (w.partial_bytes < partial_bytes) {
-        // The old block returns to the pool; kernels already queued on this stream that still use
-        // it are ordered before whatever reuses it on the same stream.
-        fth::pool_free(w.partials);
-        w.partials = nullptr;
-        w.partial_bytes = 0;
-        if (int32_t rc = fth::pool_alloc(&w.partials, partial_bytes)) return rc;
-        w.partial_bytes = partial_bytes;
+        size_t want = partial_bytes;
+        if (w.partial_bytes && want < 2 * w.partial_bytes && w.partial_bytes <= ((size_t)1 << 29)) want = 2 * w.partial_bytes;
+        void *fresh = nullptr;
+        if (int32_t rc = fth::pool_alloc(&fresh, want)) {
+            if (want == partial_bytes) return rc;
+            want = partial_bytes;  // the doubled block did not fit: take exactly what is needed
+            if (int32_t rc2 = fth::pool_alloc(&fresh, want)) return rc2;
+        }
+        if (w.partials) retired->push_back(w.partials);
+        w.partials = fresh;
+        w.partial_bytes = want;
     }
     *partials = w.partials;
     return FTH_OK;

@@ -106,6 +106,35 @@ def test_config1_block_forward_eager_graph_and_determinism(hip, oracle):
     assert rel_err(enc3.forward(x3, 3, 40), ref3) <= TOL_GEMM_F32
 
 
+def test_graph_replay_survives_a_larger_gemm_and_new_tensors_on_its_stream(hip):
+    """A captured graph keeps the address of the stream's GEMM split-tile workspace. A later, larger product on the same
+    stream outgrows that workspace; the old block must stay out of the pool, or a tensor allocated afterwards could be
+    handed the memory the replay still writes its partial tiles to."""
+    batch, seq, d, heads, f = 2, 1024, 512, 8, 2048  # 2048 tokens: the projections run the large-tile kernels with split tiles
+    layers = [make_layer(6, i, d, f, biases_zero=False) for i in range(2)]
+    x = synth.normal(6, "x", (batch * seq, d))
+    enc = fused.EncoderHip(d, heads, f, layers, 1e-5, causal=True)
+    dx, dout = DeviceBuffer.from_host(x), DeviceBuffer((batch * seq, d))
+    enc.forward_dev(dx, dout, batch, seq)
+    eager = dout.to_host()
+    enc.forward_dev(dx, dout, batch, seq, graph=True)  # capture + first replay
+    assert np.array_equal(dout.to_host(), eager)
+    # a product that needs a larger split-tile workspace (fp64, 128 x 128 tiles, every tile split), on the same stream
+    n = 2176
+    a64 = DeviceBuffer.from_host(synth.uniform(6, "a64", (n, n), -1, 1, dtype=np.float64))
+    c64 = DeviceBuffer((n, n), np.float64)
+    hip.gemm(hip.gemm_desc(n, n, n), a64, a64, c64)
+    hip.synchronize()
+    # tensors of every size class the old workspace may have had, filled with a pattern
+    canaries = [fused.HipTensor.upload(np.full((rows, 1024), 7.0, np.float32)) for rows in (4096, 8192, 16384, 32768, 4096, 8192, 16384)]
+    for _ in range(3):
+        enc.forward_dev(dx, dout, batch, seq, graph=True)
+        assert np.array_equal(dout.to_host(), eager)
+    for t in canaries:
+        assert np.all(t.download() == 7.0)
+        t.free()
+
+
 def test_small_gpt2_forward_matches_oracle(hip, oracle):
     vocab, maxpos, d, heads, f, nl, batch, seq = 1003, 48, 128, 4, 512, 3, 2, 40
     wte = synth.normal(4, "wte", (vocab, d), 0.0, 0.02)
@@ -136,14 +165,21 @@ def test_small_gpt2_forward_matches_oracle(hip, oracle):
     assert model.bad_index() == 7
 
 
+# Rows of config 5 whose oracle top-2 logit gap is so small that fp32 rounding of the LM-head product may legitimately
+# pick the other token: (sequence, position) -> gap. Empty: on the seeded inputs every compared row has a gap above
+# 6e-5 of its largest logit, three times the 2e-5 product tolerance, so any argmax difference is a failure.
+CONFIG5_ARGMAX_ALLOW = {}
+
+
 def test_config5_gpt2_small_shape_logits_and_argmax(hip, oracle):
     """Config 5: 12 layers, d 768, 12 heads, FFN 3072, vocab 50257, batch 8, seq 1024, seed 4.
-    The full CPU forward is too slow for a test, so the pipeline is pinned in three steps:
-    (1) the first 16 tokens of sequence 0 are causal-closed, so the oracle runs the whole model on
-    that prefix and must reproduce the GPU's final hidden rows; (2) on sampled rows of the GPU's
-    final hidden state the oracle's tied LM head gives the logits and the argmax, which must be
-    IDENTICAL unless the oracle's own top-2 gap is below the fp32 rounding of the product
-    (reported, never silently accepted); (3) the whole logits tensor is bitwise repeatable."""
+    (1) Two complete 1024-token sequences of the batch (5 and 7, neither the first) go through the CPU checker's whole
+    model -- embeddings, 12 blocks at S = 1024 (every SDPA tile boundary and the packed-QKV strided reads at the real
+    shape), final LayerNorm, tied LM head -- and the GPU's hidden rows, logits and argmax of those 2048 positions are
+    compared with it: hidden and logits at 2e-5, argmax identical at every position. Sequences are independent under the
+    causal per-sequence attention, so the checker runs them as batch 1. (2) On sampled rows of every other sequence the
+    checker's LM head on the GPU's hidden state must give the same logits and argmax. (3) The whole logits tensor is
+    bitwise repeatable."""
     vocab, maxpos, d, heads, f, nl, batch, seq = 50257, 1024, 768, 12, 3072, 12, 8, 1024
     wte = synth.normal(4, "wte", (vocab, d), 0.0, 0.02)
     wpe = synth.normal(4, "wpe", (maxpos, d), 0.0, 0.02)
@@ -156,27 +192,29 @@ def test_config5_gpt2_small_shape_logits_and_argmax(hip, oracle):
     model.forward_dev(dids, batch, seq, dlog, dam)
     am = dam.to_host()
     hidden = model.hidden(T)
-    assert model.bad_index() == -1
-    # (1) causal prefix through the whole model
-    P = 16
-    ref = oracle.gpt2_forward(wte, wpe, layers, np.ones(d, np.float32), np.zeros(d, np.float32), ids[:P], 1, P, heads, 1e-5,
-                              want_logits=False)
-    assert rel_err(hidden[:P], ref["hidden"]) <= TOL_GEMM_F32
-    # (2) LM head + argmax on sampled rows
-    rows = np.concatenate([np.arange(P), np.arange(97, T, 257)])
-    ref_logits = oracle.gemm(hidden[rows], wte, trans_b=True)
-    logits_rows = np.empty((rows.size, vocab), np.float32)
     full = dlog.to_host()
-    logits_rows[:] = full[rows]
-    assert rel_err(logits_rows, ref_logits) <= TOL_GEMM_F32
-    ref_am = np.argmax(ref_logits, axis=1)
-    assert np.array_equal(am[rows], np.argmax(logits_rows, axis=1).astype(np.float32))
-    mism = np.nonzero(am[rows] != ref_am)[0]
-    for i in mism:
-        top2 = np.sort(ref_logits[i])[-2:]
-        gap = float(top2[1] - top2[0])
-        print("argmax differs at row %d: oracle %d gpu %d, oracle top-2 gap %.3e" % (rows[i], ref_am[i], am[rows][i], gap))
-        assert gap <= 4 * np.finfo(np.float32).eps * float(np.max(np.abs(ref_logits[i]))), "argmax differs beyond rounding"
+    assert model.bad_index() == -1
+    assert np.array_equal(am, np.argmax(full, axis=1).astype(np.float32))  # the argmax kernel is exact on its own input
+    one, zero = np.ones(d, np.float32), np.zeros(d, np.float32)
+    # (1) whole sequences through the whole model
+    mismatches = []
+    for b in (5, 7):
+        rows = slice(b * seq, (b + 1) * seq)
+        ref = oracle.gpt2_forward(wte, wpe, layers, one, zero, ids[rows], 1, seq, heads, 1e-5, want_logits=True)
+        assert ref["bad"] == -1
+        assert rel_err(hidden[rows], ref["hidden"]) <= TOL_GEMM_F32, "hidden rows of sequence %d" % b
+        assert rel_err(full[rows], ref["logits"]) <= TOL_GEMM_F32, "logits of sequence %d" % b
+        for pos in np.nonzero(am[rows] != ref["argmax"])[0]:
+            top2 = np.sort(ref["logits"][pos])[-2:]
+            mismatches.append((b, int(pos), int(ref["argmax"][pos]), int(am[rows][pos]), float(top2[1] - top2[0])))
+    unexpected = [m for m in mismatches if (m[0], m[1]) not in CONFIG5_ARGMAX_ALLOW]
+    assert not unexpected, "argmax differs from the checker at (sequence, position, checker, gpu, checker top-2 gap): %s" % unexpected
+    assert len(mismatches) == len(CONFIG5_ARGMAX_ALLOW), "allow-listed rows that no longer differ: update CONFIG5_ARGMAX_ALLOW"
+    # (2) LM head + argmax on sampled rows of the other sequences
+    rows = np.arange(97, T, 257)
+    ref_logits = oracle.gemm(hidden[rows], wte, trans_b=True)
+    assert rel_err(full[rows], ref_logits) <= TOL_GEMM_F32
+    assert np.array_equal(am[rows], np.argmax(ref_logits, axis=1).astype(np.float32)), "argmax of sampled rows differs from the checker's LM head"
     # (3) bitwise repeatability of the whole forward
     dlog2 = DeviceBuffer((T, vocab))
     model.forward_dev(dids, batch, seq, dlog2, None)
