@@ -20,6 +20,7 @@ LIB_PATH = os.path.join(PKG_DIR, "libft_kernel_hip.so")
 
 HIP_SOURCES = [
     "runtime.hip",
+    "staging.hip",
     "rowops.hip",
     "indexops.hip",
     "gemm.hip",

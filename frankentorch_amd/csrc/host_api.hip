@@ -10,6 +10,7 @@
 
 #include "common.hpp"
 #include "pool.hpp"
+#include "staging.hpp"
 
 namespace {
 
@@ -142,11 +143,16 @@ int32_t check_out(const void *out, size_t out_cap, size_t need) {
 }
 
 // ---- staging ---------------------------------------------------------------------------------
+// Small operands go over in one asynchronous copy on the library stream; anything from 1 MiB up
+// goes through the pinned rings (parallel host copy overlapped with the DMA).
 template <typename T> int32_t stage_in(fth::Scratch &sc, const T *host, size_t n, T **dev) {
     void *p = nullptr;
     if (int32_t rc = sc.get(&p, n * sizeof(T))) return rc;
     *dev = static_cast<T *>(p);
-    if (n) FTH_HIP(hipMemcpyAsync(p, host, n * sizeof(T), hipMemcpyHostToDevice, fth::resolve_stream(nullptr)));
+    if (n == 0) return FTH_OK;
+    hipStream_t st = fth::resolve_stream(nullptr);
+    if (n * sizeof(T) >= fth::kStagedMinBytes) return fth::staged_upload(p, host, n * sizeof(T), st);
+    FTH_HIP(hipMemcpyAsync(p, host, n * sizeof(T), hipMemcpyHostToDevice, st));
     return FTH_OK;
 }
 template <typename T> int32_t stage_out(fth::Scratch &sc, size_t n, T **dev) {
@@ -155,16 +161,61 @@ template <typename T> int32_t stage_out(fth::Scratch &sc, size_t n, T **dev) {
     *dev = static_cast<T *>(p);
     return FTH_OK;
 }
-template <typename T> int32_t fetch(T *host, const T *dev, size_t n) {
-    hipStream_t st = fth::resolve_stream(nullptr);
-    if (n) FTH_HIP(hipMemcpyAsync(host, dev, n * sizeof(T), hipMemcpyDeviceToHost, st));
-    hipError_t e = hipStreamSynchronize(st);
+int32_t sync_library_stream() {
+    hipError_t e = hipStreamSynchronize(fth::resolve_stream(nullptr));
     if (e != hipSuccess) {
         fth::hip_fail(e, "hipStreamSynchronize");
         fth::last_error().code = FTH_ERR_STREAM;
         return FTH_ERR_STREAM;
     }
     return FTH_OK;
+}
+template <typename T> int32_t fetch(T *host, const T *dev, size_t n) {
+    hipStream_t st = fth::resolve_stream(nullptr);
+    if (n * sizeof(T) >= fth::kStagedMinBytes) {
+        if (int32_t rc = fth::staged_download(host, dev, n * sizeof(T), st)) return rc;
+        return sync_library_stream();
+    }
+    if (n) FTH_HIP(hipMemcpyAsync(host, dev, n * sizeof(T), hipMemcpyDeviceToHost, st));
+    return sync_library_stream();
+}
+
+// A row-wise op on host slices: `rows` independent rows of `cols` elements, one or two row-aligned
+// inputs and a row-aligned output of the same shape. Large problems run as an upload / kernel /
+// download pipeline over chunks of rows; `launch(in0, in1, out, nrows)` gets device pointers to the
+// chunk. Small ones upload, launch once and download.
+template <typename T, typename F>
+int32_t run_rows(const T *in0, const T *in1, T *out, int64_t rows, int64_t cols, F launch) {
+    const size_t total = (size_t)rows * (size_t)cols;
+    fth::Scratch sc;
+    fth::RowOp op;
+    op.n_in = in1 ? 2 : 1;
+    op.host_in[0] = in0; op.host_in[1] = in1;
+    op.in_row_bytes[0] = (size_t)cols * sizeof(T);
+    op.in_row_bytes[1] = in1 ? (size_t)cols * sizeof(T) : 0;
+    op.host_out = out;
+    op.out_row_bytes = (size_t)cols * sizeof(T);
+    op.rows = rows;
+    if (!fth::row_pipeline_applies(op)) {
+        T *d0, *d1 = nullptr, *dy;
+        if (int32_t rc = stage_in(sc, in0, total, &d0)) return rc;
+        if (in1)
+            if (int32_t rc = stage_in(sc, in1, total, &d1)) return rc;
+        if (int32_t rc = stage_out(sc, total, &dy)) return rc;
+        if (int32_t rc = launch(d0, d1, dy, rows)) return rc;
+        return fetch(out, dy, total);
+    }
+    T *d0, *d1 = nullptr, *dy;
+    if (int32_t rc = stage_out(sc, total, &d0)) return rc;
+    if (in1)
+        if (int32_t rc = stage_out(sc, total, &d1)) return rc;
+    if (int32_t rc = stage_out(sc, total, &dy)) return rc;
+    op.dev_in[0] = d0; op.dev_in[1] = d1; op.dev_out = dy;
+    if (int32_t rc = fth::row_pipeline(op, [&](int64_t row0, int64_t nrows) {
+            return launch(d0 + row0 * cols, d1 ? d1 + row0 * cols : nullptr, dy + row0 * cols, nrows);
+        }, fth::resolve_stream(nullptr)))
+        return rc;
+    return sync_library_stream();
 }
 
 template <typename T> struct Dev;
@@ -446,13 +497,20 @@ int32_t softmax_impl(const T *input, size_t input_len, const fth_meta *meta, siz
     if (int32_t rc = check_out(out, out_cap, (size_t)numel)) return rc;
     if (numel == 0) return FTH_OK;
     FTH_REQUIRE_DEVICE();
+    // log_softmax_dim_tensor_contiguous (crates/ft-kernel-cpu/src/lib.rs:39298-39375 / 18504-18590) shares the validation
+    const int64_t reduce = (int64_t)meta->shape[dim];
+    if (inner == 1 && outer <= (uint64_t)std::numeric_limits<int64_t>::max()) {
+        // last-dim form: the rows are independent, so transfers and kernels overlap chunk by chunk
+        return run_rows<T>(input + meta->storage_offset, nullptr, out, (int64_t)outer, reduce, [&](const T *x, const T *, T *y, int64_t nrows) {
+            return log_form ? Dev<T>::log_softmax(x, y, nrows, reduce, 1) : Dev<T>::softmax(x, y, nrows, reduce, 1);
+        });
+    }
     fth::Scratch sc;
     T *dx, *dy;
     if (int32_t rc = stage_in(sc, input + meta->storage_offset, (size_t)numel, &dx)) return rc;
     if (int32_t rc = stage_out(sc, (size_t)numel, &dy)) return rc;
-    // log_softmax_dim_tensor_contiguous (crates/ft-kernel-cpu/src/lib.rs:39298-39375 / 18504-18590) shares the validation
-    if (int32_t rc = log_form ? Dev<T>::log_softmax(dx, dy, (int64_t)outer, (int64_t)meta->shape[dim], (int64_t)inner)
-                              : Dev<T>::softmax(dx, dy, (int64_t)outer, (int64_t)meta->shape[dim], (int64_t)inner))
+    if (int32_t rc = log_form ? Dev<T>::log_softmax(dx, dy, (int64_t)outer, reduce, (int64_t)inner)
+                              : Dev<T>::softmax(dx, dy, (int64_t)outer, reduce, (int64_t)inner))
         return rc;
     return fetch(out, dy, (size_t)numel);
 }
@@ -469,24 +527,19 @@ int32_t layer_norm_impl(const T *x, const T *x2, size_t x_len, const T *w, const
     FTH_ARG(x_len >= total, "layer_norm: input slice shorter than batch * norm_size");
     FTH_REQUIRE_DEVICE();
     fth::Scratch sc;
-    T *dx, *dx2 = nullptr, *dw = nullptr, *db = nullptr, *dy;
-    if (int32_t rc = stage_in(sc, x, (size_t)total, &dx)) return rc;
-    if (x2)
-        if (int32_t rc = stage_in(sc, x2, (size_t)total, &dx2)) return rc;
+    T *dw = nullptr, *db = nullptr;
     if (w)
         if (int32_t rc = stage_in(sc, w, n, &dw)) return rc;
     if (b)
         if (int32_t rc = stage_in(sc, b, n, &db)) return rc;
-    if (int32_t rc = stage_out(sc, (size_t)total, &dy)) return rc;
-    int32_t rc;
-    if constexpr (std::is_same<T, float>::value) {
-        rc = x2 ? fth_dev_add_layer_norm_f32(dx, dx2, dw, db, dy, (int64_t)batch, (int64_t)n, eps, nullptr)
-                : fth_dev_layer_norm_f32(dx, dw, db, dy, (int64_t)batch, (int64_t)n, eps, nullptr);
-    } else {
-        rc = fth_dev_layer_norm_f64(dx, dw, db, dy, (int64_t)batch, (int64_t)n, eps, nullptr);
-    }
-    if (rc) return rc;
-    return fetch(out, dy, (size_t)total);
+    return run_rows<T>(x, x2, out, (int64_t)batch, (int64_t)n, [&](const T *dx, const T *dx2, T *dy, int64_t nrows) -> int32_t {
+        if constexpr (std::is_same<T, float>::value) {
+            return dx2 ? fth_dev_add_layer_norm_f32(dx, dx2, dw, db, dy, nrows, (int64_t)n, eps, nullptr)
+                       : fth_dev_layer_norm_f32(dx, dw, db, dy, nrows, (int64_t)n, eps, nullptr);
+        } else {
+            return fth_dev_layer_norm_f64(dx, dw, db, dy, nrows, (int64_t)n, eps, nullptr);
+        }
+    });
 }
 
 // rms_norm_forward (crates/ft-kernel-cpu/src/lib.rs:6459-6494 / 6418-6453)
@@ -499,13 +552,12 @@ int32_t rms_norm_impl(const T *x, size_t x_len, const T *w, size_t batch, size_t
     FTH_ARG(x_len >= total, "rms_norm: input slice shorter than batch * norm_size");
     FTH_REQUIRE_DEVICE();
     fth::Scratch sc;
-    T *dx, *dw = nullptr, *dy;
-    if (int32_t rc = stage_in(sc, x, (size_t)total, &dx)) return rc;
+    T *dw = nullptr;
     if (w)
         if (int32_t rc = stage_in(sc, w, n, &dw)) return rc;
-    if (int32_t rc = stage_out(sc, (size_t)total, &dy)) return rc;
-    if (int32_t rc = Dev<T>::rms_norm(dx, dw, dy, (int64_t)batch, (int64_t)n, eps)) return rc;
-    return fetch(out, dy, (size_t)total);
+    return run_rows<T>(x, nullptr, out, (int64_t)batch, (int64_t)n, [&](const T *dx, const T *, T *dy, int64_t nrows) {
+        return Dev<T>::rms_norm(dx, dw, dy, nrows, (int64_t)n, eps);
+    });
 }
 
 // gelu_tensor_contiguous (unary_contiguous_f32 via define_unary_f32!, crates/ft-kernel-cpu/src/
@@ -521,12 +573,11 @@ int32_t gelu_impl(const T *input, size_t input_len, const fth_meta *meta, T *out
     if (int32_t rc = check_out(out, out_cap, (size_t)numel)) return rc;
     if (numel == 0) return FTH_OK;
     FTH_REQUIRE_DEVICE();
-    fth::Scratch sc;
-    T *dx, *dy;
-    if (int32_t rc = stage_in(sc, input + meta->storage_offset, (size_t)numel, &dx)) return rc;
-    if (int32_t rc = stage_out(sc, (size_t)numel, &dy)) return rc;
-    if (int32_t rc = tanh_form ? Dev<T>::gelu_tanh(dx, dy, (int64_t)numel) : Dev<T>::gelu(dx, dy, (int64_t)numel)) return rc;
-    return fetch(out, dy, (size_t)numel);
+    // elementwise: every element is a "row" of its own, so the pipeline cuts the tensor anywhere
+    FTH_ARG(numel <= (uint64_t)std::numeric_limits<int64_t>::max(), "gelu: tensor too large");
+    return run_rows<T>(input + meta->storage_offset, nullptr, out, (int64_t)numel, 1, [&](const T *dx, const T *, T *dy, int64_t count) {
+        return tanh_form ? Dev<T>::gelu_tanh(dx, dy, count) : Dev<T>::gelu(dx, dy, count);
+    });
 }
 
 // add_tensor_contiguous (simd_elementwise_f32, crates/ft-kernel-cpu/src/lib.rs:36558-36593):
@@ -548,13 +599,10 @@ int32_t add_impl(const T *lhs, size_t lhs_len, const T *rhs, size_t rhs_len, con
     if (int32_t rc = check_out(out, out_cap, (size_t)numel)) return rc;
     if (numel == 0) return FTH_OK;
     FTH_REQUIRE_DEVICE();
-    fth::Scratch sc;
-    T *da, *db, *dy;
-    if (int32_t rc = stage_in(sc, lhs + lm->storage_offset, (size_t)numel, &da)) return rc;
-    if (int32_t rc = stage_in(sc, rhs + rm->storage_offset, (size_t)numel, &db)) return rc;
-    if (int32_t rc = stage_out(sc, (size_t)numel, &dy)) return rc;
-    if (int32_t rc = Dev<T>::add(da, db, dy, (int64_t)numel)) return rc;
-    return fetch(out, dy, (size_t)numel);
+    FTH_ARG(numel <= (uint64_t)std::numeric_limits<int64_t>::max(), "add: tensor too large");
+    return run_rows<T>(lhs + lm->storage_offset, rhs + rm->storage_offset, out, (int64_t)numel, 1, [&](const T *da, const T *db, T *dy, int64_t count) {
+        return Dev<T>::add(da, db, dy, count);
+    });
 }
 
 // sdpa_forward (crates/ft-kernel-cpu/src/lib.rs:5200-5284 / 4572-4651)

@@ -161,6 +161,31 @@ int32_t fth_memset_zero(void *dst, size_t bytes) {
     return FTH_OK;
 }
 
+int32_t fth_host_malloc(void **hptr, size_t bytes) {
+    FTH_REQUIRE_DEVICE();
+    FTH_ARG(hptr != nullptr, "fth_host_malloc: hptr is NULL");
+    *hptr = nullptr;
+    if (bytes == 0) return FTH_OK;
+    FTH_HIP(hipHostMalloc(hptr, bytes, hipHostMallocDefault));
+    return FTH_OK;
+}
+
+int32_t fth_host_free(void *hptr) {
+    if (!hptr) return FTH_OK;
+    FTH_REQUIRE_DEVICE();
+    FTH_HIP(hipHostFree(hptr));
+    return FTH_OK;
+}
+
+int32_t fth_memcpy_async(void *dst, const void *src, size_t bytes, int32_t kind, fth_stream s) {
+    FTH_REQUIRE_DEVICE();
+    FTH_ARG(kind >= 1 && kind <= 3, "fth_memcpy_async: kind %d is not 1 (H2D), 2 (D2H) or 3 (D2D)", kind);
+    if (bytes == 0) return FTH_OK;
+    const hipMemcpyKind k = kind == 1 ? hipMemcpyHostToDevice : kind == 2 ? hipMemcpyDeviceToHost : hipMemcpyDeviceToDevice;
+    FTH_HIP(hipMemcpyAsync(dst, src, bytes, k, fth::resolve_stream(s)));
+    return FTH_OK;
+}
+
 int32_t fth_stream_create(fth_stream *s) {
     FTH_REQUIRE_DEVICE();
     FTH_ARG(s != nullptr, "fth_stream_create: s is NULL");

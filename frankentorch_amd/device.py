@@ -110,6 +110,79 @@ class Event:
             pass
 
 
+class PinnedArray:
+    """A page-locked host array (fth_host_malloc) exposed as numpy; the DMA engines read and write it in place."""
+
+    def __init__(self, shape, dtype=np.float32):
+        self.shape = tuple(int(s) for s in (shape if hasattr(shape, "__len__") else (shape,)))
+        self.dtype = np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
+        p = C.c_void_p()
+        check(_lib.load().fth_host_malloc(C.byref(p), self.nbytes))
+        self.ptr = p.value or 0
+        raw = (C.c_char * self.nbytes).from_address(self.ptr) if self.nbytes else b""
+        self.array = np.frombuffer(raw, dtype=self.dtype).reshape(self.shape)
+
+    def free(self) -> None:
+        if self.ptr:
+            self.array = None
+            _lib.load().fth_host_free(self.ptr)
+        self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Stream:
+    def __init__(self):
+        s = C.c_void_p()
+        check(_lib.load().fth_stream_create(C.byref(s)))
+        self.handle = s.value
+
+    def synchronize(self) -> None:
+        check(_lib.load().fth_stream_synchronize(self.handle))
+
+    def __del__(self):
+        try:
+            _lib.load().fth_stream_destroy(self.handle)
+        except Exception:
+            pass
+
+
+def link_rates(nbytes: int, reps: int = 5) -> dict:
+    """GB/s of the host link for one pinned buffer of `nbytes`: each direction alone, then both at once on two streams."""
+    import time
+
+    L = _lib.load()
+    hin, hout = PinnedArray((nbytes,), np.uint8), PinnedArray((nbytes,), np.uint8)
+    hin.array[:] = 1
+    hout.array[:] = 0
+    din, dout = DeviceBuffer((nbytes,), np.uint8), DeviceBuffer((nbytes,), np.uint8)
+    s1, s2 = Stream(), Stream()
+
+    def timed(up, down):
+        best = float("inf")
+        for _ in range(reps + 1):
+            t0 = time.perf_counter()
+            if up:
+                check(L.fth_memcpy_async(din.ptr, hin.ptr, nbytes, 1, s1.handle))
+            if down:
+                check(L.fth_memcpy_async(hout.ptr, dout.ptr, nbytes, 2, s2.handle))
+            s1.synchronize()
+            s2.synchronize()
+            best = min(best, time.perf_counter() - t0)
+        return nbytes / best / 1e9
+
+    h2d, d2h, both = timed(True, False), timed(False, True), timed(True, True)
+    res = {"h2d": round(h2d, 2), "d2h": round(d2h, 2), "h2d_duplex": round(both, 2), "d2h_duplex": round(both, 2)}
+    hin.free()
+    hout.free()
+    return res
+
+
 def _sfx(buf: DeviceBuffer) -> str:
     if buf.dtype == np.float32:
         return "f32"

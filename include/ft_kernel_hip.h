@@ -125,6 +125,16 @@ int32_t fth_memset_zero(void *dst_dev, size_t bytes);
 
 typedef void *fth_stream; /* a hipStream_t; NULL selects the library's own ordered stream */
 typedef void *fth_event;  /* a hipEvent_t */
+
+/* Page-locked host memory (hipHostMalloc) for callers that keep hot tensors in it: the host-slice
+ * entry points recognise such slices and let the DMA engines read and write them in place, where
+ * an ordinary slice has to be copied through the library's pinned chunks first. No counterpart in
+ * the reference (its `Vec<f32>` storage is pageable, crates/ft-core/src/lib.rs:915-925). */
+int32_t fth_host_malloc(void **hptr, size_t bytes);
+int32_t fth_host_free(void *hptr);
+/* Asynchronous copy on stream `s`; kind 1 = host to device, 2 = device to host, 3 = device to
+ * device. A host side that is not page-locked makes the copy synchronous with the host. */
+int32_t fth_memcpy_async(void *dst, const void *src, size_t bytes, int32_t kind, fth_stream s);
 int32_t fth_stream_create(fth_stream *s);
 int32_t fth_stream_destroy(fth_stream s);
 int32_t fth_stream_synchronize(fth_stream s);
@@ -615,7 +625,11 @@ int32_t fth_encoder_set_activation(fth_encoder *e, int32_t activation);
 int32_t fth_encoder_forward(fth_encoder *e, const float *input, int64_t batch, int64_t seq, float *out, size_t out_cap);
 /* Resident in / resident out on stream `s`; no synchronisation. `x` [batch*seq, d_model]. */
 int32_t fth_encoder_forward_dev(fth_encoder *e, const float *x_dev, int64_t batch, int64_t seq, float *out_dev, fth_stream s);
-/* Captures forward_dev for (batch, seq) into a HIP graph and replays it: one launch per forward. */
+/* Captures forward_dev for (x_dev, out_dev, batch, seq, s) into a HIP graph and replays it: one
+ * launch per forward. The graph holds device addresses: the caller's two buffers must stay valid
+ * while the encoder lives; the encoder's activations and the stream's GEMM split-tile workspace it
+ * also records are never released before fth_encoder_free. Returns FTH_ERR_UNAVAILABLE while a
+ * rocprofiler tool library is loaded in the process (trace the eager entry point instead). */
 int32_t fth_encoder_forward_graph(fth_encoder *e, const float *x_dev, int64_t batch, int64_t seq, float *out_dev, fth_stream s);
 
 /* ------------------------------------------------------------------------------------------ */

@@ -155,3 +155,92 @@ def test_short_slices_are_errors_not_faults(hip):
         K.sdpa_forward_f32(x, x, x, 1, 4, 4, 4, 4, 1.0, True)
     with pytest.raises(HipError):
         K.rms_norm_forward_f32(x, None, 3, 4, 1e-6)
+
+
+# ---- the staged transfer paths: operands of 1 MiB and more go through the pinned rings, row-wise ops run as an
+# upload / kernel / download pipeline over chunks of rows (8 MiB chunks: the shapes below give 1, 3 and 7 chunks,
+# with a ragged last chunk) ----
+PIPE_SHAPES = [(300, 1000), (5001, 1000), (1237, 12288), (3, 1048576)]
+
+
+@pytest.mark.parametrize("rows,cols", PIPE_SHAPES)
+def test_row_pipeline_equals_the_device_tier_bit_for_bit(hip, oracle, rows, cols):
+    """Chunking a row-wise op over the pipeline cannot change a bit: every row goes through the same kernel as in one
+    launch over the resident tensor. Checked against the device tier, and against the CPU checker at the row-op bar."""
+    from frankentorch_amd.device import DeviceBuffer
+
+    x = synth.normal(41, "x", (rows, cols))
+    r = synth.normal(41, "r", (rows, cols))
+    g = synth.uniform(41, "g", (cols,), 0.5, 1.5)
+    b = synth.normal(41, "b", (cols,), 0.0, 0.1)
+    m = _m([rows, cols], np.float32)
+    dx, dr, dg, db = (DeviceBuffer.from_host(a) for a in (x, r, g, b))
+    dy = DeviceBuffer((rows, cols))
+
+    def dev(fn):
+        fn()
+        return dy.to_host().reshape(-1)
+
+    cases = [
+        ("softmax", K.softmax_dim_tensor_contiguous_f32(x, m, 1), dev(lambda: hip.softmax_lastdim(dx, dy, rows, cols)), oracle.softmax(x, 1)),
+        ("log_softmax", K.log_softmax_dim_tensor_contiguous_f32(x, m, 1), dev(lambda: hip.log_softmax_strided(dx, dy, rows, cols, 1)), None),
+        ("layer_norm", K.layer_norm_forward_f32(x, g, b, rows, cols, 1e-5), dev(lambda: hip.layer_norm(dx, dg, db, dy, rows, cols, 1e-5)),
+         oracle.layer_norm(x, g, b, 1e-5)),
+        ("add_layer_norm", K.add_layer_norm_forward_f32(x, r, g, b, rows, cols, 1e-5), dev(lambda: hip.add_layer_norm(dx, dr, dg, db, dy, rows, cols, 1e-5)), None),
+        ("rms_norm", K.rms_norm_forward_f32(x, g, rows, cols, 1e-6), dev(lambda: hip.rms_norm(dx, dg, dy, rows, cols, 1e-6)), oracle.rms_norm(x, g, 1e-6)),
+        ("gelu", K.gelu_tensor_contiguous_f32(x, m), dev(lambda: hip.gelu(dx, dy, rows * cols)), oracle.gelu(x)),
+        ("add", K.add_tensor_contiguous_f32(x, r, m, m), dev(lambda: hip.add(dx, dr, dy, rows * cols)), (x + r)),
+    ]
+    for name, got, resident, ref in cases:
+        assert got.shape == (rows * cols,), name
+        assert np.array_equal(got.view(np.uint32), resident.view(np.uint32)), name
+        # rows of a million elements: the checker's serial fp32 sums (the reference's order) are themselves 2e-4 away from
+        # the exact sums there, so only the bitwise comparison with the device tier applies
+        if ref is not None and cols <= 65536:
+            assert rel_err(got, np.asarray(ref).reshape(-1)) <= TOL_ROW_F32, name
+
+
+def test_pinned_slices_take_the_direct_path_and_give_the_same_bits(hip):
+    from frankentorch_amd.device import PinnedArray
+
+    rows, cols = 4099, 1536
+    x = synth.normal(42, "x", (rows, cols))
+    m = _m([rows, cols], np.float32)
+    ref = K.softmax_dim_tensor_contiguous_f32(x, m, 1)
+    px, py = PinnedArray((rows * cols,)), PinnedArray((rows * cols,))
+    px.array[:] = x.reshape(-1)
+    py.array[:] = -1.0
+    import ctypes as C
+
+    from frankentorch_amd import _lib
+    from frankentorch_amd.core import check
+
+    mc, n_out = m.to_c(), C.c_size_t(0)
+    check(_lib.load().fth_softmax_dim_tensor_contiguous_f32(px.ptr, rows * cols, C.byref(mc), 1, py.ptr, rows * cols, C.byref(n_out)))
+    assert n_out.value == rows * cols
+    assert np.array_equal(py.array.view(np.uint32), ref.view(np.uint32))
+    # a pinned input with a pageable output, and the other way round
+    out = np.full(rows * cols, -1.0, np.float32)
+    check(_lib.load().fth_softmax_dim_tensor_contiguous_f32(px.ptr, rows * cols, C.byref(mc), 1, out.ctypes.data, out.size, C.byref(n_out)))
+    assert np.array_equal(out.view(np.uint32), ref.view(np.uint32))
+    py.array[:] = -1.0
+    xin = np.ascontiguousarray(x.reshape(-1))
+    check(_lib.load().fth_softmax_dim_tensor_contiguous_f32(xin.ctypes.data, xin.size, C.byref(mc), 1, py.ptr, rows * cols, C.byref(n_out)))
+    assert np.array_equal(py.array.view(np.uint32), ref.view(np.uint32))
+    px.free()
+    py.free()
+
+
+def test_staged_operands_of_a_product(hip, oracle):
+    """Operands above 1 MiB are uploaded through the pinned rings (here 3 and 2 chunks) and the result comes back the same way."""
+    m_, k_, n_ = 1500, 1400, 1100
+    a = synth.uniform(43, "a", (m_, k_), -1, 1)
+    b = synth.uniform(43, "b", (k_, n_), -1, 1)
+    got = K.matmul_tensor_contiguous_f32(a, b, _m([m_, k_], np.float32), _m([k_, n_], np.float32))
+    assert rel_err(got.reshape(m_, n_), oracle.gemm(a, b)) <= TOL_GEMM_F32
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    got = K.matmul_tensor_contiguous_f64(a64, b64, _m([m_, k_], np.float64), _m([k_, n_], np.float64))
+    assert rel_err(got.reshape(m_, n_), oracle.gemm(a64, b64)) <= TOL_F64
+    # and a second call right after: the rings are idle again and reusable
+    got2 = K.matmul_tensor_contiguous_f64(a64, b64, _m([m_, k_], np.float64), _m([k_, n_], np.float64))
+    assert np.array_equal(got.view(np.uint64), got2.view(np.uint64))
