@@ -5,7 +5,7 @@ import math
 import numpy as np
 import pytest
 
-from conftest import TOL_F64, TOL_GEMM_F32, TOL_ROW_F32, rel_err
+from conftest import NORM_COLSUM_TOL_FACTOR, SDPA_BWD_MATERIALISED_TOL_FACTOR, TOL_F64, TOL_GEMM_F32, TOL_ROW_F32, rel_err
 from frankentorch_amd import synth
 from frankentorch_amd.device import DeviceBuffer
 
@@ -32,7 +32,7 @@ def test_layer_norm_backward(hip, oracle, rows, cols, dtype):
     ddx, ddw, ddb = DeviceBuffer((rows, cols), dtype), DeviceBuffer((cols,), dtype), DeviceBuffer((cols,), dtype)
     hip.layer_norm_backward(ddy, dx_, dw_, ddx, ddw, ddb, rows, cols, 1e-5)
     got = (ddx.to_host(), ddw.to_host(), ddb.to_host())
-    assert rel_err(got[0], dx_r) <= tol and rel_err(got[1], dw_r) <= tol * 4 and rel_err(got[2], db_r) <= tol * 4
+    assert rel_err(got[0], dx_r) <= tol and rel_err(got[1], dw_r) <= tol * NORM_COLSUM_TOL_FACTOR and rel_err(got[2], db_r) <= tol * NORM_COLSUM_TOL_FACTOR
     hip.layer_norm_backward(ddy, dx_, dw_, ddx, ddw, ddb, rows, cols, 1e-5)
     for a, b in zip(got, (ddx.to_host(), ddw.to_host(), ddb.to_host())):
         assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
@@ -53,7 +53,7 @@ def test_rms_norm_backward(hip, oracle, rows, cols, dtype, with_weight):
     hip.rms_norm_backward(ddy, dx_, dw_, ddx, ddw, rows, cols, 1e-6)
     assert rel_err(ddx.to_host(), dx_r) <= tol
     if with_weight:
-        assert rel_err(ddw.to_host(), dw_r) <= tol * 4
+        assert rel_err(ddw.to_host(), dw_r) <= tol * NORM_COLSUM_TOL_FACTOR
 
 
 @pytest.mark.parametrize("batch,in_f,out_f", [(96, 40, 72), (128, 256, 1024), (200, 300, 100), (1024, 768, 2304), (1, 5, 3), (33, 64, 64)])
@@ -106,7 +106,7 @@ def test_sdpa_backward(hip, oracle, bh, sq, sk, dk, dv, causal, dtype):
     hip.sdpa_backward(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, s, causal, gq, gk, gv)
     got = (gq.to_host(), gk.to_host(), gv.to_host())
     for g, r in zip(got, ref):
-        assert rel_err(g, r) <= tol * 2
+        assert rel_err(g, r) <= tol * SDPA_BWD_MATERIALISED_TOL_FACTOR
     hip.sdpa_backward(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, s, causal, gq, gk, gv)
     for a, b in zip(got, (gq.to_host(), gk.to_host(), gv.to_host())):
         assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
@@ -135,7 +135,7 @@ def test_sdpa_backward_masked(hip, oracle, bh, sq, sk, dk, dv, shared, dtype):
     hip.sdpa_backward_masked(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, s, dmask, stride, gq, gk, gv)
     got = (gq.to_host(), gk.to_host(), gv.to_host())
     for g, r in zip(got, ref):
-        assert rel_err(g, r) <= tol * 2
+        assert rel_err(g, r) <= tol * SDPA_BWD_MATERIALISED_TOL_FACTOR
     hip.sdpa_backward_masked(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, s, dmask, stride, gq, gk, gv)
     for a, b in zip(got, (gq.to_host(), gk.to_host(), gv.to_host())):
         assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
@@ -143,7 +143,7 @@ def test_sdpa_backward_masked(hip, oracle, bh, sq, sk, dk, dv, shared, dtype):
         pad = DeviceBuffer.from_host(np.concatenate([np.zeros(1, dtype), mask.ravel()]))
         hip.sdpa_backward_masked(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, s, pad.view(1), 0, gq, gk, gv)
         for g, r in zip((gq.to_host(), gk.to_host(), gv.to_host()), ref):
-            assert rel_err(g, r) <= tol * 2
+            assert rel_err(g, r) <= tol * SDPA_BWD_MATERIALISED_TOL_FACTOR
 
 
 @pytest.mark.parametrize("bh,sq,sk,dk,dv", [(2, 5, 6, 4, 3), (3, 100, 70, 32, 48), (2, 640, 640, 64, 64)])
@@ -161,7 +161,7 @@ def test_sdpa_backward_unit_dout(hip, oracle, bh, sq, sk, dk, dv, causal, dtype)
     hip.sdpa_backward_unit_dout(dq_, dk_, dv_, bh, sq, sk, dk, dv, s, causal, gq, gk, gv)
     got = (gq.to_host(), gk.to_host(), gv.to_host())
     for g, r in zip(got, ref):
-        assert rel_err(g, r) <= tol * 2
+        assert rel_err(g, r) <= tol * SDPA_BWD_MATERIALISED_TOL_FACTOR
     assert np.all(got[2] == got[2][:, :, :1])  # every value lane of a key gets the same gradient, bit for bit
     hq, hk, hv = DeviceBuffer(q.shape, dtype), DeviceBuffer(k.shape, dtype), DeviceBuffer(v.shape, dtype)
     hip.sdpa_backward(dq_, dk_, dv_, DeviceBuffer.from_host(np.ones((bh, sq, dv), dtype)), bh, sq, sk, dk, dv, s, causal, hq, hk, hv)
