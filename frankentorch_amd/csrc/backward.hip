@@ -24,6 +24,7 @@
 // the block diagonal.
 
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 #include "common.hpp"
@@ -864,9 +865,54 @@ int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, i
     return FTH_OK;
 }
 
+// ---- the allocation-free LayerNorm backward ----
+// Partial column sums live in a file-scope device array instead of a caller workspace. Every GPU
+// the library is loaded on holds its own copy at its own address, so the address is looked up once
+// per device (with that device current) and only that pointer is ever given to kernels.
+constexpr size_t kStaticScratchBytes = (size_t)24 << 20;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+int32_t static_scratch(void **out) {
+    static std::mutex mu;
+    static void *per_device[kMaxDevices] = {};
+    int dev = 0;
+    FTH_HIP(hipGetDevice(&dev));
+    FTH_ARG(dev >= 0 && dev < kMaxDevices, "static scratch: device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!per_device[dev]) {
+        void *ptr = nullptr;
+        FTH_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        FTH_ARG(ptr != nullptr, "static scratch: the device array has no address on device %d", dev);
+        per_device[dev] = ptr;
+    }
+    *out = per_device[dev];
+    return FTH_OK;
+}
+
 }  // namespace
 
 extern "C" {
+
+size_t fth_dev_layer_norm_backward_noalloc_max_bytes(void) { return kStaticScratchBytes; }
+
+int32_t fth_dev_layer_norm_backward_f32_noalloc(const float *dy, const float *x, const float *weight, int64_t rows, int64_t cols, float eps,
+                                                float *dx, float *dweight, float *dbias, fth_stream s) {
+    FTH_REQUIRE_DEVICE();
+    FTH_ARG(rows >= 0 && cols >= 0, "layer_norm backward (no allocation): negative extent");
+    FTH_ARG(cols <= 2147483647LL && rows <= 2147483647LL, "layer_norm backward (no allocation): extent too large");
+    const size_t need = norm_backward_workspace<float>(rows, cols);
+    if (need > kStaticScratchBytes)
+        return fth::set_error(FTH_ERR_BUFFER_TOO_LARGE,
+                              "layer_norm backward (no allocation): [%lld, %lld] needs %zu bytes of partial sums, the built-in scratch holds %zu; "
+                              "use fth_dev_layer_norm_backward_f32 with a workspace",
+                              (long long)rows, (long long)cols, need, kStaticScratchBytes);
+    void *ptr = nullptr;
+    if (int32_t rc = static_scratch(&ptr)) return rc;
+    // Nothing in the scratch has to start at zero: every partial row and statistic that the second
+    // pass reads is written by the first pass of the same call.
+    return norm_backward_entry<float, false>(dy, x, weight, rows, cols, eps, dx, dweight, dbias, ptr, kStaticScratchBytes, s);
+}
 
 size_t fth_dev_norm_backward_workspace_bytes(int64_t rows, int64_t cols, int32_t dtype) {
     if (rows < 0 || cols < 0) return 0;

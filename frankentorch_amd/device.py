@@ -323,6 +323,17 @@ def layer_norm_backward(dy, x, weight, dx, dweight, dbias, rows, cols, eps, work
     return ws
 
 
+def layer_norm_backward_noalloc(dy, x, weight, dx, dweight, dbias, rows, cols, eps, stream=None):
+    """fth_dev_layer_norm_backward_f32_noalloc: the fp32 LayerNorm backward with its partial sums in the library's built-in
+    device array; raises (BufferTooLarge) for shapes beyond layer_norm_backward_noalloc_max_bytes()."""
+    check(_lib.load().fth_dev_layer_norm_backward_f32_noalloc(_ptr(dy), _ptr(x), _ptr(weight), rows, cols, float(eps), _ptr(dx),
+                                                              _ptr(dweight), _ptr(dbias), stream))
+
+
+def layer_norm_backward_noalloc_max_bytes() -> int:
+    return int(_lib.load().fth_dev_layer_norm_backward_noalloc_max_bytes())
+
+
 def rms_norm_backward(dy, x, weight, dx, dweight, rows, cols, eps, workspace=None, stream=None):
     """rms_norm_backward_f32 / _f64: weight and dweight may both be None."""
     ws = _workspace(_lib.load().fth_dev_norm_backward_workspace_bytes(rows, cols, _dtype_code(x)), workspace)

@@ -297,6 +297,17 @@ int32_t fth_dev_layer_norm_backward_f32(const float *dy, const float *x, const f
 int32_t fth_dev_layer_norm_backward_f64(const double *dy, const double *x, const double *weight, int64_t rows, int64_t cols, double eps,
                                         double *dx, double *dweight, double *dbias, void *workspace, size_t workspace_bytes,
                                         fth_stream s);
+/* LayerNorm backward that allocates nothing. No counterpart in the reference: it is for callers
+ * that cannot call hipMalloc (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid it) and do not want to carry a workspace. Same kernels and results as
+ * fth_dev_layer_norm_backward_f32, with the partial column sums in a device array built into the
+ * library (fth_dev_layer_norm_backward_noalloc_max_bytes() = 24 MiB per GPU, held until the process
+ * ends). Shapes whose fth_dev_norm_backward_workspace_bytes exceeds that return
+ * FTH_ERR_BUFFER_TOO_LARGE (fp32 [8192, 4096] needs 16.1 MiB). All calls on one GPU share the
+ * array: calls that overlap in time on one GPU, on any streams, race. */
+size_t fth_dev_layer_norm_backward_noalloc_max_bytes(void);
+int32_t fth_dev_layer_norm_backward_f32_noalloc(const float *dy, const float *x, const float *weight, int64_t rows, int64_t cols, float eps,
+                                                float *dx, float *dweight, float *dbias, fth_stream s);
 /* rms_norm_backward_f32 / _f64 (:6574-6646, 6503-6570): weight and dweight may both be NULL. */
 int32_t fth_dev_rms_norm_backward_f32(const float *dy, const float *x, const float *weight, int64_t rows, int64_t cols, float eps,
                                       float *dx, float *dweight, void *workspace, size_t workspace_bytes, fth_stream s);
