@@ -46,6 +46,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "devmath.hpp"
 #include "pool.hpp"
 
 namespace {
@@ -85,7 +86,7 @@ template <> struct Mfma<float> {
     __device__ __forceinline__ static float elem(const V &v, int j) { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; }
     __device__ __forceinline__ static V zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
     __device__ __forceinline__ static V make(const float *e) { return make_float4(e[0], e[1], e[2], e[3]); }
-    __device__ __forceinline__ static float gelu(float x) { return (0.5f * x) * (1.0f + erff(x * 0.70710678118654752440f)); }
+    __device__ __forceinline__ static float gelu(float x) { return fth::gelu_erf(x); }
     // tanh-form GELU as x * sigmoid(2u), u = sqrt(2/pi) (x + 0.044715 x^3): 0.5 (1 + tanh u) = 1 / (1 + e^-2u). One
     // hardware exp2 and one division; e^-2u overflowing to inf gives x / inf = -0 where the tanh form gives -0 too.
     __device__ __forceinline__ static float gelu_tanh(float x) {

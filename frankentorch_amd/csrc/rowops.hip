@@ -1,15 +1,16 @@
 // Memory-bound row kernels for gfx950: last-dim softmax, LayerNorm, add+LayerNorm, RMSNorm,
 // erf-GELU, add, bias add, bias+residual add.
 //
-// Shape of every row kernel: one, two or four 64-lane wavefronts of a 256-thread block own one
-// row (the fewest that keep a lane at <= 4 vectors; up to 16 vectors per lane for rows of up to
-// 16 Ki elements), pull it from HBM once with 128-bit loads into registers, reduce with a fixed
-// xor-butterfly over the wavefront and a fixed left-to-right fold over the row's wavefronts, and
-// write the row back once with 128-bit non-temporal stores. No atomics anywhere: the reduction
-// tree is a function of (row length, kernel variant) only, so repeated runs are bitwise
-// identical. Rows whose base is not 16-byte aligned, whose length is not a multiple of the
-// vector width, or which do not fit the register budget take a block-per-row streaming variant
-// with the same fixed trees.
+// Shape of every row kernel: the fewest 64-lane wavefronts (1, 2, 4, 8 or 16) that keep a lane at
+// four 128-bit vectors or fewer own one row (rows beyond 16 Ki elements grow the per-lane count to
+// 8 or 16 vectors), pull it from HBM once with non-temporal 128-bit loads into registers, reduce
+// with a fixed xor-butterfly over the wavefront and a fixed left-to-right fold over the row's
+// wavefronts (one barrier per reduction, through alternating LDS halves), and write the row back
+// once with non-temporal 128-bit stores. Elementwise kernels and the bias kernels hold one vector
+// per thread. No atomics anywhere: the reduction tree is a function of (row length, kernel variant)
+// only, so repeated runs are bitwise identical. Rows whose base is not 16-byte aligned, whose
+// length is not a multiple of the vector width, or which do not fit the register budget take a
+// block-per-row streaming variant with the same fixed trees.
 //
 // Arithmetic follows crates/ft-kernel-cpu/src/lib.rs step for step (separate multiplies and adds;
 // this file is compiled with -ffp-contract=off): softmax :39219-39229, LayerNorm :5886-5909,
@@ -21,21 +22,23 @@
 #include <initializer_list>
 
 #include "common.hpp"
+#include "devmath.hpp"
 
 namespace {
 
 constexpr int kWave = 64;
 constexpr int kBlock = 256;
 
-// Streaming stores carry the non-temporal hint: an output is written once and not re-read by the
-// kernel, so it should not displace the input (which a producer kernel may just have left in the
-// last-level cache) or the reusable gamma / beta / bias lines. Loads stay temporal: measured on
-// MI355X at fp32 [8192,4096], non-temporal loads cost 8-10 % on every kernel, non-temporal stores
-// gain 2-25 %.
+// Streamed rows carry the non-temporal hint in both directions: a row is read once and written
+// once, so it should not displace the reusable gamma / beta / bias lines. Measured on MI355X at
+// fp32 [8192,4096] with every launch on a different buffer set (so that nothing is served from the
+// 256 MB last-level cache): non-temporal loads gain 2-8 %, non-temporal stores 2-25 %. (Relaunching
+// on ONE buffer set shows the opposite for loads, because the temporal loads then hit lines their
+// own previous launch left in that cache.)
 typedef float nat_f4 __attribute__((ext_vector_type(4)));
 typedef double nat_d2 __attribute__((ext_vector_type(2)));
 #ifndef FTH_NT_LOAD
-#define FTH_NT_LOAD 0
+#define FTH_NT_LOAD 1
 #endif
 #ifndef FTH_NT_STORE
 #define FTH_NT_STORE 1
@@ -98,9 +101,7 @@ __device__ __forceinline__ float dev_sqrt(float x) { return sqrtf(x); }
 __device__ __forceinline__ double dev_sqrt(double x) { return sqrt(x); }
 __device__ __forceinline__ float dev_max(float a, float b) { return fmaxf(a, b); }
 __device__ __forceinline__ double dev_max(double a, double b) { return fmax(a, b); }
-__device__ __forceinline__ float dev_gelu(float x) {
-    return (0.5f * x) * (1.0f + erff(x * 0.70710678118654752440f));
-}
+__device__ __forceinline__ float dev_gelu(float x) { return fth::gelu_erf(x); }
 __device__ __forceinline__ double dev_gelu(double x) {
     return (0.5 * x) * (1.0 + erf(x * 0.70710678118654752440));
 }
@@ -132,23 +133,46 @@ template <typename T, class F> __device__ __forceinline__ T wave_reduce(T v, F f
     return v;
 }
 
-// Reduction over the WPR wavefronts that share a row (WPR == 1: the wavefront alone; WPR == 2 or
-// 4: the row's wavefronts inside the 256-thread block, folded left to right through LDS). Every
-// thread of the block reaches the barriers (blocks with WPR > 1 never exit early).
+// Threads of the block that runs rows shared by WPR wavefronts: 256 (4 / WPR rows per block) up to
+// WPR = 4, one row per block of 64 * WPR threads beyond.
+template <int WPR> struct RowBlock {
+    static constexpr int kThreads = WPR <= 4 ? kBlock : kWave * WPR;
+    static constexpr int kRows = kThreads / (kWave * WPR);
+    // A compute unit holds 2048 threads (8 wavefronts per SIMD) at up to 64 vector registers per
+    // lane, 1024 at up to 128 and 512 at up to 256. `sets` counts the row-sized register sets the
+    // kernel keeps (row, prefetched row, gamma, beta, second operand); a set is 4 * vpl registers.
+    static constexpr int min_blocks(int vpl, int sets) {
+        const int regs = 4 * vpl * sets + 40;
+        const int threads = regs <= 64 ? 2048 : regs <= 128 ? 1024 : 512;
+        return threads / kThreads > 0 ? threads / kThreads : 1;
+    }
+};
+constexpr int kMaxWaves = 16;
+// Rows of up to this many vectors per lane keep gamma / beta in registers; longer ones fetch them
+// from cache at use.
+constexpr int kHoistVpl = 2;
+
+// Reduction over the WPR wavefronts that share a row (WPR == 1: the wavefront alone; otherwise the
+// row's wavefronts inside the block, folded left to right through LDS). `smem` holds 2 * kMaxWaves
+// values and consecutive calls alternate between its halves (`phase`), so one barrier per call is
+// enough: a wavefront can only reach the write of call n + 2 after the barrier of call n + 1, which
+// every wavefront reaches only after its reads of call n. Every thread of the block reaches the
+// barriers (blocks with WPR > 1 never exit early).
 template <int WPR, typename T, class F>
-__device__ __forceinline__ T group_reduce(T v, F f, T *smem) {
+__device__ __forceinline__ T group_reduce(T v, F f, T *smem, int &phase) {
     v = wave_reduce(v, f);
     if constexpr (WPR == 1) {
         return v;
     } else {
         const int wave = threadIdx.x / kWave;
         const int first = (wave / WPR) * WPR;
+        T *buf = smem + phase * kMaxWaves;
+        phase ^= 1;
+        if ((threadIdx.x & (kWave - 1)) == 0) buf[wave] = v;
         __syncthreads();
-        if ((threadIdx.x & (kWave - 1)) == 0) smem[wave] = v;
-        __syncthreads();
-        T r = smem[first];
+        T r = buf[first];
 #pragma unroll
-        for (int w = 1; w < WPR; ++w) r = f(r, smem[first + w]);
+        for (int w = 1; w < WPR; ++w) r = f(r, buf[first + w]);
         return r;
     }
 }
@@ -184,6 +208,20 @@ template <typename T, int VPL, int WPR> struct RowRegs {
             }
         }
     }
+    // Same lane layout, ordinary (cacheable) loads: for the per-column vectors every row re-reads.
+    __device__ __forceinline__ void load_cached(const T *vec, int nvec, T fill) {
+        const V *p = reinterpret_cast<const V *>(vec);
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            int v = lane() + i * kLanes;
+            if (v < nvec) {
+                unpack(p[v], e[i]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < EPV; ++j) e[i][j] = fill;
+            }
+        }
+    }
     __device__ __forceinline__ static void unpack(const float4 &v, float *o) {
         o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
     }
@@ -205,178 +243,235 @@ template <typename T, int VPL, int WPR> struct RowRegs {
     }
 };
 
-// A 256-thread block holds 4 / WPR rows.
-template <int WPR> __device__ __forceinline__ int64_t row_of_block() {
-    return (int64_t)blockIdx.x * (kBlock / (kWave * WPR)) + threadIdx.x / (kWave * WPR);
-}
-// Rows past the end are clamped (so every wavefront still reaches the block barriers) and their
-// stores are suppressed by passing nvec_store == 0.
-#define FTH_ROW_PROLOGUE(WPR_)                                  \
-    int64_t row = row_of_block<WPR_>();                         \
-    const bool row_live = row < rows;                           \
-    if constexpr (WPR_ == 1) {                                  \
-        if (!row_live) return;                                  \
-    } else {                                                    \
-        if (!row_live) row = rows - 1;                          \
-    }
+// The rows of one row group (the WPR wavefronts that share a row). Group g of G takes rows g, g + G,
+// g + 2 G, ... for `iters` turns, the same count in every group so that all wavefronts of a block
+// meet at the same barriers; a turn past the last row works on a clamped copy of it and stores
+// nothing. Neighbouring groups are on neighbouring rows at any time, and a group keeps its
+// per-column vectors (gamma, beta) in registers across its rows: with one row per block those
+// vectors, 32 KiB per fp32 row of 4096, crossed the L2 -> L1 path once per row, twice the volume
+// of the row itself, and LayerNorm ran at 0.63 of the HBM peak against 0.77 without them.
+template <int WPR> struct RowWalk {
+    int64_t row, stride, last;
+    __device__ __forceinline__ RowWalk(int64_t rows)
+        : row((int64_t)blockIdx.x * RowBlock<WPR>::kRows + threadIdx.x / (kWave * WPR)),
+          stride((int64_t)gridDim.x * RowBlock<WPR>::kRows), last(rows - 1) {}
+    __device__ __forceinline__ int64_t clamped(int64_t r) const { return r < last ? r : last; }
+    __device__ __forceinline__ bool live() const { return row <= last; }
+};
+// The next row is requested before the current one is reduced when a second register set fits.
+template <int VPL> constexpr bool kPrefetch = VPL <= 4;
 
 // ---- softmax ------------------------------------------------------------------------------
 template <typename T, int VPL, int WPR>
-__global__ __launch_bounds__(kBlock) void softmax_row_kernel(const T *__restrict__ x, T *__restrict__ y,
-                                                             int64_t rows, int cols) {
-    __shared__ T smem[4];
+__global__ __launch_bounds__(RowBlock<WPR>::kThreads, RowBlock<WPR>::min_blocks(VPL, 2)) void softmax_row_kernel(
+    const T *__restrict__ x, T *__restrict__ y, int64_t rows, int cols, int iters) {
+    __shared__ T smem[2 * kMaxWaves];
+    int phase = 0;
     using R = RowRegs<T, VPL, WPR>;
-    FTH_ROW_PROLOGUE(WPR)
     const int nvec = cols / R::EPV;
-    R r;
-    r.load(x + row * cols, nvec, neg_inf<T>());
-    T m = neg_inf<T>();
+    RowWalk<WPR> walk(rows);
+    R r, nxt;
+    r.load(x + walk.clamped(walk.row) * cols, nvec, neg_inf<T>());
+    for (int it = 0; it < iters; ++it) {
+        if constexpr (kPrefetch<VPL>) {
+            if (it + 1 < iters) nxt.load(x + walk.clamped(walk.row + walk.stride) * cols, nvec, neg_inf<T>());
+        }
+        T m = neg_inf<T>();
 #pragma unroll
-    for (int i = 0; i < VPL; ++i)
+        for (int i = 0; i < VPL; ++i)
 #pragma unroll
-        for (int j = 0; j < R::EPV; ++j) m = dev_max(m, r.e[i][j]);
-    m = group_reduce<WPR>(m, MaxOp{}, smem);
-    T s = 0;
+            for (int j = 0; j < R::EPV; ++j) m = dev_max(m, r.e[i][j]);
+        m = group_reduce<WPR>(m, MaxOp{}, smem, phase);
+        T s = 0;
 #pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-        const bool live = (R::lane() + i * R::kLanes) < nvec;
+        for (int i = 0; i < VPL; ++i) {
+            const bool live = (R::lane() + i * R::kLanes) < nvec;
 #pragma unroll
-        for (int j = 0; j < R::EPV; ++j) {
-            // Padding slots must stay out of the sum even when m is -inf or NaN.
-            T ev = live ? dev_exp(r.e[i][j] - m) : T(0);
-            r.e[i][j] = ev;
-            s += ev;
+            for (int j = 0; j < R::EPV; ++j) {
+                // Padding slots must stay out of the sum even when m is -inf or NaN.
+                T ev = live ? dev_exp(r.e[i][j] - m) : T(0);
+                r.e[i][j] = ev;
+                s += ev;
+            }
+        }
+        s = group_reduce<WPR>(s, SumOp{}, smem, phase);
+        // One correctly rounded 1 / s per row, then a multiply per element (the reference divides each
+        // element: the two differ by at most one rounding, far inside the parity tolerance, and the
+        // per-element IEEE division sequence would make this kernel ALU-bound).
+        const T inv = T(1) / s;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i)
+#pragma unroll
+            for (int j = 0; j < R::EPV; ++j) r.e[i][j] = r.e[i][j] * inv;
+        r.store(y + walk.clamped(walk.row) * cols, walk.live() ? nvec : 0);
+        walk.row += walk.stride;
+        if (it + 1 < iters) {
+            if constexpr (kPrefetch<VPL>) r = nxt;
+            else r.load(x + walk.clamped(walk.row) * cols, nvec, neg_inf<T>());
         }
     }
-    s = group_reduce<WPR>(s, SumOp{}, smem);
-    // One correctly rounded 1 / s per row, then a multiply per element (the reference divides each
-    // element: the two differ by at most one rounding, far inside the parity tolerance, and the
-    // per-element IEEE division sequence would make this kernel ALU-bound).
-    const T inv = T(1) / s;
-#pragma unroll
-    for (int i = 0; i < VPL; ++i)
-#pragma unroll
-        for (int j = 0; j < R::EPV; ++j) r.e[i][j] = r.e[i][j] * inv;
-    r.store(y + row * cols, row_live ? nvec : 0);
 }
 
 // ---- LayerNorm / add+LayerNorm ---------------------------------------------------------------
 template <typename T, int VPL, int WPR, bool ADD>
-__global__ __launch_bounds__(kBlock) void layernorm_row_kernel(const T *__restrict__ x, const T *__restrict__ x2,
-                                                               const T *__restrict__ w, const T *__restrict__ b,
-                                                               T *__restrict__ y, int64_t rows, int cols, T eps) {
-    __shared__ T smem[4];
+__global__ __launch_bounds__(RowBlock<WPR>::kThreads, RowBlock<WPR>::min_blocks(VPL, ADD ? 5 : 4)) void layernorm_row_kernel(
+    const T *__restrict__ x, const T *__restrict__ x2, const T *__restrict__ w, const T *__restrict__ b, T *__restrict__ y,
+    int64_t rows, int cols, T eps, int iters) {
+    __shared__ T smem[2 * kMaxWaves];
+    int phase = 0;
     using R = RowRegs<T, VPL, WPR>;
-    FTH_ROW_PROLOGUE(WPR)
     const int nvec = cols / R::EPV;
-    R r;
-    r.load(x + row * cols, nvec, T(0));
-    if constexpr (ADD) {
-        R r2;
-        r2.load(x2 + row * cols, nvec, T(0));
+    RowWalk<WPR> walk(rows);
+    const T inv_n = T(1) / (T)cols;
+    R rw, rb;  // gamma / beta of this lane's columns, kept for every row of the group
+    if constexpr (VPL <= kHoistVpl) {
+        if (w) rw.load_cached(w, nvec, T(1));
+        if (b) rb.load_cached(b, nvec, T(0));
+    }
+    R r, nxt, nxt2;
+    if constexpr (kPrefetch<VPL>) {
+        r.load(x + walk.clamped(walk.row) * cols, nvec, T(0));
+        if constexpr (ADD) nxt2.load(x2 + walk.clamped(walk.row) * cols, nvec, T(0));
+    }
+    for (int it = 0; it < iters; ++it) {
+        if constexpr (!kPrefetch<VPL>) {
+            r.load(x + walk.clamped(walk.row) * cols, nvec, T(0));
+            if constexpr (ADD) nxt2.load(x2 + walk.clamped(walk.row) * cols, nvec, T(0));
+        }
+        if constexpr (ADD) {
+#pragma unroll
+            for (int i = 0; i < VPL; ++i)
+#pragma unroll
+                for (int j = 0; j < R::EPV; ++j) r.e[i][j] = r.e[i][j] + nxt2.e[i][j];
+        }
+        if constexpr (kPrefetch<VPL>) {
+            if (it + 1 < iters) {
+                nxt.load(x + walk.clamped(walk.row + walk.stride) * cols, nvec, T(0));
+                if constexpr (ADD) nxt2.load(x2 + walk.clamped(walk.row + walk.stride) * cols, nvec, T(0));
+            }
+        }
+        T sum = 0;
 #pragma unroll
         for (int i = 0; i < VPL; ++i)
 #pragma unroll
-            for (int j = 0; j < R::EPV; ++j) r.e[i][j] = r.e[i][j] + r2.e[i][j];
-    }
-    const T inv_n = T(1) / (T)cols;
-    T sum = 0;
+            for (int j = 0; j < R::EPV; ++j) sum += r.e[i][j];
+        sum = group_reduce<WPR>(sum, SumOp{}, smem, phase);
+        const T mean = sum * inv_n;
+        T vsum = 0;
 #pragma unroll
-    for (int i = 0; i < VPL; ++i)
-#pragma unroll
-        for (int j = 0; j < R::EPV; ++j) sum += r.e[i][j];
-    sum = group_reduce<WPR>(sum, SumOp{}, smem);
-    const T mean = sum * inv_n;
-    T vsum = 0;
-#pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-        const bool live = (R::lane() + i * R::kLanes) < nvec;
-#pragma unroll
-        for (int j = 0; j < R::EPV; ++j) {
-            T d = r.e[i][j] - mean;
-            vsum += live ? d * d : T(0);
-        }
-    }
-    vsum = group_reduce<WPR>(vsum, SumOp{}, smem);
-    const T rstd = T(1) / dev_sqrt(vsum * inv_n + eps);
-#pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-        const int v = R::lane() + i * R::kLanes;
-        if (v < nvec) {
-            T wv[R::EPV], bv[R::EPV];
-            if (w) R::load_vec(w, v, wv);
-            if (b) R::load_vec(b, v, bv);
+        for (int i = 0; i < VPL; ++i) {
+            const bool live = (R::lane() + i * R::kLanes) < nvec;
 #pragma unroll
             for (int j = 0; j < R::EPV; ++j) {
-                T o = (r.e[i][j] - mean) * rstd;
-                if (w) o = o * wv[j];
-                if (b) o = o + bv[j];
-                r.e[i][j] = o;
+                T d = r.e[i][j] - mean;
+                vsum += live ? d * d : T(0);
             }
         }
+        vsum = group_reduce<WPR>(vsum, SumOp{}, smem, phase);
+        const T rstd = T(1) / dev_sqrt(vsum * inv_n + eps);
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const int v = R::lane() + i * R::kLanes;
+            if (v < nvec) {
+                T wv[R::EPV], bv[R::EPV];
+                if constexpr (VPL > kHoistVpl) {
+                    if (w) R::load_vec(w, v, wv);
+                    if (b) R::load_vec(b, v, bv);
+                }
+#pragma unroll
+                for (int j = 0; j < R::EPV; ++j) {
+                    T o = (r.e[i][j] - mean) * rstd;
+                    if (w) o = o * (VPL <= kHoistVpl ? rw.e[i][j] : wv[j]);
+                    if (b) o = o + (VPL <= kHoistVpl ? rb.e[i][j] : bv[j]);
+                    r.e[i][j] = o;
+                }
+            }
+        }
+        r.store(y + walk.clamped(walk.row) * cols, walk.live() ? nvec : 0);
+        walk.row += walk.stride;
+        if constexpr (kPrefetch<VPL>) {
+            if (it + 1 < iters) r = nxt;
+        }
     }
-    r.store(y + row * cols, row_live ? nvec : 0);
 }
 
 // ---- RMSNorm ---------------------------------------------------------------------------------
 template <typename T, int VPL, int WPR>
-__global__ __launch_bounds__(kBlock) void rmsnorm_row_kernel(const T *__restrict__ x, const T *__restrict__ w,
-                                                             T *__restrict__ y, int64_t rows, int cols, T eps) {
-    __shared__ T smem[4];
+__global__ __launch_bounds__(RowBlock<WPR>::kThreads, RowBlock<WPR>::min_blocks(VPL, 3)) void rmsnorm_row_kernel(
+    const T *__restrict__ x, const T *__restrict__ w, T *__restrict__ y, int64_t rows, int cols, T eps, int iters) {
+    __shared__ T smem[2 * kMaxWaves];
+    int phase = 0;
     using R = RowRegs<T, VPL, WPR>;
-    FTH_ROW_PROLOGUE(WPR)
     const int nvec = cols / R::EPV;
-    R r;
-    r.load(x + row * cols, nvec, T(0));
+    RowWalk<WPR> walk(rows);
     const T inv_n = T(1) / (T)cols;
-    T ss = 0;
+    R rw;
+    if constexpr (VPL <= kHoistVpl) {
+        if (w) rw.load_cached(w, nvec, T(1));
+    }
+    R r, nxt;
+    r.load(x + walk.clamped(walk.row) * cols, nvec, T(0));
+    for (int it = 0; it < iters; ++it) {
+        if constexpr (kPrefetch<VPL>) {
+            if (it + 1 < iters) nxt.load(x + walk.clamped(walk.row + walk.stride) * cols, nvec, T(0));
+        }
+        T ss = 0;
 #pragma unroll
-    for (int i = 0; i < VPL; ++i)
+        for (int i = 0; i < VPL; ++i)
 #pragma unroll
-        for (int j = 0; j < R::EPV; ++j) ss += r.e[i][j] * r.e[i][j];
-    ss = group_reduce<WPR>(ss, SumOp{}, smem);
-    const T rstd = T(1) / dev_sqrt(ss * inv_n + eps);
+            for (int j = 0; j < R::EPV; ++j) ss += r.e[i][j] * r.e[i][j];
+        ss = group_reduce<WPR>(ss, SumOp{}, smem, phase);
+        const T rstd = T(1) / dev_sqrt(ss * inv_n + eps);
 #pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-        const int v = R::lane() + i * R::kLanes;
-        if (v < nvec) {
-            T wv[R::EPV];
-            if (w) R::load_vec(w, v, wv);
+        for (int i = 0; i < VPL; ++i) {
+            const int v = R::lane() + i * R::kLanes;
+            if (v < nvec) {
+                T wv[R::EPV];
+                if constexpr (VPL > kHoistVpl) {
+                    if (w) R::load_vec(w, v, wv);
+                }
 #pragma unroll
-            for (int j = 0; j < R::EPV; ++j) {
-                T o = r.e[i][j] * rstd;
-                if (w) o = o * wv[j];
-                r.e[i][j] = o;
+                for (int j = 0; j < R::EPV; ++j) {
+                    T o = r.e[i][j] * rstd;
+                    if (w) o = o * (VPL <= kHoistVpl ? rw.e[i][j] : wv[j]);
+                    r.e[i][j] = o;
+                }
             }
         }
+        r.store(y + walk.clamped(walk.row) * cols, walk.live() ? nvec : 0);
+        walk.row += walk.stride;
+        if (it + 1 < iters) {
+            if constexpr (kPrefetch<VPL>) r = nxt;
+            else r.load(x + walk.clamped(walk.row) * cols, nvec, T(0));
+        }
     }
-    r.store(y + row * cols, row_live ? nvec : 0);
 }
 
 // ---------------------------------------------------------------------------------------------
 // Streaming variants: one 256-thread block per row, scalar loads, the row is re-read from L2.
 // ---------------------------------------------------------------------------------------------
 template <typename T, class F>
-__device__ __forceinline__ T block_reduce(T v, F f, T *smem) {
-    return group_reduce<4>(v, f, smem);
+__device__ __forceinline__ T block_reduce(T v, F f, T *smem, int &phase) {
+    return group_reduce<4>(v, f, smem, phase);
 }
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void softmax_stream_kernel(const T *__restrict__ x, T *__restrict__ y,
                                                                 int64_t rows, int64_t cols) {
-    __shared__ T smem[4];
+    __shared__ T smem[2 * kMaxWaves];
+    int phase = 0;
     const T *xr = x + (int64_t)blockIdx.x * cols;
     T *yr = y + (int64_t)blockIdx.x * cols;
     T m = neg_inf<T>();
     for (int64_t j = threadIdx.x; j < cols; j += kBlock) m = dev_max(m, xr[j]);
-    m = block_reduce(m, MaxOp{}, smem);
+    m = block_reduce(m, MaxOp{}, smem, phase);
     T s = 0;
     for (int64_t j = threadIdx.x; j < cols; j += kBlock) {
         T ev = dev_exp(xr[j] - m);
         yr[j] = ev;
         s += ev;
     }
-    s = block_reduce(s, SumOp{}, smem);
+    s = block_reduce(s, SumOp{}, smem, phase);
     for (int64_t j = threadIdx.x; j < cols; j += kBlock) yr[j] = yr[j] / s;
 }
 
@@ -407,7 +502,8 @@ __global__ __launch_bounds__(kBlock) void layernorm_stream_kernel(const T *__res
                                                                   const T *__restrict__ w, const T *__restrict__ b,
                                                                   T *__restrict__ y, int64_t rows, int64_t cols,
                                                                   T eps) {
-    __shared__ T smem[4];
+    __shared__ T smem[2 * kMaxWaves];
+    int phase = 0;
     const T *xr = x + (int64_t)blockIdx.x * cols;
     const T *x2r = ADD ? x2 + (int64_t)blockIdx.x * cols : nullptr;
     T *yr = y + (int64_t)blockIdx.x * cols;
@@ -421,7 +517,7 @@ __global__ __launch_bounds__(kBlock) void layernorm_stream_kernel(const T *__res
         }
         sum += v;
     }
-    sum = block_reduce(sum, SumOp{}, smem);
+    sum = block_reduce(sum, SumOp{}, smem, phase);
     const T mean = sum * inv_n;
     const T *src = ADD ? yr : xr;
     T vsum = 0;
@@ -429,7 +525,7 @@ __global__ __launch_bounds__(kBlock) void layernorm_stream_kernel(const T *__res
         T d = src[j] - mean;
         vsum += d * d;
     }
-    vsum = block_reduce(vsum, SumOp{}, smem);
+    vsum = block_reduce(vsum, SumOp{}, smem, phase);
     const T rstd = T(1) / dev_sqrt(vsum * inv_n + eps);
     for (int64_t j = threadIdx.x; j < cols; j += kBlock) {
         T o = (src[j] - mean) * rstd;
@@ -442,13 +538,14 @@ __global__ __launch_bounds__(kBlock) void layernorm_stream_kernel(const T *__res
 template <typename T>
 __global__ __launch_bounds__(kBlock) void rmsnorm_stream_kernel(const T *__restrict__ x, const T *__restrict__ w,
                                                                 T *__restrict__ y, int64_t rows, int64_t cols, T eps) {
-    __shared__ T smem[4];
+    __shared__ T smem[2 * kMaxWaves];
+    int phase = 0;
     const T *xr = x + (int64_t)blockIdx.x * cols;
     T *yr = y + (int64_t)blockIdx.x * cols;
     const T inv_n = T(1) / (T)cols;
     T ss = 0;
     for (int64_t j = threadIdx.x; j < cols; j += kBlock) ss += xr[j] * xr[j];
-    ss = block_reduce(ss, SumOp{}, smem);
+    ss = block_reduce(ss, SumOp{}, smem, phase);
     const T rstd = T(1) / dev_sqrt(ss * inv_n + eps);
     for (int64_t j = threadIdx.x; j < cols; j += kBlock) {
         T o = xr[j] * rstd;
@@ -462,26 +559,25 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_stream_kernel(const T *__restr
 // all before the first use, and a scalar tail covers what is left.
 // ---------------------------------------------------------------------------------------------
 enum class Ew { Gelu, Add, GeluTanh };
-constexpr int kUnr = 4;
 
-template <typename T, Ew OP>
-__global__ __launch_bounds__(kBlock) void elementwise_vec_kernel(const T *__restrict__ a, const T *__restrict__ b,
-                                                                 T *__restrict__ y, int64_t nvec) {
+template <typename T, Ew OP, int UNR, int BT>
+__global__ __launch_bounds__(BT) void elementwise_vec_kernel(const T *__restrict__ a, const T *__restrict__ b,
+                                                             T *__restrict__ y, int64_t nvec) {
     using R = RowRegs<T, 1, 1>;
     using V = typename Vec128<T>::type;
-    const int64_t base = (int64_t)blockIdx.x * (kBlock * kUnr) + threadIdx.x;
-    V va[kUnr], vb[kUnr];
+    const int64_t base = (int64_t)blockIdx.x * (BT * UNR) + threadIdx.x;
+    V va[UNR], vb[UNR];
 #pragma unroll
-    for (int u = 0; u < kUnr; ++u) {
-        int64_t v = base + (int64_t)u * kBlock;
+    for (int u = 0; u < UNR; ++u) {
+        int64_t v = base + (int64_t)u * BT;
         if (v < nvec) {
             va[u] = stream_load(reinterpret_cast<const V *>(a) + v);
             if constexpr (OP == Ew::Add) vb[u] = stream_load(reinterpret_cast<const V *>(b) + v);
         }
     }
 #pragma unroll
-    for (int u = 0; u < kUnr; ++u) {
-        int64_t v = base + (int64_t)u * kBlock;
+    for (int u = 0; u < UNR; ++u) {
+        int64_t v = base + (int64_t)u * BT;
         if (v < nvec) {
             T ea[R::EPV], eb[R::EPV];
             R::unpack(va[u], ea);
@@ -508,49 +604,31 @@ __global__ __launch_bounds__(kBlock) void elementwise_scalar_kernel(const T *__r
 }
 
 // ---- bias add / bias + residual add: y[r, j] = (x[r, j] + bias[j]) (+ res[r, j]) --------------
-// One wavefront per row so the bias index is the vector index (no division).
-template <typename T, bool RES>
-__global__ __launch_bounds__(kBlock) void bias_row_kernel(const T *x, const T *__restrict__ bias,
-                                                          const T *res, T *y, int64_t rows, int cols) {
+// One 128-bit vector per thread over the flattened tensor; the bias vector is the vector index
+// modulo the vectors of a row (the bias stays in cache).
+template <typename T, bool RES, int BT>
+__global__ __launch_bounds__(BT) void bias_flat_kernel(const T *x, const T *__restrict__ bias, const T *res, T *y,
+                                                       int64_t total_vec, int row_vec) {
     using R = RowRegs<T, 1, 1>;
     using V = typename Vec128<T>::type;
-    const int64_t row = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
-    if (row >= rows) return;
-    const int lane = threadIdx.x & (kWave - 1);
-    const int nvec = cols / R::EPV;
-    const V *xr = reinterpret_cast<const V *>(x + row * cols);
-    const V *rr = RES ? reinterpret_cast<const V *>(res + row * cols) : nullptr;
-    const V *br = reinterpret_cast<const V *>(bias);
-    V *yr = reinterpret_cast<V *>(y + row * cols);
-    for (int v0 = lane; v0 < nvec; v0 += kWave * kUnr) {
-        V vx[kUnr], vr[kUnr], vb[kUnr];
+    const int64_t v = (int64_t)blockIdx.x * BT + threadIdx.x;
+    if (v >= total_vec) return;
+    const int bv = (int)(v % row_vec);
+    const V vx = stream_load(reinterpret_cast<const V *>(x) + v);
+    const V vb = reinterpret_cast<const V *>(bias)[bv];
+    V vr;
+    if constexpr (RES) vr = stream_load(reinterpret_cast<const V *>(res) + v);
+    T ex[R::EPV], eb[R::EPV], er[R::EPV];
+    R::unpack(vx, ex);
+    R::unpack(vb, eb);
+    if constexpr (RES) R::unpack(vr, er);
 #pragma unroll
-        for (int u = 0; u < kUnr; ++u) {
-            int v = v0 + u * kWave;
-            if (v < nvec) {
-                vx[u] = stream_load(xr + v);
-                vb[u] = br[v];
-                if constexpr (RES) vr[u] = stream_load(rr + v);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < kUnr; ++u) {
-            int v = v0 + u * kWave;
-            if (v < nvec) {
-                T ex[R::EPV], eb[R::EPV], er[R::EPV];
-                R::unpack(vx[u], ex);
-                R::unpack(vb[u], eb);
-                if constexpr (RES) R::unpack(vr[u], er);
-#pragma unroll
-                for (int j = 0; j < R::EPV; ++j) {
-                    T o = ex[j] + eb[j];
-                    if constexpr (RES) o = o + er[j];
-                    ex[j] = o;
-                }
-                stream_store(yr + v, R::pack(ex));
-            }
-        }
+    for (int j = 0; j < R::EPV; ++j) {
+        T o = ex[j] + eb[j];
+        if constexpr (RES) o = o + er[j];
+        ex[j] = o;
     }
+    stream_store(reinterpret_cast<V *>(y) + v, R::pack(ex));
 }
 
 template <typename T, bool RES>
@@ -570,58 +648,74 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 constexpr int64_t kMaxGrid = 2147483647LL;
 
-// Picks (VPL, WPR) for a register-resident row of `nvec` vectors, or returns false.
-// Few vectors per lane and more wavefronts per row measured best on MI355X (fp32 [8192,4096]:
-// LayerNorm 74 % of HBM peak with 16 vectors x 1 wavefront, 85 % with 4 x 4), so the row is spread
-// over the fewest wavefronts that keep a lane at <= 4 vectors, and only longer rows grow the
-// per-lane count. `max_vpl` caps the vectors a lane may hold.
+// Picks (VPL, WPR) for a register-resident row of `nvec` vectors, or returns false. Measured on
+// MI355X over rotating buffers (rows x cols = 32 Mi fp32 elements): a row streams fastest from the
+// fewest wavefronts that keep a lane at 4 vectors or fewer -- 768 and 1024 columns on one wavefront
+// (0.75 of the HBM peak; 0.70 on two, 0.57 on four), 2048 on two, 4096 on four, 8192 and 16384 on
+// eight with 4 and 8 vectors per lane. Sixteen wavefronts (one 1024-thread block per row) lose
+// everywhere below 8192 columns. `max_vpl` caps the vectors a lane may hold.
 inline bool pick_row_shape(int64_t nvec, int max_vpl, int &vpl, int &wpr) {
-    if (nvec <= 0 || nvec > 256 * (int64_t)max_vpl) return false;
+    if (nvec <= 0 || nvec > 64 * kMaxWaves * (int64_t)max_vpl) return false;
     static const int forced = [] {
-        const char *e = std::getenv("FT_HIP_ROW_WPR");  // tuning knob: wavefronts per row (1, 2 or 4)
+        const char *e = std::getenv("FT_HIP_ROW_WPR");  // tuning knob: wavefronts per row (1, 2, 4, 8 or 16)
         return e ? std::atoi(e) : 0;
     }();
-    int w = nvec <= 64 * 4 ? 1 : nvec <= 128 * 4 ? 2 : 4;
-    if (forced == 1 || forced == 2 || forced == 4) {
+    int w = nvec <= 256 ? 1 : nvec <= 512 ? 2 : nvec <= 1024 ? 4 : nvec <= 4096 ? 8 : 16;
+    if (forced == 1 || forced == 2 || forced == 4 || forced == 8 || forced == 16) {
         if (fth::ceil_div(nvec, 64 * forced) <= max_vpl) w = forced;
     }
     const int64_t need = fth::ceil_div(nvec, 64 * w);
-    int v = need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : need <= 8 ? 8 : 16;
-    // instantiated shapes: WPR 1 x {1,2,4,8,16}, WPR 2 x {4,8,16}, WPR 4 x {2,4,8,16}
-    if (w == 2 && v < 4) v = 4;
-    if (w == 4 && v < 2) v = 2;
-    vpl = v;
+    if (w == 16 && need > 8) return false;  // 1024 threads leave a lane 128 registers: 8 vectors at most
+    vpl = need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : need <= 8 ? 8 : 16;
     wpr = w;
     return true;
 }
 
+#define FTH_ROW_DISPATCH_VPL(VPL_, W_, LAUNCH)           \
+    switch (VPL_) {                                      \
+        case 1: { LAUNCH(1, W_); } break;                \
+        case 2: { LAUNCH(2, W_); } break;                \
+        case 4: { LAUNCH(4, W_); } break;                \
+        case 8: { LAUNCH(8, W_); } break;                \
+        default: { LAUNCH(16, W_); } break;              \
+    }
 #define FTH_ROW_DISPATCH(VPL_, WPR_, LAUNCH)                         \
     do {                                                             \
-        if (WPR_ == 1) {                                             \
-            switch (VPL_) {                                          \
-                case 1: { LAUNCH(1, 1); } break;                     \
-                case 2: { LAUNCH(2, 1); } break;                     \
-                case 4: { LAUNCH(4, 1); } break;                     \
-                case 8: { LAUNCH(8, 1); } break;                     \
-                default: { LAUNCH(16, 1); } break;                   \
-            }                                                        \
-        } else if (WPR_ == 2) {                                      \
-            switch (VPL_) {                                          \
-                case 4: { LAUNCH(4, 2); } break;                     \
-                case 8: { LAUNCH(8, 2); } break;                     \
-                default: { LAUNCH(16, 2); } break;                   \
-            }                                                        \
-        } else {                                                     \
-            switch (VPL_) {                                          \
-                case 2: { LAUNCH(2, 4); } break;                     \
-                case 4: { LAUNCH(4, 4); } break;                     \
-                case 8: { LAUNCH(8, 4); } break;                     \
-                default: { LAUNCH(16, 4); } break;                   \
-            }                                                        \
+        switch (WPR_) {                                              \
+            case 1: FTH_ROW_DISPATCH_VPL(VPL_, 1, LAUNCH) break;     \
+            case 2: FTH_ROW_DISPATCH_VPL(VPL_, 2, LAUNCH) break;     \
+            case 4: FTH_ROW_DISPATCH_VPL(VPL_, 4, LAUNCH) break;     \
+            case 8: FTH_ROW_DISPATCH_VPL(VPL_, 8, LAUNCH) break;     \
+            default:                                                 \
+                switch (VPL_) {                                      \
+                    case 1: { LAUNCH(1, 16); } break;                \
+                    case 2: { LAUNCH(2, 16); } break;                \
+                    case 4: { LAUNCH(4, 16); } break;                \
+                    default: { LAUNCH(8, 16); } break;               \
+                }                                                    \
+                break;                                               \
         }                                                            \
     } while (0)
 
-inline int64_t row_grid(int64_t rows, int wpr) { return fth::ceil_div(rows, 4 / wpr); }
+inline int rows_per_block(int wpr) { return wpr <= 4 ? 4 / wpr : 1; }
+
+// Grid and turns per row group. One row per group is the default: walking several rows per group
+// (so that gamma / beta are fetched once per group) was measured at fp32 [8192,4096] over rotating
+// buffers and lost more streaming rate than the saved vector traffic gave back (softmax 0.76 ->
+// 0.72, RMSNorm 0.75 -> 0.74, LayerNorm 0.66 -> 0.68 of the HBM peak at 2 to 16 rows per group).
+inline void row_launch_shape(int64_t rows, int wpr, int64_t &grid, int &iters) {
+    static const int max_iters = [] {
+        const char *e = std::getenv("FT_HIP_ROW_ITERS");  // tuning knob: most rows one row group walks (1 = one row per group)
+        const int v = e ? std::atoi(e) : 1;
+        return v < 1 ? 1 : v;
+    }();
+    const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
+    const int64_t resident_groups = (int64_t)cus * (2048 / (kWave * wpr));
+    int64_t it = rows / resident_groups;
+    it = it < 1 ? 1 : it > max_iters ? max_iters : it;
+    grid = fth::ceil_div(fth::ceil_div(rows, it), rows_per_block(wpr));
+    iters = (int)fth::ceil_div(rows, grid * rows_per_block(wpr));
+}
 
 template <typename T>
 int32_t launch_softmax(const T *x, T *y, int64_t rows, int64_t cols, fth_stream s) {
@@ -631,10 +725,11 @@ int32_t launch_softmax(const T *x, T *y, int64_t rows, int64_t cols, fth_stream 
     FTH_ARG(x && y, "softmax: NULL operand");
     hipStream_t st = fth::resolve_stream(s);
     constexpr int EPV = Vec128<T>::n;
-    int vpl, wpr;
+    int vpl, wpr, iters = 1;
+    int64_t grid = 0;
     if (cols % EPV == 0 && aligned16(x) && aligned16(y) && pick_row_shape(cols / EPV, 16, vpl, wpr) &&
-        row_grid(rows, wpr) <= kMaxGrid) {
-#define L(V_, W_) softmax_row_kernel<T, V_, W_><<<dim3((unsigned)row_grid(rows, W_)), dim3(kBlock), 0, st>>>(x, y, rows, (int)cols)
+        (row_launch_shape(rows, wpr, grid, iters), grid <= kMaxGrid)) {
+#define L(V_, W_) softmax_row_kernel<T, V_, W_><<<dim3((unsigned)grid), dim3(RowBlock<W_>::kThreads), 0, st>>>(x, y, rows, (int)cols, iters)
         FTH_ROW_DISPATCH(vpl, wpr, L);
 #undef L
     } else {
@@ -668,11 +763,12 @@ int32_t launch_layernorm(const T *x, const T *x2, const T *w, const T *b, T *y, 
     FTH_ARG(x && y && (!ADD || x2), "layer_norm: NULL operand");
     hipStream_t st = fth::resolve_stream(s);
     constexpr int EPV = Vec128<T>::n;
-    int vpl, wpr;
+    int vpl, wpr, iters = 1;
+    int64_t grid = 0;
     bool vec_ok = cols % EPV == 0 && aligned16(x) && aligned16(y) && (!ADD || aligned16(x2)) &&
                   (!w || aligned16(w)) && (!b || aligned16(b));
-    if (vec_ok && pick_row_shape(cols / EPV, 16, vpl, wpr) && row_grid(rows, wpr) <= kMaxGrid) {
-#define L(V_, W_) layernorm_row_kernel<T, V_, W_, ADD><<<dim3((unsigned)row_grid(rows, W_)), dim3(kBlock), 0, st>>>(x, x2, w, b, y, rows, (int)cols, eps)
+    if (vec_ok && pick_row_shape(cols / EPV, ADD ? 8 : 16, vpl, wpr) && (row_launch_shape(rows, wpr, grid, iters), grid <= kMaxGrid)) {
+#define L(V_, W_) layernorm_row_kernel<T, V_, W_, ADD><<<dim3((unsigned)grid), dim3(RowBlock<W_>::kThreads), 0, st>>>(x, x2, w, b, y, rows, (int)cols, eps, iters)
         FTH_ROW_DISPATCH(vpl, wpr, L);
 #undef L
     } else {
@@ -691,10 +787,11 @@ int32_t launch_rmsnorm(const T *x, const T *w, T *y, int64_t rows, int64_t cols,
     FTH_ARG(x && y, "rms_norm: NULL operand");
     hipStream_t st = fth::resolve_stream(s);
     constexpr int EPV = Vec128<T>::n;
-    int vpl, wpr;
+    int vpl, wpr, iters = 1;
+    int64_t grid = 0;
     if (cols % EPV == 0 && aligned16(x) && aligned16(y) && (!w || aligned16(w)) &&
-        pick_row_shape(cols / EPV, 16, vpl, wpr) && row_grid(rows, wpr) <= kMaxGrid) {
-#define L(V_, W_) rmsnorm_row_kernel<T, V_, W_><<<dim3((unsigned)row_grid(rows, W_)), dim3(kBlock), 0, st>>>(x, w, y, rows, (int)cols, eps)
+        pick_row_shape(cols / EPV, 16, vpl, wpr) && (row_launch_shape(rows, wpr, grid, iters), grid <= kMaxGrid)) {
+#define L(V_, W_) rmsnorm_row_kernel<T, V_, W_><<<dim3((unsigned)grid), dim3(RowBlock<W_>::kThreads), 0, st>>>(x, w, y, rows, (int)cols, eps, iters)
         FTH_ROW_DISPATCH(vpl, wpr, L);
 #undef L
     } else {
@@ -717,9 +814,21 @@ int32_t launch_elementwise(const T *a, const T *b, T *y, int64_t n, fth_stream s
     if (aligned16(a) && aligned16(y) && (OP != Ew::Add || aligned16(b))) {
         int64_t nvec = n / EPV;
         if (nvec > 0) {
-            int64_t grid = fth::ceil_div(nvec, kBlock * kUnr);
+            static const int shape = [] {
+                const char *e = std::getenv("FT_HIP_EW_SHAPE");  // tuning knob: 100 * vectors per thread + block threads / 64
+                return e ? std::atoi(e) : 116;
+            }();
+            const int unr = shape / 100, bt = (shape % 100) * 64;
+            int64_t grid = fth::ceil_div(nvec, (int64_t)bt * unr);
             FTH_ARG(grid <= kMaxGrid, "elementwise: too long for one launch");
-            elementwise_vec_kernel<T, OP><<<dim3((unsigned)grid), dim3(kBlock), 0, st>>>(a, b, y, nvec);
+            if (unr == 4 && bt == 256) elementwise_vec_kernel<T, OP, 4, 256><<<dim3((unsigned)grid), dim3(256), 0, st>>>(a, b, y, nvec);
+            else if (unr == 1 && bt == 256) elementwise_vec_kernel<T, OP, 1, 256><<<dim3((unsigned)grid), dim3(256), 0, st>>>(a, b, y, nvec);
+            else if (unr == 2 && bt == 1024) elementwise_vec_kernel<T, OP, 2, 1024><<<dim3((unsigned)grid), dim3(1024), 0, st>>>(a, b, y, nvec);
+            else if (unr == 1 && bt == 512) elementwise_vec_kernel<T, OP, 1, 512><<<dim3((unsigned)grid), dim3(512), 0, st>>>(a, b, y, nvec);
+            else {
+                grid = fth::ceil_div(nvec, 1024);
+                elementwise_vec_kernel<T, OP, 1, 1024><<<dim3((unsigned)grid), dim3(1024), 0, st>>>(a, b, y, nvec);
+            }
             FTH_CHECK_LAUNCH("elementwise_vec");
         }
         done = nvec * EPV;
@@ -741,9 +850,17 @@ int32_t launch_bias(const T *x, const T *bias, const T *res, T *y, int64_t rows,
     FTH_ARG(x && bias && y && (!RES || res), "bias_add: NULL operand");
     hipStream_t st = fth::resolve_stream(s);
     constexpr int EPV = Vec128<T>::n;
-    if (cols % EPV == 0 && cols <= 2147483647LL && aligned16(x) && aligned16(bias) && aligned16(y) &&
-        (!RES || aligned16(res)) && fth::ceil_div(rows, 4) <= kMaxGrid) {
-        bias_row_kernel<T, RES><<<dim3((unsigned)fth::ceil_div(rows, 4)), dim3(kBlock), 0, st>>>(x, bias, res, y, rows, (int)cols);
+    int64_t total;
+    if (cols % EPV == 0 && cols <= 2147483647LL && aligned16(x) && aligned16(bias) && aligned16(y) && (!RES || aligned16(res)) &&
+        !__builtin_mul_overflow(rows, cols / EPV, &total) && fth::ceil_div(total, 256) <= kMaxGrid) {
+        static const int bt = [] {
+            const char *e = std::getenv("FT_HIP_BIAS_BLOCK");  // tuning knob: threads per block (256 or 1024)
+            return e ? std::atoi(e) : 1024;
+        }();
+        if (bt == 256)
+            bias_flat_kernel<T, RES, 256><<<dim3((unsigned)fth::ceil_div(total, 256)), dim3(256), 0, st>>>(x, bias, res, y, total, (int)(cols / EPV));
+        else
+            bias_flat_kernel<T, RES, 1024><<<dim3((unsigned)fth::ceil_div(total, 1024)), dim3(1024), 0, st>>>(x, bias, res, y, total, (int)(cols / EPV));
     } else {
         int64_t grid = fth::ceil_div(rows * cols, kBlock);
         FTH_ARG(grid <= kMaxGrid, "bias_add: too long for one launch");

@@ -121,6 +121,30 @@ def test_softmax_special_values(hip, oracle, vectors):
         assert bits[int(i)] == int(v, 16)
 
 
+def test_gelu_special_values_and_dense_accuracy(hip, oracle):
+    """The branch-free erf form against the checker (libm erff) on the values where the two could part: zeros, infinities,
+    NaN, the far tails (where 1 + erff is exactly 0 or 2), denormals; and its absolute error on a dense sweep of [-8, 8]
+    against erf in double precision (the documented bound is 4e-7; a 1-ulp erff is at 3e-7 there)."""
+    import math
+
+    x = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 6.0, -6.0, 5.7, -5.7, 1e-30, -1e-30, 1e-40, -1e-40, 3.0, -3.0, 0.5, -0.5],
+                 np.float32)
+    dx, dy = DeviceBuffer.from_host(x), DeviceBuffer(x.shape)
+    hip.gelu(dx, dy, x.size)
+    y, ref = dy.to_host(), oracle.gelu(x)
+    assert np.array_equal(np.isnan(y), np.isnan(ref))
+    fin = ~np.isnan(ref)
+    assert np.array_equal(np.isinf(y[fin]), np.isinf(ref[fin])) and np.array_equal(np.signbit(y[fin]), np.signbit(ref[fin]))
+    ok = fin & ~np.isinf(ref)
+    assert np.max(np.abs(y[ok].astype(np.float64) - ref[ok].astype(np.float64))) <= 5e-7
+    assert y[5] == 6.0 and y[6] == 0.0 and y[0] == 0.0
+    sweep = np.linspace(-8.0, 8.0, 1 << 20).astype(np.float32)
+    ds, do = DeviceBuffer.from_host(sweep), DeviceBuffer(sweep.shape)
+    hip.gelu(ds, do, sweep.size)
+    exact = 0.5 * sweep.astype(np.float64) * (1.0 + np.vectorize(math.erf)(sweep.astype(np.float64) / math.sqrt(2.0)))
+    assert np.max(np.abs(do.to_host().astype(np.float64) - exact)) <= 5e-7
+
+
 def test_empty_inputs_are_no_ops(hip):
     dx = DeviceBuffer((4,))
     hip.softmax_lastdim(dx, dx, 0, 4)
