@@ -349,27 +349,41 @@ def bench_backward(device, synth, steps, with_cpu):
     x = synth.normal(1, "x", (ROWS, COLS))
     dy = synth.normal(1, "dy", (ROWS, COLS))
     gamma = synth.uniform(1, "gamma", (COLS,), 0.5, 1.5)
-    dx_, ddy, dg = DeviceBuffer.from_host(x), DeviceBuffer.from_host(dy), DeviceBuffer.from_host(gamma)
-    gx, gw, gb = DeviceBuffer((ROWS, COLS)), DeviceBuffer((COLS,)), DeviceBuffer((COLS,))
-    ws = device.layer_norm_backward(ddy, dx_, dg, gx, gw, gb, ROWS, COLS, 1e-5)
+    # rotating buffer sets, as for the forward row ops: x, dy in and dx out per set
+    nsets = 8
+    xs_, dys, gxs = ([DeviceBuffer.from_host(x) for _ in range(nsets)], [DeviceBuffer.from_host(dy) for _ in range(nsets)],
+                     [DeviceBuffer((ROWS, COLS)) for _ in range(nsets)])
+    dg = DeviceBuffer.from_host(gamma)
+    gw, gb = DeviceBuffer((COLS,)), DeviceBuffer((COLS,))
+    ws = device.layer_norm_backward(dys[0], xs_[0], dg, gxs[0], gw, gb, ROWS, COLS, 1e-5)
+    turn = [0]
+
+    def nxt():
+        turn[0] = (turn[0] + 1) % nsets
+        return turn[0]
+
+    def ln_bwd():
+        i = nxt()
+        device.layer_norm_backward(dys[i], xs_[i], dg, gxs[i], gw, gb, ROWS, COLS, 1e-5, workspace=ws)
+
+    def rms_bwd():
+        i = nxt()
+        device.rms_norm_backward(dys[i], xs_[i], dg, gxs[i], gw, ROWS, COLS, 1e-6, workspace=ws)
+
     for name, nbytes, fn, cpu_fn in (
-        ("layer_norm_backward", 3 * ELEM * 4 + 3 * COLS * 4,
-         lambda: device.layer_norm_backward(ddy, dx_, dg, gx, gw, gb, ROWS, COLS, 1e-5, workspace=ws),
-         lambda: O.layer_norm_backward(dy, x, gamma, np.float32(1e-5))),
-        ("rms_norm_backward", 3 * ELEM * 4 + 2 * COLS * 4,
-         lambda: device.rms_norm_backward(ddy, dx_, dg, gx, gw, ROWS, COLS, 1e-6, workspace=ws),
-         lambda: O.rms_norm_backward(dy, x, gamma, np.float32(1e-6))),
+        ("layer_norm_backward", 3 * ELEM * 4 + 3 * COLS * 4, ln_bwd, lambda: O.layer_norm_backward(dy, x, gamma, np.float32(1e-5))),
+        ("rms_norm_backward", 3 * ELEM * 4 + 2 * COLS * 4, rms_bwd, lambda: O.rms_norm_backward(dy, x, gamma, np.float32(1e-6))),
     ):
         ms = timed(fn)
         gbs = nbytes / (ms * 1e-3) / 1e9
         out[name] = {"ms": round(ms, 5), "GB/s": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4), "bytes": nbytes,
-                     "workload": "fp32 [8192,4096], dx + dweight (+ dbias), all launches of the entry point"}
+                     "workload": "fp32 [8192,4096], dx + dweight (+ dbias), all launches of the entry point, %d rotating buffer sets" % nsets}
         log("[backward] %-20s %.4f ms  %7.1f GB/s  %.1f%% of HBM peak" % (name, ms, gbs, 100 * gbs / HBM_PEAK_GBS))
         if with_cpu:
             best, reps = cpu_time(cpu_fn, 2.0)
             out[name]["cpu"] = {"value": round(nbytes / best / 1e9, 2), "unit": "GB/s", "cores": O.threads(), "kind": "port",
                                 "sample": "the same tensors, best of %d" % reps}
-    del dx_, ddy, gx
+    del xs_, dys, gxs
     # linear backward at the GPT-2 FC1 shape: dx and dweight products + dbias
     batch, in_f, out_f = 8192, 768, 3072
     dyl, xl = synth.normal(4, "dyl", (batch, out_f)), synth.normal(4, "xl", (batch, in_f))

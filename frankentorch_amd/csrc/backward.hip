@@ -60,7 +60,7 @@ __device__ __forceinline__ void vset(double2 &v, int i, double x) {
     else v.y = x;
 }
 
-// Streaming (non-temporal) 16-byte stores for outputs the kernel never re-reads.
+// Streaming (non-temporal) 16-byte loads and stores: rows are read once and outputs never re-read.
 typedef float nat_f4 __attribute__((ext_vector_type(4)));
 typedef double nat_d2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ void stream_store(float4 *p, const float4 &v) {
@@ -70,6 +70,15 @@ __device__ __forceinline__ void stream_store(float4 *p, const float4 &v) {
 __device__ __forceinline__ void stream_store(double2 *p, const double2 &v) {
     nat_d2 n = {v.x, v.y};
     __builtin_nontemporal_store(n, reinterpret_cast<nat_d2 *>(p));
+}
+
+__device__ __forceinline__ float4 stream_load(const float4 *p) {
+    nat_f4 v = __builtin_nontemporal_load(reinterpret_cast<const nat_f4 *>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ double2 stream_load(const double2 *p) {
+    nat_d2 v = __builtin_nontemporal_load(reinterpret_cast<const nat_d2 *>(p));
+    return make_double2(v.x, v.y);
 }
 
 template <typename T> __device__ __forceinline__ T wave_sum(T v) {
@@ -145,8 +154,8 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
         for (int i = 0; i < VPT; ++i) {
             const int v = tid + i * kThreads;
             if (v < nvec) {
-                xd[i] = xr[v];
-                gd[i] = dyr[v];
+                xd[i] = stream_load(xr + v);
+                gd[i] = stream_load(dyr + v);
             } else {
 #pragma unroll
                 for (int e = 0; e < N; ++e) {
@@ -172,40 +181,35 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
             load_row(r, xv, gv);
         }
         if constexpr (!RMS) {
-            T s[1] = {T(0)};
+            // Two block reductions per row instead of the reference's four serial sums: neither sum(dy w) nor
+            // sum(dy w (x - mean)) needs rstd, so the first rides with sum(x) and the second with sum((x - mean)^2);
+            // c1 = rstd * sum(dy w (x - mean)) is the reference's sum(dy w xhat) with rstd factored out.
+            T s[2] = {T(0), T(0)};
 #pragma unroll
             for (int i = 0; i < VPT; ++i)
 #pragma unroll
-                for (int e = 0; e < N; ++e) s[0] += vget(xv[i], e);
-            block_sum<T, 1>(s, red, phase);
+                for (int e = 0; e < N; ++e) {
+                    s[0] += vget(xv[i], e);
+                    s[1] += vget(gv[i], e) * vget(wv[i], e);  // padding lanes hold dy = 0
+                }
+            block_sum<T, 2>(s, red, phase);
             const T mean = s[0] * inv_n;
-            T q[1] = {T(0)};
+            T q[2] = {T(0), T(0)};
 #pragma unroll
             for (int i = 0; i < VPT; ++i) {
                 const bool live = tid + i * kThreads < nvec;
 #pragma unroll
                 for (int e = 0; e < N; ++e) {
                     const T d = vget(xv[i], e) - mean;
-                    if (live) q[0] += d * d;
-                }
-            }
-            block_sum<T, 1>(q, red, phase);
-            const T rstd = t_rsqrt_of(q[0] * inv_n + eps);
-            T c[2] = {T(0), T(0)};
-#pragma unroll
-            for (int i = 0; i < VPT; ++i) {
-                const bool live = tid + i * kThreads < nvec;
-#pragma unroll
-                for (int e = 0; e < N; ++e) {
-                    const T xhat = (vget(xv[i], e) - mean) * rstd;
-                    const T dxhat = vget(gv[i], e) * vget(wv[i], e);
                     if (live) {
-                        c[0] += dxhat;
-                        c[1] += dxhat * xhat;
+                        q[0] += d * d;
+                        q[1] += (vget(gv[i], e) * vget(wv[i], e)) * d;
                     }
                 }
             }
-            block_sum<T, 2>(c, red, phase);
+            block_sum<T, 2>(q, red, phase);
+            const T rstd = t_rsqrt_of(q[0] * inv_n + eps);
+            const T c[2] = {s[1], rstd * q[1]};
             V *dxr = reinterpret_cast<V *>(dx + r * cols);
 #pragma unroll
             for (int i = 0; i < VPT; ++i) {
@@ -222,20 +226,18 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
                 if (v < nvec) stream_store(dxr + v, o);
             }
         } else {
-            T s[1] = {T(0)};
+            // one block reduction per row: sum(x^2) and sum(dy w x) do not depend on each other
+            T s[2] = {T(0), T(0)};
 #pragma unroll
             for (int i = 0; i < VPT; ++i)
 #pragma unroll
-                for (int e = 0; e < N; ++e) s[0] += vget(xv[i], e) * vget(xv[i], e);
-            block_sum<T, 1>(s, red, phase);
+                for (int e = 0; e < N; ++e) {
+                    s[0] += vget(xv[i], e) * vget(xv[i], e);
+                    s[1] += (vget(gv[i], e) * vget(wv[i], e)) * vget(xv[i], e);
+                }
+            block_sum<T, 2>(s, red, phase);
             const T rstd = t_rsqrt_of(s[0] * inv_n + eps);
-            T c[1] = {T(0)};
-#pragma unroll
-            for (int i = 0; i < VPT; ++i)
-#pragma unroll
-                for (int e = 0; e < N; ++e) c[0] += (vget(gv[i], e) * vget(wv[i], e)) * vget(xv[i], e);
-            block_sum<T, 1>(c, red, phase);
-            const T coef = rstd * rstd * rstd * c[0] * inv_n;
+            const T coef = rstd * rstd * rstd * s[1] * inv_n;
             V *dxr = reinterpret_cast<V *>(dx + r * cols);
 #pragma unroll
             for (int i = 0; i < VPT; ++i) {

@@ -67,7 +67,13 @@ __global__ __launch_bounds__(256) void quantize_rows_vec_kernel(const float *__r
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
         const int c = threadIdx.x + i * 256;
-        v[i] = c < nvec ? xr[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+        if (c < nvec) {  // read once: non-temporal
+            typedef float nat_f4 __attribute__((ext_vector_type(4)));
+            const nat_f4 t = __builtin_nontemporal_load(reinterpret_cast<const nat_f4 *>(xr + c));
+            v[i] = make_float4(t.x, t.y, t.z, t.w);
+        } else {
+            v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
         amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[i].x), fabsf(v[i].y)), fmaxf(fabsf(v[i].z), fabsf(v[i].w))));
     }
 #pragma unroll

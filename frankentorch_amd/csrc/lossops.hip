@@ -205,7 +205,7 @@ __global__ __launch_bounds__(THREADS, MINW) void resident_rows_kernel(const T *_
         for (int k = 0; k < lds_steps; ++k) {
             const T *pk = xr + (VPT + k) * THREADS + wave * kWave;  // scalar: the wavefront's 64 slots of step VPT + k
             if (tid < n_lds - k * THREADS)
-                asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" ::"v"(lane_off), "s"(pk),
+                asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1 nt" ::"v"(lane_off), "s"(pk),
                              "s"(wave_base + (unsigned)k * (THREADS * 4u))
                              : "memory", "m0");
         }
@@ -216,7 +216,7 @@ __global__ __launch_bounds__(THREADS, MINW) void resident_rows_kernel(const T *_
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
         const T *pk = uniform_ptr(xr + k * THREADS);
-        v[k] = (tid < n - k * THREADS && (k > 0 || tid >= lead)) ? pk[tid] : T(-__builtin_inf());
+        v[k] = (tid < n - k * THREADS && (k > 0 || tid >= lead)) ? __builtin_nontemporal_load(pk + tid) : T(-__builtin_inf());
     }
     T m = T(-__builtin_inf());
 #pragma unroll
