@@ -26,6 +26,7 @@ HIP_SOURCES = [
     "gemm.hip",
     "sdpa.hip",
     "backward.hip",
+    "sdpa_bwd.hip",
     "lossops.hip",
     "ingest.hip",
     "int8ops.hip",

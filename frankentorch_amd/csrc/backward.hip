@@ -28,6 +28,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "sdpa_bwd.hpp"
 
 namespace {
 
@@ -722,8 +723,10 @@ template <typename T> int sdpa_row_vpl(int64_t seq_k, const void *a, const void 
     return per <= 1 ? 1 : per <= 2 ? 2 : per <= 4 ? 4 : per <= 8 ? 8 : 16;
 }
 
+// Two score-shaped matrices (P and dU, or S and dS on the fused path), 64 elements of slack, and two per-row vectors
+// (log-sum-exp and delta of the fused path).
 template <typename T> size_t sdpa_backward_workspace(int64_t num_bh, int64_t seq_q, int64_t seq_k) {
-    return (size_t)(2 * num_bh * seq_q * seq_k + 64) * sizeof(T);
+    return (size_t)(2 * num_bh * seq_q * seq_k + 64 + 2 * num_bh * seq_q + 32) * sizeof(T);
 }
 
 template <typename T>
@@ -763,6 +766,45 @@ int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, i
     }
     const int64_t rows = num_bh * seq_q;
     FTH_ARG(fth::ceil_div(rows, kWaves) <= 2147483647LL, "sdpa backward: too many rows");
+    if constexpr (std::is_same<T, float>::value) {
+        // Fused path: the forward kernel's preparation pass (scores, log-sum-exp, delta), one key-owned kernel for dS,
+        // dK and dV, and the dQ product. P and dU are never materialised.
+        auto al = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; };
+        if (!mask && fth::sdpa_backward_fused_applies(num_bh, seq_q, seq_k, d_k, d_v, scale) && al(q) && al(k) && al(v) && al(dout) &&
+            al(dq) && al(dk) && al(dv) && al(workspace)) {
+            float *lse = p + ((2 * pe + 64 + 3) & ~(int64_t)3) + (unit_dout ? ((seq_q * d_v + 4 + 3) & ~(int64_t)3) : 0);  // behind the ones plane
+            lse = reinterpret_cast<float *>((reinterpret_cast<uintptr_t>(lse) + 15u) & ~(uintptr_t)15u);
+            float *delta = lse + ((rows + 3) & ~(int64_t)3);
+            int64_t blk = 0;
+            if (causal && seq_q == seq_k && seq_k >= 512 && seq_k % 128 == 0) {
+                blk = (seq_k / 8 + 127) / 128 * 128;
+                if (blk < 256) blk = 256;
+            }
+            if (int32_t rc = fth::sdpa_backward_prepare_f32(q, k, v, dout, dout_bs, num_bh, seq_q, seq_k, d_k, scale, causal, p, lse, delta, st))
+                return rc;
+            if (int32_t rc = fth::sdpa_backward_keys_f32(q, v, dout, dout_bs, p, lse, delta, num_bh, seq_q, seq_k, d_k, scale, causal, blk, du,
+                                                        dk, dv, st))
+                return rc;
+            // dQ = scale dS . K (the key pass leaves dS without the scale: it is the alpha here); block-causal: query block i
+            // reads the keys up to its own end
+            fth_gemm_desc g{};
+            g.batch = num_bh;
+            g.n = d_k; g.lda = seq_k; g.ldb = d_k; g.ldc = d_k;
+            g.stride_a = seq_q * seq_k; g.stride_b = seq_k * d_k; g.stride_c = seq_q * d_k;
+            if (blk > 0) {
+                for (int64_t i0 = 0; i0 < seq_q; i0 += blk) {
+                    const int64_t i1 = std::min(seq_q, i0 + blk);
+                    g.m = i1 - i0;
+                    g.k = i1;
+                    if (int32_t rc = dev_gemm<float>(&g, scale, du + i0 * seq_k, k, dq + i0 * d_k, fs)) return rc;
+                }
+                return FTH_OK;
+            }
+            g.m = seq_q;
+            g.k = seq_k;
+            return dev_gemm<float>(&g, scale, du, k, dq, fs);
+        }
+    }
     int vpl = sdpa_row_vpl<T>(seq_k, p, du);
     if (mask && ((reinterpret_cast<uintptr_t>(mask) & 15u) != 0 || mask_bh_stride % Vec16<T>::N != 0)) vpl = 0;  // unaligned mask rows
     const dim3 row_grid((unsigned)fth::ceil_div(rows, kWaves));

@@ -60,6 +60,3 @@ TOL_F64 = 1e-12
 # chain; the kernels add (rows of a workgroup) then (workgroups), and for long batches the re-associated fp32 sum of
 # thousands of terms differs from the serial one by a few ulp of the largest partial sum. Enforced bar: 4x the row-op bar.
 NORM_COLSUM_TOL_FACTOR = 4
-# The materialising SDPA backward rounds P and dU to fp32 in HBM between its five products (the reference keeps the same
-# intermediates, in a different summation order): enforced bar 2x the product bar. The tiled recompute kernels meet 1x.
-SDPA_BWD_MATERIALISED_TOL_FACTOR = 2

@@ -5,7 +5,7 @@ import math
 import numpy as np
 import pytest
 
-from conftest import NORM_COLSUM_TOL_FACTOR, SDPA_BWD_MATERIALISED_TOL_FACTOR, TOL_F64, TOL_GEMM_F32, TOL_ROW_F32, rel_err
+from conftest import NORM_COLSUM_TOL_FACTOR, TOL_F64, TOL_GEMM_F32, TOL_ROW_F32, rel_err
 from frankentorch_amd import synth
 from frankentorch_amd.device import DeviceBuffer
 
@@ -89,8 +89,11 @@ def test_linear_backward_reference_test_inputs(hip, oracle):
 
 # The last four shapes are square and long enough for the causal form to take the block-causal products
 # (blocks of 256 rows; 640 and 1152 end in a partial block).
+# Head sizes 64 and 128 with sequence lengths that are multiples of 4 take the fused path (preparation pass, key-owned
+# kernel, dQ product); the ragged ones among them end in partial query tiles and partial key blocks.
 @pytest.mark.parametrize("bh,sq,sk,dk,dv", [(2, 64, 64, 64, 64), (3, 100, 70, 32, 48), (4, 128, 128, 128, 128), (1, 5, 6, 4, 3), (2, 33, 200, 16, 16),
-                                            (2, 512, 512, 64, 64), (1, 640, 640, 32, 48), (3, 1024, 1024, 64, 64), (2, 1152, 1152, 128, 128)])
+                                            (2, 512, 512, 64, 64), (1, 640, 640, 32, 48), (3, 1024, 1024, 64, 64), (2, 1152, 1152, 128, 128),
+                                            (2, 100, 76, 64, 64), (1, 36, 260, 128, 128), (2, 256, 384, 64, 64), (2, 388, 132, 128, 128)])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_sdpa_backward(hip, oracle, bh, sq, sk, dk, dv, causal, dtype):
@@ -106,7 +109,7 @@ def test_sdpa_backward(hip, oracle, bh, sq, sk, dk, dv, causal, dtype):
     hip.sdpa_backward(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, s, causal, gq, gk, gv)
     got = (gq.to_host(), gk.to_host(), gv.to_host())
     for g, r in zip(got, ref):
-        assert rel_err(g, r) <= tol * SDPA_BWD_MATERIALISED_TOL_FACTOR
+        assert rel_err(g, r) <= tol
     hip.sdpa_backward(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, s, causal, gq, gk, gv)
     for a, b in zip(got, (gq.to_host(), gk.to_host(), gv.to_host())):
         assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
@@ -135,7 +138,7 @@ def test_sdpa_backward_masked(hip, oracle, bh, sq, sk, dk, dv, shared, dtype):
     hip.sdpa_backward_masked(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, s, dmask, stride, gq, gk, gv)
     got = (gq.to_host(), gk.to_host(), gv.to_host())
     for g, r in zip(got, ref):
-        assert rel_err(g, r) <= tol * SDPA_BWD_MATERIALISED_TOL_FACTOR
+        assert rel_err(g, r) <= tol
     hip.sdpa_backward_masked(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, s, dmask, stride, gq, gk, gv)
     for a, b in zip(got, (gq.to_host(), gk.to_host(), gv.to_host())):
         assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
@@ -143,7 +146,7 @@ def test_sdpa_backward_masked(hip, oracle, bh, sq, sk, dk, dv, shared, dtype):
         pad = DeviceBuffer.from_host(np.concatenate([np.zeros(1, dtype), mask.ravel()]))
         hip.sdpa_backward_masked(dq_, dk_, dv_, ddo, bh, sq, sk, dk, dv, s, pad.view(1), 0, gq, gk, gv)
         for g, r in zip((gq.to_host(), gk.to_host(), gv.to_host()), ref):
-            assert rel_err(g, r) <= tol * SDPA_BWD_MATERIALISED_TOL_FACTOR
+            assert rel_err(g, r) <= tol
 
 
 @pytest.mark.parametrize("bh,sq,sk,dk,dv", [(2, 5, 6, 4, 3), (3, 100, 70, 32, 48), (2, 640, 640, 64, 64)])
@@ -161,7 +164,7 @@ def test_sdpa_backward_unit_dout(hip, oracle, bh, sq, sk, dk, dv, causal, dtype)
     hip.sdpa_backward_unit_dout(dq_, dk_, dv_, bh, sq, sk, dk, dv, s, causal, gq, gk, gv)
     got = (gq.to_host(), gk.to_host(), gv.to_host())
     for g, r in zip(got, ref):
-        assert rel_err(g, r) <= tol * SDPA_BWD_MATERIALISED_TOL_FACTOR
+        assert rel_err(g, r) <= tol
     assert np.all(got[2] == got[2][:, :, :1])  # every value lane of a key gets the same gradient, bit for bit
     hq, hk, hv = DeviceBuffer(q.shape, dtype), DeviceBuffer(k.shape, dtype), DeviceBuffer(v.shape, dtype)
     hip.sdpa_backward(dq_, dk_, dv_, DeviceBuffer.from_host(np.ones((bh, sq, dv), dtype)), bh, sq, sk, dk, dv, s, causal, hq, hk, hv)
