@@ -37,4 +37,30 @@ __device__ __forceinline__ float gelu_erf(float x) {
     return x < 0.0f ? h * e : h * (2.0f - e);
 }
 
+// 2^t in double precision for the softmax weights of the fp64 attention kernel: t is a score minus a reference
+// maximum, so it is bounded above (a few units) and may be -inf. n = round(t), f = t - n in [-1/2, 1/2],
+// 2^f by its Taylor series to degree 12 (remainder 1.7e-16 at |f| = 1/2), scaled by 2^n with ldexp, which
+// underflows gradually and gives exactly 0 for the clamped -1100. Eighteen fp64 vector instructions where the
+// library exp costs about forty; in a kernel whose MFMAs and vector instructions share issue cycles that is the
+// difference that counts.
+__device__ __forceinline__ double exp2_softmax(double t) {
+    t = __builtin_fmax(t, -1100.0);
+    const double n = __builtin_rint(t);
+    const double f = t - n;
+    double p = 0x1.c3bd650fc2986p-36;
+    p = __builtin_fma(p, f, 0x1.e8cac7351bb25p-32);
+    p = __builtin_fma(p, f, 0x1.e4cf5158b8ecap-28);
+    p = __builtin_fma(p, f, 0x1.b5253d395e7c4p-24);
+    p = __builtin_fma(p, f, 0x1.62c0223a5c824p-20);
+    p = __builtin_fma(p, f, 0x1.ffcbfc588b0c7p-17);
+    p = __builtin_fma(p, f, 0x1.430912f86c787p-13);
+    p = __builtin_fma(p, f, 0x1.5d87fe78a6731p-10);
+    p = __builtin_fma(p, f, 0x1.3b2ab6fba4e77p-7);
+    p = __builtin_fma(p, f, 0x1.c6b08d704a0c0p-5);
+    p = __builtin_fma(p, f, 0x1.ebfbdff82c58fp-3);
+    p = __builtin_fma(p, f, 0x1.62e42fefa39efp-1);
+    p = __builtin_fma(p, f, 1.0);
+    return __builtin_ldexp(p, (int)n);
+}
+
 }  // namespace fth

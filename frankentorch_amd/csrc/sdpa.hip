@@ -32,6 +32,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "devmath.hpp"
 #include "sdpa_bwd.hpp"
 
 namespace {
@@ -282,6 +283,7 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
         for (int e = 0; e < NDT; ++e)
 #pragma unroll
             for (int r = 0; r < 16; ++r) o[e][r] = 0.f;
+        constexpr float kLazy = 6.0f;
         float m_run = -__builtin_inff();
         float l_run = 0.f;
 
@@ -406,20 +408,25 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
                     for (int j = 0; j < KS; ++j)
 #pragma unroll
                         for (int r = 0; r < 16; ++r) mt = fmaxf(mt, s[j][r]);
-                    float mlo, mhi;
-                    both_halves(mt, mlo, mhi);
-                    mt = fmaxf(mlo, mhi);
-                    m_new = fmaxf(m_run, mt * c2);
-                    alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-                    const float neg_m = -m_new;
-                    if (__any(alpha != 1.0f)) {
+                    // fp32 MFMAs and vector instructions share issue cycles, so the bookkeeping is kept off the common
+                    // path: the reference m of a query moves only when a score of this tile exceeds it by more than
+                    // kLazy (log2 units; weights stay below 2^kLazy and O / l does not depend on m). Only then do the two
+                    // halves of the wavefront exchange their maxima and the accumulators get rescaled; the row sum stays
+                    // a per-lane partial sum until the end.
+                    if (__any(mt * c2 > m_run + kLazy)) {
+                        float mlo, mhi;
+                        both_halves(mt, mlo, mhi);
+                        m_new = fmaxf(m_run, fmaxf(mlo, mhi) * c2);
+                        alpha = __builtin_amdgcn_exp2f(m_run - m_new);
 #pragma unroll
                         for (int e = 0; e < NDT; ++e)
 #pragma unroll
                             for (int r = 0; r < 16; ++r) o[e][r] *= alpha;
+                        l_run *= alpha;
+                        m_run = m_new;
                     }
-                    // ---- O^T += V_tile^T . P^T with the exponentials in the same instruction stream: MFMA step r needs
-                    //      only weight r, so the exponential of weight r + 1 issues while the matrix unit works on step r ----
+                    const float neg_m = -m_run;
+                    // ---- O^T += V_tile^T . P^T with the exponentials in the same instruction stream ----
 #pragma unroll
                     for (int j = 0; j < KS; ++j)
 #pragma unroll
@@ -431,10 +438,7 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
                             for (int ee = 0; ee < NDT; ++ee)
                                 o[ee] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(vv, ee), e, o[ee], 0, 0, 0);
                         }
-                    float plo, phi;
-                    both_halves(psum, plo, phi);
-                    l_run = l_run * alpha + (plo + phi);
-                    m_run = m_new;
+                    l_run += psum;
                 } else {
 #pragma unroll
                     for (int j = 0; j < KS; ++j)
@@ -485,9 +489,7 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
                             for (int ee = 0; ee < NDT; ++ee)
                                 o[ee] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(vv, ee), e, o[ee], 0, 0, 0);
                         }
-                    float plo, phi;
-                    both_halves(psum, plo, phi);
-                    l_run = l_run * alpha + (plo + phi);
+                    l_run = l_run * alpha + psum;
                     m_run = m_new;
                 }
             }
@@ -498,6 +500,11 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
         for (int kt = 0; kt < num_kt; kt += 2) {
             tile_step(kt, std::integral_constant<int, 0>{});
             if (kt + 1 < num_kt) tile_step(kt + 1, std::integral_constant<int, 1>{});
+        }
+        {  // the two halves of the wavefront hold partial row sums of the same queries
+            float llo, lhi;
+            both_halves(l_run, llo, lhi);
+            l_run = llo + lhi;
         }
 
         if constexpr (BWD) {
@@ -630,7 +637,13 @@ __global__ __launch_bounds__(64) void sdpa_generic_kernel(const SdpaArgs p) {
 //                                     element r of the lane holds: P is the B operand as it stands. Row i of
 //                                     d-tile e is d = 32 (e / 2) + 2 i + e % 2, so one 128-bit read of V feeds two
 //                                     d-tiles and a lane's outputs pair up into 16-byte stores.
-// Row max / sum: four in-lane values and two exchanges across the lane groups. exp is the library's double exp.
+// fp64 MFMAs and fp64 vector instructions share issue cycles (a vector instruction placed between two MFMAs delays the
+// second by its full issue time, also with two wavefronts per SIMD), so the softmax is written for instruction count:
+// Q is pre-multiplied by scale * log2(e) and the weights are 2^(x - ref) through an 18-instruction exp2; the reference
+// ref of a query moves only when some score of the tile exceeds it by more than kLazy (then, and only then, the lane
+// groups exchange their maxima and the accumulators are rescaled; weights stay below 2^kLazy, far from overflow, and the
+// final O / l does not depend on ref); the row sum stays a per-lane partial sum until the end; the causal / tail
+// selects run only in tiles that cross the diagonal or the end of the keys.
 // ---------------------------------------------------------------------------------------------
 using Acc4d = double __attribute__((ext_vector_type(4)));
 
@@ -666,11 +679,15 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_f64_kernel(const SdpaArgs p)
     const int q_blk0 = qb * BQ, q_wave0 = q_blk0 + wave * 16, qi = q_wave0 + lq;
     const bool q_live = qi < seq_q_i;
 
-    // Q: lane holds Q[qi][g * DQ + t], t = 0..DQ-1 (contiguous)
+    // Q: lane holds Q[qi][g * DQ + t], t = 0..DQ-1 (contiguous), times scale * log2(e): scores come out in log2 units
+    const double qmul = scale * 1.4426950408889634074;
     double2 qr[DQ / 2];
 #pragma unroll
-    for (int t = 0; t < DQ / 2; ++t)
+    for (int t = 0; t < DQ / 2; ++t) {
         qr[t] = q_live ? *reinterpret_cast<const double2 *>(Q + (int64_t)qi * d.q_row_stride + g * DQ + 2 * t) : make_double2(0.0, 0.0);
+        qr[t].x *= qmul;
+        qr[t].y *= qmul;
+    }
 
     int blk_last_q = q_blk0 + BQ - 1;
     if (blk_last_q > seq_q_i - 1) blk_last_q = seq_q_i - 1;
@@ -680,21 +697,23 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_f64_kernel(const SdpaArgs p)
     int wave_last_q = q_wave0 + 15;
     if (wave_last_q > seq_q_i - 1) wave_last_q = seq_q_i - 1;
 
-    // Tile loader through registers: thread owns vector column ld_c of rows ld_row + i * RS.
+    // Tile loader through registers: thread owns vector column ld_c of rows ld_row + i * RS. Range-checked buffer loads:
+    // the lane's byte offset is a constant, the tile and row-group part travels in the scalar offset, and rows past the
+    // last key come back as zeros without a test (the range check covers the sum of both offsets).
     constexpr int RS = 256 / (D / 2);
     const int ld_row = tid / (D / 2), ld_c = tid % (D / 2);
+    const __amdgpu_buffer_rsrc_t rs_k = __builtin_amdgcn_make_buffer_rsrc(const_cast<double *>(K), 0, (int)((unsigned)seq_k_i * (unsigned)d.k_row_stride * 8u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_v = __builtin_amdgcn_make_buffer_rsrc(const_cast<double *>(Vg), 0, (int)((unsigned)seq_k_i * (unsigned)d.v_row_stride * 8u), 0x00020000);
+    const unsigned k_lane = ((unsigned)ld_row * (unsigned)d.k_row_stride + 2u * (unsigned)ld_c) * 8u;
+    const unsigned v_lane = ((unsigned)ld_row * (unsigned)d.v_row_stride + 2u * (unsigned)ld_c) * 8u;
+    const unsigned k_row_bytes = (unsigned)d.k_row_stride * 8u, v_row_bytes = (unsigned)d.v_row_stride * 8u;
     double2 kst[NV], vst[NV];
     auto load_tile = [&](int kt) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            const int row = kt * BC + ld_row + i * RS;
-            if (row < seq_k_i) {
-                kst[i] = *reinterpret_cast<const double2 *>(K + (int64_t)row * d.k_row_stride + 2 * ld_c);
-                vst[i] = *reinterpret_cast<const double2 *>(Vg + (int64_t)row * d.v_row_stride + 2 * ld_c);
-            } else {
-                kst[i] = make_double2(0.0, 0.0);
-                vst[i] = make_double2(0.0, 0.0);
-            }
+            const unsigned row0 = (unsigned)(kt * BC + i * RS);  // uniform
+            kst[i] = __builtin_bit_cast(double2, __builtin_amdgcn_raw_buffer_load_b128(rs_k, k_lane, row0 * k_row_bytes, 0));
+            vst[i] = __builtin_bit_cast(double2, __builtin_amdgcn_raw_buffer_load_b128(rs_v, v_lane, row0 * v_row_bytes, 0));
         }
     };
     auto store_tile = [&](int buf) __attribute__((always_inline)) {
@@ -709,6 +728,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_f64_kernel(const SdpaArgs p)
 #pragma unroll
     for (int e = 0; e < NE; ++e) o[e] = (Acc4d){0.0, 0.0, 0.0, 0.0};
     const double ninf = -__builtin_inf();
+    constexpr double kLazy = 6.0;  // log2 units
     double m_run = ninf, l_run = 0.0;
 
     if (num_kt > 0) {
@@ -741,45 +761,48 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_f64_kernel(const SdpaArgs p)
                 s0 = __builtin_amdgcn_mfma_f64_16x16x4f64(kv.x, qr[t].x, s0, 0, 0, 0);
                 s1 = __builtin_amdgcn_mfma_f64_16x16x4f64(kv.y, qr[t].y, s1, 0, 0, 0);
             }
-            // ---- scale, mask, online softmax (lane-local query; keys 4 r + g) ----
-            double x[4], mt = ninf;
+            // ---- mask, online softmax in log2 units (lane-local query; keys 4 r + g) ----
+            double x[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int key = key0 + 4 * r + g;
-                double v = (s0[r] + s1[r]) * scale;
-                if constexpr (MASK) v += mk[r];
-                const bool hidden = (d.causal && key > qi) | (key >= seq_k_i);
-                v = hidden ? ninf : v;
-                x[r] = v;
-                mt = fmax(mt, v);
+                x[r] = s0[r] + s1[r];
+                if constexpr (MASK) x[r] = __builtin_fma(mk[r], 1.4426950408889634074, x[r]);
             }
-            mt = fmax(mt, __shfl_xor(mt, 16, kWave));
-            mt = fmax(mt, __shfl_xor(mt, 32, kWave));
-            const double m_new = fmax(m_run, mt);
-            // Every key so far hidden (possible only under a mask): keep the state empty instead of carrying the NaN
-            // of exp(-inf - -inf) into later tiles; a row with no visible key at all ends as 0 / 0 = NaN, as in the reference.
-            const double m_ref = (m_new == ninf) ? 0.0 : m_new;
-            // Once the running maximum has settled (after the first few tiles of most rows) no lane of the wavefront
-            // needs the rescale: skip its exp and the pass over the accumulators.
-            const bool rescale = __any(m_new != m_run);
-            const double alpha = rescale ? exp(m_run - m_ref) : 1.0;
-            if (rescale) {
+            if ((d.causal && key0 + BC - 1 > q_wave0) || key0 + BC > seq_k_i) {  // wavefront-uniform: the diagonal, the last keys
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int key = key0 + 4 * r + g;
+                    const bool hidden = (d.causal && key > qi) | (key >= seq_k_i);
+                    x[r] = hidden ? ninf : x[r];
+                }
+            }
+            const double mt = fmax(fmax(x[0], x[1]), fmax(x[2], x[3]));
+            if (__any(mt > m_run + kLazy)) {
+                // some score outgrew the reference: the query's lane groups agree on a new one and rescale
+                double mq = fmax(mt, __shfl_xor(mt, 16, kWave));
+                mq = fmax(mq, __shfl_xor(mq, 32, kWave));
+                const double m_new = fmax(m_run, mq);
+                // Every key so far hidden (possible only under a mask): m_run stays -inf and the reference below is 0, so
+                // the NaN of exp(-inf - -inf) never forms; a row with no visible key at all ends as 0 / 0 = NaN, as in
+                // the reference.
+                const double alpha = fth::exp2_softmax(m_run - ((m_new == ninf) ? 0.0 : m_new));
 #pragma unroll
                 for (int e = 0; e < NE; ++e)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) o[e][r] *= alpha;
+                l_run *= alpha;
+                m_run = m_new;
             }
+            const double m_ref = (m_run == ninf) ? 0.0 : m_run;
             // ---- O^T += V_tile^T . P^T: step r contracts keys 4 r + g; d-tiles 2 e2 and 2 e2 + 1 share one read.
-            //      Step r needs only weight r, so the exponential of weight r + 1 (some forty fp64 operations) is
-            //      spread between the MFMAs of step r. ----
+            //      Step r needs only weight r: the exponential of weight r + 1 sits between the MFMAs of step r. ----
             const double *vp = Vs + buf * KT + g * P + 2 * lq;
-            double psum = 0.0;
-            double e_cur = exp(x[0] - m_ref);
+            double e_cur = fth::exp2_softmax(x[0] - m_ref);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const double e_r = e_cur;
-                psum += e_r;
-                if (r + 1 < 4) e_cur = exp(x[r + 1] - m_ref);
+                l_run += e_r;
+                if (r + 1 < 4) e_cur = fth::exp2_softmax(x[r + 1] - m_ref);
 #pragma unroll
                 for (int e2 = 0; e2 < NE / 2; ++e2) {
                     const double2 vv = *reinterpret_cast<const double2 *>(vp + (4 * r) * P + 32 * e2);
@@ -790,14 +813,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_f64_kernel(const SdpaArgs p)
 #pragma unroll
                     for (int i = 0; i < NE; ++i) {
                         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA of step r ...
-                        __builtin_amdgcn_sched_group_barrier(0x002, 48 / NE, 0);  // ... then a share of the next exponential
+                        __builtin_amdgcn_sched_group_barrier(0x002, (24 + NE - 1) / NE, 0);  // ... then a share of the next exponential
                     }
                 }
             }
-            psum += __shfl_xor(psum, 16, kWave);
-            psum += __shfl_xor(psum, 32, kWave);
-            l_run = l_run * alpha + psum;
-            m_run = m_new;
         }
         if (kt + 1 < num_kt) store_tile(buf ^ 1);
         __syncthreads();
@@ -808,6 +827,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_mfma_f64_kernel(const SdpaArgs p)
     }
 
     // ---- normalise and store: element r of d-tile e is d = 32 (e / 2) + 2 (4 r + g) + e % 2 of query qi ----
+    l_run += __shfl_xor(l_run, 16, kWave);  // the four lane groups of a query hold partial row sums
+    l_run += __shfl_xor(l_run, 32, kWave);
     if (q_live) {
         double *orow = O + (int64_t)qi * d.o_row_stride;
 #pragma unroll
@@ -1095,7 +1116,9 @@ int32_t sdpa_entry(const fth_sdpa_desc *d, double scale, const T *q, const T *k,
             const char *e = std::getenv("FT_HIP_SDPA_F64_GENERIC");  // tuning / testing knob: 1 keeps fp64 on the generic kernel
             return e && std::atoi(e) != 0;
         }();
-        if (strides_ok && d->d_k == d->d_v && d->seq_k > 0 && !generic_only) {
+        // (the tile loads address a head's K and V through 32-bit byte offsets)
+        const bool span_ok = (d->seq_k + 16) * d->k_row_stride < ((int64_t)1 << 28) && (d->seq_k + 16) * d->v_row_stride < ((int64_t)1 << 28);
+        if (strides_ok && span_ok && d->d_k == d->d_v && d->seq_k > 0 && !generic_only) {
             if (d->d_k == 128) return launch_mfma_f64<128>(a, st);
             if (d->d_k == 64) return launch_mfma_f64<64>(a, st);
             if (d->d_k == 32) return launch_mfma_f64<32>(a, st);
