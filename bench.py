@@ -478,12 +478,19 @@ def bench_backward(device, synth, steps, with_cpu):
     ms_q = timed(quantise_next)
     ms_q_same = timed(lambda: device.quantize_rows_i8(dx8, m8, k8, qout[0][0], qout[0][1]))
     del qin, qout
+    # The same launches on all-zero operands (LAST, so that a counter run sees the product kernel's dispatches in two
+    # groups: random operands first, zeros second): the integer matrix rate of this chip depends on the operand values.
+    dxz = DeviceBuffer.from_host(np.zeros((m8, k8), np.float32))
+    dwqz = DeviceBuffer.from_host(np.zeros((n8, k8), np.int8))
+    ms_zero = timed(lambda: device.linear_int8_dynamic(dxz, m8, k8, dwqz, dws, n8, db8, dy8, workspace=ws8))
+    del dxz, dwqz
     ops = 2 * m8 * n8 * k8
     tops = ops / ((ms - ms_q_same) * 1e-3) / 1e12  # in the whole call the quantiser re-reads the same x
     qbytes = m8 * k8 * 5 + m8 * 4
     out["linear_int8_dynamic"] = {"ms": round(ms, 4), "quantize_ms": round(ms_q, 4), "product_TOP/s": round(tops, 1), "frac": round(tops / 5000.0, 4),
                                   "peak_TOP/s": 5000.0, "ops": ops, "quantize_GB/s": round(qbytes / (ms_q * 1e-3) / 1e9, 1),
                                   "quantize_same_buffer_GB/s": round(qbytes / (ms_q_same * 1e-3) / 1e9, 1),
+                                  "zero_operands": {"ms": round(ms_zero, 4), "product_TOP/s": round(2 * m8 * n8 * k8 / ((ms_zero - ms_q_same) * 1e-3) / 1e12, 1)},
                                   "workload": "x fp32 [8192,4096] . int8 W[4096,4096]^T + bias; product rate = ops / (whole call - quantiser)"}
     log("[backward] linear_int8_dynamic    %.4f ms (quantiser %.4f ms = %.0f GB/s); product %.0f TOP/s  %.1f%% of the 5.0 POP/s int8 peak"
         % (ms, ms_q, qbytes / (ms_q * 1e-3) / 1e9, tops, 100 * tops / 5000.0))

@@ -103,6 +103,7 @@ struct I8Args {
     float *c;  // [m, n]
     int64_t m, n, k;
     int tiles_m, tiles_n;
+    int vec_store;  // n % 4 == 0 and a 16-byte aligned output: interior tiles may use 128-bit stores
 };
 
 __device__ __forceinline__ void load_to_lds_16(const int8_t *src, unsigned lds_chunk) {
@@ -172,6 +173,7 @@ __global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8A
         a_src[i] = p.a + ar * p.k + q * 16;
         b_src[i] = p.b + br * p.k + q * 16;
     }
+    const int num_kt = (int)(p.k / kBK);
     auto issue = [&](int kt) __attribute__((always_inline)) {
         const unsigned base = lds0 + (unsigned)(kt % kStages) * STAGE + wave_u * (LD * 1024u);
         const int64_t koff = (int64_t)kt * kBK;
@@ -190,7 +192,6 @@ __global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8A
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    const int num_kt = (int)(p.k / kBK);
 #pragma unroll
     for (int st = 0; st < kStages - 1; ++st)
         if (st < num_kt) issue(st);
@@ -257,6 +258,44 @@ __global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8A
     __syncthreads();
     const bool interior = m0 + BM <= p.m && n0 + BN <= p.n;  // no bounds tests on the common path
     const int64_t ldc = p.n;
+    if (interior && p.vec_store) {
+        // Interior tiles leave through LDS so that the output goes out in whole rows: in the accumulator a lane holds ONE
+        // column, and storing from there writes 128-byte pieces; staged, a wavefront instruction writes 1 KiB of
+        // consecutive columns per row with 128-bit stores. One slab per MFMA tile row i: the 32 rows of both wavefront
+        // rows, 64 x BN floats.
+        float *stage = reinterpret_cast<float *>(smem) + BM;  // behind the row scales
+        constexpr int V4 = BN / 4;                            // 128-bit vectors per output row
+        constexpr int PASSES = 64 * V4 / 256;
+#pragma unroll
+        for (int i = 0; i < TW; ++i) {
+            const int lrow0 = wm * (32 * TW) + i * 32 + 4 * kg;  // tile row of accumulator element 0
+            if (i > 0) __syncthreads();                          // the previous slab has been read
+#pragma unroll
+            for (int j = 0; j < TW; ++j) {
+                const int lcol = wn * (32 * TW) + j * 32 + frow;
+                const float ws = p.b_scales[n0 + lcol];
+                const float bv = p.bias ? p.bias[n0 + lcol] : 0.0f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int dr = 8 * (r >> 2) + (r & 3);
+                    float y = (float)acc[i][j][r] * row_scale[lrow0 + dr] * ws;
+                    if (p.bias) y += bv;
+                    stage[(wm * 32 + 4 * kg + dr) * BN + lcol] = y;
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int ps = 0; ps < PASSES; ++ps) {
+                const int f = ps * 256 + tid, srow = f / V4, c4 = f % V4;
+                const float4 v = *reinterpret_cast<const float4 *>(stage + srow * BN + 4 * c4);
+                float *dst = p.c + (m0 + (srow >> 5) * (32 * TW) + i * 32 + (srow & 31)) * ldc + n0 + 4 * c4;
+                typedef float nat_f4 __attribute__((ext_vector_type(4)));
+                nat_f4 nv = {v.x, v.y, v.z, v.w};
+                __builtin_nontemporal_store(nv, reinterpret_cast<nat_f4 *>(dst));
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TW; ++i) {
         const int lrow0 = wm * (32 * TW) + i * 32 + 4 * kg;  // tile row of accumulator element 0
@@ -354,19 +393,19 @@ int32_t fth_dev_linear_int8_prequantized_f32(const int8_t *x_i8, const float *a_
     p.a = x_i8; p.b = w_i8; p.a_scales = a_scales; p.b_scales = w_scales; p.bias = bias; p.c = out;
     p.m = m; p.n = n; p.k = k;
     p.tiles_m = p.tiles_n = 0;
+    p.vec_store = (n % 4 == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0) ? 1 : 0;
     const bool aligned = ((reinterpret_cast<uintptr_t>(x_i8) | reinterpret_cast<uintptr_t>(w_i8)) & 15u) == 0;
     const int64_t tiles128 = fth::ceil_div(m, 128) * fth::ceil_div(n, 128), tiles256 = fth::ceil_div(m, 256) * fth::ceil_div(n, 256);
     if (k >= kBK && k % kBK == 0 && aligned && tiles128 <= 2147483647LL) {
         // 256 x 256 tiles once they give every compute unit a workgroup and the reduction is long enough to pay for their
-        // longer fill and drain (measured crossover between k = 4096 and k = 16384); the choice depends on the shape only.
-        // With real operands the sustained rate of either tile is set by the chip's power limit, not by the loop: the same
-        // launch runs 30% faster on all-zero operands than on operands spread over [-127, 127].
+        // longer fill and drain: they need half the L2 -> LDS traffic per MFMA, and that path (about 27 bytes per clock
+        // and compute unit in this access pattern) is what bounds the 128 x 128 loop. The choice depends on the shape only.
         const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
         static const int forced = [] {
             const char *e = std::getenv("FT_HIP_I8_TILE");  // tuning knob: 128 or 256; anything else = automatic
             return e ? std::atoi(e) : 0;
         }();
-        const bool big = forced == 256 || (forced != 128 && tiles256 >= cus && k >= 8192);
+        const bool big = forced == 256 || (forced != 128 && tiles256 >= cus && k >= 2048);
         if (int32_t rc = big ? launch_i8_gemm<4>(p, st) : launch_i8_gemm<2>(p, st)) return rc;
     } else {
         int64_t total;
