@@ -475,7 +475,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
     static_assert(LPR_A <= kWave && kWave % LPR_A == 0, "a chunk must hold whole k rows of A");
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile rows must divide into 8-row chunks per wavefront");
     static_assert(MT % 16 == 0, "swizzle assumes MFMA tile rows start on a multiple of 16");
-    static_assert(LPR <= kWave && kWave % LPR == 0, "a chunk must hold whole k rows of B");
+    static_assert(TRANS_B || (LPR <= kWave && kWave % LPR == 0), "a chunk must hold whole k rows of B");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *As = reinterpret_cast<T *>(smem_raw);  // [2][BM][BK]
@@ -1255,7 +1255,7 @@ enum class Tile { Big, Wide, Small, Tall };
 
 inline int forced_tile() {
     static const int v = [] {
-        const char *e = std::getenv("FT_HIP_GEMM_TILE");  // tuning knob: 0 = 128x128, 1 = 256x128, 2 = 64x64, 3 = 128x64 (direct fp32 only)
+        const char *e = std::getenv("FT_HIP_GEMM_TILE");  // tuning knob: 0 = 128x128, 1 = 256x128, 2 = 64x64, 3 = 128x64, 4 = 128x96 (3, 4: direct fp32 only)
         return e ? std::atoi(e) : -1;
     }();
     return v;
@@ -1284,6 +1284,17 @@ int32_t launch_shape(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
         if (!direct_off && t != Tile::Wide && p.k % DBK == 0 && p.lda <= lim && p.ldb <= lim && p.ldc <= lim) {
             constexpr int MINW_BIG = 2;
             if constexpr (std::is_same<T, float>::value) {
+                if constexpr (TRANS_B) {
+                    // 128x96 tiles (4x1 wavefronts of 32x96) when they hand every resident workgroup (two per compute
+                    // unit) a whole number of whole tiles and 128x128 tiles do not: no tile is split over K, no fix-up
+                    // pass. All GPT-2 widths are multiples of 96 (768 = 8 x 96): QKV 0.77 -> 0.82, O-proj 0.75 -> 0.78,
+                    // FC2 0.82 -> 0.83 of the matrix peak; where 128x128 tiles already divide evenly (FC1) they stay
+                    // (their main loop is 1-2 % faster).
+                    const int64_t slots = (int64_t)cus * 2;
+                    const int64_t tiles96 = fth::ceil_div(p.m, 128) * (p.n / 96) * batch;
+                    const bool n96 = f < 0 && t == Tile::Big && p.n % 96 == 0 && tiles96 % slots == 0 && big_tiles % slots != 0;
+                    if (n96 || f == 4) return launch_direct<T, 128, 96, 4, 1, 2, TRANS_B, true>(p, batch, st);
+                }
                 // Fewer 128x128 tiles than resident workgroups would split every tile over K; 128x64
                 // tiles (three workgroups per CU) give each workgroup whole tiles instead. Their main
                 // loop is about 8 % slower, which costs more than the fix-up pass (about 25 us) once
