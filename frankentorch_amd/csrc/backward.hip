@@ -93,9 +93,9 @@ template <typename T> __device__ __forceinline__ T wave_sum(T v) {
 // values: consecutive calls alternate between its halves (`phase`), so one barrier per call is
 // enough -- a wavefront can only reach the write of call n + 2 after passing the barrier of call
 // n + 1, which every wavefront reaches only after its reads of call n.
-template <typename T, int NV> __device__ __forceinline__ void block_sum(T (&v)[NV], T *red, int &phase) {
+template <typename T, int NV, int NW = kWaves> __device__ __forceinline__ void block_sum(T (&v)[NV], T *red, int &phase) {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    T *buf = red + phase * (kWaves * 2);
+    T *buf = red + phase * (NW * 2);
     phase ^= 1;
 #pragma unroll
     for (int i = 0; i < NV; ++i) v[i] = wave_sum(v[i]);
@@ -108,7 +108,7 @@ template <typename T, int NV> __device__ __forceinline__ void block_sum(T (&v)[N
     for (int i = 0; i < NV; ++i) {
         T s = buf[i];
 #pragma unroll
-        for (int w = 1; w < kWaves; ++w) s += buf[w * NV + i];
+        for (int w = 1; w < NW; ++w) s += buf[w * NV + i];
         v[i] = s;
     }
 }
@@ -117,15 +117,21 @@ template <typename T> __device__ __forceinline__ T t_rsqrt_of(T v) { return T(1)
 
 // ---- register-resident norm backward ----
 // RMS = false: LayerNorm (weight required, partial dbias written); RMS = true: RMSNorm (weight optional).
-// VPT: 16-byte vectors per thread; cols <= kThreads * VPT * N and cols % N == 0.
-template <typename T, int VPT, bool RMS>
-__global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__restrict__ dy, const T *__restrict__ x,
-                                                                 const T *__restrict__ w, int64_t rows, int cols, T eps,
-                                                                 T *__restrict__ dx, T *__restrict__ part_w,
-                                                                 T *__restrict__ part_b, int rows_per_block) {
+// NT threads own a row; VPT: 16-byte vectors per thread; cols <= NT * VPT * N and cols % N == 0.
+// DEPTH: rows requested ahead of the one being reduced (0, 1 or 2 register sets). The kernel waits for rows far more
+// than it computes, and what limits the rows in flight per compute unit is registers: a thread holds the row in hand,
+// the sets in flight, the weight and two column accumulators. Rows of up to 1024 vectors use 512 threads with two
+// vectors each and two sets in flight (two such workgroups per compute unit: four rows of 32 KiB in flight, twice what
+// 256 threads with four vectors and one set could hold).
+template <typename T, int VPT, bool RMS, int NT = kThreads, int DEPTH = (VPT * Vec16<T>::N <= 16 ? 1 : 0)>
+__global__ __launch_bounds__(NT) void norm_backward_kernel(const T *__restrict__ dy, const T *__restrict__ x,
+                                                           const T *__restrict__ w, int64_t rows, int cols, T eps,
+                                                           T *__restrict__ dx, T *__restrict__ part_w,
+                                                           T *__restrict__ part_b, int rows_per_block) {
     using V = typename Vec16<T>::type;
     constexpr int N = Vec16<T>::N;
-    __shared__ T red[2 * kWaves * 2];
+    constexpr int NW = NT / kWave;
+    __shared__ T red[2 * NW * 2];
     int phase = 0;
     const int tid = threadIdx.x;
     const int nvec = cols / N;
@@ -134,7 +140,7 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
     T aw[VPT][N], ab[VPT][N];
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-        const int v = tid + i * kThreads;
+        const int v = tid + i * NT;
 #pragma unroll
         for (int e = 0; e < N; ++e) {
             aw[i][e] = T(0);
@@ -145,15 +151,13 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
     }
     const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
     const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
-    // Rows are loaded one ahead (a second register set) when the row is short enough to afford it.
-    constexpr bool PREFETCH = VPT * N <= 16;
-    V xn[PREFETCH ? VPT : 1], gn[PREFETCH ? VPT : 1];
     auto load_row = [&](int64_t r, V *xd, V *gd) __attribute__((always_inline)) {
+        if (r >= r1) return;  // workgroup-uniform: nothing left to request
         const V *xr = reinterpret_cast<const V *>(x + r * cols);
         const V *dyr = reinterpret_cast<const V *>(dy + r * cols);
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
-            const int v = tid + i * kThreads;
+            const int v = tid + i * NT;
             if (v < nvec) {
                 xd[i] = stream_load(xr + v);
                 gd[i] = stream_load(dyr + v);
@@ -166,18 +170,16 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
             }
         }
     };
-    if constexpr (PREFETCH) {
-        if (r0 < r1) load_row(r0, xn, gn);
-    }
-    for (int64_t r = r0; r < r1; ++r) {
+    // One row: xs / gs hold it on entry (DEPTH > 0) and are handed the row DEPTH ahead as soon as they have been copied.
+    auto do_row = [&](int64_t r, V *xs, V *gs) __attribute__((always_inline)) {
         V xv[VPT], gv[VPT];
-        if constexpr (PREFETCH) {
+        if constexpr (DEPTH > 0) {
 #pragma unroll
             for (int i = 0; i < VPT; ++i) {
-                xv[i] = xn[i];
-                gv[i] = gn[i];
+                xv[i] = xs[i];
+                gv[i] = gs[i];
             }
-            if (r + 1 < r1) load_row(r + 1, xn, gn);
+            load_row(r + DEPTH, xs, gs);
         } else {
             load_row(r, xv, gv);
         }
@@ -193,12 +195,12 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
                     s[0] += vget(xv[i], e);
                     s[1] += vget(gv[i], e) * vget(wv[i], e);  // padding lanes hold dy = 0
                 }
-            block_sum<T, 2>(s, red, phase);
+            block_sum<T, 2, NW>(s, red, phase);
             const T mean = s[0] * inv_n;
             T q[2] = {T(0), T(0)};
 #pragma unroll
             for (int i = 0; i < VPT; ++i) {
-                const bool live = tid + i * kThreads < nvec;
+                const bool live = tid + i * NT < nvec;
 #pragma unroll
                 for (int e = 0; e < N; ++e) {
                     const T d = vget(xv[i], e) - mean;
@@ -208,13 +210,13 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
                     }
                 }
             }
-            block_sum<T, 2>(q, red, phase);
+            block_sum<T, 2, NW>(q, red, phase);
             const T rstd = t_rsqrt_of(q[0] * inv_n + eps);
             const T c[2] = {s[1], rstd * q[1]};
             V *dxr = reinterpret_cast<V *>(dx + r * cols);
 #pragma unroll
             for (int i = 0; i < VPT; ++i) {
-                const int v = tid + i * kThreads;
+                const int v = tid + i * NT;
                 V o;
 #pragma unroll
                 for (int e = 0; e < N; ++e) {
@@ -236,13 +238,13 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
                     s[0] += vget(xv[i], e) * vget(xv[i], e);
                     s[1] += (vget(gv[i], e) * vget(wv[i], e)) * vget(xv[i], e);
                 }
-            block_sum<T, 2>(s, red, phase);
+            block_sum<T, 2, NW>(s, red, phase);
             const T rstd = t_rsqrt_of(s[0] * inv_n + eps);
             const T coef = rstd * rstd * rstd * s[1] * inv_n;
             V *dxr = reinterpret_cast<V *>(dx + r * cols);
 #pragma unroll
             for (int i = 0; i < VPT; ++i) {
-                const int v = tid + i * kThreads;
+                const int v = tid + i * NT;
                 V o;
 #pragma unroll
                 for (int e = 0; e < N; ++e) {
@@ -253,11 +255,22 @@ __global__ __launch_bounds__(kThreads) void norm_backward_kernel(const T *__rest
                 if (v < nvec) stream_store(dxr + v, o);
             }
         }
+    };
+    V xa[DEPTH > 0 ? VPT : 1], ga[DEPTH > 0 ? VPT : 1], xb[DEPTH > 1 ? VPT : 1], gb[DEPTH > 1 ? VPT : 1];
+    if constexpr (DEPTH > 0) load_row(r0, xa, ga);
+    if constexpr (DEPTH > 1) load_row(r0 + 1, xb, gb);
+    if constexpr (DEPTH > 1) {
+        for (int64_t r = r0; r < r1; r += 2) {  // the two register sets take alternate rows
+            do_row(r, xa, ga);
+            if (r + 1 < r1) do_row(r + 1, xb, gb);
+        }
+    } else {
+        for (int64_t r = r0; r < r1; ++r) do_row(r, xa, ga);
     }
     // one row of partial column sums per workgroup
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-        const int v = tid + i * kThreads;
+        const int v = tid + i * NT;
         if (v < nvec) {
             V ow, ob;
 #pragma unroll
@@ -351,7 +364,13 @@ __global__ __launch_bounds__(kThreads) void col_partial_kernel(const T *__restri
 // part in ascending order (loads eight deep, independent of the adds), then the 8 lane sums are
 // added lane 0..7. The order is a function of (nparts) only.
 template <typename T>
-__global__ __launch_bounds__(kThreads) void col_final_kernel(const T *__restrict__ part, int nparts, int64_t cols, T *__restrict__ out) {
+__global__ __launch_bounds__(kThreads) void col_final_kernel(const T *__restrict__ part, int nparts, int64_t cols, T *__restrict__ out,
+                                                             const T *__restrict__ part2, T *__restrict__ out2) {
+    // blockIdx.y == 1: the second array of partial sums (dbias beside dweight), summed in the same launch
+    if (blockIdx.y == 1) {
+        part = part2;
+        out = out2;
+    }
     constexpr int CW = 32, PL = kThreads / CW;
     __shared__ T red[PL][CW];
     const int c = threadIdx.x % CW, pl = threadIdx.x / CW;
@@ -447,11 +466,14 @@ int32_t norm_backward_entry(const T *dy, const T *x, const T *w, int64_t rows, i
         T *pw = want_w ? part_w : nullptr, *pb = db ? part_b : nullptr;
 #define FTH_NORM_BWD(V) \
     norm_backward_kernel<T, V, RMS><<<dim3((unsigned)blocks), dim3(kThreads), 0, st>>>(dy, x, w, rows, (int)cols, eps, dx, pw, pb, rpb)
-        if (vpt <= 1) FTH_NORM_BWD(1);
-        else if (vpt <= 2) FTH_NORM_BWD(2);
-        else if (vpt <= 4) FTH_NORM_BWD(4);
+#define FTH_NORM_BWD_DEEP(V, NT_) \
+    norm_backward_kernel<T, V, RMS, NT_, 2><<<dim3((unsigned)blocks), dim3(NT_), 0, st>>>(dy, x, w, rows, (int)cols, eps, dx, pw, pb, rpb)
+        if (nvec <= kThreads) FTH_NORM_BWD_DEEP(1, kThreads);
+        else if (nvec <= 2 * kThreads) FTH_NORM_BWD_DEEP(1, 2 * kThreads);
+        else if (nvec <= 4 * kThreads) FTH_NORM_BWD_DEEP(2, 2 * kThreads);
         else if (vpt <= 8) FTH_NORM_BWD(8);
         else FTH_NORM_BWD(16);
+#undef FTH_NORM_BWD_DEEP
 #undef FTH_NORM_BWD
         FTH_CHECK_LAUNCH("norm_backward");
     } else {
@@ -468,12 +490,14 @@ int32_t norm_backward_entry(const T *dy, const T *x, const T *w, int64_t rows, i
             FTH_CHECK_LAUNCH("norm_backward_dbias");
         }
     }
-    if (want_w) {
-        col_final_kernel<T><<<dim3((unsigned)fth::ceil_div(cols, 32)), dim3(kThreads), 0, st>>>(part_w, (int)blocks, cols, dw);
+    if (want_w && db) {
+        col_final_kernel<T><<<dim3((unsigned)fth::ceil_div(cols, 32), 2), dim3(kThreads), 0, st>>>(part_w, (int)blocks, cols, dw, part_b, db);
+        FTH_CHECK_LAUNCH("norm_backward_dweight_dbias_sum");
+    } else if (want_w) {
+        col_final_kernel<T><<<dim3((unsigned)fth::ceil_div(cols, 32)), dim3(kThreads), 0, st>>>(part_w, (int)blocks, cols, dw, nullptr, nullptr);
         FTH_CHECK_LAUNCH("norm_backward_dweight_sum");
-    }
-    if (db) {
-        col_final_kernel<T><<<dim3((unsigned)fth::ceil_div(cols, 32)), dim3(kThreads), 0, st>>>(part_b, (int)blocks, cols, db);
+    } else if (db) {
+        col_final_kernel<T><<<dim3((unsigned)fth::ceil_div(cols, 32)), dim3(kThreads), 0, st>>>(part_b, (int)blocks, cols, db, nullptr, nullptr);
         FTH_CHECK_LAUNCH("norm_backward_dbias_sum");
     }
     return FTH_OK;
@@ -537,7 +561,7 @@ int32_t linear_backward_entry(const T *dy, const T *x, const T *w, int64_t batch
         col_partial_kernel<T, 0><<<dim3((unsigned)col_blocks, (unsigned)blocks), dim3(kThreads), 0, st>>>(dy, nullptr, nullptr, batch,
                                                                                                          out_f, out_f, rpb, part);
         FTH_CHECK_LAUNCH("linear_backward_dbias");
-        col_final_kernel<T><<<dim3((unsigned)fth::ceil_div(out_f, 32)), dim3(kThreads), 0, st>>>(part, (int)blocks, out_f, db);
+        col_final_kernel<T><<<dim3((unsigned)fth::ceil_div(out_f, 32)), dim3(kThreads), 0, st>>>(part, (int)blocks, out_f, db, nullptr, nullptr);
         FTH_CHECK_LAUNCH("linear_backward_dbias_sum");
     }
     return FTH_OK;
