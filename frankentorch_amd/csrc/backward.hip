@@ -799,34 +799,13 @@ int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, i
             float *lse = p + ((2 * pe + 64 + 3) & ~(int64_t)3) + (unit_dout ? ((seq_q * d_v + 4 + 3) & ~(int64_t)3) : 0);  // behind the ones plane
             lse = reinterpret_cast<float *>((reinterpret_cast<uintptr_t>(lse) + 15u) & ~(uintptr_t)15u);
             float *delta = lse + ((rows + 3) & ~(int64_t)3);
-            int64_t blk = 0;
-            if (causal && seq_q == seq_k && seq_k >= 512 && seq_k % 128 == 0) {
-                blk = (seq_k / 8 + 127) / 128 * 128;
-                if (blk < 256) blk = 256;
-            }
             if (int32_t rc = fth::sdpa_backward_prepare_f32(q, k, v, dout, dout_bs, num_bh, seq_q, seq_k, d_k, scale, causal, p, lse, delta, st))
                 return rc;
-            if (int32_t rc = fth::sdpa_backward_keys_f32(q, v, dout, dout_bs, p, lse, delta, num_bh, seq_q, seq_k, d_k, scale, causal, blk, du,
+            // (under a causal mask the key pass writes dS from each key block's own first row on: all the dQ pass reads)
+            if (int32_t rc = fth::sdpa_backward_keys_f32(q, v, dout, dout_bs, p, lse, delta, num_bh, seq_q, seq_k, d_k, scale, causal, 128, du,
                                                         dk, dv, st))
                 return rc;
-            // dQ = scale dS . K (the key pass leaves dS without the scale: it is the alpha here); block-causal: query block i
-            // reads the keys up to its own end
-            fth_gemm_desc g{};
-            g.batch = num_bh;
-            g.n = d_k; g.lda = seq_k; g.ldb = d_k; g.ldc = d_k;
-            g.stride_a = seq_q * seq_k; g.stride_b = seq_k * d_k; g.stride_c = seq_q * d_k;
-            if (blk > 0) {
-                for (int64_t i0 = 0; i0 < seq_q; i0 += blk) {
-                    const int64_t i1 = std::min(seq_q, i0 + blk);
-                    g.m = i1 - i0;
-                    g.k = i1;
-                    if (int32_t rc = dev_gemm<float>(&g, scale, du + i0 * seq_k, k, dq + i0 * d_k, fs)) return rc;
-                }
-                return FTH_OK;
-            }
-            g.m = seq_q;
-            g.k = seq_k;
-            return dev_gemm<float>(&g, scale, du, k, dq, fs);
+            return fth::sdpa_backward_dq_f32(du, k, num_bh, seq_q, seq_k, d_k, scale, causal, dq, st);
         }
     }
     int vpl = sdpa_row_vpl<T>(seq_k, p, du);

@@ -1,4 +1,4 @@
-// Fused key-owned pass of the fp32 scaled-dot-product-attention backward for gfx950
+// Fused key-owned and query-owned passes of the fp32 scaled-dot-product-attention backward for gfx950
 // (sdpa_backward_f32, crates/ft-kernel-cpu/src/lib.rs:5539-5650; the unit-dOut form :5662-5770).
 //
 // The reference materialises P = softmax(scale Q K^T) and dU per (batch, head) and runs five
@@ -8,7 +8,7 @@
 //   2. this kernel, one workgroup per block of 128 keys walking the query tiles it can see:
 //      P = 2^(S c - lse), dP = dOut V^T, dS = scale P (dP - delta) written to HBM,
 //      dV += P^T dOut, dK += dS^T Q in registers                 (products dP, dV, dK);
-//   3. dQ = dS K as a batched MFMA GEMM (csrc/gemm.hip)           (product dQ).
+//   3. a query-owned kernel, dQ = scale dS K with dS read in the accumulator layout of pass 2   (product dQ).
 // Six product-sized MFMA passes instead of five, but P and dU never make the round trip through
 // HBM between separate softmax and softmax-gradient row passes: per call S is written once and
 // read once, dS written once and read once. A recompute design that keeps nothing in HBM needs
@@ -333,6 +333,150 @@ template <int D> int32_t launch_keys(const KeysArgs &a, hipStream_t st) {
     return FTH_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Query-owned pass: dQ = scale . dS . K. One workgroup per 128 queries (a wavefront owns 32), walking the 32-key tiles
+// its queries can see; K tiles through double-buffered LDS (row order, read along d), dS straight from HBM in the
+// accumulator layout of the key-owned pass: dQ^T[d, q] += K_tile^T . dS^T, where MFMA step r contracts over the two
+// keys 8 (r / 4) + 4 half + r % 4 and a lane's B operand is dS[q = lane % 32][that key] - four 16-byte loads per lane
+// and tile, requested one tile ahead. The key-owned pass stored explicit zeros for the masked pairs of every tile on
+// the diagonal, so this loop has no mask logic: a wavefront simply stops at the last tile its queries reach. 64 MFMAs
+// (D = 128) per tile against 4 loads and 16 LDS reads, and hardly a vector instruction in between.
+// ---------------------------------------------------------------------------------------------
+struct DqArgs {
+    const float *ds, *k;
+    float *dq;
+    int64_t num_bh;
+    int seq_q, seq_k;
+    float scale;
+    int causal;
+};
+
+template <int D>
+__global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_kernel(const DqArgs p) {
+    constexpr int NDT = D / 32;
+    constexpr int VPR = D / 4;         // 16-byte vectors per row
+    constexpr int RPC = 64 / VPR;      // tile rows per 1 KiB load instruction
+    constexpr int CPW = 32 / RPC / 4;  // load instructions per wavefront per tile
+    constexpr int TILE = 32 * D;       // floats per K tile
+    using VV = typename VecN<NDT>::type;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    float *Ks = reinterpret_cast<float *>(smem_raw);  // [2][32][D], row order
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lq = lane & 31, half = lane >> 5;
+    const int64_t pid = blockIdx.x;
+    const int q_blocks = (p.seq_q + 127) / 128;
+    const int qb = q_blocks - 1 - (int)(pid / p.num_bh);  // heaviest (latest) query blocks first under a causal mask
+    const int64_t bh = pid % p.num_bh;
+    const int seq_q = p.seq_q, seq_k = p.seq_k;
+    const int q_blk0 = qb * 128, q_wave0 = q_blk0 + 32 * wave, qi = q_wave0 + lq;
+    const bool q_live = qi < seq_q;
+    const float *Kg = p.k + bh * (int64_t)seq_k * D;
+    const float *DSg = p.ds + bh * (int64_t)seq_q * seq_k;
+
+    int blk_last_q = q_blk0 + 127, wave_last_q = q_wave0 + 31;
+    if (blk_last_q > seq_q - 1) blk_last_q = seq_q - 1;
+    if (wave_last_q > seq_q - 1) wave_last_q = seq_q - 1;
+    int k_end = seq_k;
+    if (p.causal && blk_last_q + 1 < k_end) k_end = blk_last_q + 1;
+    const int ntiles = (k_end + 31) / 32;
+
+    // ---- K tile loader (rows past the last key clamped: their dS is read as zero) ----
+    const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)reinterpret_cast<uintptr_t>(smem_raw));
+    const unsigned wave_u = __builtin_amdgcn_readfirstlane((unsigned)wave);
+    auto issue_tile = [&](int t, int buf) __attribute__((always_inline)) {
+        const unsigned dst = lds0 + (unsigned)(buf * TILE * 4) + wave_u * (CPW * 1024u);
+#pragma unroll
+        for (int ci = 0; ci < CPW; ++ci) {
+            int row = 32 * t + (wave * CPW + ci) * RPC + lane / VPR;
+            row = row < seq_k ? row : seq_k - 1;
+            load_to_lds_16(Kg, (unsigned)row * (unsigned)(D * 4) + 16u * (unsigned)(lane % VPR), dst + ci * 1024u);
+        }
+    };
+
+    // ---- dS through range-checked buffer loads: lane part (its query's row, its half's keys) in the vector offset,
+    //      tile part in the scalar offset; a dead query's lane part is "nowhere" ----
+    constexpr unsigned kOut = 0x40000000u;
+    const unsigned row_bytes = (unsigned)seq_k * 4u;
+    const __amdgpu_buffer_rsrc_t rs_ds =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(DSg), 0, (int)((unsigned)seq_q * row_bytes), 0x00020000);
+    const unsigned lane_ds = q_live ? (unsigned)qi * row_bytes + 16u * (unsigned)half : kOut;
+    typedef unsigned u4v __attribute__((ext_vector_type(4)));
+    auto wave_active = [&](int t) __attribute__((always_inline)) { return !p.causal || 32 * t <= wave_last_q; };
+    auto load_ds = [&](int t, float4(&dst)[4]) __attribute__((always_inline)) {
+        const bool none = t >= ntiles || !wave_active(t);
+        const unsigned v = none ? kOut : lane_ds;
+        const bool tail = 32 * t + 32 > seq_k;  // uniform: the last keys of a row must not run into the next row
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            u4v x = __builtin_amdgcn_raw_buffer_load_b128(rs_ds, v, (unsigned)(32 * t + 8 * g) * 4u, 2);
+            if (tail && 32 * t + 8 * g + 4 * half >= seq_k) x = (u4v){0u, 0u, 0u, 0u};
+            dst[g] = __builtin_bit_cast(float4, x);
+        }
+    };
+
+    Acc16 acc[NDT];
+#pragma unroll
+    for (int e = 0; e < NDT; ++e)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[e][r] = 0.f;
+
+    float4 ds_a[4], ds_b[4];
+    if (ntiles > 0) issue_tile(0, 0);
+    load_ds(0, ds_a);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+
+    const int kvec = (4 * half) * D + NDT * lq;  // K is in row order: elements d = NDT lq .. of tile row 8 g + 4 half + j
+    auto tile_step = [&](const int t, auto buf_c, float4(&ds_cur)[4], float4(&ds_nx)[4]) __attribute__((always_inline)) {
+        constexpr int buf = decltype(buf_c)::value;
+        if (t + 1 < ntiles) issue_tile(t + 1, buf ^ 1);
+        load_ds(t + 1, ds_nx);
+        if (wave_active(t)) {
+            const float *kb = Ks + buf * TILE + kvec;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const VV kv = *reinterpret_cast<const VV *>(kb + (8 * (r >> 2) + (r & 3)) * D);
+                const float w = f4_get(ds_cur[r >> 2], r & 3);
+#pragma unroll
+                for (int e = 0; e < NDT; ++e) acc[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(kv, e), w, acc[e], 0, 0, 0);
+            }
+        }
+        // Everything requested at the top of this tile (the K copies and the next tile's dS, a whole tile of MFMAs ago)
+        // has landed by now. The explicit vmcnt(0) also tells the compiler's wait-count pass so: it does not see the
+        // K copies (inline assembly) and would otherwise place a too strict wait in front of the next tile's first MFMA.
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+    };
+    for (int t = 0; t < ntiles; t += 2) {
+        tile_step(t, std::integral_constant<int, 0>{}, ds_a, ds_b);
+        if (t + 1 < ntiles) tile_step(t + 1, std::integral_constant<int, 1>{}, ds_b, ds_a);
+    }
+
+    // ---- store: lane owns query qi, d = NDT rho + e with rho = 8 (r / 4) + 4 half + r % 4 ----
+    if (q_live) {
+        float *row = p.dq + (bh * (int64_t)seq_q + qi) * D;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int rho = 8 * (r >> 2) + 4 * half + (r & 3);
+            if constexpr (NDT == 4)
+                *reinterpret_cast<float4 *>(row + 4 * rho) =
+                    make_float4(p.scale * acc[0][r], p.scale * acc[1][r], p.scale * acc[2][r], p.scale * acc[3][r]);
+            else
+                *reinterpret_cast<float2 *>(row + 2 * rho) = make_float2(p.scale * acc[0][r], p.scale * acc[1][r]);
+        }
+    }
+}
+
+template <int D> int32_t launch_dq(const DqArgs &a, hipStream_t st) {
+    constexpr size_t smem = (size_t)2 * 32 * D * sizeof(float);
+    const int64_t grid = a.num_bh * fth::ceil_div(a.seq_q, 128);
+    FTH_ARG(grid <= 2147483647LL, "sdpa backward: grid too large");
+    sdpa_bwd_dq_kernel<D><<<dim3((unsigned)grid), dim3(256), smem, st>>>(a);
+    FTH_CHECK_LAUNCH("sdpa_bwd_dq");
+    return FTH_OK;
+}
+
 }  // namespace
 
 namespace fth {
@@ -358,6 +502,17 @@ int32_t sdpa_backward_keys_f32(const float *q, const float *v, const float *dout
     if (d == 128) return launch_keys<128>(a, st);
     if (d == 64) return launch_keys<64>(a, st);
     return fth::set_error(FTH_ERR_INVALID_ARGUMENT, "sdpa_backward_keys: head size %lld", (long long)d);
+}
+
+int32_t sdpa_backward_dq_f32(const float *ds, const float *k, int64_t num_bh, int64_t seq_q, int64_t seq_k, int64_t d, float scale,
+                             int causal, float *dq, hipStream_t st) {
+    DqArgs a;
+    a.ds = ds; a.k = k; a.dq = dq;
+    a.num_bh = num_bh; a.seq_q = (int)seq_q; a.seq_k = (int)seq_k;
+    a.scale = scale; a.causal = causal;
+    if (d == 128) return launch_dq<128>(a, st);
+    if (d == 64) return launch_dq<64>(a, st);
+    return fth::set_error(FTH_ERR_INVALID_ARGUMENT, "sdpa_backward_dq: head size %lld", (long long)d);
 }
 
 }  // namespace fth

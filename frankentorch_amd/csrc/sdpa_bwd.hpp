@@ -19,9 +19,13 @@ int32_t sdpa_backward_prepare_f32(const float *q, const float *k, const float *v
 
 // Launch 2: dS = scale P (dP - delta) into ds [num_bh, seq_q, seq_k], dK and dV. Under a causal mask dS is written
 // (zeros where masked) for the rows from the start of the `row_block`-row block that holds a key block's first key
-// (row_block a multiple of 128; 0: from row 0), which is what the block-causal dQ products read.
+// (row_block a multiple of 128; 0: from row 0); the dQ pass reads the rows from a key block's own first key on (128).
 int32_t sdpa_backward_keys_f32(const float *q, const float *v, const float *dout, int64_t dout_bh_stride, const float *s, const float *lse,
                                const float *delta, int64_t num_bh, int64_t seq_q, int64_t seq_k, int64_t d, float scale, int causal,
                                int64_t row_block, float *ds, float *dk, float *dv, hipStream_t st);
+
+// Launch 3: dQ = scale . dS . K from the dS of launch 2 (contiguous [num_bh, seq, d] operands).
+int32_t sdpa_backward_dq_f32(const float *ds, const float *k, int64_t num_bh, int64_t seq_q, int64_t seq_k, int64_t d, float scale,
+                             int causal, float *dq, hipStream_t st);
 
 }  // namespace fth
