@@ -46,6 +46,51 @@ __global__ __launch_bounds__(256) void k(float *out, const float *gin, int iters
     out[blockIdx.x * 256 + threadIdx.x] = s;
 }
 float *g_out, *g_in;
+
+// ---- second part: does the sustained MFMA rate depend on the operand VALUES? Register-only, no memory: the operands come from
+//      four register sets filled with zeros, ones or hashed bits. ----
+__device__ unsigned hash32(unsigned x) { x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16; return x; }
+template <int KIND>
+__global__ __launch_bounds__(256) void kd(float *out, int iters, int mode) {
+    F16v fa[4]; I16v ia[4];
+    for (int i = 0; i < 4; ++i) for (int r = 0; r < 16; ++r) { fa[i][r] = 0.f; ia[i][r] = 0; }
+    I4v av[4], bv[4]; float af[4], bf[4];
+    for (int s = 0; s < 4; ++s) {
+        for (int e = 0; e < 4; ++e) {
+            unsigned h = hash32(threadIdx.x * 131 + s * 17 + e * 7 + blockIdx.x * 977), g = hash32(h + 12345);
+            if (mode == 0) { h = 0; g = 0; }
+            if (mode == 1) { h = 0x01010101u; g = 0x01010101u; }
+            av[s][e] = (int)h; bv[s][e] = (int)g;
+        }
+        const unsigned h = hash32(threadIdx.x * 31 + s);
+        af[s] = mode == 0 ? 0.f : mode == 1 ? 1.f : (float)(int)(h & 0xffff) / 65536.f - 0.5f;
+        bf[s] = mode == 0 ? 0.f : mode == 1 ? 1.f : (float)(int)((h >> 16) & 0xffff) / 65536.f - 0.5f;
+    }
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (KIND == 0) fa[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[(u + i) & 3], bf[(u + 2 * i) & 3], fa[i], 0, 0, 0);
+                if (KIND == 1) ia[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[(u + i) & 3], bv[(u + 2 * i) & 3], ia[i], 0, 0, 0);
+            }
+        }
+    }
+    float s = 0;
+    for (int i = 0; i < 4; ++i) for (int r = 0; r < 16; ++r) s += fa[i][r] + ia[i][r];
+    out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+template <int KIND> void run_data(const char *name, int mode) {
+    const int iters = 20000;
+    hipEvent_t e0, e1; (void)hipEventCreate(&e0); (void)hipEventCreate(&e1);
+    kd<KIND><<<256, 256>>>(g_out, 100, mode);
+    (void)hipEventRecord(e0);
+    kd<KIND><<<256, 256>>>(g_out, iters, mode);
+    (void)hipEventRecord(e1); (void)hipEventSynchronize(e1);
+    float ms; (void)hipEventElapsedTime(&ms, e0, e1);
+    const double n = (double)iters * 32 * 1024, ops = KIND == 1 ? n * 65536 : n * 4096;
+    printf("%-44s %7.2f ms  %8.3f %s\n", name, ms, ops / (ms * 1e-3) / (KIND == 1 ? 1e15 : 1e12), KIND == 1 ? "POP/s" : "TFLOP/s");
+}
 template <int KIND, int FILL, int NF> void run(const char *name, int blocks) {
     int smem = blocks == 256 ? 100 * 1024 : 60 * 1024;
     int iters = 1000;
@@ -79,5 +124,12 @@ int main() {
     run<2, 1, 4>("f64 + 4 VALU fma", 256);
     run<2, 2, 2>("f64 + 2 ds_read_b128", 256);
     run<2, 1, 4>("f64 + 4 VALU fma", 512);
+    printf("operand values, register-only loops (no memory traffic):\n");
+    run_data<1>("i8 32x32x32, all-zero operands", 0);
+    run_data<1>("i8 32x32x32, all-one bytes", 1);
+    run_data<1>("i8 32x32x32, random bytes", 2);
+    run_data<0>("f32 32x32x2, all-zero operands", 0);
+    run_data<0>("f32 32x32x2, ones", 1);
+    run_data<0>("f32 32x32x2, random in [-0.5, 0.5)", 2);
     return 0;
 }
