@@ -39,9 +39,10 @@ def test_gemm_matches_oracle(hip, oracle, m, n, k, trans_b, dtype):
 
 # K a whole number of 128-byte K-tiles with 16-byte aligned rows: the global->LDS direct kernels.
 # Ragged m / n (clamped edge rows and columns), one-row and one-vector extents, tile counts that
-# leave every workgroup a mix of whole and split tiles (several tiles per workgroup, K split 2-3 ways).
+# leave every workgroup a mix of whole and split tiles (several tiles per workgroup, K split 2-3 ways), and the GPT-2
+# O-projection shape at a short K, which the [n, k] fp32 form runs on 128 x 96 tiles (512 whole tiles, none split).
 DIRECT_SHAPES = [(200, 300, 96), (77, 52, 64), (130, 132, 512), (1, 4, 32), (1000, 8, 32), (129, 257 * 4, 160),
-                 (2048, 2304, 768), (4096, 3072, 256), (2050, 1540, 288)]
+                 (2048, 2304, 768), (4096, 3072, 256), (2050, 1540, 288), (8192, 768, 64)]
 
 
 @pytest.mark.parametrize("m,n,k", DIRECT_SHAPES)
