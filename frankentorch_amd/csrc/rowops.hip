@@ -395,6 +395,102 @@ __global__ __launch_bounds__(RowBlock<WPR>::kThreads, RowBlock<WPR>::min_blocks(
     }
 }
 
+// ---- LayerNorm, RPT rows side by side per row group ---------------------------------------------
+// A lane holds the same columns of RPT consecutive rows, so gamma and beta are fetched once per RPT rows (with one row
+// per block they crossed the L2 -> L1 path once per row, 32 KiB for every 16 KiB fp32 row of 4096) and the RPT
+// reductions share their barriers. Per row the arithmetic and the reduction tree are those of layernorm_row_kernel:
+// the two kernels give the same bits.
+template <int WPR, int N, typename T>
+__device__ __forceinline__ void group_sum_n(T (&v)[N], T *smem, int &phase) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) v[j] = wave_reduce(v[j], SumOp{});
+    if constexpr (WPR > 1) {
+        const int wave = threadIdx.x / kWave;
+        const int first = (wave / WPR) * WPR;
+        T *buf = smem + phase * (kMaxWaves * N);
+        phase ^= 1;
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+#pragma unroll
+            for (int j = 0; j < N; ++j) buf[wave * N + j] = v[j];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            T r = buf[first * N + j];
+#pragma unroll
+            for (int w = 1; w < WPR; ++w) r = r + buf[(first + w) * N + j];
+            v[j] = r;
+        }
+    }
+}
+
+template <typename T, int VPL, int WPR, int RPT>
+__global__ __launch_bounds__(RowBlock<WPR>::kThreads) void layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ w,
+                                                                                 const T *__restrict__ b, T *__restrict__ y,
+                                                                                 int64_t rows, int cols, T eps) {
+    __shared__ T smem[2 * kMaxWaves * RPT];
+    int phase = 0;
+    using R = RowRegs<T, VPL, WPR>;
+    const int nvec = cols / R::EPV;
+    const T inv_n = T(1) / (T)cols;
+    const int64_t row0 = ((int64_t)blockIdx.x * RowBlock<WPR>::kRows + threadIdx.x / (kWave * WPR)) * RPT;
+    R r[RPT];
+#pragma unroll
+    for (int q = 0; q < RPT; ++q) {
+        const int64_t row = row0 + q < rows ? row0 + q : rows - 1;  // a turn past the last row works on a copy of it and stores nothing
+        r[q].load(x + row * cols, nvec, T(0));
+    }
+    T sum[RPT];
+#pragma unroll
+    for (int q = 0; q < RPT; ++q) {
+        sum[q] = 0;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i)
+#pragma unroll
+            for (int j = 0; j < R::EPV; ++j) sum[q] += r[q].e[i][j];
+    }
+    group_sum_n<WPR, RPT>(sum, smem, phase);
+    T mean[RPT], vsum[RPT];
+#pragma unroll
+    for (int q = 0; q < RPT; ++q) {
+        mean[q] = sum[q] * inv_n;
+        vsum[q] = 0;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const bool live = (R::lane() + i * R::kLanes) < nvec;
+#pragma unroll
+            for (int j = 0; j < R::EPV; ++j) {
+                const T d = r[q].e[i][j] - mean[q];
+                vsum[q] += live ? d * d : T(0);
+            }
+        }
+    }
+    group_sum_n<WPR, RPT>(vsum, smem, phase);
+    T rstd[RPT];
+#pragma unroll
+    for (int q = 0; q < RPT; ++q) rstd[q] = T(1) / dev_sqrt(vsum[q] * inv_n + eps);
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+        const int v = R::lane() + i * R::kLanes;
+        if (v < nvec) {
+            T wv[R::EPV], bv[R::EPV];
+            if (w) R::load_vec(w, v, wv);
+            if (b) R::load_vec(b, v, bv);
+#pragma unroll
+            for (int q = 0; q < RPT; ++q)
+#pragma unroll
+                for (int j = 0; j < R::EPV; ++j) {
+                    T o = (r[q].e[i][j] - mean[q]) * rstd[q];
+                    if (w) o = o * wv[j];
+                    if (b) o = o + bv[j];
+                    r[q].e[i][j] = o;
+                }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < RPT; ++q) r[q].store(y + (row0 + q < rows ? row0 + q : rows - 1) * cols, row0 + q < rows ? nvec : 0);
+}
+
 // ---- RMSNorm ---------------------------------------------------------------------------------
 template <typename T, int VPL, int WPR>
 __global__ __launch_bounds__(RowBlock<WPR>::kThreads, RowBlock<WPR>::min_blocks(VPL, 3)) void rmsnorm_row_kernel(
@@ -768,6 +864,31 @@ int32_t launch_layernorm(const T *x, const T *x2, const T *w, const T *b, T *y, 
     bool vec_ok = cols % EPV == 0 && aligned16(x) && aligned16(y) && (!ADD || aligned16(x2)) &&
                   (!w || aligned16(w)) && (!b || aligned16(b));
     if (vec_ok && pick_row_shape(cols / EPV, ADD ? 8 : 16, vpl, wpr) && (row_launch_shape(rows, wpr, grid, iters), grid <= kMaxGrid)) {
+        if constexpr (!ADD) {
+            // Two rows side by side (gamma / beta once per pair) where a lane's share of a row is at most four vectors and
+            // there are rows enough to fill the chip that way; FT_HIP_LN_SIDE=0 keeps one row per group. Measured at fp32
+            // [8192,4096] on rotating buffers: LayerNorm 0.70 -> 0.72 of the HBM peak with two rows, 0.64 with four (too few,
+            // too fat workgroups); without gamma and beta one row per group streams best (0.76 against 0.72), and so it does for
+            // RMSNorm with its single gamma (0.74 against 0.72 with two rows).
+            constexpr int kSide = 2;
+            static const bool side_off = [] {
+                const char *e = std::getenv("FT_HIP_LN_SIDE");
+                return e && std::atoi(e) == 0;
+            }();
+            const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
+            const int64_t side_grid = fth::ceil_div(rows, (int64_t)rows_per_block(wpr) * kSide);
+            if ((w || b) && !side_off && iters == 1 && wpr <= 4 && vpl <= 4 && side_grid >= 4 * (int64_t)cus) {
+#define LS(V_, W_) layernorm_rows_kernel<T, V_, W_, kSide><<<dim3((unsigned)side_grid), dim3(RowBlock<W_>::kThreads), 0, st>>>(x, w, b, y, rows, (int)cols, eps)
+                switch (wpr) {
+                    case 1: if (vpl == 1) { LS(1, 1); } else if (vpl == 2) { LS(2, 1); } else { LS(4, 1); } break;
+                    case 2: if (vpl == 1) { LS(1, 2); } else if (vpl == 2) { LS(2, 2); } else { LS(4, 2); } break;
+                    default: if (vpl == 1) { LS(1, 4); } else if (vpl == 2) { LS(2, 4); } else { LS(4, 4); } break;
+                }
+#undef LS
+                FTH_CHECK_LAUNCH("layer_norm");
+                return FTH_OK;
+            }
+        }
 #define L(V_, W_) layernorm_row_kernel<T, V_, W_, ADD><<<dim3((unsigned)grid), dim3(RowBlock<W_>::kThreads), 0, st>>>(x, x2, w, b, y, rows, (int)cols, eps, iters)
         FTH_ROW_DISPATCH(vpl, wpr, L);
 #undef L

@@ -189,3 +189,21 @@ def test_full_size_row_ops_parity_determinism_and_properties(hip, oracle):
     assert np.array_equal(y, (x + bias) + res)
     y = twice(lambda out: hip.add_layer_norm(dx, dr, dg, dbt, out, rows, cols, 1e-5))
     assert rel_err(y, oracle.add_layer_norm(x, res, gamma, beta, 1e-5)) <= TOL_ROW_F32
+
+
+def test_layer_norm_row_pairs_give_the_bits_of_single_rows(hip):
+    """Batches with rows enough run LayerNorm with two rows side by side per row group (gamma / beta fetched once per
+    pair); smaller batches run one row per group. Per row the arithmetic and the reduction tree are the same, so a batch
+    normalised in one call equals the same rows normalised in calls too small for the paired kernel, bit for bit -
+    also with an odd number of rows, where the last pair has a single live row."""
+    for rows, cols, piece in ((4097, 4096, 1024), (8192, 768, 1000), (5001, 2048, 512)):
+        x = synth.normal(21, "x", (rows, cols))
+        g = synth.uniform(21, "g", (cols,), 0.5, 1.5)
+        b = synth.normal(21, "b", (cols,), 0.0, 0.1)
+        dx, dg, db = DeviceBuffer.from_host(x), DeviceBuffer.from_host(g), DeviceBuffer.from_host(b)
+        whole, parts = DeviceBuffer((rows, cols)), DeviceBuffer((rows, cols))
+        hip.layer_norm(dx, dg, db, whole, rows, cols, 1e-5)
+        for r0 in range(0, rows, piece):
+            n = min(piece, rows - r0)
+            hip.layer_norm(dx.view(r0 * cols), dg, db, parts.view(r0 * cols), n, cols, 1e-5)
+        assert np.array_equal(whole.to_host().view(np.uint32), parts.to_host().view(np.uint32))
