@@ -45,7 +45,7 @@ def test_no_alloc_rejects_shapes_beyond_the_scratch(hip):
 
     cap = hip.layer_norm_backward_noalloc_max_bytes()
     assert cap == 24 << 20
-    rows, cols = 16384, 8192  # 512 workgroups x 8192 columns x 2 arrays x 4 bytes = 32 MiB of partial sums
+    rows, cols = 32768, 8192  # 512 workgroups (64 rows each) x 8192 columns x 2 arrays x 4 bytes = 32 MiB of partial sums
     assert hip.norm_backward_workspace_bytes(rows, cols, np.float32) > cap
     one = DeviceBuffer((1,))
     with pytest.raises(HipError) as exc:
