@@ -444,12 +444,15 @@ template <int N, int I = 0, typename F> __device__ __forceinline__ void static_f
     }
 }
 
-template <typename T> __device__ __forceinline__ void load_to_lds_16(const T *src, unsigned lds_chunk) {
+template <typename T> __device__ __forceinline__ void load_to_lds_16(const T *base, unsigned lane_bytes, unsigned lds_chunk) {
     // Inline assembly so that the compiler's wait-count insertion does not see an LDS write it
     // cannot disambiguate (it would drain the load queue before every LDS read and serialise the
     // prefetch); the kernel waits for vmcnt(0) itself before each barrier.
-    // The chunk address is the same in every lane; readfirstlane makes that explicit so the operand is an SGPR.
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(__builtin_amdgcn_readfirstlane(lds_chunk))
+    // Scalar base (the K-tile's uniform pointer) plus a per-lane 32-bit byte offset: no 64-bit vector address
+    // arithmetic per load (vector instructions take issue cycles from the MFMAs). The chunk address is the same in
+    // every lane; readfirstlane makes that explicit so the operand is an SGPR.
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_bytes), "s"(base),
+                 "s"(__builtin_amdgcn_readfirstlane(lds_chunk))
                  : "memory", "m0");
 }
 
@@ -520,8 +523,8 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
     int ld_left = n_iter;             // K-tiles it still has to request
     int64_t ld_tile = it / p.ktiles;
     int ld_k = (int)(it - ld_tile * p.ktiles);
-    const T *ak = nullptr, *bk = nullptr;  // uniform bases of the next K-tile to load; lane offsets fit 32 bits (launcher check)
-    unsigned a_off[A_LD], b_off[B_LD];
+    const T *ak = nullptr, *bk = nullptr;  // uniform bases of the next K-tile to load
+    unsigned a_off[A_LD], b_off[B_LD];     // per-lane BYTE offsets from them; they fit 32 bits (launcher check)
     auto setup_loader = [&]() __attribute__((always_inline)) {
         const int64_t batch = ld_tile / p.tiles_per_batch;
         int tile_m, tile_n;
@@ -534,7 +537,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
             for (int i = 0; i < A_LD; ++i) {
                 int row = (wave * A_LD + i) * 8 + lr;
                 row = row < a_rows ? row : a_rows - 1;
-                a_off[i] = (unsigned)row * (unsigned)p.lda + (unsigned)lvec(wave * A_LD + i);
+                a_off[i] = ((unsigned)row * (unsigned)p.lda + (unsigned)lvec(wave * A_LD + i)) * (unsigned)sizeof(T);
             }
         } else {
             ak = p.a + batch * p.stride_a + (int64_t)ld_k * BK * p.lda + m0;
@@ -543,7 +546,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
 #pragma unroll
             for (int i = 0; i < A_LD; ++i) {
                 const int krow = (wave * A_LD + i) * RPC_A + lane / LPR_A;
-                a_off[i] = (unsigned)krow * (unsigned)p.lda + (unsigned)col;
+                a_off[i] = ((unsigned)krow * (unsigned)p.lda + (unsigned)col) * (unsigned)sizeof(T);
             }
         }
         if constexpr (TRANS_B) {
@@ -552,7 +555,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
             for (int i = 0; i < B_LD; ++i) {
                 int row = (wave * B_LD + i) * 8 + lr;
                 row = row < b_cols ? row : b_cols - 1;
-                b_off[i] = (unsigned)row * (unsigned)p.ldb + (unsigned)lvec(wave * B_LD + i);
+                b_off[i] = ((unsigned)row * (unsigned)p.ldb + (unsigned)lvec(wave * B_LD + i)) * (unsigned)sizeof(T);
             }
         } else {
             bk = p.b + batch * p.stride_b + (int64_t)ld_k * BK * p.ldb + n0;
@@ -561,7 +564,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
 #pragma unroll
             for (int i = 0; i < B_LD; ++i) {
                 const int krow = (wave * B_LD + i) * RPC + lane / LPR;
-                b_off[i] = (unsigned)krow * (unsigned)p.ldb + (unsigned)col;
+                b_off[i] = ((unsigned)krow * (unsigned)p.ldb + (unsigned)col) * (unsigned)sizeof(T);
             }
         }
     };
@@ -570,9 +573,9 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
         const unsigned as = lds0 + (unsigned)(buf * BM * BK * (int)sizeof(T)) + wave_u * (A_LD * 1024u);
         const unsigned bs = lds0 + (unsigned)((2 * BM + buf * BN) * BK * (int)sizeof(T)) + wave_u * (B_LD * 1024u);
 #pragma unroll
-        for (int i = 0; i < A_LD; ++i) load_to_lds_16(ak + a_off[i], as + i * 1024u);
+        for (int i = 0; i < A_LD; ++i) load_to_lds_16(ak, a_off[i], as + i * 1024u);
 #pragma unroll
-        for (int i = 0; i < B_LD; ++i) load_to_lds_16(bk + b_off[i], bs + i * 1024u);
+        for (int i = 0; i < B_LD; ++i) load_to_lds_16(bk, b_off[i], bs + i * 1024u);
         ak += TRANS_A ? (int64_t)BK * p.lda : (int64_t)BK;
         bk += TRANS_B ? (int64_t)BK : (int64_t)BK * p.ldb;
         --ld_left;
@@ -1280,7 +1283,7 @@ int32_t launch_shape(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
             const char *e = std::getenv("FT_HIP_GEMM_DIRECT");  // tuning knob: 0 disables the direct-to-LDS kernels
             return e && std::atoi(e) == 0;
         }();
-        const int64_t lim = ((int64_t)1 << 31) / 128 - 128;
+        const int64_t lim = ((int64_t)1 << 32) / (128 * (int64_t)sizeof(T)) - 128;  // a tile's lane byte offsets fit 32 bits
         if (!direct_off && t != Tile::Wide && p.k % DBK == 0 && p.lda <= lim && p.ldb <= lim && p.ldc <= lim) {
             constexpr int MINW_BIG = 2;
             if constexpr (std::is_same<T, float>::value) {
@@ -1410,7 +1413,7 @@ template <typename T> int32_t launch_trans_a(GemmArgs<T> &p, const fth_gemm_desc
     constexpr int EPV = Mfma<T>::EPV;
     constexpr int64_t DBK = 128 / (int64_t)sizeof(T);
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
-    const int64_t lim = ((int64_t)1 << 31) / 128 - 128;
+    const int64_t lim = ((int64_t)1 << 32) / (128 * (int64_t)sizeof(T)) - 128;  // a tile's lane byte offsets fit 32 bits
     const bool direct = d->m % EPV == 0 && d->n % EPV == 0 && d->k % DBK == 0 && d->lda % EPV == 0 && d->ldb % EPV == 0 &&
                         d->stride_a % EPV == 0 && d->stride_b % EPV == 0 && al(p.a) && al(p.b) && d->lda <= lim && d->ldb <= lim &&
                         d->ldc <= lim;
