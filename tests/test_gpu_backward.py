@@ -186,6 +186,33 @@ def test_sdpa_backward_masked_reduces_to_the_unmasked_and_causal_forms(hip):
             assert rel_err(a.to_host(), b.to_host()) <= TOL_GEMM_F32
 
 
+@pytest.mark.parametrize("bh,sq,sk,d,causal", [(4, 2048, 2048, 128, True), (2, 1024, 1536, 64, False), (3, 1100, 1100, 64, True)])
+def test_fused_sdpa_backward_against_the_materialising_path_at_full_length(hip, bh, sq, sk, d, causal):
+    """Head sizes 64 / 128 without a mask take the fused three-pass backward (scores + statistics, key-owned pass,
+    query-owned pass); the same problem with its mask passed explicitly takes the materialising path (five batched GEMMs
+    around two row passes). Two independent implementations, compared at the benchmark's sequence length and at a
+    ragged one, plus linearity of the fused path in dOut (no checker involved)."""
+    s = 1.0 / math.sqrt(d)
+    q, k, v, do = (synth.normal(31, t, (bh, n, d), 0.0, 1.0) for t, n in (("q", sq), ("k", sk), ("v", sk), ("do", sq)))
+    dq_, dk_, dv_, ddo = _up(q, k, v, do)
+    mask = np.where(np.arange(sk)[None, :] <= np.arange(sq)[:, None], 0.0, -np.inf).astype(np.float32) if causal else np.zeros((sq, sk), np.float32)
+    fused = [DeviceBuffer(q.shape), DeviceBuffer(k.shape), DeviceBuffer(v.shape)]
+    mat = [DeviceBuffer(q.shape), DeviceBuffer(k.shape), DeviceBuffer(v.shape)]
+    ws = hip.sdpa_backward(dq_, dk_, dv_, ddo, bh, sq, sk, d, d, s, causal, *fused)
+    hip.sdpa_backward_masked(dq_, dk_, dv_, ddo, bh, sq, sk, d, d, s, DeviceBuffer.from_host(mask), 0, *mat)
+    f = [b.to_host() for b in fused]
+    for a, b in zip(f, mat):
+        assert rel_err(a, b.to_host()) <= TOL_GEMM_F32
+    # linearity: backward(2 dOut + dOut') = 2 backward(dOut) + backward(dOut')
+    do2 = synth.normal(32, "do2", (bh, sq, d))
+    g2 = [DeviceBuffer(q.shape), DeviceBuffer(k.shape), DeviceBuffer(v.shape)]
+    g3 = [DeviceBuffer(q.shape), DeviceBuffer(k.shape), DeviceBuffer(v.shape)]
+    hip.sdpa_backward(dq_, dk_, dv_, DeviceBuffer.from_host(do2), bh, sq, sk, d, d, s, causal, *g2, workspace=ws)
+    hip.sdpa_backward(dq_, dk_, dv_, DeviceBuffer.from_host(2.0 * do + do2), bh, sq, sk, d, d, s, causal, *g3, workspace=ws)
+    for a, b, c in zip(f, g2, g3):
+        assert rel_err(2.0 * a + b.to_host(), c.to_host()) <= TOL_GEMM_F32
+
+
 def test_host_slice_sdpa_backward_masked_and_its_errors(oracle):
     from frankentorch_amd import kernel_hip as K
     from frankentorch_amd.core import HipError, KernelError
