@@ -444,6 +444,14 @@ template <int N, int I = 0, typename F> __device__ __forceinline__ void static_f
     }
 }
 
+// A pointer every lane holds the same value of, made a scalar for the compiler (two v_readfirstlane_b32 where it
+// had the value in vector registers, nothing where it was scalar already).
+template <typename T> __device__ __forceinline__ const T *uniform_ptr(const T *ptr) {
+    const uint64_t v = reinterpret_cast<uint64_t>(ptr);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const T *>(((uint64_t)hi << 32) | lo);
+}
+
 template <typename T> __device__ __forceinline__ void load_to_lds_16(const T *base, unsigned lane_bytes, unsigned lds_chunk) {
     // Inline assembly so that the compiler's wait-count insertion does not see an LDS write it
     // cannot disambiguate (it would drain the load queue before every LDS read and serialise the
@@ -532,7 +540,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
         const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
         const int a_rows = (int)((p.m - m0) < BM ? (p.m - m0) : BM), b_cols = (int)((p.n - n0) < BN ? (p.n - n0) : BN);
         if constexpr (!TRANS_A) {
-            ak = p.a + batch * p.stride_a + m0 * p.lda + (int64_t)ld_k * BK;
+            ak = uniform_ptr(p.a + batch * p.stride_a + m0 * p.lda + (int64_t)ld_k * BK);
 #pragma unroll
             for (int i = 0; i < A_LD; ++i) {
                 int row = (wave * A_LD + i) * 8 + lr;
@@ -540,7 +548,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
                 a_off[i] = ((unsigned)row * (unsigned)p.lda + (unsigned)lvec(wave * A_LD + i)) * (unsigned)sizeof(T);
             }
         } else {
-            ak = p.a + batch * p.stride_a + (int64_t)ld_k * BK * p.lda + m0;
+            ak = uniform_ptr(p.a + batch * p.stride_a + (int64_t)ld_k * BK * p.lda + m0);
             int col = (lane % LPR_A) * EPV;
             col = col < a_rows ? col : a_rows - EPV;  // m is a multiple of EPV on this path
 #pragma unroll
@@ -550,7 +558,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
             }
         }
         if constexpr (TRANS_B) {
-            bk = p.b + batch * p.stride_b + n0 * p.ldb + (int64_t)ld_k * BK;
+            bk = uniform_ptr(p.b + batch * p.stride_b + n0 * p.ldb + (int64_t)ld_k * BK);
 #pragma unroll
             for (int i = 0; i < B_LD; ++i) {
                 int row = (wave * B_LD + i) * 8 + lr;
@@ -558,7 +566,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
                 b_off[i] = ((unsigned)row * (unsigned)p.ldb + (unsigned)lvec(wave * B_LD + i)) * (unsigned)sizeof(T);
             }
         } else {
-            bk = p.b + batch * p.stride_b + (int64_t)ld_k * BK * p.ldb + n0;
+            bk = uniform_ptr(p.b + batch * p.stride_b + (int64_t)ld_k * BK * p.ldb + n0);
             int col = (lane % LPR) * EPV;
             col = col < b_cols ? col : b_cols - EPV;  // n is a multiple of EPV on this path
 #pragma unroll
