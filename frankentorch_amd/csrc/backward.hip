@@ -797,19 +797,19 @@ int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, i
     const int64_t rows = num_bh * seq_q;
     FTH_ARG(fth::ceil_div(rows, kWaves) <= 2147483647LL, "sdpa backward: too many rows");
     if constexpr (std::is_same<T, float>::value) {
-        // Fused path: the forward kernel's preparation pass (scores, log-sum-exp, delta), one key-owned kernel for dS,
-        // dK and dV, and the dQ product. P and dU are never materialised.
+        // Fused path: a statistics pass (scores, dP, log-sum-exp, delta), one key-owned kernel for dS, dK and dV, and
+        // the dQ product. P and dU are never materialised.
         auto al = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; };
         if (!mask && fth::sdpa_backward_fused_applies(num_bh, seq_q, seq_k, d_k, d_v, scale) && al(q) && al(k) && al(v) && al(dout) &&
             al(dq) && al(dk) && al(dv) && al(workspace)) {
             float *lse = p + ((2 * pe + 64 + 3) & ~(int64_t)3) + (unit_dout ? ((seq_q * d_v + 4 + 3) & ~(int64_t)3) : 0);  // behind the ones plane
             lse = reinterpret_cast<float *>((reinterpret_cast<uintptr_t>(lse) + 15u) & ~(uintptr_t)15u);
             float *delta = lse + ((rows + 3) & ~(int64_t)3);
-            if (int32_t rc = fth::sdpa_backward_prepare_f32(q, k, v, dout, dout_bs, num_bh, seq_q, seq_k, d_k, scale, causal, p, lse, delta, st))
+            if (int32_t rc = fth::sdpa_backward_stats_f32(q, k, v, dout, dout_bs, num_bh, seq_q, seq_k, d_k, scale, causal, p, du, lse, delta, st))
                 return rc;
             // (under a causal mask the key pass writes dS from each key block's own first row on: all the dQ pass reads)
-            if (int32_t rc = fth::sdpa_backward_keys_f32(q, v, dout, dout_bs, p, lse, delta, num_bh, seq_q, seq_k, d_k, scale, causal, 128, du,
-                                                        dk, dv, st))
+            if (int32_t rc = fth::sdpa_backward_keys_f32(q, dout, dout_bs, p, lse, delta, num_bh, seq_q, seq_k, d_k, scale, causal, 128, du, dk,
+                                                        dv, st))
                 return rc;
             return fth::sdpa_backward_dq_f32(du, k, num_bh, seq_q, seq_k, d_k, scale, causal, dq, st);
         }

@@ -33,7 +33,6 @@
 
 #include "common.hpp"
 #include "devmath.hpp"
-#include "sdpa_bwd.hpp"
 
 namespace {
 
@@ -55,13 +54,6 @@ struct SdpaArgs {
     int64_t mask_bh_stride;  // 0: one mask for every (batch, head); else elements between consecutive bh
     int64_t group;           // query heads per K/V head (grouped-query attention), >= 1
     int mask_vec;            // mask rows can be read as aligned float4 (seq_k % 4 == 0, 16-byte aligned base and bh stride)
-    // Backward preparation pass (BWD instantiation of the fp32 MFMA kernel): instead of the output it leaves what the
-    // backward kernels need -- the raw scores Q.K^T as [num_bh, seq_q, seq_k], the log-sum-exp of every row in log2
-    // units (P = 2^(s * scale * log2e - lse)) and delta = sum_d dOut[i, d] * Out[i, d] -- all [num_bh, seq_q]-shaped
-    // operands contiguous, dout [num_bh, seq_q, d].
-    const float *dout;
-    int64_t dout_bh_stride;
-    float *s_out, *lse_out, *delta_out;
 };
 
 // exp(x - m) for x <= m as 2^((x - m) * log2 e) on the hardware exp2 unit: subtract, multiply,
@@ -120,9 +112,8 @@ __device__ __forceinline__ float f4_get(const float4 &v, int e) { return e == 0 
 // past seq_k are clamped to the last row (their scores are masked, their weights are zero).
 // MASK: an additive mask row is read for every (query, key) score, mask[bh * mask_bh_stride + qi * seq_k + key]
 // (sdpa_forward_masked_f64, crates/ft-kernel-cpu/src/lib.rs:4661-4741): score * scale + mask, then the same softmax.
-template <int D, int NW, bool PAIR, int BC, bool DIRECT, bool MASK, bool BWD = false>
+template <int D, int NW, bool PAIR, int BC, bool DIRECT, bool MASK>
 __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p) {
-    static_assert(!BWD || (!MASK && !PAIR), "the backward preparation pass is unmasked and unpaired");
     constexpr int kBC = BC;
     constexpr int KS = BC / 32;        // 32-key sub-tiles per tile
     constexpr int NTH = 64 * NW;
@@ -361,24 +352,6 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
                     }
                 }
             }
-            if constexpr (BWD) {
-                // raw scores of this wavefront's 32 queries x the tile's keys: lane (query qi) holds four runs of four
-                // consecutive keys per 32-key sub-tile (seq_k is a multiple of 4 on this path: no run straddles the row end)
-                if (wave_active && q_live) {
-                    float *srow = p.s_out + ((int64_t)bh * seq_q_i + qi) * seq_k_i;
-#pragma unroll
-                    for (int j = 0; j < KS; ++j)
-#pragma unroll
-                        for (int g = 0; g < 4; ++g) {
-                            const int key = key0 + 32 * j + 8 * g + 4 * half;
-                            if (key < seq_k_i) {
-                                // ordinary stores: the eight 16-byte pieces of a 128-byte line come from four instructions of
-                                // two lanes and merge in L2 before the line goes to HBM
-                                *reinterpret_cast<float4 *>(srow + key) = make_float4(s[j][4 * g + 0], s[j][4 * g + 1], s[j][4 * g + 2], s[j][4 * g + 3]);
-                            }
-                        }
-                }
-            }
             // The next tile's global loads are issued here, after the score MFMAs and before the
             // softmax: their latency is covered by the softmax and the P.V MFMAs, and their address
             // temporaries cannot be handed the registers the score accumulator is about to claim
@@ -507,27 +480,6 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
             l_run = llo + lhi;
         }
 
-        if constexpr (BWD) {
-            // ---- row statistics for the backward pass: lse in log2 units, delta = dOut . Out ----
-            float part = 0.f;
-            if (q_live) {
-                const float *drow = p.dout + bh * p.dout_bh_stride + (int64_t)qi * D;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int rho = 8 * (r >> 2) + 4 * half + (r & 3);
-                    const VV dv = *reinterpret_cast<const VV *>(drow + NDT * rho);
-#pragma unroll
-                    for (int e = 0; e < NDT; ++e) part += o[e][r] * vecn_get(dv, e);
-                }
-            }
-            float plo, phi;
-            both_halves(part, plo, phi);
-            if (q_live && half == 0) {
-                p.lse_out[(int64_t)bh * seq_q_i + qi] = m_run + __builtin_amdgcn_logf(l_run);  // v_log_f32 is log2
-                p.delta_out[(int64_t)bh * seq_q_i + qi] = (plo + phi) / l_run;
-            }
-            continue;
-        }
         // ---- normalise and store: lane owns query qi, d = NDT * rho + e ----
         if (q_live) {
             float *orow = O + (int64_t)qi * d.o_row_stride;
@@ -865,11 +817,11 @@ template <int D> int32_t launch_mfma_f64(SdpaArgs &a, hipStream_t st) {
     return FTH_OK;
 }
 
-template <int D, int NW, bool PAIR, bool MASK, bool BWD = false> int32_t launch_mfma_cfg(SdpaArgs &a, hipStream_t st) {
+template <int D, int NW, bool PAIR, bool MASK> int32_t launch_mfma_cfg(SdpaArgs &a, hipStream_t st) {
     constexpr int BC = (D <= 64 && (NW == 4 || D <= 32)) ? 64 : 32;  // 64-key tiles where two workgroups still fit a CU
     constexpr bool DIRECT = D >= 64 && FTH_SDPA_DIRECT;
     constexpr size_t smem = DIRECT ? (size_t)2 * BC * 2 * D * sizeof(float) : (size_t)2 * BC * ((D + 4) + (D + 8)) * sizeof(float);
-    auto kern = sdpa_mfma_kernel<D, NW, PAIR, BC, DIRECT, MASK, BWD>;
+    auto kern = sdpa_mfma_kernel<D, NW, PAIR, BC, DIRECT, MASK>;
     static bool attr_set = false;
     if (!attr_set) {
         FTH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -1079,7 +1031,6 @@ int32_t sdpa_entry(const fth_sdpa_desc *d, double scale, const T *q, const T *k,
     a.mask_bh_stride = mask_bh_stride;
     a.group = group;
     a.mask_vec = (d->seq_k % 4 == 0 && mask_bh_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(mask) & 15u) == 0) ? 1 : 0;
-    a.dout = nullptr; a.dout_bh_stride = 0; a.s_out = nullptr; a.lse_out = nullptr; a.delta_out = nullptr;
     auto al16 = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; };
     auto m4 = [](int64_t x) { return x % 4 == 0; };
     if constexpr (std::is_same<T, float>::value) {
@@ -1136,25 +1087,6 @@ int32_t sdpa_entry(const fth_sdpa_desc *d, double scale, const T *q, const T *k,
 }
 
 }  // namespace
-
-namespace fth {
-// The backward preparation pass on contiguous [num_bh, seq, d] fp32 operands, d in {64, 128}, seq_k a multiple of 4,
-// scale > 0: raw scores into s_out [num_bh, seq_q, seq_k] (only the entries a causal problem uses are written), the
-// rows' log-sum-exp (log2 units) and delta = dOut . Out.
-int32_t sdpa_backward_prepare_f32(const float *q, const float *k, const float *v, const float *dout, int64_t dout_bh_stride,
-                                  int64_t num_bh, int64_t seq_q, int64_t seq_k, int64_t d, float scale, int causal, float *s_out,
-                                  float *lse_out, float *delta_out, hipStream_t st) {
-    SdpaArgs a;
-    fth_sdpa_desc_contiguous(&a.d, num_bh, seq_q, seq_k, d, d, causal);
-    a.q = q; a.k = k; a.v = v; a.out = nullptr; a.scale = scale;
-    a.q_blocks = 0;
-    a.mask = nullptr; a.mask_bh_stride = 0; a.group = 1; a.mask_vec = 0;
-    a.dout = dout; a.dout_bh_stride = dout_bh_stride; a.s_out = s_out; a.lse_out = lse_out; a.delta_out = delta_out;
-    if (d == 128) return launch_mfma_cfg<128, 4, false, false, true>(a, st);
-    if (d == 64) return launch_mfma_cfg<64, 4, false, false, true>(a, st);
-    return fth::set_error(FTH_ERR_INVALID_ARGUMENT, "sdpa_backward_prepare: head size %lld", (long long)d);
-}
-}  // namespace fth
 
 extern "C" {
 

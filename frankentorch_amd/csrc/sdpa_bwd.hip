@@ -1,32 +1,29 @@
-// Fused key-owned and query-owned passes of the fp32 scaled-dot-product-attention backward for gfx950
-// (sdpa_backward_f32, crates/ft-kernel-cpu/src/lib.rs:5539-5650; the unit-dOut form :5662-5770).
+// Fused fp32 scaled-dot-product-attention backward for gfx950: a query-owned statistics pass, a key-owned pass and a
+// query-owned dQ pass (sdpa_backward_f32, crates/ft-kernel-cpu/src/lib.rs:5539-5650; the unit-dOut form :5662-5770).
 //
 // The reference materialises P = softmax(scale Q K^T) and dU per (batch, head) and runs five
-// products around two row passes. Here the work is three launches on [num_bh, seq, D] operands:
-//   1. the forward kernel's preparation instantiation (csrc/sdpa.hip): raw scores S = Q K^T to
-//      HBM, per-row log-sum-exp and delta = dOut . Out          (products S and P V);
-//   2. this kernel, one workgroup per block of 128 keys walking the query tiles it can see:
-//      P = 2^(S c - lse), dP = dOut V^T, dS = scale P (dP - delta) written to HBM,
-//      dV += P^T dOut, dK += dS^T Q in registers                 (products dP, dV, dK);
-//   3. a query-owned kernel, dQ = scale dS K with dS read in the accumulator layout of pass 2   (product dQ).
-// Six product-sized MFMA passes instead of five, but P and dU never make the round trip through
-// HBM between separate softmax and softmax-gradient row passes: per call S is written once and
-// read once, dS written once and read once. A recompute design that keeps nothing in HBM needs
-// eight to nine product passes (the statistics, then four in a key-owned and three in a
-// query-owned kernel); on fp32 matrix cores a product pass costs more than the HBM traffic it saves.
+// products around two row passes. Here the work is three launches on [num_bh, seq, D] operands,
+// with the reference's five products and no sixth:
+//   1. statistics, one workgroup per 128 queries walking the key tiles they can see: raw scores S = Q K^T and
+//      dP = dOut V^T to HBM, and per row the log-sum-exp and delta = sum_j P_ij dP_ij (the reference's `dot`), both
+//      from one online pass over the tiles                          (products S and dP);
+//   2. one workgroup per block of 128 keys walking the query tiles it can see:
+//      P = 2^(S c - lse), dS = P (dP - delta) written over dP,
+//      dV += P^T dOut, dK += dS^T Q in registers                    (products dV and dK);
+//   3. dQ = scale dS K with dS read in the accumulator layout of pass 2   (product dQ).
+// P and dU never make the round trip through HBM between separate softmax and softmax-gradient row passes: per call S
+// and dP are written once and read once, dS written once (in place of dP) and read once. A recompute design that keeps
+// nothing in HBM needs eight to nine product passes; on fp32 matrix cores a product pass costs more than the HBM
+// traffic it saves.
 //
-// MFMA layout (v_mfma_f32_32x32x2_f32; a wavefront owns 32 keys, the block's four wavefronts share
+// MFMA layout of pass 2 (v_mfma_f32_32x32x2_f32; a wavefront owns 32 keys, the block's four wavefronts share
 // each 32-query tile of Q and dOut through double-buffered LDS):
-//   dP[q, key]     = dOut_tile . V_blk^T    A = dOut rows from LDS (one 128-bit read feeds four MFMAs),
-//                                           B = the wavefront's V rows, resident in registers.
-//   In the accumulator a lane holds ONE key (lane % 32) and 16 of the tile's 32 queries, so S, lse,
-//   delta, P and dS are lane-local, and P / dS are the B operands of the next two products as
-//   they stand (MFMA step r contracts over exactly the two queries that register r holds):
+//   S and dP arrive from HBM in the accumulator layout of a [query, key] product: a lane holds ONE key (lane % 32) and
+//   16 of the tile's 32 queries, so S, dP, lse, delta, P and dS are lane-local, and P / dS are the B operands of the
+//   two products as they stand (MFMA step r contracts over exactly the two queries that register r holds):
 //   dV^T[d, key]  += dOut_tile^T . P        A = dOut read along d (lane = d index)
 //   dK^T[d, key]  += Q_tile^T . dS          A = Q read along d
-// dOut is read in both directions, so its LDS image is XOR-swizzled (logical 16-byte vector v of
-// tile row r in slot v ^ (r & 15)); Q is read along d only and stays in row order. No atomics:
-// each (key, d) of dK / dV is summed by one wavefront in query order, so runs are bitwise repeatable.
+// No atomics: each (key, d) of dK / dV is summed by one wavefront in query order, so runs are bitwise repeatable.
 
 #include <cstdlib>
 #include <type_traits>
@@ -37,12 +34,16 @@
 namespace {
 
 constexpr int kWave = 64;
+#ifndef FTH_SDPA_BWD_KEYS_OCC
+#define FTH_SDPA_BWD_KEYS_OCC 1
+#endif
 using Acc16 = float __attribute__((ext_vector_type(16)));
 typedef float nat_f4 __attribute__((ext_vector_type(4)));
 
 struct KeysArgs {
-    const float *q, *v, *dout, *s, *lse, *delta;
-    float *ds, *dk, *dv;
+    const float *q, *dout, *s, *lse, *delta;
+    float *dpds;  // dP in, dS out, element for element
+    float *dk, *dv;
     int64_t num_bh, dout_bh_stride;
     int seq_q, seq_k;
     float scale;
@@ -72,8 +73,277 @@ __device__ __forceinline__ float vecn_get(const float2 &v, int e) { return e == 
 __device__ __forceinline__ float vecn_get(const float4 &v, int e) { return e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w; }
 __device__ __forceinline__ float f4_get(const float4 &v, int e) { return e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w; }
 
+// x of lanes 0..31 and x of lanes 32..63, each broadcast to both halves (one v_permlane32_swap, no LDS round trip).
+__device__ __forceinline__ void both_halves(float x, float &lo, float &hi) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    lo = __uint_as_float(r[0]);
+    hi = __uint_as_float(r[1]);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Statistics pass. One workgroup per 128 queries (a wavefront owns 32; a lane one query, whose Q and dOut rows it keeps
+// in registers as B operands), walking BC-key tiles of K and V through double-buffered LDS:
+//   S^T[key, q]  = K_tile . Q^T,   dP^T[key, q] = V_tile . dOut^T      (the same product shape twice)
+// In the accumulators a lane holds its query's scores and dP against 16 keys per 32-key sub-tile, so the row maximum,
+// the row sum and delta = sum_j P_ij dP_ij need no exchange between lanes until the very end (the two halves of a
+// wavefront hold the same queries against different keys). The reference weight 2^m of a row moves only when a score
+// exceeds it by more than kLazy (log2 units): both running sums are then rescaled, which happens a few times per row.
+// Both tiles are read one 16-byte vector per lane with 16 consecutive lanes on 16 consecutive rows, so logical vector
+// v of tile row r is stored in slot v ^ (r & 15) (the permutation applied on the global side of the copy).
+// ---------------------------------------------------------------------------------------------
+struct StatsArgs {
+    const float *q, *k, *v, *dout;
+    float *s, *dp, *lse, *delta;
+    int64_t num_bh, dout_bh_stride;
+    int seq_q, seq_k;
+    float scale;
+    int causal;
+};
+
+template <int D, int BC>
+__global__ __launch_bounds__(256, 2) void sdpa_bwd_stats_kernel(const StatsArgs p) {
+    constexpr int KS = BC / 32;        // 32-key sub-tiles per tile
+    constexpr int VPR = D / 4;         // 16-byte vectors per row
+    constexpr int RPC = 64 / VPR;      // tile rows per 1 KiB load instruction
+    constexpr int CPW = BC / RPC / 4;  // load instructions per wavefront per operand tile
+    constexpr int TILE = BC * D;       // floats per operand tile
+    constexpr int NST = 2 * KS * 4;    // 16-byte stores per wavefront and tile
+    static_assert(NST == 8 || NST == 16, "the end-of-tile wait is written for 8 or 16 stores");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    float *Ks = reinterpret_cast<float *>(smem_raw);  // [2][BC][D], swizzled
+    float *Vs = Ks + 2 * TILE;                        // [2][BC][D], swizzled
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lq = lane & 31, half = lane >> 5;
+    const int seq_q = p.seq_q, seq_k = p.seq_k;
+    const int q_blocks = (seq_q + 127) / 128;
+    // Query blocks are issued heaviest (latest) first across all heads, and when the head count allows it every query
+    // block of a head lands on the same XCD, whose L2 then serves the head's K and V to all of them.
+    int64_t bh;
+    int unit;
+    {
+        const int64_t pid = blockIdx.x;
+        if (p.num_bh % 8 == 0) {
+            const int64_t xcd = pid % 8, w = pid / 8, per = p.num_bh / 8;
+            unit = (int)(w / per);
+            bh = (w % per) * 8 + xcd;
+        } else {
+            unit = (int)(pid / p.num_bh);
+            bh = pid % p.num_bh;
+        }
+    }
+    const int qb = q_blocks - 1 - unit;
+    const int q_blk0 = qb * 128, q_wave0 = q_blk0 + 32 * wave, qi = q_wave0 + lq;
+    const bool q_live = qi < seq_q;
+    const float *Kg = p.k + bh * (int64_t)seq_k * D, *Vg = p.v + bh * (int64_t)seq_k * D;
+    const float c2 = p.scale * 1.44269502162933349609375f;  // scale * log2(e)
+
+    // ---- Q and dOut rows into registers: lane holds row[8 t + 4 half + e] ----
+    float4 qr[D / 8], dor[D / 8];
+    {
+        const int qc = q_live ? qi : seq_q - 1;
+        const float *qrow = p.q + (bh * (int64_t)seq_q + qc) * D + 4 * half;
+        const float *drow = p.dout + bh * p.dout_bh_stride + (int64_t)qc * D + 4 * half;
+#pragma unroll
+        for (int t = 0; t < D / 8; ++t) {
+            qr[t] = *reinterpret_cast<const float4 *>(qrow + 8 * t);
+            dor[t] = *reinterpret_cast<const float4 *>(drow + 8 * t);
+        }
+    }
+
+    int blk_last_q = q_blk0 + 127, wave_last_q = q_wave0 + 31;
+    if (blk_last_q > seq_q - 1) blk_last_q = seq_q - 1;
+    if (wave_last_q > seq_q - 1) wave_last_q = seq_q - 1;
+    int k_end = seq_k;
+    if (p.causal && blk_last_q + 1 < k_end) k_end = blk_last_q + 1;
+    const int num_kt = (k_end + BC - 1) / BC;
+
+    // ---- tile loader: this wavefront owns CPW 1 KiB chunks of each tile; lane L of chunk c covers tile row
+    //      c RPC + L / VPR, physical vector slot L % VPR ----
+    const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)reinterpret_cast<uintptr_t>(smem_raw));
+    const unsigned wave_u = __builtin_amdgcn_readfirstlane((unsigned)wave);
+    int ld_row[CPW];
+    unsigned ld_col[CPW];
+#pragma unroll
+    for (int ci = 0; ci < CPW; ++ci) {
+        const int trow = (wave * CPW + ci) * RPC + lane / VPR;
+        const int slot = lane % VPR;
+        ld_row[ci] = trow;
+        ld_col[ci] = 16u * (unsigned)((slot & ~15) | ((slot ^ trow) & 15));  // the logical vector that lives in this slot
+    }
+    auto issue_tile = [&](int kt, int buf) __attribute__((always_inline)) {
+        const int row0 = kt * BC;
+        const unsigned kdst = lds0 + (unsigned)(buf * TILE * 4) + wave_u * (CPW * 1024u);
+        const unsigned vdst = lds0 + (unsigned)((2 * TILE + buf * TILE) * 4) + wave_u * (CPW * 1024u);
+#pragma unroll
+        for (int ci = 0; ci < CPW; ++ci) {
+            int row = row0 + ld_row[ci];
+            row = row < seq_k ? row : seq_k - 1;  // rows past the end repeat the last one: their scores are masked
+            const unsigned off = (unsigned)row * (unsigned)(D * 4) + ld_col[ci];
+            load_to_lds_16(Kg, off, kdst + ci * 1024u);
+            load_to_lds_16(Vg, off, vdst + ci * 1024u);
+        }
+    };
+
+    // ---- S and dP out through range-checked buffer stores: the lane part (its query's row, its half's keys; "nowhere"
+    //      for a query past the end) in the vector offset, the tile part in the scalar offset ----
+    constexpr unsigned kOut = 0x40000000u;
+    constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
+    const unsigned row_bytes = (unsigned)seq_k * 4u, slab_bytes = (unsigned)seq_q * row_bytes;
+    const __amdgpu_buffer_rsrc_t rs_s =
+        __builtin_amdgcn_make_buffer_rsrc(p.s + bh * (int64_t)seq_q * seq_k, 0, (int)slab_bytes, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rs_dp =
+        __builtin_amdgcn_make_buffer_rsrc(p.dp + bh * (int64_t)seq_q * seq_k, 0, (int)slab_bytes, kRsrcFlags);
+    const unsigned lane_st = q_live ? (unsigned)qi * row_bytes + 16u * (unsigned)half : kOut;
+    typedef unsigned u4v __attribute__((ext_vector_type(4)));
+
+    // fragment read t of tile row lq: vector 2 t + half sits in slot (2 t) ^ lx (bits 1..3 take eight per-lane values,
+    // bit 4 is 2 t's own), lx = half ^ (lq & 15)
+    const int lx = half ^ (lq & 15);
+    int frag[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) frag[u] = lq * D + 4 * (((2 * u) ^ lx) & 15);
+
+    constexpr float kLazy = 6.0f;
+    float m_run = -__builtin_inff(), l_run = 0.f, a_run = 0.f;
+
+    if (num_kt > 0) issue_tile(0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): own tile parts have landed
+    __syncthreads();
+
+    auto tile_step = [&](const int kt, auto buf_c) __attribute__((always_inline)) {
+        constexpr int buf = decltype(buf_c)::value;
+        const int key0 = kt * BC;
+        if (kt + 1 < num_kt) issue_tile(kt + 1, buf ^ 1);
+        // A wavefront whose every query precedes this tile's first key has nothing to add.
+        const bool wave_active = !p.causal || key0 <= wave_last_q;
+        if (wave_active) {
+            Acc16 s[KS], dp[KS];
+#pragma unroll
+            for (int j = 0; j < KS; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    s[j][r] = 0.f;
+                    dp[j][r] = 0.f;
+                }
+            const float *kb = Ks + buf * TILE, *vb = Vs + buf * TILE;
+#pragma unroll
+            for (int t = 0; t < D / 8; ++t) {
+#pragma unroll
+                for (int j = 0; j < KS; ++j) {
+                    const int off = frag[t & 7] + j * 32 * D + 4 * ((2 * t) & 16);
+                    const float4 kv = *reinterpret_cast<const float4 *>(kb + off);
+                    const float4 vv = *reinterpret_cast<const float4 *>(vb + off);
+                    s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.x, qr[t].x, s[j], 0, 0, 0);
+                    s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.y, qr[t].y, s[j], 0, 0, 0);
+                    s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.z, qr[t].z, s[j], 0, 0, 0);
+                    s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.w, qr[t].w, s[j], 0, 0, 0);
+                    dp[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, dor[t].x, dp[j], 0, 0, 0);
+                    dp[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, dor[t].y, dp[j], 0, 0, 0);
+                    dp[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.z, dor[t].z, dp[j], 0, 0, 0);
+                    dp[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.w, dor[t].w, dp[j], 0, 0, 0);
+                }
+            }
+            // ---- raw scores and dP of this wavefront's 32 queries x the tile's keys: a lane holds four runs of four
+            //      consecutive keys per sub-tile (seq_k is a multiple of 4 on this path: no run straddles the row end) ----
+            const bool tail = key0 + BC > seq_k;  // uniform
+            auto store_tile = [&](auto tail_c) __attribute__((always_inline)) {
+#pragma unroll
+                for (int j = 0; j < KS; ++j)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        unsigned v = lane_st + (unsigned)(32 * j + 8 * g) * 4u;
+                        if constexpr (decltype(tail_c)::value)
+                            if (key0 + 32 * j + 8 * g + 4 * half >= seq_k) v = kOut;
+                        // (element by element through float temporaries: a bit cast applied to a vector element directly reads element 0)
+                        const float s0 = s[j][4 * g + 0], s1 = s[j][4 * g + 1], s2 = s[j][4 * g + 2], s3 = s[j][4 * g + 3];
+                        const float d0 = dp[j][4 * g + 0], d1 = dp[j][4 * g + 1], d2 = dp[j][4 * g + 2], d3 = dp[j][4 * g + 3];
+                        const u4v sv = {__builtin_bit_cast(unsigned, s0), __builtin_bit_cast(unsigned, s1), __builtin_bit_cast(unsigned, s2),
+                                        __builtin_bit_cast(unsigned, s3)};
+                        const u4v dv = {__builtin_bit_cast(unsigned, d0), __builtin_bit_cast(unsigned, d1), __builtin_bit_cast(unsigned, d2),
+                                        __builtin_bit_cast(unsigned, d3)};
+                        __builtin_amdgcn_raw_buffer_store_b128(sv, rs_s, v, (unsigned)key0 * 4u, 0);
+                        __builtin_amdgcn_raw_buffer_store_b128(dv, rs_dp, v, (unsigned)key0 * 4u, 0);
+                    }
+            };
+            if (tail) store_tile(std::true_type{});
+            else store_tile(std::false_type{});
+            // ---- online row statistics (lane-local query) ----
+            const bool need_mask = (p.causal && key0 + BC - 1 > q_wave0) || tail;
+            if (need_mask) {  // wavefront-uniform; selects, no per-element branches
+#pragma unroll
+                for (int j = 0; j < KS; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int key = key0 + 32 * j + 8 * (r >> 2) + 4 * half + (r & 3);
+                        const bool hidden = (p.causal && key > qi) | (key >= seq_k);
+                        s[j][r] = hidden ? -__builtin_inff() : s[j][r];
+                    }
+            }
+            float mt = -__builtin_inff();
+#pragma unroll
+            for (int j = 0; j < KS; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) mt = fmaxf(mt, s[j][r]);
+            if (__any(mt * c2 > m_run + kLazy)) {
+                float mlo, mhi;
+                both_halves(mt, mlo, mhi);
+                const float m_new = fmaxf(m_run, fmaxf(mlo, mhi) * c2);
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                l_run *= alpha;
+                a_run *= alpha;
+                m_run = m_new;
+            }
+            const float neg_m = -m_run;
+#pragma unroll
+            for (int j = 0; j < KS; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][r], c2, neg_m));
+                    l_run += e;
+                    a_run = __builtin_fmaf(e, dp[j][r], a_run);
+                }
+            // the stores of this tile may stay in flight; the copies issued before them may not (in-order completion)
+            if constexpr (NST == 8) __builtin_amdgcn_s_waitcnt(0x0F78);
+            else __builtin_amdgcn_s_waitcnt(0x4F70);
+        } else {
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+        }
+        __syncthreads();
+    };
+    for (int kt = 0; kt < num_kt; kt += 2) {
+        tile_step(kt, std::integral_constant<int, 0>{});
+        if (kt + 1 < num_kt) tile_step(kt + 1, std::integral_constant<int, 1>{});
+    }
+    // the two halves of the wavefront hold partial sums of the same queries
+    float llo, lhi, alo, ahi;
+    both_halves(l_run, llo, lhi);
+    both_halves(a_run, alo, ahi);
+    if (q_live && half == 0) {
+        const float l = llo + lhi;
+        p.lse[bh * (int64_t)seq_q + qi] = m_run + __builtin_amdgcn_logf(l);  // v_log_f32 is log2
+        p.delta[bh * (int64_t)seq_q + qi] = (alo + ahi) / l;
+    }
+}
+
+template <int D> int32_t launch_stats(const StatsArgs &a, hipStream_t st) {
+    constexpr int BC = D <= 64 ? 64 : 32;  // two workgroups per compute unit either way
+    constexpr size_t smem = (size_t)2 * 2 * BC * D * sizeof(float);
+    static bool attr_set = false;
+    if (!attr_set) {
+        FTH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(sdpa_bwd_stats_kernel<D, BC>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem));
+        attr_set = true;
+    }
+    const int64_t grid = a.num_bh * fth::ceil_div(a.seq_q, 128);
+    FTH_ARG(grid <= 2147483647LL, "sdpa backward: grid too large");
+    sdpa_bwd_stats_kernel<D, BC><<<dim3((unsigned)grid), dim3(256), smem, st>>>(a);
+    FTH_CHECK_LAUNCH("sdpa_bwd_stats");
+    return FTH_OK;
+}
+
 template <int D>
-__global__ __launch_bounds__(256, 1) void sdpa_bwd_keys_kernel(const KeysArgs p) {
+__global__ __launch_bounds__(256, FTH_SDPA_BWD_KEYS_OCC) void sdpa_bwd_keys_kernel(const KeysArgs p) {
     constexpr int NDT = D / 32;        // 32-wide d-tiles of dK^T / dV^T
     constexpr int VPR = D / 4;         // 16-byte vectors per row
     constexpr int RPC = 64 / VPR;      // tile rows per 1 KiB load instruction
@@ -82,7 +352,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_keys_kernel(const KeysArgs p)
     using VV = typename VecN<NDT>::type;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     float *Qs = reinterpret_cast<float *>(smem_raw);  // [2][32][D], row order
-    float *Os = Qs + 2 * TILE;                        // [2][32][D], swizzled
+    float *Os = Qs + 2 * TILE;                        // [2][32][D], row order
     float *Ls = Os + 2 * TILE;                        // [2][2][64]: log-sum-exp and delta of the tile's queries (32 used)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -93,21 +363,12 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_keys_kernel(const KeysArgs p)
     const int seq_q = p.seq_q, seq_k = p.seq_k;
     const int key0 = kb * 128, kw0 = key0 + 32 * wave, kw = kw0 + lq;
     const bool key_live = kw < seq_k;
-    const int kc = key_live ? kw : seq_k - 1;
     const float *Qg = p.q + bh * (int64_t)seq_q * D;
     const float *Og = p.dout + bh * p.dout_bh_stride;
     const float *Sg = p.s + bh * (int64_t)seq_q * seq_k;
-    float *DSg = p.ds + bh * (int64_t)seq_q * seq_k;
+    float *DSg = p.dpds + bh * (int64_t)seq_q * seq_k;
     const float *Lg = p.lse + bh * (int64_t)seq_q, *Dg = p.delta + bh * (int64_t)seq_q;
     const float c2 = p.scale * 1.44269502162933349609375f;  // scale * log2(e): the statistics are in log2 units
-
-    // V rows of this lane's key: V[kc][8 t + 4 half + e]
-    float4 vr[D / 8];
-    {
-        const float *vrow = p.v + (bh * (int64_t)seq_k + kc) * D + 4 * half;
-#pragma unroll
-        for (int t = 0; t < D / 8; ++t) vr[t] = *reinterpret_cast<const float4 *>(vrow + 8 * t);
-    }
 
     int q_lo = 0;
     if (p.causal) q_lo = p.row_block > 0 ? (key0 / p.row_block) * p.row_block : 0;
@@ -117,16 +378,9 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_keys_kernel(const KeysArgs p)
     const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)reinterpret_cast<uintptr_t>(smem_raw));
     const unsigned wave_u = __builtin_amdgcn_readfirstlane((unsigned)wave);
     int ld_row[CPW];
-    unsigned q_col[CPW], o_col[CPW];  // byte offsets inside a row
 #pragma unroll
-    for (int ci = 0; ci < CPW; ++ci) {
-        const int trow = (wave * CPW + ci) * RPC + lane / VPR;
-        const int slot = lane % VPR;
-        const int oq = (slot & ~15) | ((slot ^ trow) & 15);  // the logical vector that lives in physical slot `slot` of dOut's image
-        ld_row[ci] = trow;
-        q_col[ci] = 16u * (unsigned)slot;
-        o_col[ci] = 16u * (unsigned)oq;
-    }
+    for (int ci = 0; ci < CPW; ++ci) ld_row[ci] = (wave * CPW + ci) * RPC + lane / VPR;
+    const unsigned ld_col = 16u * (unsigned)(lane % VPR);  // byte offset inside a row
     auto issue_tile = [&](int t, int buf) __attribute__((always_inline)) {
         const int row0 = q_lo + 32 * t;
         const unsigned qdst = lds0 + (unsigned)(buf * TILE * 4) + wave_u * (CPW * 1024u);
@@ -135,8 +389,9 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_keys_kernel(const KeysArgs p)
         for (int ci = 0; ci < CPW; ++ci) {
             int row = row0 + ld_row[ci];
             row = row < seq_q ? row : seq_q - 1;
-            load_to_lds_16(Qg, (unsigned)row * (unsigned)(D * 4) + q_col[ci], qdst + ci * 1024u);
-            load_to_lds_16(Og, (unsigned)row * (unsigned)(D * 4) + o_col[ci], odst + ci * 1024u);
+            const unsigned off = (unsigned)row * (unsigned)(D * 4) + ld_col;
+            load_to_lds_16(Qg, off, qdst + ci * 1024u);
+            load_to_lds_16(Og, off, odst + ci * 1024u);
         }
         if (wave_u < 2) {  // wavefront 0 brings the log-sum-exps, wavefront 1 the deltas: one dword per lane
             int row = row0 + lane;
@@ -145,22 +400,9 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_keys_kernel(const KeysArgs p)
         }
     };
 
-    // ---- per-lane LDS read offsets ----
-    // dP product: 128-bit vector 2 t + half of tile row lq sits in slot (2 t) ^ lx (bits 1..3 take eight per-lane values,
-    // bit 4 is 2 t's own), lx = half ^ (lq & 15).
-    const int lx = half ^ (lq & 15);
-    int ofrag[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) ofrag[u] = lq * D + 4 * (((2 * u) ^ lx) & 15);
-    // dV product: elements d = NDT lq .. NDT lq + NDT - 1 of tile row qrow(r) = 8 (r / 4) + 4 half + r % 4
-    int ovec[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int qrow = 8 * (r >> 2) + 4 * half + (r & 3);
-        const int lv = (NDT * lq) / 4, within = (NDT * lq) % 4;
-        ovec[r] = qrow * D + 4 * ((lv & ~15) | ((lv ^ qrow) & 15)) + within;
-    }
-    const int qvec = (4 * half) * D + NDT * lq;  // dK product: Q is in row order
+    // Both products read their A operand along d: elements d = NDT lq .. NDT lq + NDT - 1 of tile row
+    // 8 (r / 4) + 4 half + r % 4; consecutive lanes read consecutive vectors of one row.
+    const int avec = (4 * half) * D + NDT * lq;
 
     Acc16 dvT[NDT], dkT[NDT];
 #pragma unroll
@@ -171,7 +413,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_keys_kernel(const KeysArgs p)
             dkT[e][r] = 0.f;
         }
 
-    // ---- S in and dS out go through buffer instructions: their range check drops what lies past the end of the
+    // ---- S and dP in, dS out through buffer instructions: their range check drops what lies past the end of the
     //      (batch, head) slab (rows past seq_q, the keys of dead lanes, the tile after the last, the store before the
     //      first), so no access needs a branch. A lane's byte offset is lane part + wavefront-uniform tile part + uniform
     //      row part; every valid sum stays below 2^30 (the launcher checks it) and kOut, the "nowhere" value of the lane
@@ -194,12 +436,13 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_keys_kernel(const KeysArgs p)
         return qt + 32 <= seq_q && kw0 + 32 <= seq_k && (!p.causal || qt >= kw0 + 31);
     };
 
-    // Two register sets of scores alternate: one is consumed by the tile in hand while the other receives the next
-    // tile's (requested during this tile's dP product). dS is stored as it is made, WITHOUT the softmax scale: the dQ
-    // product applies it as its alpha and dK is scaled once when it is stored. Vector memory operations complete in
-    // issue order, and a tile issues its operand copies for the next tile FIRST, then exactly 16 score loads and 16 dS
-    // stores: the wait that ends a tile is vmcnt(32), which covers the copies and leaves the rest in flight.
-    float s_a[16], s_b[16];
+    // Two register sets of scores and dP alternate: one is consumed by the tile in hand while the other receives the
+    // next tile's, requested element by element inside this tile's product loop. dS goes out as it is made, to the very
+    // address its dP came from, WITHOUT the softmax scale: the dQ product applies it when it stores and dK is scaled once
+    // when it is stored. Vector memory operations complete in issue order, and a tile issues its operand copies for the
+    // next tile FIRST, then exactly 32 loads and 16 stores: the wait that ends a tile is vmcnt(48), which covers the
+    // copies and leaves the rest in flight.
+    float s_a[16], s_b[16], dp_a[16], dp_b[16];
     unsigned ld_tile = kOut;  // uniform tile part of the next loads
     auto aim_loads = [&](int t) __attribute__((always_inline)) {
         const unsigned qt = (unsigned)(q_lo + 32 * t);
@@ -210,8 +453,10 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_keys_kernel(const KeysArgs p)
     if (ntiles > 0) issue_tile(0, 0);
     aim_loads(0);
 #pragma unroll
-    for (int r = 0; r < 16; ++r)
-        s_a[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_s, lane_sd + ld_tile + row_part[r], 0, 2));
+    for (int r = 0; r < 16; ++r) {
+        s_a[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_s, lane_sd + ld_tile, row_part[r], 2));
+        dp_a[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_ds, lane_sd + ld_tile, row_part[r], 2));
+    }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): own tile parts have landed
     __syncthreads();
 
@@ -220,19 +465,16 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_keys_kernel(const KeysArgs p)
     // wavefront per SIMD or two), so what counts is the NUMBER of non-MFMA instructions per tile. The loop body therefore
     // carries no mask logic: a tile that needs masking (the diagonal, the last rows, the last keys) first sets the scores
     // of its hidden pairs to -inf, whose weight 2^(-inf) is an exact zero, and then runs the same body.
-    auto tile_step = [&](const int t, auto buf_c, float(&s_cur)[16], float(&s_nx)[16]) __attribute__((always_inline)) {
+    auto tile_step = [&](const int t, auto buf_c, float(&s_cur)[16], float(&dp_cur)[16], float(&s_nx)[16], float(&dp_nx)[16])
+                         __attribute__((always_inline)) {
         constexpr int buf = decltype(buf_c)::value;
-        constexpr int STEPS = D / 8, RPS = 16 / STEPS;  // dP steps, score rows requested per step
         const int qt = q_lo + 32 * t;
         if (t + 1 < ntiles) issue_tile(t + 1, buf ^ 1);
         aim_loads(t + 1);
         const unsigned v_ld = lane_sd + ld_tile, v_st = lane_sd + (unsigned)qt * row_bytes;
-        auto request = [&](int step) __attribute__((always_inline)) {
-#pragma unroll
-            for (int u = 0; u < RPS; ++u) {
-                const int r = step * RPS + u;
-                s_nx[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_s, v_ld, row_part[r], 2));
-            }
+        auto request = [&](int r) __attribute__((always_inline)) {
+            s_nx[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_s, v_ld, row_part[r], 2));
+            dp_nx[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_ds, v_ld, row_part[r], 2));
         };
         auto store_ds = [&](int r, float x) __attribute__((always_inline)) {
             __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x), rs_ds, v_st, row_part[r], 0);
@@ -246,40 +488,21 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_keys_kernel(const KeysArgs p)
                     s_cur[r] = hidden ? -__builtin_inff() : s_cur[r];
                 }
             }
-            // ---- dP = dOut_tile . V_blk^T; the fragment of step t8 + 1 is requested before the MFMAs of step t8 ----
-            Acc16 dp;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) dp[r] = 0.f;
-            const float *ob = Os + buf * TILE;
-            auto frag = [&](int t8) __attribute__((always_inline)) {
-                return *reinterpret_cast<const float4 *>(ob + ofrag[t8 & 7] + 4 * ((2 * t8) & 16));
-            };
-            float4 ov_n = frag(0);
-#pragma unroll
-            for (int t8 = 0; t8 < STEPS; ++t8) {
-                const float4 ov = ov_n;
-                if (t8 + 1 < STEPS) ov_n = frag(t8 + 1);
-                __builtin_amdgcn_sched_barrier(0);  // the scheduler would otherwise sink the read to just before its use
-                dp = __builtin_amdgcn_mfma_f32_32x32x2f32(ov.x, vr[t8].x, dp, 0, 0, 0);
-                request(t8);
-                dp = __builtin_amdgcn_mfma_f32_32x32x2f32(ov.y, vr[t8].y, dp, 0, 0, 0);
-                dp = __builtin_amdgcn_mfma_f32_32x32x2f32(ov.z, vr[t8].z, dp, 0, 0, 0);
-                dp = __builtin_amdgcn_mfma_f32_32x32x2f32(ov.w, vr[t8].w, dp, 0, 0, 0);
-            }
             // ---- P, dS (lane-local) and the two output products ----
-            const float *qb = Qs + buf * TILE + qvec;
+            const float *ob = Os + buf * TILE + avec, *qb = Qs + buf * TILE + avec;
             const float *stats = Ls + buf * 128 + 4 * half;
             float4 lse4, del4;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
+                request(r);
                 if ((r & 3) == 0) {
                     lse4 = *reinterpret_cast<const float4 *>(stats + 2 * r);
                     del4 = *reinterpret_cast<const float4 *>(stats + 64 + 2 * r);
                 }
                 const float pw = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[r], c2, -f4_get(lse4, r & 3)));
-                const float dsv = pw * (dp[r] - f4_get(del4, r & 3));
+                const float dsv = pw * (dp_cur[r] - f4_get(del4, r & 3));
                 store_ds(r, dsv);
-                const VV ov = *reinterpret_cast<const VV *>(ob + ovec[r]);
+                const VV ov = *reinterpret_cast<const VV *>(ob + (8 * (r >> 2) + (r & 3)) * D);
                 const VV qv = *reinterpret_cast<const VV *>(qb + (8 * (r >> 2) + (r & 3)) * D);
 #pragma unroll
                 for (int e = 0; e < NDT; ++e) {
@@ -290,16 +513,16 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_keys_kernel(const KeysArgs p)
         } else {
             // every (query, key) of this wavefront's part of the tile is masked: dS is zero there
 #pragma unroll
-            for (int st = 0; st < STEPS; ++st) request(st);
+            for (int r = 0; r < 16; ++r) request(r);
 #pragma unroll
             for (int r = 0; r < 16; ++r) store_ds(r, 0.f);
         }
-        __builtin_amdgcn_s_waitcnt(0x8F70);  // vmcnt(32)
+        __builtin_amdgcn_s_waitcnt(0xCF70);  // vmcnt(48)
         __syncthreads();
     };
     for (int t = 0; t < ntiles; t += 2) {
-        tile_step(t, std::integral_constant<int, 0>{}, s_a, s_b);
-        if (t + 1 < ntiles) tile_step(t + 1, std::integral_constant<int, 1>{}, s_b, s_a);
+        tile_step(t, std::integral_constant<int, 0>{}, s_a, dp_a, s_b, dp_b);
+        if (t + 1 < ntiles) tile_step(t + 1, std::integral_constant<int, 1>{}, s_b, dp_b, s_a, dp_a);
     }
     // ---- store: lane owns key kw, d = NDT rho + e with rho = 8 (r / 4) + 4 half + r % 4 ----
     if (key_live) {
@@ -490,12 +713,26 @@ bool sdpa_backward_fused_applies(int64_t num_bh, int64_t seq_q, int64_t seq_k, i
            scale > 0.f && (seq_q + 64) * seq_k < ((int64_t)1 << 28) && seq_q * d_k < (1 << 28);  // byte offsets inside one slab of S stay below 2^30
 }
 
-int32_t sdpa_backward_keys_f32(const float *q, const float *v, const float *dout, int64_t dout_bh_stride, const float *s, const float *lse,
+int32_t sdpa_backward_stats_f32(const float *q, const float *k, const float *v, const float *dout, int64_t dout_bh_stride, int64_t num_bh,
+                                int64_t seq_q, int64_t seq_k, int64_t d, float scale, int causal, float *s_out, float *dp_out,
+                                float *lse_out, float *delta_out, hipStream_t st) {
+    StatsArgs a;
+    a.q = q; a.k = k; a.v = v; a.dout = dout;
+    a.s = s_out; a.dp = dp_out; a.lse = lse_out; a.delta = delta_out;
+    a.num_bh = num_bh; a.dout_bh_stride = dout_bh_stride;
+    a.seq_q = (int)seq_q; a.seq_k = (int)seq_k;
+    a.scale = scale; a.causal = causal;
+    if (d == 128) return launch_stats<128>(a, st);
+    if (d == 64) return launch_stats<64>(a, st);
+    return fth::set_error(FTH_ERR_INVALID_ARGUMENT, "sdpa_backward_stats: head size %lld", (long long)d);
+}
+
+int32_t sdpa_backward_keys_f32(const float *q, const float *dout, int64_t dout_bh_stride, const float *s, const float *lse,
                                const float *delta, int64_t num_bh, int64_t seq_q, int64_t seq_k, int64_t d, float scale, int causal,
-                               int64_t row_block, float *ds, float *dk, float *dv, hipStream_t st) {
+                               int64_t row_block, float *dpds, float *dk, float *dv, hipStream_t st) {
     KeysArgs a;
-    a.q = q; a.v = v; a.dout = dout; a.s = s; a.lse = lse; a.delta = delta;
-    a.ds = ds; a.dk = dk; a.dv = dv;
+    a.q = q; a.dout = dout; a.s = s; a.lse = lse; a.delta = delta;
+    a.dpds = dpds; a.dk = dk; a.dv = dv;
     a.num_bh = num_bh; a.dout_bh_stride = dout_bh_stride;
     a.seq_q = (int)seq_q; a.seq_k = (int)seq_k;
     a.scale = scale; a.causal = causal; a.row_block = (int)row_block;
