@@ -753,10 +753,19 @@ template <typename T> int sdpa_row_vpl(int64_t seq_k, const void *a, const void 
     return per <= 1 ? 1 : per <= 2 ? 2 : per <= 4 ? 4 : per <= 8 ? 8 : 16;
 }
 
-// Two score-shaped matrices (P and dU, or S and dS on the fused path), 64 elements of slack, and two per-row vectors
-// (log-sum-exp and delta of the fused path).
+// Two score-shaped matrices (P and dU; on the fused fp32 path S and dP / dS in whole 32 x 32 tiles with one spare tile
+// row, which is what the size allows for), 64 elements of slack, and two per-row vectors (log-sum-exp and delta of the
+// fused path).
+template <typename T> int64_t sdpa_backward_score_elems(int64_t num_bh, int64_t seq_q, int64_t seq_k) {
+    if (std::is_same<T, float>::value) {
+        int64_t s_floats, d_floats;
+        fth::sdpa_backward_fused_workspace(num_bh, seq_q, seq_k, &s_floats, &d_floats);
+        return s_floats + d_floats;  // >= 2 * num_bh * seq_q * seq_k
+    }
+    return 2 * num_bh * seq_q * seq_k;
+}
 template <typename T> size_t sdpa_backward_workspace(int64_t num_bh, int64_t seq_q, int64_t seq_k) {
-    return (size_t)(2 * num_bh * seq_q * seq_k + 64 + 2 * num_bh * seq_q + 32) * sizeof(T);
+    return (size_t)(sdpa_backward_score_elems<T>(num_bh, seq_q, seq_k) + 64 + 2 * num_bh * seq_q + 32) * sizeof(T);
 }
 
 template <typename T>
@@ -785,11 +794,12 @@ int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, i
             workspace_bytes);
     T *p = static_cast<T *>(workspace);
     T *du = p + pe;
+    const int64_t score_elems = sdpa_backward_score_elems<T>(num_bh, seq_q, seq_k);
     // dOut = ones (sdpa_backward_f32_unit_dout, :5662-5770): one [seq_q, d_v] plane of ones shared by every (batch, head)
     // through a zero batch stride stands in for the gradient; nothing of size num_bh is materialised.
     int64_t dout_bs = seq_q * d_v;
     if (unit_dout) {
-        T *ones = p + ((2 * pe + 64 + 3) & ~(int64_t)3);  // keeps the 16-byte alignment of the workspace base
+        T *ones = p + ((score_elems + 64 + 3) & ~(int64_t)3);  // keeps the 16-byte alignment of the workspace base
         if (int32_t rc = value_fill<T>(ones, seq_q * d_v, T(1), st)) return rc;
         dout = ones;
         dout_bs = 0;
@@ -802,16 +812,18 @@ int32_t sdpa_backward_entry(const T *q, const T *k, const T *v, const T *dout, i
         auto al = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; };
         if (!mask && fth::sdpa_backward_fused_applies(num_bh, seq_q, seq_k, d_k, d_v, scale) && al(q) && al(k) && al(v) && al(dout) &&
             al(dq) && al(dk) && al(dv) && al(workspace)) {
-            float *lse = p + ((2 * pe + 64 + 3) & ~(int64_t)3) + (unit_dout ? ((seq_q * d_v + 4 + 3) & ~(int64_t)3) : 0);  // behind the ones plane
+            float *lse = p + ((score_elems + 64 + 3) & ~(int64_t)3) + (unit_dout ? ((seq_q * d_v + 4 + 3) & ~(int64_t)3) : 0);  // behind the ones plane
             lse = reinterpret_cast<float *>((reinterpret_cast<uintptr_t>(lse) + 15u) & ~(uintptr_t)15u);
             float *delta = lse + ((rows + 3) & ~(int64_t)3);
-            if (int32_t rc = fth::sdpa_backward_stats_f32(q, k, v, dout, dout_bs, num_bh, seq_q, seq_k, d_k, scale, causal, p, du, lse, delta, st))
+            int64_t s_floats, d_floats;
+            fth::sdpa_backward_fused_workspace(num_bh, seq_q, seq_k, &s_floats, &d_floats);
+            float *dpds = p + s_floats;
+            if (int32_t rc = fth::sdpa_backward_stats_f32(q, k, v, dout, dout_bs, num_bh, seq_q, seq_k, d_k, scale, causal, p, dpds, lse, delta, st))
                 return rc;
-            // (under a causal mask the key pass writes dS from each key block's own first row on: all the dQ pass reads)
-            if (int32_t rc = fth::sdpa_backward_keys_f32(q, dout, dout_bs, p, lse, delta, num_bh, seq_q, seq_k, d_k, scale, causal, 128, du, dk,
+            if (int32_t rc = fth::sdpa_backward_keys_f32(q, dout, dout_bs, p, lse, delta, num_bh, seq_q, seq_k, d_k, scale, causal, 128, dpds, dk,
                                                         dv, st))
                 return rc;
-            return fth::sdpa_backward_dq_f32(du, k, num_bh, seq_q, seq_k, d_k, scale, causal, dq, st);
+            return fth::sdpa_backward_dq_f32(dpds, k, num_bh, seq_q, seq_k, d_k, scale, causal, dq, st);
         }
     }
     int vpl = sdpa_row_vpl<T>(seq_k, p, du);

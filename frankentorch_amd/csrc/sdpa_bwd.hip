@@ -73,23 +73,63 @@ __device__ __forceinline__ float vecn_get(const float2 &v, int e) { return e == 
 __device__ __forceinline__ float vecn_get(const float4 &v, int e) { return e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w; }
 __device__ __forceinline__ float f4_get(const float4 &v, int e) { return e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w; }
 
-// x of lanes 0..31 and x of lanes 32..63, each broadcast to both halves (one v_permlane32_swap, no LDS round trip).
-__device__ __forceinline__ void both_halves(float x, float &lo, float &hi) {
-    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    lo = __uint_as_float(r[0]);
-    hi = __uint_as_float(r[1]);
+// Workspace layout of the three score-shaped intermediates. Per (batch, head) the [seq_q, seq_k] plane is cut into
+// 32 x 32 tiles of 4 KiB, tile (qt, kt) at tile index qt * KT + kt; partial tiles at the edges are stored whole.
+// Inside a tile the 16-byte vector number (2 g + h) * 32 + c holds, for S and dP, the four elements
+//   [row 8 g + 4 h + i][column c], i = 0..3     (the accumulator registers 4 g .. 4 g + 3 of lane 32 h + c when the
+//                                                lanes run along the keys: what passes 1 and 2 hold), and for dS
+//   [row c][column 8 g + 4 h + i], i = 0..3     (the B operand registers of lane 32 h + c of the dQ pass, whose lanes
+//                                                run along the queries).
+// Every access of every pass is then one 16-byte vector per lane and 1 KiB in one piece per instruction, except the dS
+// stores of pass 2 (single elements, sixteen 16-byte pieces per instruction).
+// S has QT tile rows. dP and dS share a slab of QT + 1 tile rows: dP tile (qt, kt) sits in tile row qt + 1 and dS
+// tile (qt, kt) in tile row qt, so pass 2 writes the dS of a tile over the dP of the tile it finished before (every
+// load of that one has long returned) and never over anything it has yet to read.
+struct TileMap {
+    unsigned qt_n, kt_n;
+    __host__ __device__ TileMap(int seq_q, int seq_k) : qt_n((unsigned)(seq_q + 31) >> 5), kt_n((unsigned)(seq_k + 31) >> 5) {}
+    __host__ __device__ int64_t s_slab_floats() const { return (int64_t)qt_n * kt_n * 1024; }
+    __host__ __device__ int64_t d_slab_floats() const { return (int64_t)(qt_n + 1) * kt_n * 1024; }
+    __host__ __device__ unsigned s_slab_bytes() const { return qt_n * kt_n * 4096u; }
+    __host__ __device__ unsigned d_slab_bytes() const { return (qt_n + 1) * kt_n * 4096u; }
+    __host__ __device__ unsigned row_bytes() const { return kt_n * 4096u; }  // one tile row
+    __host__ __device__ unsigned tile_bytes(unsigned qt, unsigned kt) const { return (qt * kt_n + kt) * 4096u; }
+    // byte offset of a lane's vector g = 0 inside a tile; vector g is 1024 g further on
+    __host__ __device__ static unsigned lane_vec(int half, int c) { return (unsigned)(half * 32 + c) * 16u; }
+};
+
+// Reductions over the 32 lanes of each half of a wavefront, result in every lane: four data-parallel-primitive steps
+// inside rows of 16 lanes (quad swaps, then the mirrored halves of 8 and of 16) and one swizzle across the two rows.
+template <typename F> __device__ __forceinline__ float half_reduce(float x, F op) {
+    auto dpp = [](float v, auto ctrl) __attribute__((always_inline)) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), decltype(ctrl)::value, 0xF, 0xF, true));
+    };
+    x = op(x, dpp(x, std::integral_constant<int, 0xB1>{}));   // quad_perm [1, 0, 3, 2]
+    x = op(x, dpp(x, std::integral_constant<int, 0x4E>{}));   // quad_perm [2, 3, 0, 1]
+    x = op(x, dpp(x, std::integral_constant<int, 0x141>{}));  // row_half_mirror
+    x = op(x, dpp(x, std::integral_constant<int, 0x140>{}));  // row_mirror
+    return op(x, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, x), 0x401F)));  // lane ^ 16
+}
+__device__ __forceinline__ float half_max(float x) {
+    return half_reduce(x, [](float a, float b) { return fmaxf(a, b); });
+}
+__device__ __forceinline__ float half_sum(float x) {
+    return half_reduce(x, [](float a, float b) { return a + b; });
 }
 
 // ---------------------------------------------------------------------------------------------
-// Statistics pass. One workgroup per 128 queries (a wavefront owns 32; a lane one query, whose Q and dOut rows it keeps
-// in registers as B operands), walking BC-key tiles of K and V through double-buffered LDS:
-//   S^T[key, q]  = K_tile . Q^T,   dP^T[key, q] = V_tile . dOut^T      (the same product shape twice)
-// In the accumulators a lane holds its query's scores and dP against 16 keys per 32-key sub-tile, so the row maximum,
-// the row sum and delta = sum_j P_ij dP_ij need no exchange between lanes until the very end (the two halves of a
-// wavefront hold the same queries against different keys). The reference weight 2^m of a row moves only when a score
-// exceeds it by more than kLazy (log2 units): both running sums are then rescaled, which happens a few times per row.
-// Both tiles are read one 16-byte vector per lane with 16 consecutive lanes on 16 consecutive rows, so logical vector
-// v of tile row r is stored in slot v ^ (r & 15) (the permutation applied on the global side of the copy).
+// Statistics pass. One workgroup per 128 queries (a wavefront owns 32; a lane keeps the Q and dOut rows of query
+// lane % 32 in registers as A operands), walking BC-key tiles of K and V through double-buffered LDS:
+//   S[q, key]  = Q . K_tile^T,   dP[q, key] = dOut . V_tile^T      (the same product shape twice)
+// In the accumulators a lane then holds ONE key column (lane % 32) of 16 of its wavefront's queries - the layout the
+// key-owned pass reads - so a store instruction writes two whole 128-byte row segments. (With the operand roles the
+// other way round a lane owns a query and its statistics need no exchange at all, but every store instruction then
+// scatters thirty-two 32-byte pieces over as many rows; that variant ran 15% slower, and twice as slow with streaming
+// stores, which shows what the L2 has to merge.) The price is that each lane keeps its own running (reference, sum,
+// sum of P dP) triple for each of its 16 rows over the keys IT has seen; the 32 lanes of a row are merged once, at
+// the end of the pass. A lane's reference 2^m moves only when one of its scores exceeds it by more than kLazy (log2
+// units). Both tiles are read one 16-byte vector per lane with 16 consecutive lanes on 16 consecutive rows, so logical
+// vector v of tile row r is stored in slot v ^ (r & 15) (the permutation applied on the global side of the copy).
 // ---------------------------------------------------------------------------------------------
 struct StatsArgs {
     const float *q, *k, *v, *dout;
@@ -138,7 +178,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_stats_kernel(const StatsArgs 
     const float *Kg = p.k + bh * (int64_t)seq_k * D, *Vg = p.v + bh * (int64_t)seq_k * D;
     const float c2 = p.scale * 1.44269502162933349609375f;  // scale * log2(e)
 
-    // ---- Q and dOut rows into registers: lane holds row[8 t + 4 half + e] ----
+    // ---- Q and dOut rows of query lane % 32 into registers: lane holds row[8 t + 4 half + e] ----
     float4 qr[D / 8], dor[D / 8];
     {
         const int qc = q_live ? qi : seq_q - 1;
@@ -185,16 +225,16 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_stats_kernel(const StatsArgs 
         }
     };
 
-    // ---- S and dP out through range-checked buffer stores: the lane part (its query's row, its half's keys; "nowhere"
-    //      for a query past the end) in the vector offset, the tile part in the scalar offset ----
+    // ---- S and dP go out in whole 32 x 32 tiles of 4 KiB (workspace layout, see TileMap): a lane's four registers
+    //      r = 4 g .. 4 g + 3 are one 16-byte vector of the tile, a store instruction writes 1 KiB in one piece. Range-
+    //      checked buffer stores: the tile row of a wavefront whose queries lie wholly past seq_q is outside the slab. ----
     constexpr unsigned kOut = 0x40000000u;
     constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
-    const unsigned row_bytes = (unsigned)seq_k * 4u, slab_bytes = (unsigned)seq_q * row_bytes;
-    const __amdgpu_buffer_rsrc_t rs_s =
-        __builtin_amdgcn_make_buffer_rsrc(p.s + bh * (int64_t)seq_q * seq_k, 0, (int)slab_bytes, kRsrcFlags);
-    const __amdgpu_buffer_rsrc_t rs_dp =
-        __builtin_amdgcn_make_buffer_rsrc(p.dp + bh * (int64_t)seq_q * seq_k, 0, (int)slab_bytes, kRsrcFlags);
-    const unsigned lane_st = q_live ? (unsigned)qi * row_bytes + 16u * (unsigned)half : kOut;
+    const TileMap tm(seq_q, seq_k);
+    const __amdgpu_buffer_rsrc_t rs_s = __builtin_amdgcn_make_buffer_rsrc(p.s + bh * tm.s_slab_floats(), 0, (int)tm.s_slab_bytes(), kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rs_dp = __builtin_amdgcn_make_buffer_rsrc(p.dp + bh * tm.d_slab_floats(), 0, (int)tm.d_slab_bytes(), kRsrcFlags);
+    const unsigned lane_st = TileMap::lane_vec(half, lq);
+    const unsigned qt_wave = (unsigned)(q_blk0 >> 5) + wave_u;  // from the scalar copy of the wavefront index: stays scalar
     typedef unsigned u4v __attribute__((ext_vector_type(4)));
 
     // fragment read t of tile row lq: vector 2 t + half sits in slot (2 t) ^ lx (bits 1..3 take eight per-lane values,
@@ -204,8 +244,16 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_stats_kernel(const StatsArgs 
 #pragma unroll
     for (int u = 0; u < 8; ++u) frag[u] = lq * D + 4 * (((2 * u) ^ lx) & 15);
 
-    constexpr float kLazy = 6.0f;
-    float m_run = -__builtin_inff(), l_run = 0.f, a_run = 0.f;
+    // Per lane and row: reference m (log2 units; a large finite negative start, so that a lane that never sees a key of
+    // a row keeps weight zero without an inf - inf), sum l of 2^(s c - m), sum a of 2^(s c - m) dP.
+    constexpr float kLazy = 6.0f, kNone = -1.0e30f;
+    float m_run[16], l_run[16], a_run[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        m_run[r] = kNone;
+        l_run[r] = 0.f;
+        a_run[r] = 0.f;
+    }
 
     if (num_kt > 0) issue_tile(0, 0);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): own tile parts have landed
@@ -226,84 +274,100 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_stats_kernel(const StatsArgs 
                     s[j][r] = 0.f;
                     dp[j][r] = 0.f;
                 }
+            // One step = one 16-byte fragment and the four MFMAs it feeds; steps alternate between the two products. The
+            // fragment of step st + 2 is requested before the MFMAs of step st (the scheduler, left alone, sinks every
+            // read to just before its use and each group of four MFMAs then waits out the LDS latency).
             const float *kb = Ks + buf * TILE, *vb = Vs + buf * TILE;
+            constexpr int NSTEP = (D / 8) * KS * 2;
+            auto frag_at = [&](int st) __attribute__((always_inline)) {
+                const int t = st / (2 * KS), j = (st >> 1) % KS;
+                const int off = frag[t & 7] + j * 32 * D + 4 * ((2 * t) & 16);
+                return *reinterpret_cast<const float4 *>(((st & 1) ? vb : kb) + off);
+            };
+            float4 fr[3];
+            fr[0] = frag_at(0);
+            fr[1] = frag_at(1);
 #pragma unroll
-            for (int t = 0; t < D / 8; ++t) {
+            for (int st = 0; st < NSTEP; ++st) {
+                if (st + 2 < NSTEP) fr[(st + 2) % 3] = frag_at(st + 2);
+                __builtin_amdgcn_sched_barrier(0);
+                const float4 f = fr[st % 3];
+                const int t = st / (2 * KS), j = (st >> 1) % KS;
+                if (st & 1) {
+                    dp[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(dor[t].x, f.x, dp[j], 0, 0, 0);
+                    dp[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(dor[t].y, f.y, dp[j], 0, 0, 0);
+                    dp[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(dor[t].z, f.z, dp[j], 0, 0, 0);
+                    dp[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(dor[t].w, f.w, dp[j], 0, 0, 0);
+                } else {
+                    s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(qr[t].x, f.x, s[j], 0, 0, 0);
+                    s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(qr[t].y, f.y, s[j], 0, 0, 0);
+                    s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(qr[t].z, f.z, s[j], 0, 0, 0);
+                    s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(qr[t].w, f.w, s[j], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // ---- raw scores and dP of this wavefront's 32 queries x the tile's keys: element r of sub-tile j is query
+            //      q_wave0 + 8 (r / 4) + 4 half + r % 4 against key key0 + 32 j + lane % 32 ----
+            const bool tail = key0 + BC > seq_k;  // uniform
 #pragma unroll
-                for (int j = 0; j < KS; ++j) {
-                    const int off = frag[t & 7] + j * 32 * D + 4 * ((2 * t) & 16);
-                    const float4 kv = *reinterpret_cast<const float4 *>(kb + off);
-                    const float4 vv = *reinterpret_cast<const float4 *>(vb + off);
-                    s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.x, qr[t].x, s[j], 0, 0, 0);
-                    s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.y, qr[t].y, s[j], 0, 0, 0);
-                    s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.z, qr[t].z, s[j], 0, 0, 0);
-                    s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.w, qr[t].w, s[j], 0, 0, 0);
-                    dp[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, dor[t].x, dp[j], 0, 0, 0);
-                    dp[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, dor[t].y, dp[j], 0, 0, 0);
-                    dp[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.z, dor[t].z, dp[j], 0, 0, 0);
-                    dp[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.w, dor[t].w, dp[j], 0, 0, 0);
+            for (int j = 0; j < KS; ++j) {
+                // (a second sub-tile that starts past the last key has no tile of its own: its stores go nowhere)
+                const unsigned v = (KS > 1 && key0 + 32 * j >= seq_k) ? kOut : lane_st;
+                const unsigned ts = tm.tile_bytes(qt_wave, (unsigned)(key0 >> 5) + j);
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    // (element by element through float temporaries: a bit cast applied to a vector element directly reads element 0)
+                    const float s0 = s[j][4 * g + 0], s1 = s[j][4 * g + 1], s2 = s[j][4 * g + 2], s3 = s[j][4 * g + 3];
+                    const float d0 = dp[j][4 * g + 0], d1 = dp[j][4 * g + 1], d2 = dp[j][4 * g + 2], d3 = dp[j][4 * g + 3];
+                    const u4v sx = {__builtin_bit_cast(unsigned, s0), __builtin_bit_cast(unsigned, s1), __builtin_bit_cast(unsigned, s2),
+                                    __builtin_bit_cast(unsigned, s3)};
+                    const u4v dx = {__builtin_bit_cast(unsigned, d0), __builtin_bit_cast(unsigned, d1), __builtin_bit_cast(unsigned, d2),
+                                    __builtin_bit_cast(unsigned, d3)};
+                    __builtin_amdgcn_raw_buffer_store_b128(sx, rs_s, v + (unsigned)g * 1024u, ts, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(dx, rs_dp, v + (unsigned)g * 1024u, ts + tm.row_bytes(), 0);
                 }
             }
-            // ---- raw scores and dP of this wavefront's 32 queries x the tile's keys: a lane holds four runs of four
-            //      consecutive keys per sub-tile (seq_k is a multiple of 4 on this path: no run straddles the row end) ----
-            const bool tail = key0 + BC > seq_k;  // uniform
-            auto store_tile = [&](auto tail_c) __attribute__((always_inline)) {
-#pragma unroll
-                for (int j = 0; j < KS; ++j)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        unsigned v = lane_st + (unsigned)(32 * j + 8 * g) * 4u;
-                        if constexpr (decltype(tail_c)::value)
-                            if (key0 + 32 * j + 8 * g + 4 * half >= seq_k) v = kOut;
-                        // (element by element through float temporaries: a bit cast applied to a vector element directly reads element 0)
-                        const float s0 = s[j][4 * g + 0], s1 = s[j][4 * g + 1], s2 = s[j][4 * g + 2], s3 = s[j][4 * g + 3];
-                        const float d0 = dp[j][4 * g + 0], d1 = dp[j][4 * g + 1], d2 = dp[j][4 * g + 2], d3 = dp[j][4 * g + 3];
-                        const u4v sv = {__builtin_bit_cast(unsigned, s0), __builtin_bit_cast(unsigned, s1), __builtin_bit_cast(unsigned, s2),
-                                        __builtin_bit_cast(unsigned, s3)};
-                        const u4v dv = {__builtin_bit_cast(unsigned, d0), __builtin_bit_cast(unsigned, d1), __builtin_bit_cast(unsigned, d2),
-                                        __builtin_bit_cast(unsigned, d3)};
-                        __builtin_amdgcn_raw_buffer_store_b128(sv, rs_s, v, (unsigned)key0 * 4u, 0);
-                        __builtin_amdgcn_raw_buffer_store_b128(dv, rs_dp, v, (unsigned)key0 * 4u, 0);
-                    }
-            };
-            if (tail) store_tile(std::true_type{});
-            else store_tile(std::false_type{});
-            // ---- online row statistics (lane-local query) ----
+            // ---- online statistics, per lane and row ----
             const bool need_mask = (p.causal && key0 + BC - 1 > q_wave0) || tail;
             if (need_mask) {  // wavefront-uniform; selects, no per-element branches
 #pragma unroll
                 for (int j = 0; j < KS; ++j)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        const int key = key0 + 32 * j + 8 * (r >> 2) + 4 * half + (r & 3);
-                        const bool hidden = (p.causal && key > qi) | (key >= seq_k);
+                        const int key = key0 + 32 * j + lq, qrow = q_wave0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                        const bool hidden = (p.causal && key > qrow) | (key >= seq_k);
                         s[j][r] = hidden ? -__builtin_inff() : s[j][r];
                     }
             }
-            float mt = -__builtin_inff();
+            // exponents against the lane's references; the references move (rarely) when one exceeds kLazy
+            float big = -__builtin_inff();
 #pragma unroll
             for (int j = 0; j < KS; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) mt = fmaxf(mt, s[j][r]);
-            if (__any(mt * c2 > m_run + kLazy)) {
-                float mlo, mhi;
-                both_halves(mt, mlo, mhi);
-                const float m_new = fmaxf(m_run, fmaxf(mlo, mhi) * c2);
-                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-                l_run *= alpha;
-                a_run *= alpha;
-                m_run = m_new;
+                for (int r = 0; r < 16; ++r) big = fmaxf(big, __builtin_fmaf(s[j][r], c2, -m_run[r]));
+            if (__any(big > kLazy)) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float mx = s[0][r];
+#pragma unroll
+                    for (int j = 1; j < KS; ++j) mx = fmaxf(mx, s[j][r]);
+                    const float m_new = fmaxf(m_run[r], mx * c2);
+                    const float alpha = __builtin_amdgcn_exp2f(m_run[r] - m_new);
+                    l_run[r] *= alpha;
+                    a_run[r] *= alpha;
+                    m_run[r] = m_new;
+                }
             }
-            const float neg_m = -m_run;
 #pragma unroll
             for (int j = 0; j < KS; ++j)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][r], c2, neg_m));
-                    l_run += e;
-                    a_run = __builtin_fmaf(e, dp[j][r], a_run);
+                    const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][r], c2, -m_run[r]));
+                    l_run[r] += e;
+                    a_run[r] = __builtin_fmaf(e, dp[j][r], a_run[r]);
                 }
-            // the stores of this tile may stay in flight; the copies issued before them may not (in-order completion)
+            // the stores of this tile may stay in flight; the copies issued before them may not (in-order completion;
+            // the counter holds 63 at most)
             if constexpr (NST == 8) __builtin_amdgcn_s_waitcnt(0x0F78);
             else __builtin_amdgcn_s_waitcnt(0x4F70);
         } else {
@@ -315,14 +379,18 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_stats_kernel(const StatsArgs 
         tile_step(kt, std::integral_constant<int, 0>{});
         if (kt + 1 < num_kt) tile_step(kt + 1, std::integral_constant<int, 1>{});
     }
-    // the two halves of the wavefront hold partial sums of the same queries
-    float llo, lhi, alo, ahi;
-    both_halves(l_run, llo, lhi);
-    both_halves(a_run, alo, ahi);
-    if (q_live && half == 0) {
-        const float l = llo + lhi;
-        p.lse[bh * (int64_t)seq_q + qi] = m_run + __builtin_amdgcn_logf(l);  // v_log_f32 is log2
-        p.delta[bh * (int64_t)seq_q + qi] = (alo + ahi) / l;
+    // ---- merge the 32 lanes of every row (lanes 0..31 and 32..63 hold different rows): common reference, then the two
+    //      sums rescaled to it ----
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const float m_all = half_max(m_run[r]);
+        const float w = __builtin_amdgcn_exp2f(m_run[r] - m_all);
+        const float l = half_sum(l_run[r] * w), a = half_sum(a_run[r] * w);
+        const int qrow = q_wave0 + 8 * (r >> 2) + 4 * half + (r & 3);
+        if (lq == 0 && qrow < seq_q) {
+            p.lse[bh * (int64_t)seq_q + qrow] = m_all + __builtin_amdgcn_logf(l);  // v_log_f32 is log2
+            p.delta[bh * (int64_t)seq_q + qrow] = a / l;
+        }
     }
 }
 
@@ -361,12 +429,11 @@ __global__ __launch_bounds__(256, FTH_SDPA_BWD_KEYS_OCC) void sdpa_bwd_keys_kern
     const int kb = (int)(pid / p.num_bh);  // key blocks in ascending order: under a causal mask the heaviest come first
     const int64_t bh = pid % p.num_bh;
     const int seq_q = p.seq_q, seq_k = p.seq_k;
-    const int key0 = kb * 128, kw0 = key0 + 32 * wave, kw = kw0 + lq;
+    const unsigned wave_u = __builtin_amdgcn_readfirstlane((unsigned)wave);  // scalar copy: what derives from it stays scalar
+    const int key0 = kb * 128, kw0 = key0 + 32 * (int)wave_u, kw = kw0 + lq;
     const bool key_live = kw < seq_k;
     const float *Qg = p.q + bh * (int64_t)seq_q * D;
     const float *Og = p.dout + bh * p.dout_bh_stride;
-    const float *Sg = p.s + bh * (int64_t)seq_q * seq_k;
-    float *DSg = p.dpds + bh * (int64_t)seq_q * seq_k;
     const float *Lg = p.lse + bh * (int64_t)seq_q, *Dg = p.delta + bh * (int64_t)seq_q;
     const float c2 = p.scale * 1.44269502162933349609375f;  // scale * log2(e): the statistics are in log2 units
 
@@ -376,7 +443,6 @@ __global__ __launch_bounds__(256, FTH_SDPA_BWD_KEYS_OCC) void sdpa_bwd_keys_kern
 
     // ---- tile loader (Q and dOut rows q_lo + 32 t .. + 31, rows past the end clamped: their weights are zero) ----
     const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)reinterpret_cast<uintptr_t>(smem_raw));
-    const unsigned wave_u = __builtin_amdgcn_readfirstlane((unsigned)wave);
     int ld_row[CPW];
 #pragma unroll
     for (int ci = 0; ci < CPW; ++ci) ld_row[ci] = (wave * CPW + ci) * RPC + lane / VPR;
@@ -413,116 +479,136 @@ __global__ __launch_bounds__(256, FTH_SDPA_BWD_KEYS_OCC) void sdpa_bwd_keys_kern
             dkT[e][r] = 0.f;
         }
 
-    // ---- S and dP in, dS out through buffer instructions: their range check drops what lies past the end of the
-    //      (batch, head) slab (rows past seq_q, the keys of dead lanes, the tile after the last, the store before the
-    //      first), so no access needs a branch. A lane's byte offset is lane part + wavefront-uniform tile part + uniform
-    //      row part; every valid sum stays below 2^30 (the launcher checks it) and kOut, the "nowhere" value of the lane
-    //      and tile parts, is 2^30: any sum with a kOut in it is out of range and below 2^32. Lane and tile part travel in
-    //      the instruction's vector offset (one add per tile), the row part in its scalar offset (none per row); the range
-    //      check of this part covers the sum of both. ----
+    // ---- S and dP in, dS out through buffer instructions on whole 4 KiB tiles (TileMap). Their range check is what
+    //      drops the request for "the tile after the last" and for tiles this wavefront does not use: kOut, the "nowhere"
+    //      value of the uniform tile part of an offset, is 2^30, every valid offset stays below it (the launcher checks
+    //      the slab sizes), and any sum with a kOut in it is out of range and below 2^32. ----
     constexpr unsigned kOut = 0x40000000u;
     constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
-    const unsigned slab_bytes = (unsigned)seq_q * (unsigned)seq_k * 4u, row_bytes = (unsigned)seq_k * 4u;
-    const __amdgpu_buffer_rsrc_t rs_s = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(Sg), 0, (int)slab_bytes, kRsrcFlags);
-    const __amdgpu_buffer_rsrc_t rs_ds = __builtin_amdgcn_make_buffer_rsrc(DSg, 0, (int)slab_bytes, kRsrcFlags);
-    const unsigned lane_sd = key_live ? (unsigned)(4 * half) * row_bytes + 4u * (unsigned)kw : kOut;
-    unsigned row_part[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) row_part[r] = (unsigned)(8 * (r >> 2) + (r & 3)) * row_bytes;
+    const TileMap tm(seq_q, seq_k);
+    const __amdgpu_buffer_rsrc_t rs_s =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.s) + bh * tm.s_slab_floats(), 0, (int)tm.s_slab_bytes(), kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rs_d = __builtin_amdgcn_make_buffer_rsrc(p.dpds + bh * tm.d_slab_floats(), 0, (int)tm.d_slab_bytes(), kRsrcFlags);
+    const unsigned lane_ld = TileMap::lane_vec(half, lq);
+    // dS element [row, column lq] of a tile: vector (lq / 4) * 32 + row, component lq % 4; row = 8 (r / 4) + 4 half + r % 4
+    const unsigned lane_st = (unsigned)(lq >> 2) * 512u + (unsigned)(lq & 3) * 4u + (unsigned)half * 64u;
+    const unsigned kt_wave = (unsigned)(kw0 >> 5), qt_lo = (unsigned)(q_lo >> 5);
+    const bool wave_dead = kw0 >= seq_k;  // no key of this wavefront exists: it has no tile column
     auto wave_hidden = [&](int t) __attribute__((always_inline)) { return p.causal && q_lo + 32 * t + 31 < kw0; };
     // a tile of which this wavefront masks nothing: every row and key exists, every query sees every key
     auto wave_plain = [&](int t) __attribute__((always_inline)) {
         const int qt = q_lo + 32 * t;
         return qt + 32 <= seq_q && kw0 + 32 <= seq_k && (!p.causal || qt >= kw0 + 31);
     };
+    typedef unsigned u4v __attribute__((ext_vector_type(4)));
 
-    // Two register sets of scores and dP alternate: one is consumed by the tile in hand while the other receives the
-    // next tile's, requested element by element inside this tile's product loop. dS goes out as it is made, to the very
-    // address its dP came from, WITHOUT the softmax scale: the dQ product applies it when it stores and dK is scaled once
-    // when it is stored. Vector memory operations complete in issue order, and a tile issues its operand copies for the
-    // next tile FIRST, then exactly 32 loads and 16 stores: the wait that ends a tile is vmcnt(48), which covers the
-    // copies and leaves the rest in flight.
-    float s_a[16], s_b[16], dp_a[16], dp_b[16];
+    // The scores and dP of a tile sit in one register set, filled a whole tile ahead: as soon as the four elements of a
+    // group of the tile in hand have been turned into P and dS, their registers are the destination of the next tile's
+    // group. dS goes out as it is made, WITHOUT the softmax scale: the dQ product applies it when it stores and dK is
+    // scaled once when it is stored. Vector memory operations complete in issue order, and a tile issues its operand
+    // copies for the next tile FIRST, then exactly 8 loads and 16 stores (8 loads and no store where the wavefront sees
+    // nothing of the tile): the wait that ends a tile is vmcnt(24) (vmcnt(8)), which covers the copies and leaves the
+    // rest in flight.
+    float sv[16], dv[16];
     unsigned ld_tile = kOut;  // uniform tile part of the next loads
     auto aim_loads = [&](int t) __attribute__((always_inline)) {
-        const unsigned qt = (unsigned)(q_lo + 32 * t);
-        const bool none = t >= ntiles || wave_hidden(t);
-        ld_tile = none ? kOut : qt * row_bytes;
+        const bool none = t >= ntiles || wave_hidden(t) || wave_dead;
+        ld_tile = none ? kOut : tm.tile_bytes(qt_lo + (unsigned)t, kt_wave);
+    };
+    auto request = [&](int g) __attribute__((always_inline)) {
+        const u4v x = __builtin_amdgcn_raw_buffer_load_b128(rs_s, lane_ld + (unsigned)g * 1024u, ld_tile, 2);
+        const u4v y = __builtin_amdgcn_raw_buffer_load_b128(rs_d, lane_ld + (unsigned)g * 1024u + tm.row_bytes(), ld_tile, 2);
+        // (whole vectors are cast: a bit cast applied to a vector element directly reads element 0)
+        const nat_f4 xf = __builtin_bit_cast(nat_f4, x), yf = __builtin_bit_cast(nat_f4, y);
+        sv[4 * g + 0] = xf.x; sv[4 * g + 1] = xf.y; sv[4 * g + 2] = xf.z; sv[4 * g + 3] = xf.w;
+        dv[4 * g + 0] = yf.x; dv[4 * g + 1] = yf.y; dv[4 * g + 2] = yf.z; dv[4 * g + 3] = yf.w;
     };
 
     if (ntiles > 0) issue_tile(0, 0);
     aim_loads(0);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        s_a[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_s, lane_sd + ld_tile, row_part[r], 2));
-        dp_a[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_ds, lane_sd + ld_tile, row_part[r], 2));
-    }
+    for (int g = 0; g < 4; ++g) request(g);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): own tile parts have landed
     __syncthreads();
 
     // fp32 MFMAs and ordinary vector instructions do not overlap on this part (a wavefront's stream of
     // v_mfma_f32_32x32x2_f32 slows by the full issue time of every VALU instruction placed between them, with one
-    // wavefront per SIMD or two), so what counts is the NUMBER of non-MFMA instructions per tile. The loop body therefore
-    // carries no mask logic: a tile that needs masking (the diagonal, the last rows, the last keys) first sets the scores
-    // of its hidden pairs to -inf, whose weight 2^(-inf) is an exact zero, and then runs the same body.
-    auto tile_step = [&](const int t, auto buf_c, float(&s_cur)[16], float(&dp_cur)[16], float(&s_nx)[16], float(&dp_nx)[16])
-                         __attribute__((always_inline)) {
+    // wavefront per SIMD or two), and a vector memory instruction costs about 20 cycles of it, so what counts is the
+    // NUMBER of non-MFMA instructions per tile. The loop body therefore carries no mask logic: a tile that needs masking
+    // (the diagonal, the last rows, the last keys) first sets the scores of its hidden pairs to -inf, whose weight
+    // 2^(-inf) is an exact zero, and then runs the same body.
+    auto tile_step = [&](const int t, auto buf_c) __attribute__((always_inline)) {
         constexpr int buf = decltype(buf_c)::value;
         const int qt = q_lo + 32 * t;
         if (t + 1 < ntiles) issue_tile(t + 1, buf ^ 1);
+        const unsigned st_tile = wave_dead ? kOut : tm.tile_bytes(qt_lo + (unsigned)t, kt_wave);
         aim_loads(t + 1);
-        const unsigned v_ld = lane_sd + ld_tile, v_st = lane_sd + (unsigned)qt * row_bytes;
-        auto request = [&](int r) __attribute__((always_inline)) {
-            s_nx[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_s, v_ld, row_part[r], 2));
-            dp_nx[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_ds, v_ld, row_part[r], 2));
-        };
         auto store_ds = [&](int r, float x) __attribute__((always_inline)) {
-            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x), rs_ds, v_st, row_part[r], 0);
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x), rs_d, lane_st + (unsigned)(8 * (r >> 2) + (r & 3)) * 16u,
+                                                  st_tile, 0);
         };
         if (!wave_hidden(t)) {
+            // the tile's statistics: log-sum-exp and delta of the four queries of each element group
+            const float *stats = Ls + buf * 128 + 4 * half;
+            float4 lse_g[4], del_g[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                lse_g[g] = *reinterpret_cast<const float4 *>(stats + 8 * g);
+                del_g[g] = *reinterpret_cast<const float4 *>(stats + 64 + 8 * g);
+            }
             if (!wave_plain(t)) {  // wavefront-uniform, a few tiles per key block
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int qi = qt + 8 * (r >> 2) + 4 * half + (r & 3);
                     const bool hidden = (p.causal && kw > qi) | (qi >= seq_q) | !key_live;
-                    s_cur[r] = hidden ? -__builtin_inff() : s_cur[r];
+                    sv[r] = hidden ? -__builtin_inff() : sv[r];
                 }
             }
-            // ---- P, dS (lane-local) and the two output products ----
+            // ---- P, dS (lane-local) and the two output products, software-pipelined by hand: step r reads the LDS
+            //      operands of element r + 1 and does its P / dS arithmetic among the MFMAs of element r, whose operands
+            //      step r - 1 left in registers; the last step of each group of four requests the next tile's group. The
+            //      scheduling fences keep the compiler from sinking reads and requests to just before their first use. ----
             const float *ob = Os + buf * TILE + avec, *qb = Qs + buf * TILE + avec;
-            const float *stats = Ls + buf * 128 + 4 * half;
-            float4 lse4, del4;
+            VV ov_c = *reinterpret_cast<const VV *>(ob), qv_c = *reinterpret_cast<const VV *>(qb);
+            float pw_c = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[0], c2, -lse_g[0].x));
+            float ds_c = pw_c * (dv[0] - del_g[0].x);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                request(r);
-                if ((r & 3) == 0) {
-                    lse4 = *reinterpret_cast<const float4 *>(stats + 2 * r);
-                    del4 = *reinterpret_cast<const float4 *>(stats + 64 + 2 * r);
+                const int rn = r + 1 < 16 ? r + 1 : 15;
+                VV ov_n = ov_c, qv_n = qv_c;
+                if (r + 1 < 16) {
+                    ov_n = *reinterpret_cast<const VV *>(ob + (8 * (rn >> 2) + (rn & 3)) * D);
+                    qv_n = *reinterpret_cast<const VV *>(qb + (8 * (rn >> 2) + (rn & 3)) * D);
                 }
-                const float pw = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[r], c2, -f4_get(lse4, r & 3)));
-                const float dsv = pw * (dp_cur[r] - f4_get(del4, r & 3));
-                store_ds(r, dsv);
-                const VV ov = *reinterpret_cast<const VV *>(ob + (8 * (r >> 2) + (r & 3)) * D);
-                const VV qv = *reinterpret_cast<const VV *>(qb + (8 * (r >> 2) + (r & 3)) * D);
+                __builtin_amdgcn_sched_barrier(0);
+                float pw_n = 0.f, ds_n = 0.f;
+                if (r + 1 < 16) {
+                    pw_n = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[rn], c2, -f4_get(lse_g[rn >> 2], rn & 3)));
+                    ds_n = pw_n * (dv[rn] - f4_get(del_g[rn >> 2], rn & 3));
+                }
+                store_ds(r, ds_c);
 #pragma unroll
                 for (int e = 0; e < NDT; ++e) {
-                    dvT[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(ov, e), pw, dvT[e], 0, 0, 0);
-                    dkT[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(qv, e), dsv, dkT[e], 0, 0, 0);
+                    dvT[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(ov_c, e), pw_c, dvT[e], 0, 0, 0);
+                    dkT[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(qv_c, e), ds_c, dkT[e], 0, 0, 0);
                 }
+                __builtin_amdgcn_sched_barrier(0);
+                // elements 4 g .. 4 g + 3 were all consumed by the end of step 4 g + 2 (step r computes element r + 1)
+                if ((r & 3) == 3) request(r >> 2);
+                ov_c = ov_n; qv_c = qv_n; pw_c = pw_n; ds_c = ds_n;
             }
+            __builtin_amdgcn_s_waitcnt(0x4F78);  // vmcnt(24)
         } else {
-            // every (query, key) of this wavefront's part of the tile is masked: dS is zero there
+            // every (query, key) of this wavefront's part of the tile is masked, and the dQ pass does not read it
 #pragma unroll
-            for (int r = 0; r < 16; ++r) request(r);
-#pragma unroll
-            for (int r = 0; r < 16; ++r) store_ds(r, 0.f);
+            for (int g = 0; g < 4; ++g) request(g);
+            __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8)
         }
-        __builtin_amdgcn_s_waitcnt(0xCF70);  // vmcnt(48)
         __syncthreads();
     };
     for (int t = 0; t < ntiles; t += 2) {
-        tile_step(t, std::integral_constant<int, 0>{}, s_a, dp_a, s_b, dp_b);
-        if (t + 1 < ntiles) tile_step(t + 1, std::integral_constant<int, 1>{}, s_b, dp_b, s_a, dp_a);
+        tile_step(t, std::integral_constant<int, 0>{});
+        if (t + 1 < ntiles) tile_step(t + 1, std::integral_constant<int, 1>{});
     }
     // ---- store: lane owns key kw, d = NDT rho + e with rho = 8 (r / 4) + 4 half + r % 4 ----
     if (key_live) {
@@ -558,12 +644,13 @@ template <int D> int32_t launch_keys(const KeysArgs &a, hipStream_t st) {
 
 // ---------------------------------------------------------------------------------------------
 // Query-owned pass: dQ = scale . dS . K. One workgroup per 128 queries (a wavefront owns 32), walking the 32-key tiles
-// its queries can see; K tiles through double-buffered LDS (row order, read along d), dS straight from HBM in the
-// accumulator layout of the key-owned pass: dQ^T[d, q] += K_tile^T . dS^T, where MFMA step r contracts over the two
-// keys 8 (r / 4) + 4 half + r % 4 and a lane's B operand is dS[q = lane % 32][that key] - four 16-byte loads per lane
-// and tile, requested one tile ahead. The key-owned pass stored explicit zeros for the masked pairs of every tile on
-// the diagonal, so this loop has no mask logic: a wavefront simply stops at the last tile its queries reach. 64 MFMAs
-// (D = 128) per tile against 4 loads and 16 LDS reads, and hardly a vector instruction in between.
+// its queries can see; K tiles through double-buffered LDS (row order, read along d), dS straight from HBM:
+// dQ^T[d, q] += K_tile^T . dS^T, where MFMA step r contracts over the two keys 8 (r / 4) + 4 half + r % 4 and a lane's
+// B operand is dS[q = lane % 32][that key] - four 16-byte loads per lane and tile (the workspace tiles hold dS in
+// exactly that order, 1 KiB in one piece per instruction), requested one tile ahead. The key-owned pass stored
+// explicit zeros for the masked pairs of every tile on the diagonal, so this loop has no mask logic: a wavefront simply
+// stops at the last tile its queries reach. 64 MFMAs (D = 128) per tile against 4 loads and 16 LDS reads, and hardly a
+// vector instruction in between.
 // ---------------------------------------------------------------------------------------------
 struct DqArgs {
     const float *ds, *k;
@@ -592,10 +679,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_kernel(const DqArgs p) {
     const int qb = q_blocks - 1 - (int)(pid / p.num_bh);  // heaviest (latest) query blocks first under a causal mask
     const int64_t bh = pid % p.num_bh;
     const int seq_q = p.seq_q, seq_k = p.seq_k;
-    const int q_blk0 = qb * 128, q_wave0 = q_blk0 + 32 * wave, qi = q_wave0 + lq;
+    const unsigned wave_u = __builtin_amdgcn_readfirstlane((unsigned)wave);  // scalar copy: what derives from it stays scalar
+    const int q_blk0 = qb * 128, q_wave0 = q_blk0 + 32 * (int)wave_u, qi = q_wave0 + lq;
     const bool q_live = qi < seq_q;
     const float *Kg = p.k + bh * (int64_t)seq_k * D;
-    const float *DSg = p.ds + bh * (int64_t)seq_q * seq_k;
 
     int blk_last_q = q_blk0 + 127, wave_last_q = q_wave0 + 31;
     if (blk_last_q > seq_q - 1) blk_last_q = seq_q - 1;
@@ -606,7 +693,6 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_kernel(const DqArgs p) {
 
     // ---- K tile loader (rows past the last key clamped: their dS is read as zero) ----
     const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)reinterpret_cast<uintptr_t>(smem_raw));
-    const unsigned wave_u = __builtin_amdgcn_readfirstlane((unsigned)wave);
     auto issue_tile = [&](int t, int buf) __attribute__((always_inline)) {
         const unsigned dst = lds0 + (unsigned)(buf * TILE * 4) + wave_u * (CPW * 1024u);
 #pragma unroll
@@ -617,22 +703,24 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_kernel(const DqArgs p) {
         }
     };
 
-    // ---- dS through range-checked buffer loads: lane part (its query's row, its half's keys) in the vector offset,
-    //      tile part in the scalar offset; a dead query's lane part is "nowhere" ----
+    // ---- dS through range-checked buffer loads on whole 4 KiB tiles (TileMap): a lane's vector g of tile (its
+    //      wavefront's query tile, key tile t) is dS[its query][keys 8 g + 4 half .. + 3]; "nowhere" for a tile the
+    //      wavefront does not use ----
     constexpr unsigned kOut = 0x40000000u;
-    const unsigned row_bytes = (unsigned)seq_k * 4u;
+    const TileMap tm(seq_q, seq_k);
     const __amdgpu_buffer_rsrc_t rs_ds =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(DSg), 0, (int)((unsigned)seq_q * row_bytes), 0x00020000);
-    const unsigned lane_ds = q_live ? (unsigned)qi * row_bytes + 16u * (unsigned)half : kOut;
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.ds) + bh * tm.d_slab_floats(), 0, (int)tm.d_slab_bytes(), 0x00020000);
+    const unsigned lane_ds = TileMap::lane_vec(half, lq);
+    const unsigned qt_wave = (unsigned)(q_wave0 >> 5);
     typedef unsigned u4v __attribute__((ext_vector_type(4)));
     auto wave_active = [&](int t) __attribute__((always_inline)) { return !p.causal || 32 * t <= wave_last_q; };
     auto load_ds = [&](int t, float4(&dst)[4]) __attribute__((always_inline)) {
-        const bool none = t >= ntiles || !wave_active(t);
-        const unsigned v = none ? kOut : lane_ds;
-        const bool tail = 32 * t + 32 > seq_k;  // uniform: the last keys of a row must not run into the next row
+        const bool none = t >= ntiles || !wave_active(t) || q_wave0 >= seq_q;
+        const unsigned ts = none ? kOut : tm.tile_bytes(qt_wave, (unsigned)t);
+        const bool tail = 32 * t + 32 > seq_k;  // uniform: columns past the last key count as zero whatever the tile holds
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            u4v x = __builtin_amdgcn_raw_buffer_load_b128(rs_ds, v, (unsigned)(32 * t + 8 * g) * 4u, 2);
+            u4v x = __builtin_amdgcn_raw_buffer_load_b128(rs_ds, lane_ds + (unsigned)g * 1024u, ts, 2);
             if (tail && 32 * t + 8 * g + 4 * half >= seq_k) x = (u4v){0u, 0u, 0u, 0u};
             dst[g] = __builtin_bit_cast(float4, x);
         }
@@ -656,13 +744,24 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_kernel(const DqArgs p) {
         if (t + 1 < ntiles) issue_tile(t + 1, buf ^ 1);
         load_ds(t + 1, ds_nx);
         if (wave_active(t)) {
+            // the K fragment of step r + 2 is requested before the MFMAs of step r (the scheduler, left alone, sinks each
+            // read to just before its use and every group of MFMAs then waits out the LDS latency)
             const float *kb = Ks + buf * TILE + kvec;
+            auto frag_at = [&](int r) __attribute__((always_inline)) {
+                return *reinterpret_cast<const VV *>(kb + (8 * (r >> 2) + (r & 3)) * D);
+            };
+            VV fr[3];
+            fr[0] = frag_at(0);
+            fr[1] = frag_at(1);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const VV kv = *reinterpret_cast<const VV *>(kb + (8 * (r >> 2) + (r & 3)) * D);
+                if (r + 2 < 16) fr[(r + 2) % 3] = frag_at(r + 2);
+                __builtin_amdgcn_sched_barrier(0);
+                const VV kv = fr[r % 3];
                 const float w = f4_get(ds_cur[r >> 2], r & 3);
 #pragma unroll
                 for (int e = 0; e < NDT; ++e) acc[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(vecn_get(kv, e), w, acc[e], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         // Everything requested at the top of this tile (the K copies and the next tile's dS, a whole tile of MFMAs ago)
@@ -709,8 +808,16 @@ bool sdpa_backward_fused_applies(int64_t num_bh, int64_t seq_q, int64_t seq_k, i
         const char *e = std::getenv("FT_HIP_SDPA_BWD_FUSED");  // tuning / testing knob: 0 keeps the materialising backward
         return e && std::atoi(e) == 0;
     }();
-    return !off && d_k == d_v && (d_k == 64 || d_k == 128) && seq_q % 4 == 0 && seq_k % 4 == 0 && seq_q >= 32 && seq_k >= 32 &&
-           scale > 0.f && (seq_q + 64) * seq_k < ((int64_t)1 << 28) && seq_q * d_k < (1 << 28);  // byte offsets inside one slab of S stay below 2^30
+    if (off || d_k != d_v || (d_k != 64 && d_k != 128) || seq_q % 4 != 0 || seq_k % 4 != 0 || seq_q < 32 || seq_k < 32 || !(scale > 0.f)) return false;
+    // byte offsets inside one (batch, head) slab of tiles stay below 2^30, and so do those inside its operands
+    const int64_t qt = (seq_q + 31) / 32, kt = (seq_k + 31) / 32;
+    return (qt + 4) * kt * 4096 < ((int64_t)1 << 30) && seq_q * d_k < (1 << 28) && seq_k * d_k < (1 << 28);
+}
+
+void sdpa_backward_fused_workspace(int64_t num_bh, int64_t seq_q, int64_t seq_k, int64_t *s_floats, int64_t *d_floats) {
+    const int64_t qt = (seq_q + 31) / 32, kt = (seq_k + 31) / 32;
+    *s_floats = num_bh * qt * kt * 1024;
+    *d_floats = num_bh * (qt + 1) * kt * 1024;
 }
 
 int32_t sdpa_backward_stats_f32(const float *q, const float *k, const float *v, const float *dout, int64_t dout_bh_stride, int64_t num_bh,
