@@ -20,6 +20,8 @@
 
 #include <cstdlib>
 
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace {
@@ -106,11 +108,21 @@ struct I8Args {
     int vec_store;  // n % 4 == 0 and a 16-byte aligned output: interior tiles may use 128-bit stores
 };
 
-__device__ __forceinline__ void load_to_lds_16(const int8_t *src, unsigned lds_chunk) {
-    // Inline assembly so that the compiler's wait-count insertion does not see an LDS write it cannot
-    // disambiguate; the kernel waits for vmcnt(0) itself before each barrier.
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(__builtin_amdgcn_readfirstlane(lds_chunk))
+// One wavefront-wide global -> LDS copy of 16 bytes per lane: scalar base, one unsigned 32-bit byte offset per lane (no
+// 64-bit vector address arithmetic: vector instructions take issue cycles from the MFMAs). Inline assembly so that the
+// compiler's wait-count insertion does not see an LDS write it cannot disambiguate; the kernel waits for its loads
+// itself before each barrier.
+__device__ __forceinline__ void load_to_lds_16(const int8_t *base, unsigned lane_off, unsigned lds_chunk) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base),
+                 "s"(__builtin_amdgcn_readfirstlane(lds_chunk))
                  : "memory", "m0");
+}
+
+// A pointer every lane holds the same value of, made a scalar for the compiler.
+__device__ __forceinline__ const int8_t *uniform_ptr(const int8_t *ptr) {
+    const uint64_t v = reinterpret_cast<uint64_t>(ptr);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const int8_t *>(((uint64_t)hi << 32) | lo);
 }
 
 constexpr int kBK = 64;     // bytes of K per stage
@@ -162,7 +174,11 @@ __global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8A
     const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)reinterpret_cast<uintptr_t>(smem));
     const unsigned wave_u = __builtin_amdgcn_readfirstlane((unsigned)wave);
     const int lrow = lane >> 2, lslot = lane & 3;
-    const int8_t *a_src[LD], *b_src[LD];
+    // Scalar tile bases and per-lane byte offsets from them (a tile spans at most 256 rows of k bytes: the launcher
+    // checks that this fits 32 bits). Rows past the end repeat the last row; their results are not stored.
+    const int64_t a_row0 = m0 < p.m ? m0 : p.m - 1, b_row0 = n0 < p.n ? n0 : p.n - 1;
+    const int8_t *a_base = uniform_ptr(p.a + a_row0 * p.k), *b_base = uniform_ptr(p.b + b_row0 * p.k);
+    unsigned a_off[LD], b_off[LD];
 #pragma unroll
     for (int i = 0; i < LD; ++i) {
         const int r = wave * (16 * LD) + i * 16 + lrow;  // row inside the tile
@@ -170,17 +186,17 @@ __global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8A
         int64_t ar = m0 + r, br = n0 + r;
         ar = ar < p.m ? ar : p.m - 1;
         br = br < p.n ? br : p.n - 1;
-        a_src[i] = p.a + ar * p.k + q * 16;
-        b_src[i] = p.b + br * p.k + q * 16;
+        a_off[i] = (unsigned)((ar - a_row0) * p.k) + (unsigned)q * 16u;
+        b_off[i] = (unsigned)((br - b_row0) * p.k) + (unsigned)q * 16u;
     }
     const int num_kt = (int)(p.k / kBK);
     auto issue = [&](int kt) __attribute__((always_inline)) {
         const unsigned base = lds0 + (unsigned)(kt % kStages) * STAGE + wave_u * (LD * 1024u);
-        const int64_t koff = (int64_t)kt * kBK;
+        const int8_t *ak = a_base + (int64_t)kt * kBK, *bk = b_base + (int64_t)kt * kBK;  // scalar arithmetic
 #pragma unroll
         for (int i = 0; i < LD; ++i) {
-            load_to_lds_16(a_src[i] + koff, base + i * 1024u);
-            load_to_lds_16(b_src[i] + koff, base + A_BYTES + i * 1024u);
+            load_to_lds_16(ak, a_off[i], base + i * 1024u);
+            load_to_lds_16(bk, b_off[i], base + A_BYTES + i * 1024u);
         }
     };
 
@@ -195,17 +211,27 @@ __global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8A
 #pragma unroll
     for (int st = 0; st < kStages - 1; ++st)
         if (st < num_kt) issue(st);
-    // Fragment addresses: lane (row = lane % 32 of a 32-row MFMA tile, k group = lane / 32).
+    // Fragment addresses: lane (row = lane % 32 of a 32-row MFMA tile, k group = lane / 32). The swizzle term of a row
+    // depends on lane % 32 only (tile rows of a wavefront start at multiples of 32), so two per-lane byte offsets per
+    // operand - one for each 32-byte K step - serve every read, with the stage, the MFMA tile row and the operand as
+    // immediate offsets: the loop below is unrolled over the ring of stages so that the stage index is a constant.
     const int frow = lane & 31, kg = lane >> 5;
+    const unsigned swz = (unsigned)(frow >> 2) & 3u;
+    unsigned fa[2], fb[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+        const unsigned slot = ((unsigned)(ks * 2 + kg) ^ swz) << 4;
+        fa[ks] = (unsigned)(wm * (32 * TW) + frow) * kBK + slot;
+        fb[ks] = (unsigned)A_BYTES + (unsigned)(wn * (32 * TW) + frow) * kBK + slot;
+    }
     V4i af[2][TW], bf[2][TW];  // fragment registers of the two 32-byte K steps of a stage
-    auto fetch = [&](int kt, int ks) __attribute__((always_inline)) {
-        const unsigned char *As = smem + (kt % kStages) * STAGE, *Bs = As + A_BYTES;
-        const int q = ks * 2 + kg;
+    auto fetch = [&](auto stage_c, int ks) __attribute__((always_inline)) {
+        constexpr int stage = decltype(stage_c)::value;
+        const unsigned char *base = smem + stage * STAGE;
 #pragma unroll
         for (int i = 0; i < TW; ++i) {
-            const int ra = wm * (32 * TW) + i * 32 + frow, rb = wn * (32 * TW) + i * 32 + frow;
-            af[ks][i] = *reinterpret_cast<const V4i *>(As + ra * kBK + ((q ^ ((ra >> 2) & 3)) << 4));
-            bf[ks][i] = *reinterpret_cast<const V4i *>(Bs + rb * kBK + ((q ^ ((rb >> 2) & 3)) << 4));
+            af[ks][i] = *reinterpret_cast<const V4i *>(base + fa[ks] + i * 32 * kBK);
+            bf[ks][i] = *reinterpret_cast<const V4i *>(base + fb[ks] + i * 32 * kBK);
         }
     };
     auto mma = [&](int ks) __attribute__((always_inline)) {
@@ -225,26 +251,44 @@ __global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8A
     };
     land(0);
     if (kStages - 1 < num_kt) issue(kStages - 1);
-    fetch(0, 0);
-    // Steady state, one stage per iteration: the fragments of a K step are read from LDS while the MFMAs of the step
+    fetch(std::integral_constant<int, 0>{}, 0);
+    // Steady state, one stage per step: the fragments of a K step are read from LDS while the MFMAs of the step
     // before it run, across the stage boundary as well, so neither the LDS latency nor the barrier wait is followed
-    // by an MFMA that needs what was just requested.
-    // The last stage is peeled off so that the loop body is straight-line code: with a conditional fetch the
+    // by an MFMA that needs what was just requested. A step is straight-line code (with a conditional fetch the
     // compiler's wait-count pass joins two paths in front of the second batch of MFMAs and makes it wait for the
-    // reads that were only just issued.
-    for (int kt = 0; kt + 1 < num_kt; ++kt) {
-        fetch(kt, 1);
+    // reads that were only just issued); the last stage is finished after the loop.
+    auto step = [&](int kt, auto stage_c) __attribute__((always_inline)) {
+        constexpr int stage = decltype(stage_c)::value;
+        fetch(stage_c, 1);
         __builtin_amdgcn_sched_barrier(0);
         mma(0);
         __builtin_amdgcn_sched_barrier(0);
         land(kt + 1);  // also: every wavefront has finished reading stage kt, whose buffer takes stage kt + kStages
         if (kt + kStages < num_kt) issue(kt + kStages);
-        fetch(kt + 1, 0);
+        fetch(std::integral_constant<int, (stage + 1) % kStages>{}, 0);
         __builtin_amdgcn_sched_barrier(0);
         mma(1);
         __builtin_amdgcn_sched_barrier(0);
+    };
+    static_assert(kStages == 4, "the main loop is unrolled over four stages");
+    int kt = 0;
+    for (; kt + kStages < num_kt; kt += kStages) {
+        step(kt + 0, std::integral_constant<int, 0>{});
+        step(kt + 1, std::integral_constant<int, 1>{});
+        step(kt + 2, std::integral_constant<int, 2>{});
+        step(kt + 3, std::integral_constant<int, 3>{});
     }
-    fetch(num_kt - 1, 1);
+    // one to four stages are left (kt is a multiple of four): all but the last as steps, then the last one's second half
+    const int left = num_kt - kt;
+    if (left > 1) step(kt + 0, std::integral_constant<int, 0>{});
+    if (left > 2) step(kt + 1, std::integral_constant<int, 1>{});
+    if (left > 3) step(kt + 2, std::integral_constant<int, 2>{});
+    switch (left) {
+        case 1: fetch(std::integral_constant<int, 0>{}, 1); break;
+        case 2: fetch(std::integral_constant<int, 1>{}, 1); break;
+        case 3: fetch(std::integral_constant<int, 2>{}, 1); break;
+        default: fetch(std::integral_constant<int, 3>{}, 1); break;
+    }
     __builtin_amdgcn_sched_barrier(0);
     mma(0);
     mma(1);
@@ -396,7 +440,7 @@ int32_t fth_dev_linear_int8_prequantized_f32(const int8_t *x_i8, const float *a_
     p.vec_store = (n % 4 == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0) ? 1 : 0;
     const bool aligned = ((reinterpret_cast<uintptr_t>(x_i8) | reinterpret_cast<uintptr_t>(w_i8)) & 15u) == 0;
     const int64_t tiles128 = fth::ceil_div(m, 128) * fth::ceil_div(n, 128), tiles256 = fth::ceil_div(m, 256) * fth::ceil_div(n, 256);
-    if (k >= kBK && k % kBK == 0 && aligned && tiles128 <= 2147483647LL) {
+    if (k >= kBK && k % kBK == 0 && k <= (1 << 23) && aligned && tiles128 <= 2147483647LL) {  // (256 rows of k bytes within 32 bits)
         // 256 x 256 tiles once they give every compute unit a workgroup and the reduction is long enough to pay for their
         // longer fill and drain: they need half the L2 -> LDS traffic per MFMA, and that path (about 27 bytes per clock
         // and compute unit in this access pattern) is what bounds the 128 x 128 loop. The choice depends on the shape only.
