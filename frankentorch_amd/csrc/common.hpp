@@ -27,6 +27,28 @@ int compute_units();
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Causal attention launches whose workgroups are ALL resident at once (grid <= workgroups per compute unit x compute
+// units) cannot rely on heaviest-first issue to balance: nothing is left to hand out when a light workgroup ends. The
+// hardware deals workgroup ids round-robin over the 8 XCDs and, inside an XCD, over its compute units in id order, so a
+// compute unit holds ids j, j + P, j + 2 P, ... of its XCD (P = compute units per XCD). Walking every other pass
+// backwards pairs the heavy end of one pass with the light end of the next; a compute unit's workgroups then add up to
+// about the same work. Returns the pass length P when the launch qualifies, else 0.
+template <typename K> int snake_pass_length(K kernel, int threads, size_t smem, int64_t grid, bool causal) {
+    if (!causal) return 0;
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, smem) != hipSuccess || per_cu <= 0) return 0;
+    const int cus = compute_units() > 0 ? compute_units() : 256;
+    return (cus % 8 == 0 && grid <= (int64_t)per_cu * cus && grid > cus) ? cus / 8 : 0;
+}
+
+// Position i of an XCD's id sequence of `total` entries -> the position whose work it takes (see snake_pass_length).
+__host__ __device__ inline int64_t snake_order(int64_t i, int pass_len, int64_t total) {
+    if (pass_len <= 0) return i;
+    const int64_t pass = i / pass_len, j = i % pass_len, lo = pass * pass_len;
+    const int64_t hi = lo + pass_len < total ? lo + pass_len : total;
+    return (pass & 1) ? hi - 1 - j : i;
+}
+
 }  // namespace fth
 
 #define FTH_HIP(expr)                                             \

@@ -54,6 +54,7 @@ struct SdpaArgs {
     int64_t mask_bh_stride;  // 0: one mask for every (batch, head); else elements between consecutive bh
     int64_t group;           // query heads per K/V head (grouped-query attention), >= 1
     int mask_vec;            // mask rows can be read as aligned float4 (seq_k % 4 == 0, 16-byte aligned base and bh stride)
+    int snake;               // > 0: every workgroup is resident at once; pass length of fth::snake_order
 };
 
 // exp(x - m) for x <= m as 2^((x - m) * log2 e) on the hardware exp2 unit: subtract, multiply,
@@ -112,8 +113,8 @@ __device__ __forceinline__ float f4_get(const float4 &v, int e) { return e == 0 
 // past seq_k are clamped to the last row (their scores are masked, their weights are zero).
 // MASK: an additive mask row is read for every (query, key) score, mask[bh * mask_bh_stride + qi * seq_k + key]
 // (sdpa_forward_masked_f64, crates/ft-kernel-cpu/src/lib.rs:4661-4741): score * scale + mask, then the same softmax.
-template <int D, int NW, bool PAIR, int BC, bool DIRECT, bool MASK>
-__global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p) {
+template <int D, int NW, bool PAIR, int BC, bool DIRECT, bool MASK, int MINW = 2>
+__global__ __launch_bounds__(64 * NW, MINW) void sdpa_mfma_kernel(const SdpaArgs p) {
     constexpr int kBC = BC;
     constexpr int KS = BC / 32;        // 32-key sub-tiles per tile
     constexpr int NTH = 64 * NW;
@@ -146,7 +147,9 @@ __global__ __launch_bounds__(64 * NW, 2) void sdpa_mfma_kernel(const SdpaArgs p)
         const int64_t pid = blockIdx.x;
         const int64_t g = p.group, kv_heads = d.num_bh / g;
         if (kv_heads % kXcds == 0) {
-            const int64_t xcd = pid % kXcds, w = pid / kXcds, per = d.num_bh / kXcds;
+            const int64_t xcd = pid % kXcds, per = d.num_bh / kXcds;
+            int64_t w = pid / kXcds;
+            w = fth::snake_order(w, p.snake, (int64_t)units * per);
             unit = (int)(w / per);
             const int64_t idx = w % per;
             bh = ((idx / g) * kXcds + xcd) * g + idx % g;
@@ -817,11 +820,12 @@ template <int D> int32_t launch_mfma_f64(SdpaArgs &a, hipStream_t st) {
     return FTH_OK;
 }
 
-template <int D, int NW, bool PAIR, bool MASK> int32_t launch_mfma_cfg(SdpaArgs &a, hipStream_t st) {
-    constexpr int BC = (D <= 64 && (NW == 4 || D <= 32)) ? 64 : 32;  // 64-key tiles where two workgroups still fit a CU
+template <int D, int NW, bool PAIR, bool MASK, bool OCC3 = false> int32_t launch_mfma_cfg(SdpaArgs &a, hipStream_t st) {
+    // 64-key tiles where two workgroups still fit a CU; 32-key tiles (and a register budget for three) where three should
+    constexpr int BC = OCC3 ? 32 : (D <= 64 && (NW == 4 || D <= 32)) ? 64 : 32;
     constexpr bool DIRECT = D >= 64 && FTH_SDPA_DIRECT;
     constexpr size_t smem = DIRECT ? (size_t)2 * BC * 2 * D * sizeof(float) : (size_t)2 * BC * ((D + 4) + (D + 8)) * sizeof(float);
-    auto kern = sdpa_mfma_kernel<D, NW, PAIR, BC, DIRECT, MASK>;
+    auto kern = sdpa_mfma_kernel<D, NW, PAIR, BC, DIRECT, MASK, OCC3 ? 3 : 2>;
     static bool attr_set = false;
     if (!attr_set) {
         FTH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -831,6 +835,7 @@ template <int D, int NW, bool PAIR, bool MASK> int32_t launch_mfma_cfg(SdpaArgs 
     const int64_t units = PAIR ? (a.q_blocks + 1) / 2 : a.q_blocks;
     const int64_t grid = a.d.num_bh * units;
     FTH_ARG(grid <= 2147483647LL, "sdpa: grid too large");
+    a.snake = PAIR ? 0 : fth::snake_pass_length(kern, 64 * NW, smem, grid, a.d.causal != 0);
     kern<<<dim3((unsigned)grid), dim3(64 * NW), smem, st>>>(a);
     FTH_CHECK_LAUNCH("sdpa_mfma");
     return FTH_OK;
@@ -995,12 +1000,20 @@ template <int D> int32_t launch_mfma(SdpaArgs &a, hipStream_t st) {
     const int64_t wg128 = a.d.num_bh * fth::ceil_div(a.d.seq_q, 128);
     bool wide = D >= 128 || 2 * wg128 >= (int64_t)cus;  // D = 128 staging does not fit 2-wavefront blocks
     static const int forced = [] {
-        const char *e = std::getenv("FT_HIP_SDPA_CFG");  // tuning knob: bit 0 = 4 wavefronts, bit 1 = pairing; -1 = auto
+        const char *e = std::getenv("FT_HIP_SDPA_CFG");  // tuning knob: bit 0 = 4 wavefronts, bit 1 = pairing, bit 2 = 32-key tiles at head size 64; -1 = auto
         return e ? std::atoi(e) : -1;
     }();
     if (forced >= 0) {
         wide = D >= 128 || (forced & 1);
         pair = a.d.causal != 0 && (forced & 2);
+    }
+    if constexpr (D == 64) {
+        // Between two and four workgroups per compute unit a causal launch takes 32-key tiles, of which four workgroups
+        // fit a compute unit (two of the 64-key ones do): everything is resident at once and the order of
+        // fth::snake_order balances the compute units, which heaviest-first issue on two slots cannot (GPT-2's 96 heads
+        // x 8 query blocks: the heaviest block alone is 8 of the 6.75 work units per slot).
+        const bool three = forced >= 0 ? (forced & 4) != 0 : (a.d.causal != 0 && wg128 > 2 * (int64_t)cus && wg128 <= 4 * (int64_t)cus);
+        if (!a.mask && !pair && wide && three) return launch_mfma_cfg<D, 4, false, false, true>(a, st);
     }
     if (a.mask) return wide ? launch_mfma_cfg<D, 4, false, true>(a, st) : launch_mfma_cfg<D, 2, false, true>(a, st);
     if (pair) return wide ? launch_mfma_cfg<D, 4, true, false>(a, st) : launch_mfma_cfg<D, 2, true, false>(a, st);
@@ -1030,6 +1043,7 @@ int32_t sdpa_entry(const fth_sdpa_desc *d, double scale, const T *q, const T *k,
     a.mask = masked ? mask : nullptr;
     a.mask_bh_stride = mask_bh_stride;
     a.group = group;
+    a.snake = 0;
     a.mask_vec = (d->seq_k % 4 == 0 && mask_bh_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(mask) & 15u) == 0) ? 1 : 0;
     auto al16 = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; };
     auto m4 = [](int64_t x) { return x % 4 == 0; };

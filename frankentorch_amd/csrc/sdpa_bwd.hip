@@ -34,9 +34,6 @@
 namespace {
 
 constexpr int kWave = 64;
-#ifndef FTH_SDPA_BWD_KEYS_OCC
-#define FTH_SDPA_BWD_KEYS_OCC 1
-#endif
 using Acc16 = float __attribute__((ext_vector_type(16)));
 typedef float nat_f4 __attribute__((ext_vector_type(4)));
 
@@ -49,6 +46,7 @@ struct KeysArgs {
     float scale;
     int causal;
     int row_block;  // dS is defined (zero where masked) from the start of the row block that holds a key block's first key; 0: from row 0
+    int snake;      // > 0: every workgroup is resident at once; pass length of fth::snake_order
 };
 
 // One wavefront-wide global -> LDS copy of 16 bytes per lane (scalar base, per-lane byte offset): lane L's bytes land
@@ -138,6 +136,7 @@ struct StatsArgs {
     int seq_q, seq_k;
     float scale;
     int causal;
+    int snake;  // > 0: every workgroup is resident at once; pass length of fth::snake_order
 };
 
 template <int D, int BC>
@@ -164,7 +163,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_stats_kernel(const StatsArgs 
     {
         const int64_t pid = blockIdx.x;
         if (p.num_bh % 8 == 0) {
-            const int64_t xcd = pid % 8, w = pid / 8, per = p.num_bh / 8;
+            const int64_t xcd = pid % 8, per = p.num_bh / 8;
+            const int64_t w = fth::snake_order(pid / 8, p.snake, (int64_t)q_blocks * per);
             unit = (int)(w / per);
             bh = (w % per) * 8 + xcd;
         } else {
@@ -405,13 +405,15 @@ template <int D> int32_t launch_stats(const StatsArgs &a, hipStream_t st) {
     }
     const int64_t grid = a.num_bh * fth::ceil_div(a.seq_q, 128);
     FTH_ARG(grid <= 2147483647LL, "sdpa backward: grid too large");
-    sdpa_bwd_stats_kernel<D, BC><<<dim3((unsigned)grid), dim3(256), smem, st>>>(a);
+    StatsArgs b = a;
+    b.snake = a.num_bh % 8 == 0 ? fth::snake_pass_length(sdpa_bwd_stats_kernel<D, BC>, 256, smem, grid, a.causal != 0) : 0;
+    sdpa_bwd_stats_kernel<D, BC><<<dim3((unsigned)grid), dim3(256), smem, st>>>(b);
     FTH_CHECK_LAUNCH("sdpa_bwd_stats");
     return FTH_OK;
 }
 
 template <int D>
-__global__ __launch_bounds__(256, FTH_SDPA_BWD_KEYS_OCC) void sdpa_bwd_keys_kernel(const KeysArgs p) {
+__global__ __launch_bounds__(256, D == 64 ? 3 : 2) void sdpa_bwd_keys_kernel(const KeysArgs p) {
     constexpr int NDT = D / 32;        // 32-wide d-tiles of dK^T / dV^T
     constexpr int VPR = D / 4;         // 16-byte vectors per row
     constexpr int RPC = 64 / VPR;      // tile rows per 1 KiB load instruction
@@ -425,8 +427,10 @@ __global__ __launch_bounds__(256, FTH_SDPA_BWD_KEYS_OCC) void sdpa_bwd_keys_kern
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lq = lane & 31, half = lane >> 5;
-    const int64_t pid = blockIdx.x;
-    const int kb = (int)(pid / p.num_bh);  // key blocks in ascending order: under a causal mask the heaviest come first
+    // key blocks in ascending order: under a causal mask the heaviest come first (or, when every workgroup is resident
+    // at once, in the back-and-forth order of fth::snake_order over each XCD's ids)
+    const int64_t pid = p.snake > 0 ? (int64_t)(blockIdx.x % 8) + 8 * fth::snake_order(blockIdx.x / 8, p.snake, gridDim.x / 8) : (int64_t)blockIdx.x;
+    const int kb = (int)(pid / p.num_bh);
     const int64_t bh = pid % p.num_bh;
     const int seq_q = p.seq_q, seq_k = p.seq_k;
     const unsigned wave_u = __builtin_amdgcn_readfirstlane((unsigned)wave);  // scalar copy: what derives from it stays scalar
@@ -637,7 +641,9 @@ template <int D> int32_t launch_keys(const KeysArgs &a, hipStream_t st) {
     }
     const int64_t k_blocks = fth::ceil_div(a.seq_k, 128), grid = a.num_bh * k_blocks;
     FTH_ARG(grid <= 2147483647LL, "sdpa backward: grid too large");
-    sdpa_bwd_keys_kernel<D><<<dim3((unsigned)grid), dim3(256), smem, st>>>(a);
+    KeysArgs b = a;
+    b.snake = grid % 8 == 0 ? fth::snake_pass_length(sdpa_bwd_keys_kernel<D>, 256, smem, grid, a.causal != 0) : 0;
+    sdpa_bwd_keys_kernel<D><<<dim3((unsigned)grid), dim3(256), smem, st>>>(b);
     FTH_CHECK_LAUNCH("sdpa_bwd_keys");
     return FTH_OK;
 }
@@ -659,6 +665,7 @@ struct DqArgs {
     int seq_q, seq_k;
     float scale;
     int causal;
+    int snake;  // > 0: every workgroup is resident at once; pass length of fth::snake_order
 };
 
 template <int D>
@@ -674,7 +681,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_kernel(const DqArgs p) {
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lq = lane & 31, half = lane >> 5;
-    const int64_t pid = blockIdx.x;
+    const int64_t pid = p.snake > 0 ? (int64_t)(blockIdx.x % 8) + 8 * fth::snake_order(blockIdx.x / 8, p.snake, gridDim.x / 8) : (int64_t)blockIdx.x;
     const int q_blocks = (p.seq_q + 127) / 128;
     const int qb = q_blocks - 1 - (int)(pid / p.num_bh);  // heaviest (latest) query blocks first under a causal mask
     const int64_t bh = pid % p.num_bh;
@@ -794,7 +801,9 @@ template <int D> int32_t launch_dq(const DqArgs &a, hipStream_t st) {
     constexpr size_t smem = (size_t)2 * 32 * D * sizeof(float);
     const int64_t grid = a.num_bh * fth::ceil_div(a.seq_q, 128);
     FTH_ARG(grid <= 2147483647LL, "sdpa backward: grid too large");
-    sdpa_bwd_dq_kernel<D><<<dim3((unsigned)grid), dim3(256), smem, st>>>(a);
+    DqArgs b = a;
+    b.snake = grid % 8 == 0 ? fth::snake_pass_length(sdpa_bwd_dq_kernel<D>, 256, smem, grid, a.causal != 0) : 0;
+    sdpa_bwd_dq_kernel<D><<<dim3((unsigned)grid), dim3(256), smem, st>>>(b);
     FTH_CHECK_LAUNCH("sdpa_bwd_dq");
     return FTH_OK;
 }
