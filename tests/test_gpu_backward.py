@@ -188,7 +188,7 @@ def test_sdpa_backward_masked_reduces_to_the_unmasked_and_causal_forms(hip):
             assert rel_err(a.to_host(), b.to_host()) <= TOL_GEMM_F32
 
 
-@pytest.mark.parametrize("bh,sq,sk,d,causal", [(4, 2048, 2048, 128, True), (2, 1024, 1536, 64, False), (3, 1100, 1100, 64, True)])
+@pytest.mark.parametrize("bh,sq,sk,d,causal", [(4, 2048, 2048, 128, True), (2, 1024, 1536, 64, False), (3, 1100, 1100, 64, True), (96, 1024, 1024, 64, True)])
 def test_fused_sdpa_backward_against_the_materialising_path_at_full_length(hip, bh, sq, sk, d, causal):
     """Head sizes 64 / 128 without a mask take the fused three-pass backward (scores + statistics, key-owned pass,
     query-owned pass); the same problem with its mask passed explicitly takes the materialising path (five batched GEMMs

@@ -123,3 +123,25 @@ def test_config4_full_size_sampled_heads_determinism_and_checksum(hip, oracle):
         assert rel_err(out[bh:bh + 1], ref) <= TOL_GEMM_F32
     assert np.all(out.max(axis=1) <= v.max(axis=1) + 1e-6) and np.all(out.min(axis=1) >= v.min(axis=1) - 1e-6)
     assert np.array_equal(out[:, 0], v[:, 0])
+
+
+@pytest.mark.parametrize("bh,seq", [(96, 1024), (64, 1152), (32, 4096)])
+def test_fully_resident_causal_launch_sampled_heads(hip, oracle, bh, seq):
+    """Causal, head size 64, between two and four query blocks per compute unit: every workgroup of the launch is
+    resident at once and the query blocks are handed out in the back-and-forth order (32-key tiles). Sampled
+    (batch, head) slices against the oracle, the first row, and bitwise equality of two runs."""
+    D = 64
+    s = 1.0 / math.sqrt(D)
+    q, k, v = (synth.normal(21, n, (bh, seq, D)) for n in ("Q", "K", "V"))
+    dq, dk, dv = DeviceBuffer.from_host(q), DeviceBuffer.from_host(k), DeviceBuffer.from_host(v)
+    do, do2 = DeviceBuffer(q.shape), DeviceBuffer(q.shape)
+    desc = hip.sdpa_desc_contiguous(bh, seq, seq, D, D, True)
+    hip.sdpa_forward(desc, s, dq, dk, dv, do)
+    hip.sdpa_forward(desc, s, dq, dk, dv, do2)
+    out = do.to_host()
+    assert np.array_equal(out.view(np.uint32), do2.to_host().view(np.uint32))
+    for h in (0, bh // 2 + 3, bh - 1):
+        ref = oracle.sdpa_forward(q[h:h + 1], k[h:h + 1], v[h:h + 1], s, True)
+        assert rel_err(out[h:h + 1], ref) <= TOL_GEMM_F32
+    assert np.array_equal(out[:, 0], v[:, 0])
+    assert np.all(out.max(axis=1) <= v.max(axis=1) + 1e-5) and np.all(out.min(axis=1) >= v.min(axis=1) - 1e-5)
