@@ -817,7 +817,7 @@ bool sdpa_backward_fused_applies(int64_t num_bh, int64_t seq_q, int64_t seq_k, i
         const char *e = std::getenv("FT_HIP_SDPA_BWD_FUSED");  // tuning / testing knob: 0 keeps the materialising backward
         return e && std::atoi(e) == 0;
     }();
-    if (off || d_k != d_v || (d_k != 64 && d_k != 128) || seq_q % 4 != 0 || seq_k % 4 != 0 || seq_q < 32 || seq_k < 32 || !(scale > 0.f)) return false;
+    if (off || d_k != d_v || (d_k != 64 && d_k != 128) || seq_q < 32 || seq_k < 32 || !(scale > 0.f)) return false;
     // byte offsets inside one (batch, head) slab of tiles stay below 2^30, and so do those inside its operands
     const int64_t qt = (seq_q + 31) / 32, kt = (seq_k + 31) / 32;
     return (qt + 4) * kt * 4096 < ((int64_t)1 << 30) && seq_q * d_k < (1 << 28) && seq_k * d_k < (1 << 28);

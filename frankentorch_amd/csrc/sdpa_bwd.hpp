@@ -7,8 +7,7 @@
 
 namespace fth {
 
-// True when the fused path covers the problem: d_k == d_v in {64, 128}, sequence lengths multiples of 4 and at least 32,
-// a positive scale. Operands are contiguous [num_bh, seq, d] and 16-byte aligned (the caller checks the pointers).
+// True when the fused path covers the problem: d_k == d_v in {64, 128}, sequence lengths of at least 32, a positive scale. Operands are contiguous [num_bh, seq, d] and 16-byte aligned (the caller checks the pointers).
 bool sdpa_backward_fused_applies(int64_t num_bh, int64_t seq_q, int64_t seq_k, int64_t d_k, int64_t d_v, float scale);
 
 // Sizes, in floats, of the two score-shaped workspace arrays of the fused path: `s` holds the raw scores, `d` holds dP

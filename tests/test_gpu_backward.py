@@ -89,13 +89,14 @@ def test_linear_backward_reference_test_inputs(hip, oracle):
 
 # The last four shapes are square and long enough for the causal form to take the block-causal products
 # (blocks of 256 rows; 640 and 1152 end in a partial block).
-# Head sizes 64 and 128 with sequence lengths that are multiples of 4 take the fused path (statistics pass, key-owned
+# Head sizes 64 and 128 with sequence lengths of at least 32 take the fused path (statistics pass, key-owned
 # kernel, dQ product; intermediates in whole 32 x 32 tiles); the ragged ones among them end in partial query tiles and
-# partial key blocks, the last three in a single tile, in fewer keys than a key block holds and in more queries than keys.
+# partial key blocks: a single tile, fewer keys than a key block holds, more queries than keys, odd lengths.
 @pytest.mark.parametrize("bh,sq,sk,dk,dv", [(2, 64, 64, 64, 64), (3, 100, 70, 32, 48), (4, 128, 128, 128, 128), (1, 5, 6, 4, 3), (2, 33, 200, 16, 16),
                                             (2, 512, 512, 64, 64), (1, 640, 640, 32, 48), (3, 1024, 1024, 64, 64), (2, 1152, 1152, 128, 128),
                                             (2, 100, 76, 64, 64), (1, 36, 260, 128, 128), (2, 256, 384, 64, 64), (2, 388, 132, 128, 128),
-                                            (1, 32, 32, 64, 64), (2, 132, 36, 128, 128), (1, 580, 68, 64, 64)])
+                                            (1, 32, 32, 64, 64), (2, 132, 36, 128, 128), (1, 580, 68, 64, 64),
+                                            (2, 101, 77, 64, 64), (1, 45, 131, 128, 128), (2, 333, 333, 64, 64)])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_sdpa_backward(hip, oracle, bh, sq, sk, dk, dv, causal, dtype):
@@ -151,7 +152,7 @@ def test_sdpa_backward_masked(hip, oracle, bh, sq, sk, dk, dv, shared, dtype):
             assert rel_err(g, r) <= tol
 
 
-@pytest.mark.parametrize("bh,sq,sk,dk,dv", [(2, 5, 6, 4, 3), (3, 100, 70, 32, 48), (2, 640, 640, 64, 64)])
+@pytest.mark.parametrize("bh,sq,sk,dk,dv", [(2, 5, 6, 4, 3), (3, 100, 70, 32, 48), (2, 640, 640, 64, 64), (2, 99, 71, 64, 64)])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_sdpa_backward_unit_dout(hip, oracle, bh, sq, sk, dk, dv, causal, dtype):
