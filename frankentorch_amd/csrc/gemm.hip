@@ -486,7 +486,10 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
     static_assert(LPR_A <= kWave && kWave % LPR_A == 0, "a chunk must hold whole k rows of A");
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile rows must divide into 8-row chunks per wavefront");
     static_assert(MT % 16 == 0, "swizzle assumes MFMA tile rows start on a multiple of 16");
-    static_assert(TRANS_B || (LPR <= kWave && kWave % LPR == 0), "a chunk must hold whole k rows of B");
+    // [k,n] B: chunks of whole k rows where a row's vectors divide the wavefront (BN = 64, 128); otherwise (BN = 96: 24
+    // vectors a row) the tile's vectors are dealt to the lanes in row-major order and a chunk ends mid-row.
+    constexpr bool B_WHOLE_ROWS = LPR <= kWave && kWave % LPR == 0;
+    static_assert(TRANS_B || B_WHOLE_ROWS || BK * LPR % kWave == 0, "the [k,n] tile must be a whole number of chunks");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *As = reinterpret_cast<T *>(smem_raw);  // [2][BM][BK]
@@ -567,12 +570,23 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
             }
         } else {
             bk = uniform_ptr(p.b + batch * p.stride_b + (int64_t)ld_k * BK * p.ldb + n0);
-            int col = (lane % LPR) * EPV;
-            col = col < b_cols ? col : b_cols - EPV;  // n is a multiple of EPV on this path
+            if constexpr (B_WHOLE_ROWS) {
+                int col = (lane % LPR) * EPV;
+                col = col < b_cols ? col : b_cols - EPV;  // n is a multiple of EPV on this path
 #pragma unroll
-            for (int i = 0; i < B_LD; ++i) {
-                const int krow = (wave * B_LD + i) * RPC + lane / LPR;
-                b_off[i] = ((unsigned)krow * (unsigned)p.ldb + (unsigned)col) * (unsigned)sizeof(T);
+                for (int i = 0; i < B_LD; ++i) {
+                    const int krow = (wave * B_LD + i) * RPC + lane / LPR;
+                    b_off[i] = ((unsigned)krow * (unsigned)p.ldb + (unsigned)col) * (unsigned)sizeof(T);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < B_LD; ++i) {
+                    const int vec = (wave * B_LD + i) * kWave + lane;  // vector index in the [BK][LPR] tile
+                    const int krow = vec / LPR;
+                    int col = (vec % LPR) * EPV;
+                    col = col < b_cols ? col : b_cols - EPV;
+                    b_off[i] = ((unsigned)krow * (unsigned)p.ldb + (unsigned)col) * (unsigned)sizeof(T);
+                }
             }
         }
     };
@@ -1295,12 +1309,13 @@ int32_t launch_shape(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
         if (!direct_off && t != Tile::Wide && p.k % DBK == 0 && p.lda <= lim && p.ldb <= lim && p.ldc <= lim) {
             constexpr int MINW_BIG = 2;
             if constexpr (std::is_same<T, float>::value) {
-                if constexpr (TRANS_B) {
+                {
                     // 128x96 tiles (4x1 wavefronts of 32x96) when they hand every resident workgroup (two per compute
                     // unit) a whole number of whole tiles and 128x128 tiles do not: no tile is split over K, no fix-up
                     // pass. All GPT-2 widths are multiples of 96 (768 = 8 x 96): QKV 0.77 -> 0.82, O-proj 0.75 -> 0.78,
                     // FC2 0.82 -> 0.83 of the matrix peak; where 128x128 tiles already divide evenly (FC1) they stay
-                    // (their main loop is 1-2 % faster).
+                    // (their main loop is 1-2 % faster). With B stored [k, n] the same holds for the input gradient of
+                    // a linear layer (dy . W at FC2's shape).
                     const int64_t slots = (int64_t)cus * 2;
                     const int64_t tiles96 = fth::ceil_div(p.m, 128) * (p.n / 96) * batch;
                     const bool n96 = f < 0 && t == Tile::Big && p.n % 96 == 0 && tiles96 % slots == 0 && big_tiles % slots != 0;
