@@ -7,6 +7,8 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
+#include <vector>
 
 #include "ft_kernel_hip.h"
 
@@ -35,8 +37,21 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // about the same work. Returns the pass length P when the launch qualifies, else 0.
 template <typename K> int snake_pass_length(K kernel, int threads, size_t smem, int64_t grid, bool causal) {
     if (!causal) return 0;
-    int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, smem) != hipSuccess || per_cu <= 0) return 0;
+    // The occupancy of a (kernel, block size, LDS size) never changes: asked once, kept (a handful of entries).
+    struct Seen { const void *k; int threads; size_t smem; int per_cu; };
+    static std::mutex mu;
+    static std::vector<Seen> seen;
+    int per_cu = -1;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        for (const Seen &e : seen)
+            if (e.k == reinterpret_cast<const void *>(kernel) && e.threads == threads && e.smem == smem) per_cu = e.per_cu;
+        if (per_cu < 0) {
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, smem) != hipSuccess) per_cu = 0;
+            seen.push_back({reinterpret_cast<const void *>(kernel), threads, smem, per_cu});
+        }
+    }
+    if (per_cu <= 0) return 0;
     const int cus = compute_units() > 0 ? compute_units() : 256;
     return (cus % 8 == 0 && grid <= (int64_t)per_cu * cus && grid > cus) ? cus / 8 : 0;
 }
