@@ -139,12 +139,16 @@ template <int WPR> struct RowBlock {
     static constexpr int kThreads = WPR <= 4 ? kBlock : kWave * WPR;
     static constexpr int kRows = kThreads / (kWave * WPR);
     // A compute unit holds 2048 threads (8 wavefronts per SIMD) at up to 64 vector registers per
-    // lane, 1024 at up to 128 and 512 at up to 256. `sets` counts the row-sized register sets the
-    // kernel keeps (row, prefetched row, gamma, beta, second operand); a set is 4 * vpl registers.
-    static constexpr int min_blocks(int vpl, int sets) {
+    // lane, 1536 at up to 85, 1024 at up to 128 and 512 at up to 256. `sets` counts the row-sized register sets the
+    // kernel keeps (row, prefetched row, gamma, beta, second operand); a set is 4 * vpl registers. The result is
+    // the second argument of __launch_bounds__, which hipcc reads as wavefronts per SIMD (not blocks per
+    // compute unit): the register budget the kernel is compiled for, whatever its block size.
+    static constexpr int min_blocks(int vpl, int sets, int elem_bytes) {
         const int regs = 4 * vpl * sets + 40;
-        const int threads = regs <= 64 ? 2048 : regs <= 128 ? 1024 : 512;
-        return threads / kThreads > 0 ? threads / kThreads : 1;
+        // (1536 threads: fp32 only; the fp64 kernels need the room for their exponential)
+        const int threads = regs <= 64 ? 2048 : (regs <= 80 && elem_bytes == 4) ? 1536 : regs <= 128 ? 1024 : 512;
+        const int waves = threads / 256, own = kThreads / 256;
+        return waves > own ? waves : own;
     }
 };
 constexpr int kMaxWaves = 16;
@@ -263,7 +267,7 @@ template <int VPL> constexpr bool kPrefetch = VPL <= 4;
 
 // ---- softmax ------------------------------------------------------------------------------
 template <typename T, int VPL, int WPR>
-__global__ __launch_bounds__(RowBlock<WPR>::kThreads, RowBlock<WPR>::min_blocks(VPL, 2)) void softmax_row_kernel(
+__global__ __launch_bounds__(RowBlock<WPR>::kThreads, RowBlock<WPR>::min_blocks(VPL, 2, (int)sizeof(T))) void softmax_row_kernel(
     const T *__restrict__ x, T *__restrict__ y, int64_t rows, int cols, int iters) {
     __shared__ T smem[2 * kMaxWaves];
     int phase = 0;
@@ -314,7 +318,7 @@ __global__ __launch_bounds__(RowBlock<WPR>::kThreads, RowBlock<WPR>::min_blocks(
 
 // ---- LayerNorm / add+LayerNorm ---------------------------------------------------------------
 template <typename T, int VPL, int WPR, bool ADD>
-__global__ __launch_bounds__(RowBlock<WPR>::kThreads, RowBlock<WPR>::min_blocks(VPL, ADD ? 5 : 4)) void layernorm_row_kernel(
+__global__ __launch_bounds__(RowBlock<WPR>::kThreads, RowBlock<WPR>::min_blocks(VPL, ADD ? 5 : 4, (int)sizeof(T))) void layernorm_row_kernel(
     const T *__restrict__ x, const T *__restrict__ x2, const T *__restrict__ w, const T *__restrict__ b, T *__restrict__ y,
     int64_t rows, int cols, T eps, int iters) {
     __shared__ T smem[2 * kMaxWaves];
@@ -493,7 +497,7 @@ __global__ __launch_bounds__(RowBlock<WPR>::kThreads) void layernorm_rows_kernel
 
 // ---- RMSNorm ---------------------------------------------------------------------------------
 template <typename T, int VPL, int WPR>
-__global__ __launch_bounds__(RowBlock<WPR>::kThreads, RowBlock<WPR>::min_blocks(VPL, 3)) void rmsnorm_row_kernel(
+__global__ __launch_bounds__(RowBlock<WPR>::kThreads, RowBlock<WPR>::min_blocks(VPL, 3, (int)sizeof(T))) void rmsnorm_row_kernel(
     const T *__restrict__ x, const T *__restrict__ w, T *__restrict__ y, int64_t rows, int cols, T eps, int iters) {
     __shared__ T smem[2 * kMaxWaves];
     int phase = 0;
@@ -756,7 +760,9 @@ inline bool pick_row_shape(int64_t nvec, int max_vpl, int &vpl, int &wpr) {
         const char *e = std::getenv("FT_HIP_ROW_WPR");  // tuning knob: wavefronts per row (1, 2, 4, 8 or 16)
         return e ? std::atoi(e) : 0;
     }();
-    int w = nvec <= 256 ? 1 : nvec <= 512 ? 2 : nvec <= 1024 ? 4 : nvec <= 4096 ? 8 : 16;
+    // (rows of 769 to 1024 vectors on eight wavefronts, two vectors a lane: at fp32 [8192, 4096] on rotating buffers softmax
+    // 0.754 -> 0.777 of the HBM peak, LayerNorm 0.719 -> 0.725, RMSNorm 0.739 -> 0.746 against four wavefronts with four vectors)
+    int w = nvec <= 256 ? 1 : nvec <= 512 ? 2 : nvec <= 768 ? 4 : nvec <= 4096 ? 8 : 16;
     if (forced == 1 || forced == 2 || forced == 4 || forced == 8 || forced == 16) {
         if (fth::ceil_div(nvec, 64 * forced) <= max_vpl) w = forced;
     }
@@ -865,6 +871,8 @@ int32_t launch_layernorm(const T *x, const T *x2, const T *w, const T *b, T *y, 
                   (!w || aligned16(w)) && (!b || aligned16(b));
     if (vec_ok && pick_row_shape(cols / EPV, ADD ? 8 : 16, vpl, wpr) && (row_launch_shape(rows, wpr, grid, iters), grid <= kMaxGrid)) {
         if constexpr (!ADD) {
+            // (Three 512-thread workgroups per compute unit, which is what the kernel's 65 registers allow, stream best at
+            // this shape: compiled for 64 registers and four per unit 0.704 of the HBM peak against 0.721, held to two 0.675.)
             // Two rows side by side (gamma / beta once per pair) where a lane's share of a row is at most four vectors and
             // there are rows enough to fill the chip that way; FT_HIP_LN_SIDE=0 keeps one row per group. Measured at fp32
             // [8192,4096] on rotating buffers: LayerNorm 0.70 -> 0.72 of the HBM peak with two rows, 0.64 with four (too few,
@@ -877,11 +885,12 @@ int32_t launch_layernorm(const T *x, const T *x2, const T *w, const T *b, T *y, 
             }();
             const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
             const int64_t side_grid = fth::ceil_div(rows, (int64_t)rows_per_block(wpr) * kSide);
-            if ((w || b) && !side_off && iters == 1 && wpr <= 4 && vpl <= 4 && side_grid >= 4 * (int64_t)cus) {
+            if ((w || b) && !side_off && iters == 1 && wpr <= 8 && vpl <= 4 && side_grid >= 4 * (int64_t)cus) {
 #define LS(V_, W_) layernorm_rows_kernel<T, V_, W_, kSide><<<dim3((unsigned)side_grid), dim3(RowBlock<W_>::kThreads), 0, st>>>(x, w, b, y, rows, (int)cols, eps)
                 switch (wpr) {
                     case 1: if (vpl == 1) { LS(1, 1); } else if (vpl == 2) { LS(2, 1); } else { LS(4, 1); } break;
                     case 2: if (vpl == 1) { LS(1, 2); } else if (vpl == 2) { LS(2, 2); } else { LS(4, 2); } break;
+                    case 8: if (vpl == 1) { LS(1, 8); } else if (vpl == 2) { LS(2, 8); } else { LS(4, 8); } break;
                     default: if (vpl == 1) { LS(1, 4); } else if (vpl == 2) { LS(2, 4); } else { LS(4, 4); } break;
                 }
 #undef LS
