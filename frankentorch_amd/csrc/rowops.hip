@@ -921,7 +921,12 @@ int32_t launch_rmsnorm(const T *x, const T *w, T *y, int64_t rows, int64_t cols,
     int64_t grid = 0;
     if (cols % EPV == 0 && aligned16(x) && aligned16(y) && (!w || aligned16(w)) &&
         pick_row_shape(cols / EPV, 16, vpl, wpr) && (row_launch_shape(rows, wpr, grid, iters), grid <= kMaxGrid)) {
-#define L(V_, W_) rmsnorm_row_kernel<T, V_, W_><<<dim3((unsigned)grid), dim3(RowBlock<W_>::kThreads), 0, st>>>(x, w, y, rows, (int)cols, eps, iters)
+        // 512-thread workgroups with a gamma vector stream best three to a compute unit, as the two-row LayerNorm kernel does
+        // by its registers (measured at fp32 [8192, 4096] on rotating buffers: four per unit 0.744 of the HBM peak, three 0.759,
+        // two 0.733; softmax, which reads no second vector, is best at four). The kernel's registers would allow four, so 48 KiB
+        // of unused dynamic LDS per workgroup hold the count at three.
+        const size_t pad = (wpr == 8 && w) ? (size_t)48 * 1024 : 0;
+#define L(V_, W_) rmsnorm_row_kernel<T, V_, W_><<<dim3((unsigned)grid), dim3(RowBlock<W_>::kThreads), pad, st>>>(x, w, y, rows, (int)cols, eps, iters)
         FTH_ROW_DISPATCH(vpl, wpr, L);
 #undef L
     } else {
