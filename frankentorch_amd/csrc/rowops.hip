@@ -877,7 +877,10 @@ int32_t launch_layernorm(const T *x, const T *x2, const T *w, const T *b, T *y, 
             // there are rows enough to fill the chip that way; FT_HIP_LN_SIDE=0 keeps one row per group. Measured at fp32
             // [8192,4096] on rotating buffers: LayerNorm 0.70 -> 0.72 of the HBM peak with two rows, 0.64 with four (too few,
             // too fat workgroups); without gamma and beta one row per group streams best (0.76 against 0.72), and so it does for
-            // RMSNorm with its single gamma (0.74 against 0.72 with two rows).
+            // RMSNorm with its single gamma (0.74 against 0.72 with two rows). At eight wavefronts per row (two vectors a
+            // lane) three rows side by side measure 0.696 and four 0.659 against 0.722 with two. Across all variants the
+            // rate follows the bytes a row moves from L2 into the compute unit: 16 KiB (softmax) 0.776, 32 KiB (RMSNorm;
+            // LayerNorm two rows at a time) 0.72-0.76, 48 KiB (LayerNorm one row at a time) 0.67.
             constexpr int kSide = 2;
             static const bool side_off = [] {
                 const char *e = std::getenv("FT_HIP_LN_SIDE");
