@@ -74,6 +74,28 @@ def test_linear_backward(hip, oracle, batch, in_f, out_f, dtype):
     assert np.all(ddb2.to_host() == 7)
 
 
+def test_linear_backward_at_the_benchmark_shape_sampled(hip, oracle):
+    """Batch 8192, 768 -> 3072 (the FC1 layer of the GPT-2 shape): dx = dy . W is an 8192 x 768 x 3072 product with W stored
+    [k, n], which runs on 128 x 96 tiles (512 whole tiles, one per resident workgroup); dweight splits its 8192-deep reduction
+    across workgroups. Sampled rows of both against the checker's GEMM, dbias against its column sum, and a bitwise repeat."""
+    batch, in_f, out_f = 8192, 768, 3072
+    dy = synth.normal(33, "dy", (batch, out_f))
+    x = synth.normal(33, "x", (batch, in_f))
+    w = synth.normal(33, "w", (out_f, in_f), 0.0, 0.02)
+    ddy, dx_, dw_ = _up(dy, x, w)
+    ddx, ddw, ddb = DeviceBuffer((batch, in_f)), DeviceBuffer((out_f, in_f)), DeviceBuffer((out_f,))
+    hip.linear_backward(ddy, dx_, dw_, ddx, ddw, ddb, batch, in_f, out_f)
+    gx, gw, gb = ddx.to_host(), ddw.to_host(), ddb.to_host()
+    rows = np.unique(np.concatenate([np.arange(3, batch, 131), [0, 127, 128, batch - 1]]))
+    assert rel_err(gx[rows], oracle.gemm(dy[rows], w, False)) <= TOL_GEMM_F32
+    outs = np.unique(np.concatenate([np.arange(5, out_f, 67), [0, 95, 96, out_f - 1]]))
+    assert rel_err(gw[outs], oracle.gemm(np.ascontiguousarray(dy[:, outs].T), x, False)) <= TOL_GEMM_F32
+    assert rel_err(gb, oracle.gemm(np.ones((1, batch), np.float32), dy, False)[0]) <= TOL_GEMM_F32
+    hip.linear_backward(ddy, dx_, dw_, ddx, ddw, ddb, batch, in_f, out_f)
+    for a, b in zip((gx, gw, gb), (ddx.to_host(), ddw.to_host(), ddb.to_host())):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
 def test_linear_backward_reference_test_inputs(hip, oracle):
     """The inputs of the reference's own dweight test (crates/ft-kernel-cpu/src/lib.rs:43862-43911), fp64."""
     batch, in_f, out_f = 96, 40, 72
