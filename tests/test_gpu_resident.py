@@ -106,6 +106,61 @@ def test_config1_block_forward_eager_graph_and_determinism(hip, oracle):
     assert rel_err(enc3.forward(x3, 3, 40), ref3) <= TOL_GEMM_F32
 
 
+def test_block_equals_its_separate_launches_bit_for_bit(hip):
+    """The resident block is a fixed sequence of the library's own launches (LayerNorm, GEMM + epilogue, SDPA on the strided
+    operands of the packed QKV projection). Issued one by one through the public device operations it must give the same
+    bits, at config 1 and at a token count that is not a multiple of any tile (d_model 384, 45 tokens, non-causal)."""
+    from frankentorch_amd import _lib
+    batch, seq, d, heads, f = 1, 128, 256, 4, 1024
+    T, hd = batch * seq, d // heads
+    L = make_layer(0, 1, d, f, biases_zero=False)
+    x = synth.normal(0, "x", (T, d))
+    got = fused.EncoderHip(d, heads, f, [L], 1e-5, causal=True).forward(x, batch, seq)
+    up = DeviceBuffer.from_host
+    dx = up(x)
+    wqkv, bqkv = up(np.concatenate([L["wq"], L["wk"], L["wv"]])), up(np.concatenate([L["bq"], L["bk"], L["bv"]]))
+    h, qkv, ctx, xa, ff, out = (DeviceBuffer(s_) for s_ in ((T, d), (T, 3 * d), (T, d), (T, d), (T, f), (T, d)))
+    hip.layer_norm(dx, up(L["ln1_w"]), up(L["ln1_b"]), h, T, d, 1e-5)
+    hip.gemm(hip.gemm_desc(T, 3 * d, d, trans_b=True, epilogue=hip.EPI_BIAS), h, wqkv, qkv, bqkv)
+    a = _lib.SdpaDesc()
+    a.num_bh, a.heads, a.seq_q, a.seq_k, a.d_k, a.d_v = batch * heads, heads, seq, seq, hd, hd
+    a.q_batch_stride = a.k_batch_stride = a.v_batch_stride = seq * 3 * d
+    a.q_head_stride = a.k_head_stride = a.v_head_stride = hd
+    a.q_row_stride = a.k_row_stride = a.v_row_stride = 3 * d
+    a.o_batch_stride, a.o_head_stride, a.o_row_stride = seq * d, hd, d
+    a.causal, a.kv_group = 1, 0
+    hip.sdpa_forward(a, 1.0 / math.sqrt(hd), qkv, qkv.view(d), qkv.view(2 * d), ctx)
+    hip.gemm(hip.gemm_desc(T, d, d, trans_b=True, epilogue=hip.EPI_BIAS | hip.EPI_RESIDUAL), ctx, up(L["wo"]), xa, up(L["bo"]), dx)
+    hip.layer_norm(xa, up(L["ln2_w"]), up(L["ln2_b"]), h, T, d, 1e-5)
+    hip.gemm(hip.gemm_desc(T, f, d, trans_b=True, epilogue=hip.EPI_BIAS | hip.EPI_GELU), h, up(L["w1"]), ff, up(L["b1"]))
+    hip.gemm(hip.gemm_desc(T, d, f, trans_b=True, epilogue=hip.EPI_BIAS | hip.EPI_RESIDUAL), ff, up(L["w2"]), out, up(L["b2"]), xa)
+    assert np.array_equal(out.to_host().view(np.uint32), got.view(np.uint32))
+    # a token count that is not a multiple of the 32-row tile
+    d2, f2, heads2, seq2 = 384, 512, 6, 45
+    L2 = make_layer(1, 0, d2, f2, biases_zero=False)
+    x2 = synth.normal(1, "x", (seq2, d2))
+    got2 = fused.EncoderHip(d2, heads2, f2, [L2], 1e-5, causal=False).forward(x2, 1, seq2)
+    dx2, h2 = up(x2), DeviceBuffer((seq2, d2))
+    q2 = DeviceBuffer((seq2, 3 * d2))
+    hip.layer_norm(dx2, up(L2["ln1_w"]), up(L2["ln1_b"]), h2, seq2, d2, 1e-5)
+    hip.gemm(hip.gemm_desc(seq2, 3 * d2, d2, trans_b=True, epilogue=hip.EPI_BIAS), h2, up(np.concatenate([L2["wq"], L2["wk"], L2["wv"]])), q2,
+             up(np.concatenate([L2["bq"], L2["bk"], L2["bv"]])))
+    hd2 = d2 // heads2
+    a.num_bh, a.heads, a.seq_q, a.seq_k, a.d_k, a.d_v = heads2, heads2, seq2, seq2, hd2, hd2
+    a.q_batch_stride = a.k_batch_stride = a.v_batch_stride = seq2 * 3 * d2
+    a.q_head_stride = a.k_head_stride = a.v_head_stride = hd2
+    a.q_row_stride = a.k_row_stride = a.v_row_stride = 3 * d2
+    a.o_batch_stride, a.o_head_stride, a.o_row_stride = seq2 * d2, hd2, d2
+    a.causal = 0
+    c2, xa2, ff2, o2 = DeviceBuffer((seq2, d2)), DeviceBuffer((seq2, d2)), DeviceBuffer((seq2, f2)), DeviceBuffer((seq2, d2))
+    hip.sdpa_forward(a, 1.0 / math.sqrt(hd2), q2, q2.view(d2), q2.view(2 * d2), c2)
+    hip.gemm(hip.gemm_desc(seq2, d2, d2, trans_b=True, epilogue=hip.EPI_BIAS | hip.EPI_RESIDUAL), c2, up(L2["wo"]), xa2, up(L2["bo"]), dx2)
+    hip.layer_norm(xa2, up(L2["ln2_w"]), up(L2["ln2_b"]), h2, seq2, d2, 1e-5)
+    hip.gemm(hip.gemm_desc(seq2, f2, d2, trans_b=True, epilogue=hip.EPI_BIAS | hip.EPI_GELU), h2, up(L2["w1"]), ff2, up(L2["b1"]))
+    hip.gemm(hip.gemm_desc(seq2, d2, f2, trans_b=True, epilogue=hip.EPI_BIAS | hip.EPI_RESIDUAL), ff2, up(L2["w2"]), o2, up(L2["b2"]), xa2)
+    assert np.array_equal(o2.to_host().view(np.uint32), got2.view(np.uint32))
+
+
 def test_graph_replay_survives_a_larger_gemm_and_new_tensors_on_its_stream(hip):
     """A captured graph keeps the address of the stream's GEMM split-tile workspace. A later, larger product on the same
     stream outgrows that workspace; the old block must stay out of the pool, or a tensor allocated afterwards could be
