@@ -15,6 +15,9 @@
 // [0, classes) (the reference would panic on the slice index) is reported through `bad_index` as
 // the lowest offending row, and that row's outputs are left unwritten.
 
+#include <cstdlib>
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace {
@@ -270,6 +273,76 @@ __global__ __launch_bounds__(THREADS, MINW) void resident_rows_kernel(const T *_
     }
 }
 
+// Cross-entropy loss of long fp32 rows in one streaming pass. The loss needs only the row's log-sum-exp and one
+// element, so nothing of the row has to stay on chip: each lane keeps a running maximum m and the sum s of exp(v - m) over
+// the elements it has seen, rescaling s when a batch of 32 values raises m (one extra exponential per batch at most), and
+// the lanes' pairs are merged at the end. Against the two-pass form (maximum first, then the sum) only the rounding of s
+// differs, by a few ulp. The row is read as a scalar head up to the first 16-byte boundary, 128-bit non-temporal vectors
+// eight deep per lane, and a scalar tail (rows such as 50 257 floats start at arbitrary 4-byte offsets). m starts at the
+// lowest finite value, not -inf: a -inf element then adds exp(-inf) = 0 instead of exp(-inf + inf), as it does in the
+// two-pass form whenever the row holds one finite value; a row of nothing but -inf ends as m + ln 0 - (-inf) = NaN, as
+// there. NaN elements never raise m (strict >) and poison s, +inf gives exp(inf - inf): NaN, as there.
+__global__ __launch_bounds__(256) void cross_entropy_forward_stream_kernel(const float *__restrict__ logits, const int64_t *__restrict__ target,
+                                                                           int64_t classes, float *__restrict__ loss, int64_t *bad_index) {
+    constexpr int NT = 256, WAVES = NT / kWave;
+    typedef float nat_f4 __attribute__((ext_vector_type(4)));
+    __shared__ float red[2 * WAVES];
+    int phase = 0;
+    const int64_t i = blockIdx.x;
+    const int64_t t = target[i];
+    if (t < 0 || t >= classes) {  // uniform over the workgroup
+        note_bad(bad_index, i);
+        return;
+    }
+    const float *xr = logits + i * classes;
+    float m = -3.402823466e+38f, s = 0.f;
+    auto feed1 = [&](float v) __attribute__((always_inline)) {
+        const float nm = max_gt(m, v);
+        if (nm > m) {
+            s *= t_exp<float>(m - nm);
+            m = nm;
+        }
+        s += t_exp<float>(v - m);
+    };
+    int64_t lead = (int64_t)(((16u - (unsigned)(reinterpret_cast<uintptr_t>(xr) & 15u)) & 15u) / sizeof(float));
+    if (lead > classes) lead = classes;
+    if ((int64_t)threadIdx.x < lead) feed1(xr[threadIdx.x]);
+    const int64_t nvec = (classes - lead) / 4;
+    const nat_f4 *xv = reinterpret_cast<const nat_f4 *>(xr + lead);
+    int64_t j = threadIdx.x;
+    for (; j + 7 * NT < nvec; j += 8 * NT) {
+        nat_f4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(xv + j + u * NT);
+        float nm = m;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) nm = max_gt(max_gt(max_gt(max_gt(nm, v[u].x), v[u].y), v[u].z), v[u].w);
+        if (nm > m) {
+            s *= t_exp<float>(m - nm);
+            m = nm;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            s += t_exp<float>(v[u].x - m);
+            s += t_exp<float>(v[u].y - m);
+            s += t_exp<float>(v[u].z - m);
+            s += t_exp<float>(v[u].w - m);
+        }
+    }
+    for (; j < nvec; j += NT) {
+        const nat_f4 v = __builtin_nontemporal_load(xv + j);
+        feed1(v.x);
+        feed1(v.y);
+        feed1(v.z);
+        feed1(v.w);
+    }
+    const int64_t t0 = lead + nvec * 4 + threadIdx.x;
+    if (t0 < classes) feed1(xr[t0]);
+    const float m_all = block_reduce<float, MaxGtOp, WAVES>(m, MaxGtOp{}, red, phase);
+    const float s_all = block_reduce<float, SumOp, WAVES>(s * t_exp<float>(m - m_all), SumOp{}, red, phase);
+    if (threadIdx.x == 0) loss[i] = (m_all + t_log<float>(s_all)) - xr[t];
+}
+
 // Launches the register-resident kernel if the row fits; returns false if it does not (the caller streams).
 template <typename T, int MODE>
 bool launch_resident(const T *x, const int64_t *target, const T *dloss, int64_t rows, int64_t cols, T *out, int64_t *bad_index,
@@ -363,7 +436,18 @@ int32_t cross_entropy_entry(bool backward, const T *logits, const int64_t *targe
             if (!launch_resident<T, kLossBackward>(logits, target, dloss, batch, classes, out, bad_index, st))
                 cross_entropy_backward_kernel<T><<<dim3((unsigned)batch), dim3(kThreads), 0, st>>>(logits, target, dloss, classes, out, bad_index);
         } else {
-            if (!launch_resident<T, kLossForward>(logits, target, nullptr, batch, classes, out, bad_index, st))
+            bool streamed = false;
+            if constexpr (std::is_same<T, float>::value) {
+                static const bool stream_off = [] {
+                    const char *e = std::getenv("FT_HIP_CE_STREAM");  // tuning knob: 0 keeps the row-resident loss kernel for long rows
+                    return e && std::atoi(e) == 0;
+                }();
+                if (!stream_off && classes >= 8192) {  // long rows: one streaming pass, nothing of the row kept on chip
+                    cross_entropy_forward_stream_kernel<<<dim3((unsigned)batch), dim3(256), 0, st>>>(logits, target, classes, out, bad_index);
+                    streamed = true;
+                }
+            }
+            if (!streamed && !launch_resident<T, kLossForward>(logits, target, nullptr, batch, classes, out, bad_index, st))
                 cross_entropy_forward_kernel<T><<<dim3((unsigned)batch), dim3(kThreads), 0, st>>>(logits, target, classes, out, bad_index);
         }
         FTH_CHECK_LAUNCH("cross_entropy");

@@ -107,6 +107,40 @@ def test_cross_entropy_forward_backward(hip, oracle, rows, cols, dtype):
     assert np.array_equal(got_d.view(np.uint8), dlogits.to_host().view(np.uint8))
 
 
+@pytest.mark.parametrize("cols", [8192, 8229, 20003])
+def test_cross_entropy_forward_long_rows_specials(hip, oracle, cols):
+    """fp32 rows of 8192 classes and more take the one-pass loss kernel (running maximum and rescaled sum per lane). Rows that
+    start at every 4-byte offset inside a 16-byte vector (odd class counts), targets in the scalar head, body and tail, and the
+    special values: -inf entries (weight zero), a row whose maximum comes last, huge spreads, NaN, +inf and a row of nothing
+    but -inf (NaN in the reference's two-pass form as well)."""
+    rows = 12
+    logits = synth.normal(41, "logits", (rows, cols)) * np.float32(3.0)
+    logits[1, ::3] = -np.inf
+    logits[2, -1] = 60.0                      # the maximum is the last element (tail)
+    logits[3, 0] = 75.0                       # ... or the first (head)
+    logits[4] = np.linspace(-80.0, 80.0, cols, dtype=np.float32)   # ascending: every batch raises the maximum
+    logits[5] = np.linspace(80.0, -80.0, cols, dtype=np.float32)
+    logits[6, 5] = np.nan
+    logits[7, cols // 2] = np.inf
+    logits[8] = -np.inf
+    logits[9] = -3.0e38                        # every value below any practical start of a running maximum
+    logits[10, : cols - 1] = -np.inf          # one finite value, in the tail
+    target = np.array([0, 1, cols - 1, 3, cols // 2, 2, 7, 9, 4, cols - 2, cols - 1, 5], np.int64)
+    dl, dt = DeviceBuffer.from_host(logits), DeviceBuffer.from_host(target)
+    loss, bad = DeviceBuffer((rows,)), DeviceBuffer((1,), np.int64)
+    hip.cross_entropy_forward(dl, dt, rows, cols, loss, bad)
+    assert int(bad.to_host()[0]) == -1
+    got, ref = loss.to_host(), oracle.cross_entropy_forward(logits, target)
+    assert np.array_equal(np.isnan(got), np.isnan(ref)), (got, ref)
+    assert np.isnan(ref[[6, 7, 8]]).all()
+    ok = ~np.isnan(ref)
+    assert np.array_equal(np.isinf(got[ok]), np.isinf(ref[ok])) and np.array_equal(got[ok][np.isinf(ref[ok])], ref[ok][np.isinf(ref[ok])])
+    fin = ok & np.isfinite(ref)
+    assert np.max(np.abs(got[fin] - ref[fin])) <= TOL_ROW_F32 * np.max(np.abs(ref[fin]))
+    hip.cross_entropy_forward(dl, dt, rows, cols, loss)
+    assert np.array_equal(got.view(np.uint8), loss.to_host().view(np.uint8))
+
+
 def test_cross_entropy_reports_the_first_bad_target(hip, oracle):
     rows, cols = 40, 33
     logits = synth.normal(24, "logits", (rows, cols))
