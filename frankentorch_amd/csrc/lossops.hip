@@ -443,7 +443,10 @@ int32_t cross_entropy_entry(bool backward, const T *logits, const int64_t *targe
                     return e && std::atoi(e) == 0;
                 }();
                 if (!stream_off && classes >= 8192) {  // long rows: one streaming pass, nothing of the row kept on chip
-                    cross_entropy_forward_stream_kernel<<<dim3((unsigned)batch), dim3(256), 0, st>>>(logits, target, classes, out, bad_index);
+                    // (three workgroups per compute unit read the stream fastest, as for the argmax kernel: 48 KiB of unused dynamic LDS
+                    //  per workgroup hold the count there, whatever the register allocation would allow)
+                    cross_entropy_forward_stream_kernel<<<dim3((unsigned)batch), dim3(256), (size_t)48 * 1024, st>>>(logits, target, classes, out,
+                                                                                                                    bad_index);
                     streamed = true;
                 }
             }
