@@ -111,14 +111,25 @@ def bench_rowops(device, synth, steps, warmup, with_cpu):
         return fn
 
     launches = {k: rotating(c) for k, c in calls.items()}
+    # The ceiling of a read-once / write-once kernel at this shape, measured in the same run on the same rotating sets:
+    # the library's plain 128-bit streaming copy (128 MiB in, 128 MiB out). Not part of the step.
+    copy_launch = rotating(lambda i: device.copy(xs[i], ys[i], ELEM))
 
     def step():
         for fn in launches.values():
             fn()
 
+    # Untimed warm-up: the W steps asked for, and then more of the same step until WARM_SECONDS of load have passed (what
+    # every per-kernel figure below gets too): at 0.25 ms a step, five warm-up steps end before the clocks have settled
+    # and the timed steps read 4-5 % low.
     for _ in range(warmup):
         step()
     device.synchronize()
+    t_end = time.perf_counter() + WARM_SECONDS
+    while time.perf_counter() < t_end:
+        for _ in range(8):
+            step()
+        device.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
         step()
@@ -141,7 +152,18 @@ def bench_rowops(device, synth, steps, warmup, with_cpu):
                             "same_buffer": {"ms": round(ms_same, 5), "GB/s": round(gbs_same, 1), "frac": round(gbs_same / HBM_PEAK_GBS, 4)}}
         log("[rowops] %-18s %.4f ms  %7.1f GB/s  %.1f%% of HBM peak over %d rotating buffer sets (same buffer: %.4f ms, %.1f%%)"
             % (name, ms, gbs, 100 * gbs / HBM_PEAK_GBS, ROTATE_SETS, ms_same, 100 * gbs_same / HBM_PEAK_GBS))
+    copy_launch()
+    device.synchronize()
+    ms_copy = event_time_ms(device, copy_launch, max(20, steps))
+    ms_copy_same = event_time_ms(device, lambda: device.copy(xs[0], ys[0], ELEM), max(20, steps))
+    copy_ceiling = {"ms": round(ms_copy, 5), "GB/s": round(2 * ELEM * 4 / (ms_copy * 1e-3) / 1e9, 1),
+                    "frac": round(2 * ELEM * 4 / (ms_copy * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "bytes": 2 * ELEM * 4,
+                    "same_buffer": {"ms": round(ms_copy_same, 5), "frac": round(2 * ELEM * 4 / (ms_copy_same * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+                    "workload": "plain streaming copy fp32 [8192,4096] -> [8192,4096], one 128-bit vector per lane, same rotating buffer sets"}
+    log("[rowops] %-18s %.4f ms  %7.1f GB/s  %.1f%% of HBM peak (the ceiling of a read-once / write-once kernel here; same buffer %.1f%%)"
+        % ("copy_ceiling", ms_copy, copy_ceiling["GB/s"], 100 * copy_ceiling["frac"], 100 * copy_ceiling["same_buffer"]["frac"]))
     dominant = max(per_kernel, key=lambda k: per_kernel[k]["ms"])
+    per_kernel["copy_ceiling"] = copy_ceiling
     roof = {"bound": "hbm", "kernel": dominant, "achieved": per_kernel[dominant]["GB/s"], "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": per_kernel[dominant]["frac"], "traffic": MEASURED_HBM_TRAFFIC.get(dominant),
             "buffers": "%d rotating input/output sets per kernel (no reuse from the last-level cache)" % ROTATE_SETS}

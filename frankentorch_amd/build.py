@@ -84,19 +84,5 @@ def build_library(jobs: int = 8) -> str:
     return LIB_PATH
 
 
-MICROBENCH_SRC = os.path.join(CSRC, "microbench", "mfma_issue.hip")
-MICROBENCH_BIN = os.path.join(PKG_DIR, "microbench_mfma_issue.bin")
-
-
-def build_microbench() -> str:
-    """Compiles the MFMA / vector-instruction issue microbenchmark (a stand-alone program, not part of the library)."""
-    tmp = MICROBENCH_BIN + ".tmp"
-    _run([_hipcc(), "-O3", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-          "-Wno-unused-command-line-argument", "-o", tmp, MICROBENCH_SRC])
-    os.replace(tmp, MICROBENCH_BIN)
-    return MICROBENCH_BIN
-
-
 if __name__ == "__main__":
     print(build_library())
-    print(build_microbench())

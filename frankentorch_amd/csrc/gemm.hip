@@ -1203,6 +1203,13 @@ int32_t launch_persistent(Kern kern, size_t smem, int BK, int &blocks_per_cu, Ge
     int64_t grid = (int64_t)cus * blocks_per_cu;
     const int64_t cap = total / kMinItersPerBlock > 0 ? total / kMinItersPerBlock : 1;
     if (grid > cap) grid = cap;
+    {
+        static const int forced_grid = [] {
+            const char *e = std::getenv("FT_HIP_GEMM_GRID");  // tuning knob: workgroups of the persistent kernels
+            return e ? std::atoi(e) : 0;
+        }();
+        if (forced_grid > 0 && forced_grid <= grid) grid = forced_grid;
+    }
     p.tiles_m = (int)tm;
     p.tiles_n = (int)tn;
     p.ktiles = (int)ktiles;

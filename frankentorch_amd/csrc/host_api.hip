@@ -976,6 +976,29 @@ int32_t sdpa_backward_impl(const T *q, size_t q_len, const T *k, size_t k_len, c
     return fetch(dq, gq, (size_t)nq);
 }
 
+// transpose_2d_into_f32 / _f64 (crates/ft-kernel-cpu/src/lib.rs:42415-42439, 42294-42318) and
+// transpose_batched_materialize_f32 / _f64 (:42526-42556, 42490-42519): dst[b][c][r] = src[b][r][c]. The reference
+// asserts src.len() == dst.len() == batch * rows * cols in debug builds and indexes past a short slice otherwise.
+template <typename T>
+int32_t transpose_impl(const T *src, size_t src_len, size_t batch, size_t rows, size_t cols, T *out, size_t out_cap) {
+    uint64_t plane, total;
+    FTH_ARG(checked_mul(rows, cols, &plane) && checked_mul(plane, batch, &total), "transpose: batch * rows * cols overflows");
+    if (int32_t rc = check_out(out, out_cap, (size_t)total)) return rc;
+    if (total == 0) return FTH_OK;
+    FTH_ARG(src != nullptr && src_len >= total, "transpose: source slice shorter than batch * rows * cols");
+    FTH_ARG(total <= (uint64_t)std::numeric_limits<int64_t>::max(), "transpose: tensor too large");
+    FTH_REQUIRE_DEVICE();
+    fth::Scratch sc;
+    T *ds, *dd;
+    if (int32_t rc = stage_in(sc, src, (size_t)total, &ds)) return rc;
+    if (int32_t rc = stage_out(sc, (size_t)total, &dd)) return rc;
+    int32_t rc;
+    if constexpr (sizeof(T) == 4) rc = fth_dev_transpose_batched_f32(ds, dd, (int64_t)batch, (int64_t)rows, (int64_t)cols, nullptr);
+    else rc = fth_dev_transpose_batched_f64(ds, dd, (int64_t)batch, (int64_t)rows, (int64_t)cols, nullptr);
+    if (rc) return rc;
+    return fetch(out, dd, (size_t)total);
+}
+
 }  // namespace
 
 extern "C" {
@@ -1221,6 +1244,21 @@ int32_t fth_quantize_rows_i8(const float *x, size_t x_len, size_t rows, size_t c
 int32_t fth_linear_int8_dynamic_f32(const float *x, size_t x_len, size_t m, size_t k, const int8_t *w_i8, size_t w_len, const float *w_scales,
                                     size_t w_scales_len, size_t n, const float *bias, size_t bias_len, float *out, size_t out_cap) {
     return linear_int8_impl(x, x_len, m, k, w_i8, w_len, w_scales, w_scales_len, n, bias, bias_len, out, out_cap);
+}
+
+int32_t fth_transpose_2d_into_f32(const float *src, size_t src_len, float *dst, size_t dst_cap, size_t rows, size_t cols) {
+    return transpose_impl<float>(src, src_len, 1, rows, cols, dst, dst_cap);
+}
+int32_t fth_transpose_2d_into_f64(const double *src, size_t src_len, double *dst, size_t dst_cap, size_t rows, size_t cols) {
+    return transpose_impl<double>(src, src_len, 1, rows, cols, dst, dst_cap);
+}
+int32_t fth_transpose_batched_materialize_f32(const float *src, size_t src_len, size_t batch, size_t rows, size_t cols, float *out,
+                                              size_t out_cap) {
+    return transpose_impl<float>(src, src_len, batch, rows, cols, out, out_cap);
+}
+int32_t fth_transpose_batched_materialize_f64(const double *src, size_t src_len, size_t batch, size_t rows, size_t cols, double *out,
+                                              size_t out_cap) {
+    return transpose_impl<double>(src, src_len, batch, rows, cols, out, out_cap);
 }
 
 }  // extern "C"

@@ -246,6 +246,70 @@ __global__ __launch_bounds__(kBlock) void permute_0213_kernel(const T *__restric
     }
 }
 
+// ---- batched 2-D transpose: dst[b][c][r] = src[b][r][c] -------------------------------------------
+// A 64 x 64 tile goes through LDS so that both sides move whole 128-bit vectors along their contiguous dimension: a
+// lane reads four consecutive columns of one source row and writes four consecutive rows' worth of one destination row.
+// The tile is kept [column][row + pad]: the vector of a source row lands as four scalars 65 words apart (conflict-free
+// over the 16 lanes of a row), and a destination row is read back as four consecutive words.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void transpose_tile_kernel(const T *__restrict__ src, T *__restrict__ dst, int64_t rows,
+                                                                int64_t cols, int64_t tiles_x) {
+    constexpr int TS = 64, EPV = 16 / (int)sizeof(T), VPR = TS / EPV;  // vectors per tile row: 16 (fp32) or 32 (fp64)
+    using V = typename std::conditional<sizeof(T) == 4, float4, double2>::type;
+    __shared__ T tile[TS][TS + 1];
+    const int64_t plane = rows * cols;
+    const T *sp = src + (int64_t)blockIdx.y * plane;
+    T *dp = dst + (int64_t)blockIdx.y * plane;
+    const int64_t r0 = ((int64_t)blockIdx.x / tiles_x) * TS, c0 = ((int64_t)blockIdx.x % tiles_x) * TS;
+    const int vx = threadIdx.x % VPR, vy = threadIdx.x / VPR;
+    constexpr int RPP = kBlock / VPR;  // tile rows covered per pass
+#pragma unroll
+    for (int p = 0; p < TS / RPP; ++p) {
+        const int r = vy + p * RPP;
+        if (r0 + r < rows && c0 + vx * EPV < cols) {
+            const V v = *reinterpret_cast<const V *>(sp + (r0 + r) * cols + c0 + vx * EPV);
+            const T *e = reinterpret_cast<const T *>(&v);
+#pragma unroll
+            for (int j = 0; j < EPV; ++j) tile[vx * EPV + j][r] = e[j];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < TS / RPP; ++p) {
+        const int c = vy + p * RPP;
+        if (c0 + c < cols && r0 + vx * EPV < rows) {
+            V v;
+            T *e = reinterpret_cast<T *>(&v);
+#pragma unroll
+            for (int j = 0; j < EPV; ++j) e[j] = tile[c][vx * EPV + j];
+            *reinterpret_cast<V *>(dp + (c0 + c) * rows + r0 + vx * EPV) = v;
+        }
+    }
+}
+
+// Any extents and alignments: 32 x 32 tiles of single elements, both sides coalesced.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void transpose_scalar_kernel(const T *__restrict__ src, T *__restrict__ dst, int64_t rows,
+                                                                  int64_t cols, int64_t tiles_x) {
+    __shared__ T tile[32][33];
+    const int64_t plane = rows * cols;
+    const T *sp = src + (int64_t)blockIdx.y * plane;
+    T *dp = dst + (int64_t)blockIdx.y * plane;
+    const int64_t r0 = ((int64_t)blockIdx.x / tiles_x) * 32, c0 = ((int64_t)blockIdx.x % tiles_x) * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int64_t r = r0 + ty + 8 * k, c = c0 + tx;
+        if (r < rows && c < cols) tile[ty + 8 * k][tx] = sp[r * cols + c];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int64_t c = c0 + ty + 8 * k, r = r0 + tx;
+        if (r < rows && c < cols) dp[c * rows + r] = tile[tx][ty + 8 * k];
+    }
+}
+
 template <typename T>
 int32_t launch_index_select(const T *input, int64_t outer, int64_t dim_size, int64_t inner, const double *indices,
                             int64_t num_indices, T *out, int64_t *bad, fth_stream s) {
@@ -312,6 +376,31 @@ int32_t launch_permute(const T *src, T *dst, int64_t d0, int64_t d1, int64_t d2,
     return FTH_OK;
 }
 
+template <typename T>
+int32_t launch_transpose(const T *src, T *dst, int64_t batch, int64_t rows, int64_t cols, fth_stream s) {
+    FTH_REQUIRE_DEVICE();
+    FTH_ARG(batch >= 0 && rows >= 0 && cols >= 0, "transpose: negative extent");
+    if (batch == 0 || rows == 0 || cols == 0) return FTH_OK;
+    FTH_ARG(src && dst, "transpose: NULL operand");
+    FTH_ARG(src != dst, "transpose: source and destination must not be the same buffer");
+    constexpr int EPV = 16 / (int)sizeof(T);
+    const bool vec = rows % EPV == 0 && cols % EPV == 0 &&
+                     ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0;
+    const int ts = vec ? 64 : 32;
+    const int64_t tiles_x = fth::ceil_div(cols, ts), tiles = tiles_x * fth::ceil_div(rows, ts);
+    FTH_ARG(tiles <= kMaxGrid, "transpose: matrix too large for one launch");
+    hipStream_t st = fth::resolve_stream(s);
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {  // the grid's second extent is limited to 65535
+        const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
+        const T *sp = src + b0 * rows * cols;
+        T *dp = dst + b0 * rows * cols;
+        if (vec) transpose_tile_kernel<T><<<dim3((unsigned)tiles, (unsigned)nb), dim3(kBlock), 0, st>>>(sp, dp, rows, cols, tiles_x);
+        else transpose_scalar_kernel<T><<<dim3((unsigned)tiles, (unsigned)nb), dim3(kBlock), 0, st>>>(sp, dp, rows, cols, tiles_x);
+        FTH_CHECK_LAUNCH("transpose");
+    }
+    return FTH_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -354,6 +443,18 @@ int32_t fth_dev_argmax_f32(const float *x, int64_t outer, int64_t reduce, int64_
 }
 int32_t fth_dev_argmax_f64(const double *x, int64_t outer, int64_t reduce, int64_t inner, double *out, fth_stream s) {
     return launch_argmax<double>(x, outer, reduce, inner, out, s);
+}
+int32_t fth_dev_transpose_2d_f32(const float *src, float *dst, int64_t rows, int64_t cols, fth_stream s) {
+    return launch_transpose<float>(src, dst, 1, rows, cols, s);
+}
+int32_t fth_dev_transpose_2d_f64(const double *src, double *dst, int64_t rows, int64_t cols, fth_stream s) {
+    return launch_transpose<double>(src, dst, 1, rows, cols, s);
+}
+int32_t fth_dev_transpose_batched_f32(const float *src, float *dst, int64_t batch, int64_t rows, int64_t cols, fth_stream s) {
+    return launch_transpose<float>(src, dst, batch, rows, cols, s);
+}
+int32_t fth_dev_transpose_batched_f64(const double *src, double *dst, int64_t batch, int64_t rows, int64_t cols, fth_stream s) {
+    return launch_transpose<double>(src, dst, batch, rows, cols, s);
 }
 int32_t fth_dev_permute_0213_f32(const float *src, float *dst, int64_t d0, int64_t d1, int64_t d2, int64_t d3,
                                  fth_stream s) {

@@ -18,6 +18,7 @@
 // bias pass :17336-17351. Only the summation ORDER differs (tree instead of sequential /
 // pairwise-128), which is what the 1e-5 tolerance of the parity tests covers.
 
+#include <algorithm>
 #include <cstdlib>
 #include <initializer_list>
 
@@ -495,6 +496,19 @@ __global__ __launch_bounds__(RowBlock<WPR>::kThreads) void layernorm_rows_kernel
     for (int q = 0; q < RPT; ++q) r[q].store(y + (row0 + q < rows ? row0 + q : rows - 1) * cols, row0 + q < rows ? nvec : 0);
 }
 
+// Direct global -> LDS copy of 16 bytes per lane: the wavefront's 64 lanes fill 1 KiB of LDS at `lds_byte` in lane
+// order, with no staging registers. The compiler does not see the LDS write, so the reader waits for vmcnt(0) itself.
+__device__ __forceinline__ void vec_to_lds(const void *base, unsigned lane_bytes, unsigned lds_byte) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_bytes), "s"(base),
+                 "s"(__builtin_amdgcn_readfirstlane(lds_byte))
+                 : "memory", "m0");
+}
+template <typename T> __device__ __forceinline__ const T *uniform_base(const T *ptr) {
+    const uint64_t v = reinterpret_cast<uint64_t>(ptr);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const T *>(((uint64_t)hi << 32) | lo);
+}
+
 // ---- RMSNorm ---------------------------------------------------------------------------------
 template <typename T, int VPL, int WPR>
 __global__ __launch_bounds__(RowBlock<WPR>::kThreads, RowBlock<WPR>::min_blocks(VPL, 3, (int)sizeof(T))) void rmsnorm_row_kernel(
@@ -545,6 +559,145 @@ __global__ __launch_bounds__(RowBlock<WPR>::kThreads, RowBlock<WPR>::min_blocks(
             else r.load(x + walk.clamped(walk.row) * cols, nvec, T(0));
         }
     }
+}
+
+// ---- Row ops, walking rows: few workgroups, each owning rows r, r + G, r + 2 G, ... ---------------
+// Two 512-lane workgroups per compute unit, each in a plain load -> reduce -> store loop over its rows, with the
+// per-column vectors (gamma, beta) copied into LDS once per workgroup. Same arithmetic and reduction trees as the
+// one-row-per-workgroup kernels above (the results are bit-identical); what changes is how the memory system is driven.
+enum class RowOp { Softmax, LayerNorm, RmsNorm };
+
+template <typename T, int VPL, int WPR, RowOp OP>
+__global__ __launch_bounds__(RowBlock<WPR>::kThreads) void row_walk_kernel(const T *__restrict__ x, const T *__restrict__ w,
+                                                                           const T *__restrict__ b, T *__restrict__ y,
+                                                                           int64_t rows, int cols, T eps) {
+    static_assert(RowBlock<WPR>::kRows == 1, "one row group per workgroup");
+    constexpr int NT = RowBlock<WPR>::kThreads;
+    using R = RowRegs<T, VPL, WPR>;
+    using V = typename Vec128<T>::type;
+    extern __shared__ __align__(16) unsigned char dyn_lds[];  // the only LDS object (offset 0): gamma, beta, exchange buffer
+    T *smem = reinterpret_cast<T *>(dyn_lds + (size_t)2 * VPL * NT * 16);
+    int phase = 0;
+    const int nvec = cols / R::EPV;
+    const T inv_n = T(1) / (T)cols;
+    const bool has_w = OP != RowOp::Softmax && w != nullptr, has_b = OP == RowOp::LayerNorm && b != nullptr;
+    if constexpr (OP != RowOp::Softmax) {
+        const unsigned wave_byte = (threadIdx.x / kWave) * (kWave * 16);
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            int v = (int)threadIdx.x + i * NT;
+            v = v < nvec ? v : nvec - 1;
+            if (has_w) vec_to_lds(uniform_base(w), (unsigned)v * 16u, (unsigned)(i * NT * 16) + wave_byte);
+            if (has_b) vec_to_lds(uniform_base(b), (unsigned)v * 16u, (unsigned)((VPL + i) * NT * 16) + wave_byte);
+        }
+    }
+    const V *lw = reinterpret_cast<const V *>(dyn_lds), *lb = lw + VPL * NT;
+    bool first = OP != RowOp::Softmax;
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        R r;
+        r.load(x + row * cols, nvec, OP == RowOp::Softmax ? neg_inf<T>() : T(0));
+        if (first) {
+            // gamma / beta were requested before the first row and vector memory operations complete in issue order;
+            // the explicit wait is for the compiler, which does not know of the LDS writes.
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            first = false;
+        }
+        if constexpr (OP == RowOp::Softmax) {
+            T m = neg_inf<T>();
+#pragma unroll
+            for (int i = 0; i < VPL; ++i)
+#pragma unroll
+                for (int j = 0; j < R::EPV; ++j) m = dev_max(m, r.e[i][j]);
+            m = group_reduce<WPR>(m, MaxOp{}, smem, phase);
+            T s = 0;
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) {
+                const bool live = (R::lane() + i * R::kLanes) < nvec;
+#pragma unroll
+                for (int j = 0; j < R::EPV; ++j) {
+                    T ev = live ? dev_exp(r.e[i][j] - m) : T(0);
+                    r.e[i][j] = ev;
+                    s += ev;
+                }
+            }
+            s = group_reduce<WPR>(s, SumOp{}, smem, phase);
+            const T inv = T(1) / s;
+#pragma unroll
+            for (int i = 0; i < VPL; ++i)
+#pragma unroll
+                for (int j = 0; j < R::EPV; ++j) r.e[i][j] = r.e[i][j] * inv;
+        } else {
+            T mean = 0, rstd;
+            if constexpr (OP == RowOp::LayerNorm) {
+                T sum = 0;
+#pragma unroll
+                for (int i = 0; i < VPL; ++i)
+#pragma unroll
+                    for (int j = 0; j < R::EPV; ++j) sum += r.e[i][j];
+                sum = group_reduce<WPR>(sum, SumOp{}, smem, phase);
+                mean = sum * inv_n;
+                T vsum = 0;
+#pragma unroll
+                for (int i = 0; i < VPL; ++i) {
+                    const bool live = (R::lane() + i * R::kLanes) < nvec;
+#pragma unroll
+                    for (int j = 0; j < R::EPV; ++j) {
+                        const T d = r.e[i][j] - mean;
+                        vsum += live ? d * d : T(0);
+                    }
+                }
+                vsum = group_reduce<WPR>(vsum, SumOp{}, smem, phase);
+                rstd = T(1) / dev_sqrt(vsum * inv_n + eps);
+            } else {
+                T ss = 0;
+#pragma unroll
+                for (int i = 0; i < VPL; ++i)
+#pragma unroll
+                    for (int j = 0; j < R::EPV; ++j) ss += r.e[i][j] * r.e[i][j];
+                ss = group_reduce<WPR>(ss, SumOp{}, smem, phase);
+                rstd = T(1) / dev_sqrt(ss * inv_n + eps);
+            }
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) {
+                const int v = R::lane() + i * R::kLanes;
+                if (v < nvec) {
+                    T wv[R::EPV], bv[R::EPV];
+                    if (has_w) R::unpack(lw[i * NT + threadIdx.x], wv);
+                    if (has_b) R::unpack(lb[i * NT + threadIdx.x], bv);
+#pragma unroll
+                    for (int j = 0; j < R::EPV; ++j) {
+                        T o = OP == RowOp::LayerNorm ? (r.e[i][j] - mean) * rstd : r.e[i][j] * rstd;
+                        if (has_w) o = o * wv[j];
+                        if (has_b) o = o + bv[j];
+                        r.e[i][j] = o;
+                    }
+                }
+            }
+        }
+        r.store(y + row * cols, nvec);
+    }
+}
+
+// Launches row_walk_kernel when the shape fits it (rows of 513 to 1024 vectors, enough rows to give every workgroup a
+// few); returns false when the caller should take its one-row-per-workgroup path.
+template <typename T, RowOp OP>
+bool try_row_walk(const T *x, const T *w, const T *b, T *y, int64_t rows, int64_t cols, T eps, int vpl, int wpr, hipStream_t st) {
+    // Measured at fp32 [8192, 4096] on rotating buffers, fractions of the HBM peak, one row per workgroup against walking
+    // with 2 / 3 / 4 workgroups per compute unit: LayerNorm (gamma and beta) 0.724 against 0.751 / 0.713 / 0.711; RMSNorm
+    // 0.760 against 0.759 / 0.739 / 0.743; softmax 0.775 against 0.750 / 0.715 / 0.723. So only the op that reads two
+    // per-column vectors walks by default.
+    static const int forced = [] {
+        const char *e = std::getenv("FT_HIP_ROW_WALK");  // tuning knob: workgroups per compute unit of the walking kernel, every op (0 = off)
+        return e ? std::atoi(e) : -1;
+    }();
+    const int per_cu = forced >= 0 ? forced : (OP == RowOp::LayerNorm && w != nullptr && b != nullptr) ? 2 : 0;
+    if (per_cu <= 0 || wpr != 8 || vpl != 2) return false;
+    const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
+    const int64_t grid = (int64_t)cus * per_cu;
+    if (rows < 4 * grid) return false;
+    const size_t lds = (size_t)2 * 2 * 512 * 16 + 2 * kMaxWaves * sizeof(T);
+    row_walk_kernel<T, 2, 8, OP><<<dim3((unsigned)grid), dim3(512), lds, st>>>(x, w, b, y, rows, (int)cols, eps);
+    return true;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -658,7 +811,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_stream_kernel(const T *__restr
 // Elementwise: GELU, add. Each thread owns UNR 128-bit vectors a block-stride apart, loads them
 // all before the first use, and a scalar tail covers what is left.
 // ---------------------------------------------------------------------------------------------
-enum class Ew { Gelu, Add, GeluTanh };
+enum class Ew { Gelu, Add, GeluTanh, Copy };
 
 template <typename T, Ew OP, int UNR, int BT>
 __global__ __launch_bounds__(BT) void elementwise_vec_kernel(const T *__restrict__ a, const T *__restrict__ b,
@@ -686,7 +839,7 @@ __global__ __launch_bounds__(BT) void elementwise_vec_kernel(const T *__restrict
             for (int j = 0; j < R::EPV; ++j) {
                 if constexpr (OP == Ew::Gelu) ea[j] = dev_gelu(ea[j]);
                 else if constexpr (OP == Ew::GeluTanh) ea[j] = dev_gelu_tanh(ea[j]);
-                else ea[j] = ea[j] + eb[j];
+                else if constexpr (OP == Ew::Add) ea[j] = ea[j] + eb[j];
             }
             stream_store(reinterpret_cast<V *>(y) + v, R::pack(ea));
         }
@@ -700,7 +853,8 @@ __global__ __launch_bounds__(kBlock) void elementwise_scalar_kernel(const T *__r
     if (i >= n) return;
     if constexpr (OP == Ew::Gelu) y[i] = dev_gelu(a[i]);
     else if constexpr (OP == Ew::GeluTanh) y[i] = dev_gelu_tanh(a[i]);
-    else y[i] = a[i] + b[i];
+    else if constexpr (OP == Ew::Add) y[i] = a[i] + b[i];
+    else y[i] = a[i];
 }
 
 // ---- bias add / bias + residual add: y[r, j] = (x[r, j] + bias[j]) (+ res[r, j]) --------------
@@ -831,6 +985,10 @@ int32_t launch_softmax(const T *x, T *y, int64_t rows, int64_t cols, fth_stream 
     int64_t grid = 0;
     if (cols % EPV == 0 && aligned16(x) && aligned16(y) && pick_row_shape(cols / EPV, 16, vpl, wpr) &&
         (row_launch_shape(rows, wpr, grid, iters), grid <= kMaxGrid)) {
+        if (try_row_walk<T, RowOp::Softmax>(x, nullptr, nullptr, y, rows, cols, T(0), vpl, wpr, st)) {
+            FTH_CHECK_LAUNCH("softmax");
+            return FTH_OK;
+        }
 #define L(V_, W_) softmax_row_kernel<T, V_, W_><<<dim3((unsigned)grid), dim3(RowBlock<W_>::kThreads), 0, st>>>(x, y, rows, (int)cols, iters)
         FTH_ROW_DISPATCH(vpl, wpr, L);
 #undef L
@@ -871,6 +1029,10 @@ int32_t launch_layernorm(const T *x, const T *x2, const T *w, const T *b, T *y, 
                   (!w || aligned16(w)) && (!b || aligned16(b));
     if (vec_ok && pick_row_shape(cols / EPV, ADD ? 8 : 16, vpl, wpr) && (row_launch_shape(rows, wpr, grid, iters), grid <= kMaxGrid)) {
         if constexpr (!ADD) {
+            if (try_row_walk<T, RowOp::LayerNorm>(x, w, b, y, rows, cols, eps, vpl, wpr, st)) {
+                FTH_CHECK_LAUNCH("layer_norm");
+                return FTH_OK;
+            }
             // (Three 512-thread workgroups per compute unit, which is what the kernel's 65 registers allow, stream best at
             // this shape: compiled for 64 registers and four per unit 0.704 of the HBM peak against 0.721, held to two 0.675.)
             // Two rows side by side (gamma / beta once per pair) where a lane's share of a row is at most four vectors and
@@ -928,6 +1090,10 @@ int32_t launch_rmsnorm(const T *x, const T *w, T *y, int64_t rows, int64_t cols,
         // by its registers (measured at fp32 [8192, 4096] on rotating buffers: four per unit 0.744 of the HBM peak, three 0.759,
         // two 0.733; softmax, which reads no second vector, is best at four). The kernel's registers would allow four, so 48 KiB
         // of unused dynamic LDS per workgroup hold the count at three.
+        if (try_row_walk<T, RowOp::RmsNorm>(x, w, nullptr, y, rows, cols, eps, vpl, wpr, st)) {
+            FTH_CHECK_LAUNCH("rms_norm");
+            return FTH_OK;
+        }
         const size_t pad = (wpr == 8 && w) ? (size_t)48 * 1024 : 0;
 #define L(V_, W_) rmsnorm_row_kernel<T, V_, W_><<<dim3((unsigned)grid), dim3(RowBlock<W_>::kThreads), pad, st>>>(x, w, y, rows, (int)cols, eps, iters)
         FTH_ROW_DISPATCH(vpl, wpr, L);
@@ -1063,6 +1229,12 @@ int32_t fth_dev_add_f32(const float *a, const float *b, float *y, int64_t n, fth
 }
 int32_t fth_dev_add_f64(const double *a, const double *b, double *y, int64_t n, fth_stream s) {
     return launch_elementwise<double, Ew::Add>(a, b, y, n, s);
+}
+int32_t fth_dev_copy_f32(const float *x, float *y, int64_t n, fth_stream s) {
+    return launch_elementwise<float, Ew::Copy>(x, nullptr, y, n, s);
+}
+int32_t fth_dev_copy_f64(const double *x, double *y, int64_t n, fth_stream s) {
+    return launch_elementwise<double, Ew::Copy>(x, nullptr, y, n, s);
 }
 int32_t fth_dev_bias_add_f32(const float *x, const float *bias, float *y, int64_t rows, int64_t cols, fth_stream s) {
     return launch_bias<float, false>(x, bias, nullptr, y, rows, cols, s);

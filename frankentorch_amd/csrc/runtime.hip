@@ -161,6 +161,15 @@ int32_t fth_memset_zero(void *dst, size_t bytes) {
     return FTH_OK;
 }
 
+int32_t fth_device_memory_info(uint64_t *free_bytes, uint64_t *total_bytes) {
+    FTH_REQUIRE_DEVICE();
+    size_t f = 0, tot = 0;
+    FTH_HIP(hipMemGetInfo(&f, &tot));
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = tot;
+    return FTH_OK;
+}
+
 int32_t fth_host_malloc(void **hptr, size_t bytes) {
     FTH_REQUIRE_DEVICE();
     FTH_ARG(hptr != nullptr, "fth_host_malloc: hptr is NULL");

@@ -273,6 +273,25 @@ def argmax(x, outer, reduce, inner, out, stream=None):
     check(getattr(_lib.load(), "fth_dev_argmax_" + _sfx(x))(_ptr(x), outer, reduce, inner, _ptr(out), stream))
 
 
+def copy(x, y, n, stream=None):
+    check(getattr(_lib.load(), "fth_dev_copy_" + _sfx(x))(_ptr(x), _ptr(y), n, stream))
+
+
+def transpose_2d(src, dst, rows, cols, stream=None):
+    check(getattr(_lib.load(), "fth_dev_transpose_2d_" + _sfx(src))(_ptr(src), _ptr(dst), rows, cols, stream))
+
+
+def transpose_batched(src, dst, batch, rows, cols, stream=None):
+    check(getattr(_lib.load(), "fth_dev_transpose_batched_" + _sfx(src))(_ptr(src), _ptr(dst), batch, rows, cols, stream))
+
+
+def memory_info():
+    """(free, total) device memory in bytes."""
+    f, tot = C.c_uint64(), C.c_uint64()
+    check(_lib.load().fth_device_memory_info(C.byref(f), C.byref(tot)))
+    return f.value, tot.value
+
+
 def permute_0213(src, dst, d0, d1, d2, d3, stream=None):
     check(getattr(_lib.load(), "fth_dev_permute_0213_" + _sfx(src))(_ptr(src), _ptr(dst), d0, d1, d2, d3, stream))
 

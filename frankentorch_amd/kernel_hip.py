@@ -11,7 +11,8 @@ Reference lines (crates/ft-kernel-cpu/src/lib.rs): matmul :37752 / :17355, bmm :
 addmm :41562 / :17514, linear :17306 / :17162, matmul_rhs_transposed :17408 / :17381,
 softmax_dim :39193 / :18350, layer_norm_forward :5877 / :5824, add_layer_norm_forward :5932,
 rms_norm_forward :6459 / :6418, gelu :37123, add :36870, sdpa_forward :5200 / :4572,
-index_select :40216, argmax_dim :39443 / :18653.
+index_select :40216, argmax_dim :39443 / :18653, transpose_2d :42406 / :42286,
+transpose_batched_materialize :42526 / :42490.
 """
 from __future__ import annotations
 
@@ -447,3 +448,33 @@ def sdpa_forward_f32(q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal):
 
 def sdpa_forward_f64(q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal):
     return _sdpa("fth_sdpa_forward_f64", np.float64, q, k, v, num_bh, seq_q, seq_k, d_k, d_v, scale, causal)
+
+
+def _transpose(name, dtype, src, batch, rows, cols, batched):
+    src = _slice(src, dtype)
+    total = batch * rows * cols
+    out = np.empty(total if total < 2 ** 62 else 0, dtype=dtype)  # an overflowing extent is for the library to report
+    fn = getattr(_lib.load(), name)
+    if batched:
+        check(fn(_p(src), src.size, batch, rows, cols, _p(out), out.size))
+    else:
+        check(fn(_p(src), src.size, _p(out), out.size, rows, cols))
+    return out
+
+
+def transpose_2d_f32(src, rows, cols):
+    """src [rows, cols] -> [cols, rows] (transpose_2d_f32 / transpose_2d_into_f32, crates/ft-kernel-cpu/src/lib.rs:42406-42439)."""
+    return _transpose("fth_transpose_2d_into_f32", np.float32, src, 1, rows, cols, False)
+
+
+def transpose_2d_f64(src, rows, cols):
+    return _transpose("fth_transpose_2d_into_f64", np.float64, src, 1, rows, cols, False)
+
+
+def transpose_batched_materialize_f32(src, batch, rows, cols):
+    """src [batch, rows, cols] -> [batch, cols, rows] (crates/ft-kernel-cpu/src/lib.rs:42526-42556)."""
+    return _transpose("fth_transpose_batched_materialize_f32", np.float32, src, batch, rows, cols, True)
+
+
+def transpose_batched_materialize_f64(src, batch, rows, cols):
+    return _transpose("fth_transpose_batched_materialize_f64", np.float64, src, batch, rows, cols, True)

@@ -122,6 +122,8 @@ int32_t fth_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes);
 int32_t fth_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes);
 int32_t fth_memcpy_d2d(void *dst_dev, const void *src_dev, size_t bytes);
 int32_t fth_memset_zero(void *dst_dev, size_t bytes);
+/* Free and total device memory in bytes as the driver reports them (hipMemGetInfo). */
+int32_t fth_device_memory_info(uint64_t *free_bytes, uint64_t *total_bytes);
 
 typedef void *fth_stream; /* a hipStream_t; NULL selects the library's own ordered stream */
 typedef void *fth_event;  /* a hipEvent_t */
@@ -185,6 +187,11 @@ int32_t fth_dev_gelu_tanh_f64(const double *x, double *y, int64_t n, fth_stream 
 /* add_tensor_contiguous_f32 (crates/ft-kernel-cpu/src/lib.rs:36870-36877): exact IEEE l + r. */
 int32_t fth_dev_add_f32(const float *a, const float *b, float *y, int64_t n, fth_stream s);
 int32_t fth_dev_add_f64(const double *a, const double *b, double *y, int64_t n, fth_stream s);
+/* The materialising copy behind contiguous / narrow / expand (`copy_from_slice` into a `build_uninit` buffer,
+ * crates/ft-kernel-cpu/src/lib.rs:2585-2639): y[i] = x[i], one 128-bit vector per lane, streaming both ways. It is also
+ * what the benchmark times as the ceiling of a read-once / write-once kernel on this part. */
+int32_t fth_dev_copy_f32(const float *x, float *y, int64_t n, fth_stream s);
+int32_t fth_dev_copy_f64(const double *x, double *y, int64_t n, fth_stream s);
 /* The bias pass of linear_tensor_f32 (crates/ft-kernel-cpu/src/lib.rs:17336-17351):
  * y[r, j] = x[r, j] + bias[j]. x == y is allowed. */
 int32_t fth_dev_bias_add_f32(const float *x, const float *bias, float *y, int64_t rows, int64_t cols, fth_stream s);
@@ -225,6 +232,14 @@ int32_t fth_dev_argmax_f64(const double *x, int64_t outer, int64_t reduce, int64
  * (TensorTape::permute_slice, perm [0,2,1,3], crates/ft-autograd/src/lib.rs:10733-10882). */
 int32_t fth_dev_permute_0213_f32(const float *src, float *dst, int64_t d0, int64_t d1, int64_t d2, int64_t d3, fth_stream s);
 int32_t fth_dev_permute_0213_f64(const double *src, double *dst, int64_t d0, int64_t d1, int64_t d2, int64_t d3, fth_stream s);
+
+/* 2-D and batched 2-D transposes: dst[b][c][r] = src[b][r][c] for `batch` row-major [rows, cols] planes
+ * (transpose_2d_into_f32 / _f64, crates/ft-kernel-cpu/src/lib.rs:42415-42439, 42294-42318;
+ * transpose_batched_materialize_f32 / _f64, :42526-42556, 42490-42519). Exact copies of the bits; dst must not be src. */
+int32_t fth_dev_transpose_2d_f32(const float *src, float *dst, int64_t rows, int64_t cols, fth_stream s);
+int32_t fth_dev_transpose_2d_f64(const double *src, double *dst, int64_t rows, int64_t cols, fth_stream s);
+int32_t fth_dev_transpose_batched_f32(const float *src, float *dst, int64_t batch, int64_t rows, int64_t cols, fth_stream s);
+int32_t fth_dev_transpose_batched_f64(const double *src, double *dst, int64_t batch, int64_t rows, int64_t cols, fth_stream s);
 
 /* Dense contraction on MFMA. C[b] = alpha * A[b] * op(B[b]) (+ epilogue), beta = 0 (C is fully
  * overwritten, crates/ft-kernel-cpu/src/lib.rs:1310-1338).
@@ -303,8 +318,10 @@ int32_t fth_dev_layer_norm_backward_f64(const double *dy, const double *x, const
  * fth_dev_layer_norm_backward_f32, with the partial column sums in a device array built into the
  * library (fth_dev_layer_norm_backward_noalloc_max_bytes() = 24 MiB per GPU, held until the process
  * ends). Shapes whose fth_dev_norm_backward_workspace_bytes exceeds that return
- * FTH_ERR_BUFFER_TOO_LARGE (fp32 [8192, 4096] needs 16.1 MiB). All calls on one GPU share the
- * array: calls that overlap in time on one GPU, on any streams, race. */
+ * FTH_ERR_BUFFER_TOO_LARGE (fp32 [8192, 4096] needs 8.1 MiB, [16384, 8192] 16.1 MiB; ask
+ * fth_dev_norm_backward_workspace_bytes). All calls on one GPU share the array: calls that overlap
+ * in time on one GPU, on any streams, race. The first call on a device looks the array's address
+ * up (hipGetSymbolAddress), so make it outside any stream capture; later calls only launch kernels. */
 size_t fth_dev_layer_norm_backward_noalloc_max_bytes(void);
 int32_t fth_dev_layer_norm_backward_f32_noalloc(const float *dy, const float *x, const float *weight, int64_t rows, int64_t cols, float eps,
                                                 float *dx, float *dweight, float *dbias, fth_stream s);
@@ -548,6 +565,14 @@ int32_t fth_add_tensor_contiguous_f32(const float *lhs, size_t lhs_len, const fl
 int32_t fth_add_tensor_contiguous_f64(const double *lhs, size_t lhs_len, const double *rhs, size_t rhs_len,
                                       const fth_meta *lhs_meta, const fth_meta *rhs_meta,
                                       double *out, size_t out_cap, size_t *out_len);
+/* transpose_2d_into_f32 (:42415) / _f64 (:42294): src [rows, cols] -> dst [cols, rows], caller buffer;
+ * transpose_batched_materialize_f32 (:42526) / _f64 (:42490): src [batch, rows, cols] -> out [batch, cols, rows]. */
+int32_t fth_transpose_2d_into_f32(const float *src, size_t src_len, float *dst, size_t dst_cap, size_t rows, size_t cols);
+int32_t fth_transpose_2d_into_f64(const double *src, size_t src_len, double *dst, size_t dst_cap, size_t rows, size_t cols);
+int32_t fth_transpose_batched_materialize_f32(const float *src, size_t src_len, size_t batch, size_t rows, size_t cols, float *out,
+                                              size_t out_cap);
+int32_t fth_transpose_batched_materialize_f64(const double *src, size_t src_len, size_t batch, size_t rows, size_t cols, double *out,
+                                              size_t out_cap);
 /* sdpa_forward_f32 (:5200) / _f64 (:4572) */
 int32_t fth_sdpa_forward_f32(const float *q, size_t q_len, const float *k, size_t k_len, const float *v,
                              size_t v_len, size_t num_bh, size_t seq_q, size_t seq_k, size_t d_k, size_t d_v,

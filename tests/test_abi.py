@@ -145,6 +145,21 @@ def test_fused_entry_points_check_slice_lengths_before_any_device_call():
         assert ei.value.kind != "Unavailable", "the length check must come before the device check"
 
 
+def test_transposes_check_lengths_before_any_device_call():
+    x = np.zeros(12, np.float32)
+    assert K.transpose_2d_f32(np.zeros(0, np.float32), 0, 5).size == 0          # empty result: no device needed
+    assert K.transpose_batched_materialize_f64(np.zeros(0), 3, 0, 4).size == 0
+    with pytest.raises(core.HipError) as ei:
+        K.transpose_2d_f32(x[:-1], 3, 4)                                          # source shorter than rows * cols
+    assert ei.value.kind == "InvalidArgument"
+    with pytest.raises(core.HipError) as ei:
+        K.transpose_batched_materialize_f32(x, 2 ** 40, 2 ** 40, 2 ** 40)         # extent product overflows
+    assert ei.value.kind == "InvalidArgument"
+    out = np.zeros(11, np.float32)
+    rc = _lib.load().fth_transpose_2d_into_f32(x.ctypes.data, x.size, out.ctypes.data, out.size, 3, 4)
+    assert _lib.load().fth_status_name(rc) == b"OutputTooSmall"
+
+
 def test_empty_results_need_no_device():
     f32 = lambda s: TensorMeta.from_shape(s, DType.F32)
     z = np.zeros(0, np.float32)
