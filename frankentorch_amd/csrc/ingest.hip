@@ -20,6 +20,17 @@
 // other) and, when the stored type or layout differs from the one asked for, converts
 // (F16 / BF16 / F64 <-> F32 / F64) and transposes on the GPU, so no converted host copy is made.
 
+//
+// The same handle also reads the reference's NATIVE state-dict format (fth_statedict_*), the loading direction of
+// load_state_dict / load_state_dict_from_bytes (crates/ft-serialize/src/lib.rs:996-1160; layout written by
+// write_state_dict_to_writer :786-860), all integers little-endian:
+//
+//   "FTSV" | version u32 (<= 1) | tensor count u64 | per tensor: key length u64, key (UTF-8), ndim u64, ndim x u64 dims,
+//   dtype tag u8 (0 F64, 1 F32, 2 F16, 3 BF16), numel x width payload bytes | end of file.
+//
+// Its failures keep the reference's variants and reason strings: InvalidMagic, UnsupportedVersion{found, max},
+// Corrupt{reason}.
+
 #include <fcntl.h>
 #include <sys/mman.h>
 #include <sys/stat.h>
@@ -568,8 +579,98 @@ int32_t read_dev(const fth_safetensors *f, const char *name, int32_t transpose_2
     return FTH_OK;
 }
 
-int32_t finish_open(fth_safetensors *f, fth_safetensors **out) {
-    if (int32_t rc = parse(f)) {
+// ---- the reference's native state-dict container -------------------------------------------------
+// load_state_dict_from_bytes (crates/ft-serialize/src/lib.rs:1005-1160), check for check and in its order. Tensors are
+// not copied: an entry records where its payload sits in the mapped bytes.
+constexpr uint32_t kNativeVersion = 1;        // FT_STATE_FORMAT_VERSION (:596)
+constexpr uint64_t kNativeMinTensorBytes = 17;  // FT_MIN_NATIVE_TENSOR_HEADER_BYTES (:601): key length + ndim + dtype tag
+
+bool native_u64(const uint8_t *base, size_t len, size_t &pos, uint64_t &v) {
+    if (len - pos < 8) return false;  // pos <= len always
+    v = 0;
+    for (int i = 7; i >= 0; --i) v = (v << 8) | base[pos + (size_t)i];
+    pos += 8;
+    return true;
+}
+
+int32_t parse_native(fth_safetensors *f) {
+    const uint8_t *d = f->base;
+    const size_t len = f->len;
+    size_t pos = 0;
+    if (len < 4 || std::memcmp(d, "FTSV", 4) != 0)
+        return fth::set_error(FTH_ERR_INVALID_MAGIC, "invalid magic bytes: not a FrankenTorch state file");
+    pos = 4;
+    if (len - pos < 4) return corrupt("truncated u32");
+    const uint32_t version = (uint32_t)d[4] | ((uint32_t)d[5] << 8) | ((uint32_t)d[6] << 16) | ((uint32_t)d[7] << 24);
+    pos = 8;
+    if (version > kNativeVersion) {
+        fth::set_error(FTH_ERR_UNSUPPORTED_VERSION, "unsupported format version %u (max supported: %u)", version, kNativeVersion);
+        fth::last_error().a = version;
+        fth::last_error().b = kNativeVersion;
+        return FTH_ERR_UNSUPPORTED_VERSION;
+    }
+    uint64_t count = 0;
+    if (!native_u64(d, len, pos, count)) return corrupt("truncated u64");
+    const uint64_t remaining = len - pos;
+    if (count > remaining / kNativeMinTensorBytes)
+        return fth::set_error(FTH_ERR_CORRUPT, "claimed %llu tensors but only %llu bytes remain (min %llu per tensor)",
+                              (unsigned long long)count, (unsigned long long)remaining, (unsigned long long)kNativeMinTensorBytes);
+    std::map<std::string, Entry> seen;  // name order, as the reference's BTreeMap
+    static const char *const kNames[4] = {"f64", "f32", "f16", "bf16"};
+    static const int kWidth[4] = {8, 4, 2, 2};
+    for (uint64_t i = 0; i < count; ++i) {
+        uint64_t key_len = 0;
+        if (!native_u64(d, len, pos, key_len)) return corrupt("truncated u64");
+        if (key_len > UINT64_MAX - pos) return corrupt("key length overflow");
+        if (key_len > len - pos) return corrupt("truncated key data");
+        if (!valid_utf8(d + pos, (size_t)key_len)) return corrupt("invalid UTF-8 in key");
+        std::string key(reinterpret_cast<const char *>(d + pos), (size_t)key_len);
+        pos += (size_t)key_len;
+        if (seen.count(key)) return corrupt("duplicate tensor key in native state dict: '%s'", key);
+        // (The reference accepts any UTF-8 key. One with a NUL byte cannot be named through a C string, so this reader
+        // refuses the container instead of listing a key that could not be looked up.)
+        if (key.find('\0') != std::string::npos) return corrupt("tensor key contains a NUL byte, which this interface cannot address");
+        uint64_t ndim = 0;
+        if (!native_u64(d, len, pos, ndim)) return corrupt("truncated u64");
+        if (ndim > (len - pos) / 8) return corrupt("truncated shape data for tensor '%s'", key);
+        Entry e;
+        e.name = key;
+        e.shape.reserve((size_t)ndim);
+        uint64_t numel = 1;
+        bool overflow = false;
+        for (uint64_t k = 0; k < ndim; ++k) {
+            uint64_t dim = 0;
+            if (!native_u64(d, len, pos, dim)) return corrupt("truncated u64");
+            if (!overflow && __builtin_mul_overflow(numel, dim, &numel)) overflow = true;
+            e.shape.push_back(dim);
+        }
+        if (pos >= len) return corrupt("truncated dtype");
+        const uint8_t tag = d[pos];
+        if (tag > 3) return fth::set_error(FTH_ERR_CORRUPT, "unknown dtype tag: %u", (unsigned)tag);
+        pos += 1;
+        if (overflow) return corrupt("shape overflow in native state dict tensor '%s'", key);
+        uint64_t needed = 0, end = 0;
+        if (__builtin_mul_overflow(numel, (uint64_t)kWidth[tag], &needed) || __builtin_add_overflow((uint64_t)pos, needed, &end))
+            return corrupt("byte count overflow for %s tensor '%s'", kNames[tag], key);
+        if (end > len) return corrupt("truncated %s data", kNames[tag]);
+        e.dtype = tag;  // the tags are the FTH_DTYPE_* values (crates/ft-serialize/src/lib.rs:597-600)
+        e.bits = 8 * kWidth[tag];
+        e.begin = pos;
+        e.end = end;
+        e.numel = numel;
+        pos = (size_t)end;
+        seen.emplace(std::move(key), std::move(e));
+    }
+    if (pos != len)
+        return fth::set_error(FTH_ERR_CORRUPT, "trailing bytes after state dict payload: remaining=%llu", (unsigned long long)(len - pos));
+    f->data = f->base;  // payload positions are absolute
+    f->tensors.reserve(seen.size());
+    for (auto &kv : seen) f->tensors.push_back(std::move(kv.second));
+    return FTH_OK;
+}
+
+int32_t finish_open(fth_safetensors *f, fth_safetensors **out, bool native = false) {
+    if (int32_t rc = native ? parse_native(f) : parse(f)) {
         delete f;
         return rc;
     }
@@ -577,12 +678,8 @@ int32_t finish_open(fth_safetensors *f, fth_safetensors **out) {
     return FTH_OK;
 }
 
-}  // namespace
-
-extern "C" {
-
-int32_t fth_safetensors_open(const char *path, fth_safetensors **out) {
-    FTH_ARG(path != nullptr && out != nullptr, "safetensors_open: NULL argument");
+int32_t open_path(const char *path, fth_safetensors **out, bool native) {
+    FTH_ARG(path != nullptr && out != nullptr, "open: NULL argument");
     *out = nullptr;
     const int fd = ::open(path, O_RDONLY | O_CLOEXEC);
     if (fd < 0) return fth::set_error(FTH_ERR_IO, "cannot open '%s': %s", path, std::strerror(errno));
@@ -599,7 +696,7 @@ int32_t fth_safetensors_open(const char *path, fth_safetensors **out) {
     fth_safetensors *f = new (std::nothrow) fth_safetensors();
     if (!f) {
         ::close(fd);
-        return fth::set_error(FTH_ERR_KERNEL, "safetensors_open: host allocation failed");
+        return fth::set_error(FTH_ERR_KERNEL, "open: host allocation failed");
     }
     f->len = (size_t)sb.st_size;
     if (f->len > 0) {
@@ -615,18 +712,27 @@ int32_t fth_safetensors_open(const char *path, fth_safetensors **out) {
         (void)madvise(m, f->len, MADV_SEQUENTIAL);
     }
     ::close(fd);
-    return finish_open(f, out);
+    return finish_open(f, out, native);
 }
 
-int32_t fth_safetensors_open_bytes(const void *data, size_t len, fth_safetensors **out) {
-    FTH_ARG(out != nullptr && (data != nullptr || len == 0), "safetensors_open_bytes: NULL argument");
+
+int32_t open_bytes(const void *data, size_t len, fth_safetensors **out, bool native) {
+    FTH_ARG(out != nullptr && (data != nullptr || len == 0), "open_bytes: NULL argument");
     *out = nullptr;
     fth_safetensors *f = new (std::nothrow) fth_safetensors();
-    if (!f) return fth::set_error(FTH_ERR_KERNEL, "safetensors_open_bytes: host allocation failed");
+    if (!f) return fth::set_error(FTH_ERR_KERNEL, "open_bytes: host allocation failed");
     f->base = static_cast<const uint8_t *>(data);
     f->len = len;
-    return finish_open(f, out);
+    return finish_open(f, out, native);
 }
+
+}  // namespace
+
+extern "C" {
+
+int32_t fth_safetensors_open(const char *path, fth_safetensors **out) { return open_path(path, out, false); }
+
+int32_t fth_safetensors_open_bytes(const void *data, size_t len, fth_safetensors **out) { return open_bytes(data, len, out, false); }
 
 int32_t fth_safetensors_close(fth_safetensors *f) {
     delete f;
@@ -682,6 +788,21 @@ const char *fth_safetensors_metadata(const fth_safetensors *f, const char *key) 
     if (!f || !key || !f->has_metadata) return nullptr;
     auto it = f->metadata.find(key);
     return it == f->metadata.end() ? nullptr : it->second.c_str();
+}
+
+// The native state-dict container through the same handle: listing, info and reads are the safetensors functions.
+int32_t fth_statedict_open(const char *path, fth_statedict **out) { return open_path(path, out, true); }
+int32_t fth_statedict_open_bytes(const void *data, size_t len, fth_statedict **out) { return open_bytes(data, len, out, true); }
+int32_t fth_statedict_close(fth_statedict *f) { return fth_safetensors_close(f); }
+int64_t fth_statedict_count(const fth_statedict *f) { return fth_safetensors_count(f); }
+const char *fth_statedict_name(const fth_statedict *f, int64_t index) { return fth_safetensors_name(f, index); }
+int32_t fth_statedict_info(const fth_statedict *f, const char *name, fth_safetensors_tensor *info) { return fth_safetensors_info(f, name, info); }
+int32_t fth_statedict_read(const fth_statedict *f, const char *name, void *dst, size_t dst_bytes) { return fth_safetensors_read(f, name, dst, dst_bytes); }
+int32_t fth_statedict_read_f32_dev(const fth_statedict *f, const char *name, int32_t transpose_2d, float *dst_dev, size_t dst_elems, fth_stream s) {
+    return read_dev<float>(f, name, transpose_2d, dst_dev, dst_elems, s);
+}
+int32_t fth_statedict_read_f64_dev(const fth_statedict *f, const char *name, int32_t transpose_2d, double *dst_dev, size_t dst_elems, fth_stream s) {
+    return read_dev<double>(f, name, transpose_2d, dst_dev, dst_elems, s);
 }
 
 }  // extern "C"

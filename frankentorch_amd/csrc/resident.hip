@@ -795,6 +795,11 @@ int32_t fth_gpt2_from_safetensors(const fth_safetensors *f, int64_t n_heads, flo
     return FTH_OK;
 }
 
+int32_t fth_gpt2_from_statedict(const fth_statedict *f, int64_t n_heads, float ln_eps, int32_t activation, fth_gpt2 **out) {
+    // The two containers share their handle type: the reader only asks for names, shapes and device reads.
+    return fth_gpt2_from_safetensors(f, n_heads, ln_eps, activation, out);
+}
+
 int32_t fth_gpt2_dims(const fth_gpt2 *g, int64_t *vocab, int64_t *max_pos, int64_t *d_model, int64_t *n_heads, int64_t *d_ff,
                       int64_t *n_layers) {
     FTH_ARG(g != nullptr, "gpt2_dims: model is NULL");

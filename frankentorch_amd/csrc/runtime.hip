@@ -96,6 +96,8 @@ const char *fth_status_name(int32_t code) {
         case FTH_ERR_OUTPUT_TOO_SMALL: return "OutputTooSmall";
         case FTH_ERR_CORRUPT: return "Corrupt";
         case FTH_ERR_IO: return "Io";
+        case FTH_ERR_INVALID_MAGIC: return "InvalidMagic";
+        case FTH_ERR_UNSUPPORTED_VERSION: return "UnsupportedVersion";
         default: return "Unknown";
     }
 }

@@ -206,6 +206,13 @@ class Gpt2Hip:
         self.vocab, self.max_pos, self.d_model, self.n_heads, self.d_ff, self.n_layers = (d.value for d in dims)
         return self
 
+    @classmethod
+    def from_state_dict(cls, source, n_heads: int, ln_eps: float = 1e-5, gelu_tanh: bool = True) -> "Gpt2Hip":
+        """The same from a native state-dict container ("FTSV"; path, bytes or an open serialize.StateDictFile)."""
+        from .serialize import StateDictFile
+
+        return cls.from_safetensors(source if isinstance(source, StateDictFile) else StateDictFile(source), n_heads, ln_eps, gelu_tanh)
+
     def forward_dev(self, ids: DeviceBuffer, batch: int, seq: int, logits: Optional[DeviceBuffer],
                     argmax: Optional[DeviceBuffer], stream=None) -> None:
         check(_lib.load().fth_gpt2_forward_dev(self._g, ids.ptr, batch, seq, None if logits is None else logits.ptr,

@@ -1,11 +1,13 @@
-"""Host-side mirror of the safetensors loading surface of `ft-serialize`
-(crates/ft-serialize/src/lib.rs:2170-2286): `load_safetensors`, `load_safetensors_from_bytes`,
-`load_safetensors_metadata`, over the C ABI's memory-mapped reader. The device-side path
+"""Host-side mirror of the loading surface of `ft-serialize`: the safetensors functions
+(crates/ft-serialize/src/lib.rs:2170-2286: `load_safetensors`, `load_safetensors_from_bytes`,
+`load_safetensors_metadata`) and the native state-dict ones (:996-1160: `load_state_dict`,
+`load_state_dict_from_bytes`), over the C ABI's memory-mapped reader. The device-side path
 (`SafeTensorsFile.read_dev`, `fused.Gpt2Hip.from_safetensors`) moves tensors straight into resident
 buffers instead of building host tensors first.
 
-Errors: `core.HipError` with kind "Corrupt" where the reference returns TensorIOError::Corrupt and
-"Io" where it returns TensorIOError::Io.
+Errors: `core.HipError` with kind "Corrupt" where the reference returns TensorIOError::Corrupt,
+"Io" for TensorIOError::Io, "InvalidMagic" and "UnsupportedVersion" for the native container's
+two header variants.
 """
 from __future__ import annotations
 
@@ -35,14 +37,17 @@ def bf16_to_f32(bits: np.ndarray) -> np.ndarray:
 class SafeTensorsFile:
     """An open, validated safetensors container (a path, or bytes that stay referenced)."""
 
+    _OPEN, _OPEN_BYTES = "fth_safetensors_open", "fth_safetensors_open_bytes"
+
     def __init__(self, source):
         h = C.c_void_p()
+        lib = _lib.load()
         if isinstance(source, (bytes, bytearray, memoryview)):
             self._keep = bytes(source)
-            check(_lib.load().fth_safetensors_open_bytes(self._keep, len(self._keep), C.byref(h)))
+            check(getattr(lib, self._OPEN_BYTES)(self._keep, len(self._keep), C.byref(h)))
         else:
             self._keep = None
-            check(_lib.load().fth_safetensors_open(str(source).encode(), C.byref(h)))
+            check(getattr(lib, self._OPEN)(str(source).encode(), C.byref(h)))
         self._h = h.value
 
     def close(self) -> None:
@@ -132,3 +137,21 @@ def load_safetensors_metadata(path) -> Optional[Dict[str, str]]:
     does not enumerate keys through the C ABI, so the view object is returned."""
     f = SafeTensorsFile(path)
     return f.metadata()
+
+
+class StateDictFile(SafeTensorsFile):
+    """An open, validated native state-dict container ("FTSV"). Same listing and read calls; no metadata map."""
+
+    _OPEN, _OPEN_BYTES = "fth_statedict_open", "fth_statedict_open_bytes"
+
+
+def load_state_dict_from_bytes(data) -> Dict[str, np.ndarray]:
+    """crates/ft-serialize/src/lib.rs:1005: name -> tensor, in name order (BF16 tensors as uint16 bit patterns)."""
+    with StateDictFile(data) as f:
+        return {n: f.read(n) for n in f.names()}
+
+
+def load_state_dict(path) -> Dict[str, np.ndarray]:
+    """crates/ft-serialize/src/lib.rs:996."""
+    with StateDictFile(path) as f:
+        return {n: f.read(n) for n in f.names()}

@@ -61,7 +61,9 @@ enum {
     FTH_ERR_INVALID_ARGUMENT = 105,    /* reference would panic         */
     FTH_ERR_OUTPUT_TOO_SMALL = 106,    /* caller's out buffer < result  */
     FTH_ERR_CORRUPT = 107,             /* TensorIOError::Corrupt{reason} (crates/ft-serialize) */
-    FTH_ERR_IO = 108                   /* TensorIOError::Io{path, source}                     */
+    FTH_ERR_IO = 108,                  /* TensorIOError::Io{path, source}                     */
+    FTH_ERR_INVALID_MAGIC = 109,       /* TensorIOError::InvalidMagic                         */
+    FTH_ERR_UNSUPPORTED_VERSION = 110  /* TensorIOError::UnsupportedVersion{found, max}: fth_error_info a = found, b = max */
 };
 
 /* DType / Device tags: crates/ft-core/src/lib.rs:23-35 and :176-179, plus the HIP device id the
@@ -705,6 +707,28 @@ int32_t fth_safetensors_read_f64_dev(const fth_safetensors *f, const char *name,
 int32_t fth_safetensors_metadata_count(const fth_safetensors *f);
 const char *fth_safetensors_metadata(const fth_safetensors *f, const char *key);
 
+/* The reference's NATIVE state-dict container, load_state_dict (crates/ft-serialize/src/lib.rs:996-1002) and
+ * load_state_dict_from_bytes (:1005-1160), through the same kind of handle: "FTSV", version u32 (<= 1), tensor count u64,
+ * then per tensor key length u64, key, ndim u64, u64 dims, dtype tag u8 (0 F64, 1 F32, 2 F16, 3 BF16) and the payload,
+ * all little-endian (written by write_state_dict_to_writer :786-860). open / open_bytes validate the whole container in
+ * the reference's order and fail as it does: FTH_ERR_INVALID_MAGIC, FTH_ERR_UNSUPPORTED_VERSION, and FTH_ERR_CORRUPT with
+ * the reference's reason text (truncated key / shape / dtype / payload, duplicate key, a tensor count or byte count the
+ * file cannot hold, trailing bytes). One deviation: a key that contains a NUL byte, which the reference accepts, cannot be
+ * named through a C string and makes open fail with FTH_ERR_CORRUPT. Listing (name order), info and the host and device
+ * reads behave as for safetensors; there is no metadata map. */
+typedef struct fth_safetensors fth_statedict;
+int32_t fth_statedict_open(const char *path, fth_statedict **out);
+int32_t fth_statedict_open_bytes(const void *data, size_t len, fth_statedict **out);
+int32_t fth_statedict_close(fth_statedict *f);
+int64_t fth_statedict_count(const fth_statedict *f);
+const char *fth_statedict_name(const fth_statedict *f, int64_t index);
+int32_t fth_statedict_info(const fth_statedict *f, const char *name, fth_safetensors_tensor *info);
+int32_t fth_statedict_read(const fth_statedict *f, const char *name, void *dst, size_t dst_bytes);
+int32_t fth_statedict_read_f32_dev(const fth_statedict *f, const char *name, int32_t transpose_2d, float *dst_dev, size_t dst_elems,
+                                   fth_stream s);
+int32_t fth_statedict_read_f64_dev(const fth_statedict *f, const char *name, int32_t transpose_2d, double *dst_dev, size_t dst_elems,
+                                   fth_stream s);
+
 /* GPT-2-shaped decoder: learned positions, pre-LN blocks, final LN, LM head tied to wte. */
 typedef struct fth_gpt2 fth_gpt2;
 int32_t fth_gpt2_new(int64_t vocab, int64_t max_pos, int64_t d_model, int64_t n_heads, int64_t d_ff, float ln_eps,
@@ -718,6 +742,8 @@ int32_t fth_gpt2_new(int64_t vocab, int64_t max_pos, int64_t d_model, int64_t n_
  * converted to f32 there. Shapes are taken from the file; other tensors in it (attention mask buffers) are ignored.
  * A missing or mis-shaped tensor is FTH_ERR_CORRUPT. activation: FTH_ACT_GELU_TANH is what GPT-2 was trained with. */
 int32_t fth_gpt2_from_safetensors(const fth_safetensors *f, int64_t n_heads, float ln_eps, int32_t activation, fth_gpt2 **out);
+/* The same from a native state-dict container holding the same tensor names. */
+int32_t fth_gpt2_from_statedict(const fth_statedict *f, int64_t n_heads, float ln_eps, int32_t activation, fth_gpt2 **out);
 /* vocab, max_pos, d_model, n_heads, d_ff, n_layers of a model (any pointer may be NULL). */
 int32_t fth_gpt2_dims(const fth_gpt2 *g, int64_t *vocab, int64_t *max_pos, int64_t *d_model, int64_t *n_heads, int64_t *d_ff,
                       int64_t *n_layers);

@@ -442,3 +442,128 @@ def gpt2_forward(wte, wpe, layers, lnf_w, lnf_b, ids, batch, seq, heads, eps, wa
                                      _p(am))
     del keep
     return {"hidden": hidden, "logits": logits, "argmax": am, "bad": int(bad)}
+
+
+def transpose_2d(x):
+    """transpose_2d_f32 / _f64 (crates/ft-kernel-cpu/src/lib.rs:42406-42439, 42286-42318): [rows, cols] -> [cols, rows], a
+    copy of the bits."""
+    x = np.asarray(x)
+    return np.ascontiguousarray(x.T)
+
+
+def transpose_batched(x):
+    """transpose_batched_materialize_f32 / _f64 (crates/ft-kernel-cpu/src/lib.rs:42526-42556, 42490-42519):
+    [batch, rows, cols] -> [batch, cols, rows]."""
+    x = np.asarray(x)
+    return np.ascontiguousarray(x.transpose(0, 2, 1))
+
+
+# ---- native state-dict container ---------------------------------------------------------------
+class StateDictError(Exception):
+    """kind: "InvalidMagic" | "UnsupportedVersion" | "Corrupt" (TensorIOError, crates/ft-serialize/src/lib.rs:607-619)."""
+
+    def __init__(self, kind, reason=""):
+        self.kind, self.reason = kind, reason
+        super().__init__("%s: %s" % (kind, reason))
+
+
+def load_state_dict_from_bytes(data):
+    """load_state_dict_from_bytes (crates/ft-serialize/src/lib.rs:1005-1160) restated step for step in plain Python:
+    returns {key: (dtype_tag, shape tuple, payload bytes)} in key order, or raises StateDictError with the reference's
+    variant and reason text. (The rank-1 width-4 F64 fast path :1165-1260 returns the same map and is not restated.)"""
+    data = bytes(data)
+    n = len(data)
+    pos = 0
+
+    def corrupt(reason):
+        return StateDictError("Corrupt", reason)
+
+    def u64(what="truncated u64"):
+        nonlocal pos
+        if pos + 8 > n:  # read_fixed_bytes :1472-1486
+            raise corrupt(what)
+        v = int.from_bytes(data[pos:pos + 8], "little")
+        pos += 8
+        return v
+
+    if n < 4 or data[:4] != b"FTSV":  # :1011
+        raise StateDictError("InvalidMagic")
+    pos = 4
+    if pos + 4 > n:
+        raise corrupt("truncated u32")
+    version = int.from_bytes(data[4:8], "little")
+    pos = 8
+    if version > 1:  # :1018
+        raise StateDictError("UnsupportedVersion", "found %d max 1" % version)
+    count = u64()
+    remaining = n - pos
+    if count > remaining // 17:  # :1029-1040
+        raise corrupt("claimed %d tensors but only %d bytes remain (min 17 per tensor)" % (count, remaining))
+    width = {0: 8, 1: 4, 2: 2, 3: 2}
+    names = {0: "f64", 1: "f32", 2: "f16", 3: "bf16"}
+    out = {}
+    for _ in range(count):
+        key_len = u64()
+        key_end = pos + key_len
+        if key_end >= 1 << 64:
+            raise corrupt("key length overflow")
+        if key_end > n:
+            raise corrupt("truncated key data")
+        try:
+            key = data[pos:key_end].decode("utf-8")
+        except UnicodeDecodeError:
+            raise corrupt("invalid UTF-8 in key")
+        pos = key_end
+        if key in out:
+            raise corrupt("duplicate tensor key in native state dict: '%s'" % key)
+        ndim = u64()
+        if ndim > (n - pos) // 8:
+            raise corrupt("truncated shape data for tensor '%s'" % key)
+        shape, numel, overflow = [], 1, False
+        for _ in range(ndim):
+            dim = u64()
+            if not overflow:
+                if numel * dim >= 1 << 64:
+                    overflow = True
+                else:
+                    numel *= dim
+            shape.append(dim)
+        if pos >= n:
+            raise corrupt("truncated dtype")
+        tag = data[pos]
+        if tag > 3:
+            raise corrupt("unknown dtype tag: %d" % tag)
+        pos += 1
+        if overflow:
+            raise corrupt("shape overflow in native state dict tensor '%s'" % key)
+        needed = numel * width[tag]
+        if needed >= 1 << 64 or pos + needed >= 1 << 64:
+            raise corrupt("byte count overflow for %s tensor '%s'" % (names[tag], key))
+        if pos + needed > n:
+            raise corrupt("truncated %s data" % names[tag])
+        out[key] = (tag, tuple(shape), data[pos:pos + needed])
+        pos += needed
+    if pos != n:
+        raise corrupt("trailing bytes after state dict payload: remaining=%d" % (n - pos))
+    # BTreeMap<String, _> iterates in byte order of the UTF-8 keys
+    return {k: out[k] for k in sorted(out, key=lambda s: s.encode("utf-8"))}
+
+
+def encode_state_dict(tensors):
+    """The layout write_state_dict_to_writer produces (crates/ft-serialize/src/lib.rs:786-860), for building test inputs:
+    `tensors` is {key: numpy array of float64 / float32 / float16, or (uint16 array, "bf16")}; keys are written in
+    byte order."""
+    tag_of = {np.dtype(np.float64): 0, np.dtype(np.float32): 1, np.dtype(np.float16): 2}
+    out = [b"FTSV", (1).to_bytes(4, "little"), len(tensors).to_bytes(8, "little")]
+    for key in sorted(tensors, key=lambda s: s.encode("utf-8")):
+        v = tensors[key]
+        if isinstance(v, tuple):
+            arr, tag = np.ascontiguousarray(v[0], dtype=np.uint16), 3
+        else:
+            arr = np.ascontiguousarray(v)
+            tag = tag_of[arr.dtype]
+        kb = key.encode("utf-8")
+        out += [len(kb).to_bytes(8, "little"), kb, arr.ndim.to_bytes(8, "little")]
+        out += [int(d).to_bytes(8, "little") for d in arr.shape]
+        out += [bytes([tag]), arr.astype(arr.dtype.newbyteorder("<"), copy=False).tobytes()]
+    return b"".join(out)

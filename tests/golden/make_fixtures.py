@@ -6,6 +6,9 @@ Sources (read as text / JSON from the reference checkout; nothing is imported or
   * artifacts/optimization/golden_outputs/*.txt    golden output text files (numbers parsed out)
   * artifacts/perf/frankentorch-kgs4.54/pass1_golden_gemm_bt.digest_lines   f64 GEMM checksums
   * fuzz/corpus/ft_serialize_safetensors/*         seed containers of the safetensors fuzz target (hex)
+  * fuzz/corpus/ft_serialize_state_dict/*          seed containers of the native state-dict fuzz target (hex)
+  * artifacts/optimization/golden_outputs/ft_serialize_*.txt   encoded native state dicts (hex) with their keys, dtypes,
+                                                   shapes and value bit patterns
   * in-source #[test] literals of crates/ft-kernel-cpu/src/lib.rs, transcribed by hand below with
     their line numbers (the literal input vectors and the asserted outputs)
 
@@ -172,11 +175,46 @@ def safetensors_corpus():
     return [{"name": n, "hex": open(os.path.join(d, n), "rb").read().hex()} for n in sorted(os.listdir(d))]
 
 
+def native_state_dict():
+    """Known answers for the native ("FTSV") state-dict container: the reference's golden encodings with the tensors
+    they hold (artifacts/optimization/golden_outputs/ft_serialize_*save*.txt: `encoded_hex=` is the container, every
+    `key=... dtype=... shape=[...] bits=a,b,...` line one tensor's raw element bit patterns), the decode summary of its
+    generated many-small-tensors payload (ft_serialize_decode_pass19.txt; the payload itself is built by the test
+    helper native_many_small_f64_payload, crates/ft-serialize/src/lib.rs:3847-3870, restated in the test that uses
+    it), and the seed inputs of its fuzz target (fuzz/corpus/ft_serialize_state_dict/*, read by its unit test
+    fuzz_corpus_state_dict_does_not_panic :4945-4971, which only asks for no panic)."""
+    gdir = os.path.join(REF, "artifacts", "optimization", "golden_outputs")
+    encodings = []
+    for fn in sorted(os.listdir(gdir)):
+        if not (fn.startswith("ft_serialize_") and "save" in fn):
+            continue
+        text = open(os.path.join(gdir, fn)).read()
+        hexs = re.search(r"^encoded_hex=([0-9a-f]+)$", text, re.M).group(1)
+        total = int(re.search(r"^total_len=(\d+)$", text, re.M).group(1))
+        tensors = []
+        for m in re.finditer(r"^key=(\S+) dtype=(\w+) shape=\[([^\]]*)\] bits=([0-9a-f,]*)$", text, re.M):
+            shape = [int(v) for v in m.group(3).split(",") if v.strip()]
+            tensors.append({"key": m.group(1), "dtype": m.group(2), "shape": shape, "bits": [b for b in m.group(4).split(",") if b]})
+        encodings.append({"source": "artifacts/optimization/golden_outputs/" + fn, "total_len": total, "encoded_hex": hexs, "tensors": tensors})
+    summary = open(os.path.join(gdir, "ft_serialize_decode_pass19.txt")).read()
+    decoded = []
+    for m in re.finditer(r"^key=(\S+) dtype=(\w+) shape=\[([^\]]*)\] values=\[([^\]]*)\]$", summary, re.M):
+        decoded.append({"key": m.group(1), "dtype": m.group(2), "shape": [int(v) for v in m.group(3).split(",") if v.strip()],
+                        "values": [float(v) for v in m.group(4).split(",") if v.strip()]})
+    d = os.path.join(REF, "fuzz", "corpus", "ft_serialize_state_dict")
+    corpus = [{"name": n, "hex": open(os.path.join(d, n), "rb").read().hex()} for n in sorted(os.listdir(d))]
+    return {"encodings": encodings,
+            "decode_pass19": {"source": "artifacts/optimization/golden_outputs/ft_serialize_decode_pass19.txt",
+                              "generator": "4 tensors 'layer.%04d.weight', rank 1, width 4, F64, value = tensor_index * 4 + position",
+                              "tensors": decoded},
+            "fuzz_corpus": corpus}
+
+
 def main():
     if not os.path.isdir(REF):
         sys.exit("reference checkout not found at %s" % REF)
     doc = {"conformance": conformance_cases(), "in_source": IN_SOURCE, "golden_text": golden_texts(),
-           "safetensors_corpus": safetensors_corpus()}
+           "safetensors_corpus": safetensors_corpus(), "native_state_dict": native_state_dict()}
     with open(OUT, "w") as f:
         json.dump(doc, f, indent=1, sort_keys=True)
         f.write("\n")
