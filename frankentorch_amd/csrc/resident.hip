@@ -587,14 +587,15 @@ int32_t fth_encoder_forward(fth_encoder *e, const float *input, int64_t batch, i
 int32_t fth_encoder_forward_graph(fth_encoder *e, const float *x_dev, int64_t batch, int64_t seq, float *out_dev, fth_stream s) {
     FTH_ARG(e != nullptr, "encoder_forward_graph: encoder is NULL");
     FTH_ARG(batch > 0 && seq > 0 && x_dev && out_dev && x_dev != out_dev, "encoder_forward_graph: bad arguments");
-    FTH_REQUIRE_DEVICE();
     // A run of this entry point under a rocprofiler tool library (rocprofv3 --kernel-trace) once
     // ended in a host segmentation fault inside the HIP runtime, below this function, between the
     // capture and the first replay; the same binary replays graphs without that tool. No cause
     // was found on this side of the runtime, so the combination is refused rather than retried.
+    // (Checked before the device is touched, so the refusal can be tested without one.)
     if (profiler_tool_loaded())
         return fth::set_error(FTH_ERR_UNAVAILABLE, "encoder_forward_graph: HIP-graph replay is refused while a rocprofiler tool "
                                                    "library is loaded; use fth_encoder_forward_dev");
+    FTH_REQUIRE_DEVICE();
     hipStream_t st = fth::resolve_stream(s);
     GraphKey key{x_dev, out_dev, batch, seq, s};
     hipGraphExec_t exec = nullptr;

@@ -123,17 +123,33 @@ Stager &stager() {
     return *s;
 }
 
-// True when [p, p + bytes) is page-locked host memory the DMA engines can address (hipHostMalloc).
+// True when [p, p + bytes) is page-locked host memory the DMA engines can address (hipHostMalloc): both ends must be
+// page-locked AND belong to one allocation (a slice that starts in one pinned block and ends in another, with pageable
+// memory between them, must not be handed to the DMA engine whole).
 bool is_pinned(const void *p, size_t bytes) {
-    auto one = [](const void *q) {
-        hipPointerAttribute_t a;
-        if (hipPointerGetAttributes(&a, q) != hipSuccess) {
-            (void)hipGetLastError();  // an ordinary pointer is reported as an error by some runtimes
-            return false;
-        }
-        return a.type == hipMemoryTypeHost;
-    };
-    return bytes > 0 && one(p) && one(static_cast<const char *>(p) + bytes - 1);
+    if (bytes == 0) return false;
+    hipPointerAttribute_t a;
+    if (hipPointerGetAttributes(&a, p) != hipSuccess) {
+        (void)hipGetLastError();  // an ordinary pointer is reported as an error by some runtimes
+        return false;
+    }
+    if (a.type != hipMemoryTypeHost) return false;
+    hipPointerAttribute_t b;
+    const char *last = static_cast<const char *>(p) + bytes - 1;
+    if (hipPointerGetAttributes(&b, last) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    if (b.type != hipMemoryTypeHost) return false;
+    // Same allocation: ask the runtime for the block that holds the first byte and require the last byte inside it.
+    // (Where the runtime cannot answer for host memory the two page-locked ends are all there is to go by.)
+    hipDeviceptr_t base = nullptr;
+    size_t size = 0;
+    if (hipMemGetAddressRange(&base, &size, const_cast<void *>(p)) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;
+    }
+    return last < static_cast<const char *>(base) + size && static_cast<const char *>(p) >= static_cast<const char *>(base);
 }
 
 #define FTH_STAGE(expr)                                      \

@@ -160,6 +160,36 @@ def test_transposes_check_lengths_before_any_device_call():
     assert _lib.load().fth_status_name(rc) == b"OutputTooSmall"
 
 
+def test_graph_replay_is_refused_under_a_profiler_tool(env={"LD_PRELOAD": "/nonexistent/librocprofiler-sdk-tool.so"}):
+    """fth_encoder_forward_graph returns Unavailable, with its own message, whenever a rocprofiler tool library is named in
+    the process environment; the check precedes any device call, so a child process without a GPU can show it (the dynamic
+    loader only warns about a preload it cannot find; naming a missing file in ROCP_TOOL_LIBRARIES, the other trigger, makes
+    the HIP runtime itself abort at load, so that one is not exercised here). The handle and the two buffers are never
+    dereferenced before the check."""
+    import subprocess
+    import sys
+
+    code = (
+        "import ctypes as C, sys\n"
+        "sys.path.insert(0, %r)\n"
+        "from frankentorch_amd import _lib\n"
+        "L = _lib.load()\n"
+        "rc = L.fth_encoder_forward_graph(C.c_void_p(4096), C.c_void_p(8192), 1, 8, C.c_void_p(12288), None)\n"
+        "print(rc, _lib.last_error().message.decode())\n" % os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    )
+    child_env = dict(os.environ)
+    child_env.update(env)
+    out = subprocess.run([sys.executable, "-c", code], env=child_env, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    rc, message = out.stdout.strip().split(" ", 1)
+    assert int(rc) == 100 and "rocprofiler tool" in message and "fth_encoder_forward_dev" in message
+    # without the variable the same call gets as far as the device check (or, on a GPU box, would run): not this message
+    clean = {k: v for k, v in os.environ.items() if k not in ("ROCP_TOOL_LIBRARIES",) and not (k == "LD_PRELOAD" and "rocprofiler" in v)}
+    if not os.path.exists("/dev/kfd"):
+        out = subprocess.run([sys.executable, "-c", code], env=clean, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+        assert out.returncode == 0 and out.stdout.startswith("100 ") and "rocprofiler tool" not in out.stdout
+
+
 def test_empty_results_need_no_device():
     f32 = lambda s: TensorMeta.from_shape(s, DType.F32)
     z = np.zeros(0, np.float32)

@@ -285,6 +285,28 @@ def test_norm_backward_at_the_row_op_benchmark_shape(hip, oracle):
     assert rel_err(ddw.to_host(), (dy64 * x64 * rstd).sum(0)) <= 4 * TOL_ROW_F32
 
 
+@pytest.mark.parametrize("rows,cols", [(8192, 4096), (8192, 768), (3000, 1024)])
+def test_column_sums_are_no_further_from_the_f64_sum_than_the_serial_f32_sum_is(hip, oracle, rows, cols):
+    """What NORM_COLSUM_TOL_FACTOR stands on. dweight / dbias are sums over the batch; the reference adds the rows in one
+    serial fp32 chain, the kernels add (rows of a workgroup) then (workgroups). Both are fp32 roundings of the same exact
+    sum, so the fair question is not how far they are from each other but how far each is from the float64 sum of the
+    same terms: the GPU's re-associated sum must not be the worse of the two."""
+    x = synth.normal(41, "x", (rows, cols))
+    dy = synth.normal(41, "dy", (rows, cols))
+    w = synth.uniform(41, "w", (cols,), 0.5, 1.5)
+    _, dw_o, db_o = oracle.layer_norm_backward(dy, x, w, np.float32(1e-5))   # the reference's serial fp32 sums
+    ddy, dx_, dw_ = _up(dy, x, w)
+    ddx, ddw, ddb = DeviceBuffer((rows, cols)), DeviceBuffer((cols,)), DeviceBuffer((cols,))
+    hip.layer_norm_backward(ddy, dx_, dw_, ddx, ddw, ddb, rows, cols, 1e-5)
+    x64, dy64 = x.astype(np.float64), dy.astype(np.float64)
+    xhat = (x64 - x64.mean(1, keepdims=True)) / np.sqrt(x64.var(1, keepdims=True) + 1e-5)
+    for name, gpu, serial, truth in (("dweight", ddw.to_host(), dw_o, (dy64 * xhat).sum(0)), ("dbias", ddb.to_host(), db_o, dy64.sum(0))):
+        e_gpu, e_serial = rel_err(gpu, truth), rel_err(serial, truth)
+        assert e_gpu <= max(e_serial, 1e-6), "%s: GPU %.3g from the f64 sum, the serial fp32 sum %.3g" % (name, e_gpu, e_serial)
+        assert e_gpu <= TOL_ROW_F32  # and against the truth the plain row-op bar holds, without the factor
+        assert rel_err(gpu, serial) <= TOL_ROW_F32 * NORM_COLSUM_TOL_FACTOR
+
+
 def test_host_slice_backward_entry_points(oracle):
     """The ft_kernel_cpu-named functions on host slices (upload, kernels, download), and their error statuses."""
     from frankentorch_amd import kernel_hip as K

@@ -228,13 +228,12 @@ CONFIG5_ARGMAX_ALLOW = {}
 
 def test_config5_gpt2_small_shape_logits_and_argmax(hip, oracle):
     """Config 5: 12 layers, d 768, 12 heads, FFN 3072, vocab 50257, batch 8, seq 1024, seed 4.
-    (1) Two complete 1024-token sequences of the batch (5 and 7, neither the first) go through the CPU checker's whole
-    model -- embeddings, 12 blocks at S = 1024 (every SDPA tile boundary and the packed-QKV strided reads at the real
-    shape), final LayerNorm, tied LM head -- and the GPU's hidden rows, logits and argmax of those 2048 positions are
-    compared with it: hidden and logits at 2e-5, argmax identical at every position. Sequences are independent under the
-    causal per-sequence attention, so the checker runs them as batch 1. (2) On sampled rows of every other sequence the
-    checker's LM head on the GPU's hidden state must give the same logits and argmax. (3) The whole logits tensor is
-    bitwise repeatable."""
+    (1) ALL EIGHT 1024-token sequences of the batch go through the CPU checker's whole model -- embeddings, 12 blocks at
+    S = 1024 (every SDPA tile boundary and the packed-QKV strided reads at the real shape), final LayerNorm, tied LM
+    head -- and the GPU's hidden rows, logits and argmax of all 8192 positions are compared with it: hidden and logits at
+    2e-5, argmax identical at every position. Sequences are independent under the causal per-sequence attention, so the
+    checker runs them one at a time as batch 1 (about four seconds each on sixteen threads). (2) The whole logits tensor
+    is bitwise repeatable."""
     vocab, maxpos, d, heads, f, nl, batch, seq = 50257, 1024, 768, 12, 3072, 12, 8, 1024
     wte = synth.normal(4, "wte", (vocab, d), 0.0, 0.02)
     wpe = synth.normal(4, "wpe", (maxpos, d), 0.0, 0.02)
@@ -253,7 +252,7 @@ def test_config5_gpt2_small_shape_logits_and_argmax(hip, oracle):
     one, zero = np.ones(d, np.float32), np.zeros(d, np.float32)
     # (1) whole sequences through the whole model
     mismatches = []
-    for b in (5, 7):
+    for b in range(batch):
         rows = slice(b * seq, (b + 1) * seq)
         ref = oracle.gpt2_forward(wte, wpe, layers, one, zero, ids[rows], 1, seq, heads, 1e-5, want_logits=True)
         assert ref["bad"] == -1
@@ -265,12 +264,45 @@ def test_config5_gpt2_small_shape_logits_and_argmax(hip, oracle):
     unexpected = [m for m in mismatches if (m[0], m[1]) not in CONFIG5_ARGMAX_ALLOW]
     assert not unexpected, "argmax differs from the checker at (sequence, position, checker, gpu, checker top-2 gap): %s" % unexpected
     assert len(mismatches) == len(CONFIG5_ARGMAX_ALLOW), "allow-listed rows that no longer differ: update CONFIG5_ARGMAX_ALLOW"
-    # (2) LM head + argmax on sampled rows of the other sequences
-    rows = np.arange(97, T, 257)
-    ref_logits = oracle.gemm(hidden[rows], wte, trans_b=True)
-    assert rel_err(full[rows], ref_logits) <= TOL_GEMM_F32
-    assert np.array_equal(am[rows], np.argmax(ref_logits, axis=1).astype(np.float32)), "argmax of sampled rows differs from the checker's LM head"
-    # (3) bitwise repeatability of the whole forward
+    # (2) bitwise repeatability of the whole forward
     dlog2 = DeviceBuffer((T, vocab))
     model.forward_dev(dids, batch, seq, dlog2, None)
     assert np.array_equal(full.view(np.uint32), dlog2.to_host().view(np.uint32))
+
+
+def test_graph_replay_is_refused_in_a_process_that_names_a_profiler_tool(hip):
+    """A fresh child process whose LD_PRELOAD names a (non-existent) rocprofiler library: the loader only warns, the eager
+    block runs and matches this process's result bit for bit, and the graph entry point returns Unavailable."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import sys, numpy as np\n"
+        "sys.path.insert(0, %r); sys.path.insert(0, %r)\n"
+        "from frankentorch_amd import fused, synth\n"
+        "from frankentorch_amd.core import HipError\n"
+        "from frankentorch_amd.device import DeviceBuffer\n"
+        "from test_gpu_resident import make_layer\n"
+        "enc = fused.EncoderHip(256, 4, 1024, [make_layer(0, 0, 256, 1024)], 1e-5, causal=True)\n"
+        "x = synth.normal(0, 'x', (128, 256)); dx, dout = DeviceBuffer.from_host(x), DeviceBuffer((128, 256))\n"
+        "enc.forward_dev(dx, dout, 1, 128)\n"
+        "print('eager', int(dout.to_host().view(np.uint32).astype(np.uint64).sum()))\n"
+        "try:\n"
+        "    enc.forward_dev(dx, dout, 1, 128, graph=True)\n"
+        "    print('graph ran')\n"
+        "except HipError as e:\n"
+        "    print('graph', e.kind)\n" % (root, os.path.join(root, "tests"))
+    )
+    env = dict(os.environ)
+    env["LD_PRELOAD"] = (env.get("LD_PRELOAD", "") + " /nonexistent/librocprofiler-sdk-tool.so").strip()
+    out = subprocess.run([sys.executable, "-c", code], env=env, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    lines = out.stdout.strip().splitlines()
+    assert lines[-1] == "graph Unavailable", out.stdout
+    enc = fused.EncoderHip(256, 4, 1024, [make_layer(0, 0, 256, 1024)], 1e-5, causal=True)
+    x = synth.normal(0, "x", (128, 256))
+    dx, dout = DeviceBuffer.from_host(x), DeviceBuffer((128, 256))
+    enc.forward_dev(dx, dout, 1, 128)
+    assert lines[-2] == "eager %d" % int(dout.to_host().view(np.uint32).astype(np.uint64).sum())

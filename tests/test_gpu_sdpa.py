@@ -103,9 +103,10 @@ def test_packed_qkv_strides_equal_the_permuted_copies(hip, oracle):
 
 
 def test_config4_full_size_sampled_heads_determinism_and_checksum(hip, oracle):
-    """B4 H32 S2048 D128, seed 3, causal. Two (batch, head) slices are compared with the oracle in
-    full; the whole output is bitwise equal across two runs; rows are convex combinations of V
-    rows, so every output lies inside V's per-head range (a property that needs no oracle)."""
+    """B4 H32 S2048 D128, seed 3, causal. Every fourth (batch, head) slice, from all four batches, and the last one
+    (bh = 127) are compared with the oracle in full, each held to the tolerance on its own; the whole output is bitwise
+    equal across two runs; rows are convex combinations of V rows, so every output lies inside V's per-head range (a
+    property that needs no oracle)."""
     B, H, S, D = 4, 32, 2048, 128
     s = 1.0 / math.sqrt(D)
     q = synth.normal(3, "Q", (B * H, S, D), 0.0, s)
@@ -118,9 +119,10 @@ def test_config4_full_size_sampled_heads_determinism_and_checksum(hip, oracle):
     hip.sdpa_forward(desc, s, dq, dk, dv, do2)
     out = do.to_host()
     assert np.array_equal(out.view(np.uint32), do2.to_host().view(np.uint32))
-    for bh in (0, 77):
-        ref = oracle.sdpa_forward(q[bh:bh + 1], k[bh:bh + 1], v[bh:bh + 1], s, True)
-        assert rel_err(out[bh:bh + 1], ref) <= TOL_GEMM_F32
+    heads = sorted(set(range(0, B * H, 4)) | {77, B * H - 1})
+    ref = oracle.sdpa_forward(q[heads], k[heads], v[heads], s, True)
+    for i, bh in enumerate(heads):
+        assert rel_err(out[bh], ref[i]) <= TOL_GEMM_F32, "(batch, head) slice %d" % bh
     assert np.all(out.max(axis=1) <= v.max(axis=1) + 1e-6) and np.all(out.min(axis=1) >= v.min(axis=1) - 1e-6)
     assert np.array_equal(out[:, 0], v[:, 0])
 

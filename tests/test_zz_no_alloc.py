@@ -40,6 +40,34 @@ def test_no_alloc_layer_norm_backward_equals_the_workspace_form(hip, oracle):
     assert rel_err(got[1], dw_r) <= TOL_ROW_F32 * NORM_COLSUM_TOL_FACTOR and rel_err(got[2], db_r) <= TOL_ROW_F32 * NORM_COLSUM_TOL_FACTOR
 
 
+def test_no_alloc_call_allocates_nothing(hip):
+    """The property the entry point exists for: after a first call (which looks the scratch array's address up), a call
+    changes neither the library pool's block and byte counts nor the device's free memory, for the register-resident shape
+    and for a streaming one (columns not a multiple of the vector width)."""
+    import ctypes as C
+
+    from frankentorch_amd import _lib
+
+    def pool():
+        used, cached = C.c_uint64(), C.c_uint64()
+        assert _lib.load().fth_pool_stats(C.byref(used), C.byref(cached)) == 0
+        return used.value, cached.value
+
+    for rows, cols in ((4096, 4096), (700, 1026)):
+        x = synth.normal(35, "x", (rows, cols))
+        dy = synth.normal(35, "dy", (rows, cols))
+        w = synth.uniform(35, "w", (cols,), 0.5, 1.5)
+        ddy, dx_, dw_ = (DeviceBuffer.from_host(a) for a in (dy, x, w))
+        out = [DeviceBuffer((rows, cols)), DeviceBuffer((cols,)), DeviceBuffer((cols,))]
+        hip.layer_norm_backward_noalloc(ddy, dx_, dw_, out[0], out[1], out[2], rows, cols, 1e-5)  # warm-up
+        hip.synchronize()
+        before = (pool(), hip.memory_info()[0])
+        for _ in range(3):
+            hip.layer_norm_backward_noalloc(ddy, dx_, dw_, out[0], out[1], out[2], rows, cols, 1e-5)
+        hip.synchronize()
+        assert (pool(), hip.memory_info()[0]) == before, (rows, cols)
+
+
 def test_no_alloc_rejects_shapes_beyond_the_scratch(hip):
     from frankentorch_amd.core import HipError
 
