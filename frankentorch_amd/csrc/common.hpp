@@ -29,6 +29,12 @@ int compute_units();
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Softmax over contiguous rows too long or too ragged for the 128-bit row kernels (any length up to 65 536 floats /
+// 32 768 doubles, any 4- / 8-byte alignment): the register-resident row kernel of the loss unit. Returns false, with
+// nothing launched, when a row does not fit.
+bool softmax_resident_rows(const float *x, float *y, int64_t rows, int64_t cols, hipStream_t st);
+bool softmax_resident_rows(const double *x, double *y, int64_t rows, int64_t cols, hipStream_t st);
+
 // Causal attention launches whose workgroups are ALL resident at once (grid <= workgroups per compute unit x compute
 // units) cannot rely on heaviest-first issue to balance: nothing is left to hand out when a light workgroup ends. The
 // hardware deals workgroup ids round-robin over the 8 XCDs and, inside an XCD, over its compute units in id order, so a

@@ -63,4 +63,23 @@ __device__ __forceinline__ double exp2_softmax(double t) {
     return __builtin_ldexp(p, (int)n);
 }
 
+// exp(x) = 2^(x * log2 e) on the hardware exp2 unit. The product x * log2 e is carried in two
+// pieces (t + r, with the rounding error of the multiply recovered by an FMA and the low bits of
+// log2 e added), and 2^r is folded back as 1 + r ln 2, so the result stays within about 1.5 ULP
+// instead of the |x| * 2^-24 relative error of a bare exp2(x * log2e). -inf (and anything below -126)
+// maps to exactly 0 and NaN propagates, which the softmax special cases rely on. Results below 2^-126 flush to
+// zero. Meant for arguments that are not large and positive (a value minus a maximum): where 2^t overflows the
+// correction term gives NaN, not +inf.
+__device__ __forceinline__ float exp_hw(float x) {
+    const float kL2eHi = 1.44269502162933349609375f;  // float(log2 e)
+    const float kL2eLo = 1.925963033500011e-8f;       // log2 e - float(log2 e)
+    const float kLn2 = 0.693147182464599609375f;
+    const float t = x * kL2eHi;
+    float r = __builtin_fmaf(x, kL2eHi, -t);
+    r = __builtin_fmaf(x, kL2eLo, r);
+    r = (x < -126.0f) ? 0.0f : r;  // 2^t is 0 from here on; keeps t = -inf (x = -inf, or x * log2 e overflowing) out of r
+    const float e = __builtin_amdgcn_exp2f(t);
+    return __builtin_fmaf(e * r, kLn2, e);
+}
+
 }  // namespace fth

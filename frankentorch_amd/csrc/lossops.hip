@@ -19,6 +19,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "devmath.hpp"
 
 namespace {
 
@@ -27,7 +28,7 @@ constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
 
 template <typename T> __device__ __forceinline__ T t_exp(T v);
-template <> __device__ __forceinline__ float t_exp<float>(float v) { return expf(v); }
+template <> __device__ __forceinline__ float t_exp<float>(float v) { return fth::exp_hw(v); }
 template <> __device__ __forceinline__ double t_exp<double>(double v) { return exp(v); }
 template <typename T> __device__ __forceinline__ T t_log(T v);
 template <> __device__ __forceinline__ float t_log<float>(float v) { return logf(v); }
@@ -152,27 +153,59 @@ __global__ __launch_bounds__(kThreads) void cross_entropy_backward_kernel(const 
     for (int64_t c = threadIdx.x; c < classes; c += kThreads) drow[c] = g * (t_exp<T>(row[c] - lse) - (c == t ? T(1) : T(0)));
 }
 
-// Keeps a workgroup-uniform pointer in scalar registers and stops the compiler from folding what is added to it
-// later into a per-lane offset.
-template <typename P> __device__ __forceinline__ P *uniform_ptr(P *p) {
-    asm volatile("" : "+s"(p));
-    return p;
+// ---- bounds-checked row accesses ----
+// A buffer resource over [base, base + bytes): the hardware returns 0 for a load and drops a store whose byte offset is
+// not below `bytes`, so the ragged end of a row needs no per-lane predicate, and the resource lives in scalar registers:
+// the only vector register an access needs is the lane's byte offset, shared by every step of the row.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t span_of(const void *base, int bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes < 0 ? 0 : bytes, 0x00020000);
 }
+typedef unsigned int raw_u2 __attribute__((ext_vector_type(2)));
+// non-temporal: rows are read once and outputs never re-read
+template <typename T> __device__ __forceinline__ T span_load(__amdgpu_buffer_rsrc_t r, int byte_off);
+template <> __device__ __forceinline__ float span_load<float>(__amdgpu_buffer_rsrc_t r, int byte_off) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, 2));
+}
+template <> __device__ __forceinline__ double span_load<double>(__amdgpu_buffer_rsrc_t r, int byte_off) {
+    return __builtin_bit_cast(double, __builtin_amdgcn_raw_buffer_load_b64(r, byte_off, 0, 2));
+}
+__device__ __forceinline__ void span_store(float v, __amdgpu_buffer_rsrc_t r, int byte_off) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned int, v), r, byte_off, 0, 2);
+}
+__device__ __forceinline__ void span_store(double v, __amdgpu_buffer_rsrc_t r, int byte_off) {
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(raw_u2, v), r, byte_off, 0, 2);
+}
+// max that returns the other operand for a NaN (one instruction; of +0 and -0 it returns +0)
+__device__ __forceinline__ float max_skip_nan(float a, float b) { return __builtin_fmaxf(a, b); }
+__device__ __forceinline__ double max_skip_nan(double a, double b) { return __builtin_fmax(a, b); }
+
+struct MaxSkipNanOp {
+    template <typename T> __device__ __forceinline__ T operator()(T a, T b) const { return max_skip_nan(a, b); }
+};
 
 // One row per workgroup, held in registers: lane t owns elements t, t + THREADS, ... (VPT of them).
-// MODE 0: log-softmax (max that skips NaN); 1: cross-entropy loss; 2: cross-entropy dlogits (strict `>` max).
-enum { kLogSoftmax = 0, kLossForward = 1, kLossBackward = 2 };
+// MODE 0: log-softmax; 1: cross-entropy loss; 2: cross-entropy dlogits; 3: softmax. The maximum of all skips NaN elements
+// (f32::max in the reference's log-softmax fold, a strict `>` scan in its cross-entropy: the same value, up to the
+// sign of a zero maximum, which none of the outputs depends on beyond the sign of a zero).
+enum { kLogSoftmax = 0, kLossForward = 1, kLossBackward = 2, kSoftmax = 3 };
 
 // `lds_steps` further steps of the row (after the VPT register steps) live in dynamic LDS, filled by direct-to-LDS
 // loads: with 19 steps (76 KiB) there and at most 64 registers per lane, two 1024-lane workgroups share a compute unit
 // and one's loads overlap the other's arithmetic and stores. Each lane reads back only the LDS words its own loads
 // wrote, so a wait for the loads is enough and no barrier is needed. MINW: minimum wavefronts per SIMD (sets the
-// register budget).
-template <typename T, int VPT, int THREADS, int MODE, int MINW>
+// register budget). FULL: the caller guarantees cols >= VPT * THREADS, so every register step is fully occupied
+// (apart from the alignment lead of step 0) and needs no padding.
+//
+// The kernel is as much bound by vector instructions as by memory (at [8192, 50257] the vector units were busy 60 % of
+// the time with the library exponential and per-element predicates), so each pass is kept to the arithmetic proper:
+// the step's address and bound are scalar work, padding is applied only where a step can be ragged, and the
+// cross-entropy gradient keeps exp(x - max) from the sum pass instead of taking a second exponential.
+template <typename T, int VPT, int THREADS, int MODE, int MINW, bool FULL>
 __global__ __launch_bounds__(THREADS, MINW) void resident_rows_kernel(const T *__restrict__ x, const int64_t *__restrict__ target,
                                                                      const T *__restrict__ dloss, int64_t cols, T *__restrict__ out,
                                                                      int64_t *bad_index, int lds_steps) {
     constexpr int WAVES = THREADS / kWave;
+    constexpr int kElt = (int)sizeof(T);
     // Left free, the scheduler overlaps the exponentials of many elements and spills the row once the register budget
     // is nearly all row data; there the per-element steps are kept in program order instead.
     constexpr bool kPinOrder = THREADS == 1024 && VPT * (int)sizeof(T) * MINW > 384;
@@ -182,7 +215,7 @@ __global__ __launch_bounds__(THREADS, MINW) void resident_rows_kernel(const T *_
     int phase = 0;
     const int64_t i = blockIdx.x;
     int64_t t = 0;
-    if (MODE != kLogSoftmax) {
+    if (MODE == kLossForward || MODE == kLossBackward) {
         t = target[i];
         if (t < 0 || t >= cols) {  // uniform over the workgroup
             note_bad(bad_index, i);
@@ -195,11 +228,14 @@ __global__ __launch_bounds__(THREADS, MINW) void resident_rows_kernel(const T *_
     // (fp64: 512-byte) pieces: rows of an odd length start at arbitrary element offsets, and partial-line
     // writes from different wavefronts cost far more HBM time than they carry. Slot j holds element j - lead;
     // slots below `lead` (only in step 0) and from `n` on are empty.
+    const T *row_in = x + i * cols;
     const T *row_out = (MODE == kLossForward ? x : out) + i * cols;
     const int lead = (int)((reinterpret_cast<uintptr_t>(row_out) / sizeof(T)) % kWave);
-    const T *xr = x + i * cols - lead;   // slot 0 of the row
+    const T *xr = row_in - lead;         // slot 0 of the row
     const int n = (int)cols + lead;      // one past the last occupied slot
-    const int n_lds = n - VPT * THREADS;  // occupied slots that live in LDS (<= 0: none)
+    const int kfull = n / THREADS;       // steps below this one are full, step kfull is ragged, later ones are empty
+    // LDS steps [0, lds_full) are full; the (at most two) remaining ones take a per-lane bound
+    const int lds_full = kfull - VPT < 0 ? 0 : (kfull - VPT < lds_steps ? kfull - VPT : lds_steps);
     if constexpr (sizeof(T) == 4) {
         // oldest in the load queue, so the compiler's own counted waits for the register loads below stay exact
         const unsigned wave = __builtin_amdgcn_readfirstlane((unsigned)(tid / kWave));
@@ -207,70 +243,86 @@ __global__ __launch_bounds__(THREADS, MINW) void resident_rows_kernel(const T *_
         const unsigned lane_off = (unsigned)(tid & (kWave - 1)) * 4u;
         for (int k = 0; k < lds_steps; ++k) {
             const T *pk = xr + (VPT + k) * THREADS + wave * kWave;  // scalar: the wavefront's 64 slots of step VPT + k
-            if (tid < n_lds - k * THREADS)
+            if (k < lds_full || tid < n - (VPT + k) * THREADS)
                 asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1 nt" ::"v"(lane_off), "s"(pk),
                              "s"(wave_base + (unsigned)k * (THREADS * 4u))
                              : "memory", "m0");
         }
     }
-    // Step k touches slots [k * THREADS, (k + 1) * THREADS): a scalar base per step plus the one per-lane offset
-    // `tid`, so no per-element address or bounds predicate stays live in a vector register between the passes.
+    // Step k touches slots [k * THREADS, (k + 1) * THREADS) through a resource that starts at the step's slot 0 and ends
+    // with the row: scalar work per step, and the one per-lane offset `off` for all of them.
+    const int off = tid * kElt;
+    const bool lead_ok = tid >= lead;
+    auto step_span = [&](const T *slot0, int k, int end) __attribute__((always_inline)) {
+        return span_of(slot0 + k * THREADS, (end - k * THREADS) * kElt);
+    };
     T v[VPT];
+    {
+        // step 0: the `lead` empty slots lie before the row (for row 0, before the allocation): their lanes read
+        // element 0 and drop it
+        const int e0 = tid - lead;
+        const T t0 = span_load<T>(span_of(row_in, (int)cols * kElt), (e0 < 0 ? 0 : e0) * kElt);
+        v[0] = (lead_ok && tid < n) ? t0 : T(-__builtin_inf());
+    }
 #pragma unroll
-    for (int k = 0; k < VPT; ++k) {
-        const T *pk = uniform_ptr(xr + k * THREADS);
-        v[k] = (tid < n - k * THREADS && (k > 0 || tid >= lead)) ? __builtin_nontemporal_load(pk + tid) : T(-__builtin_inf());
+    for (int k = 1; k < VPT; ++k) {
+        const T tk = span_load<T>(step_span(xr, k, n), off);
+        v[k] = (FULL || tid < n - k * THREADS) ? tk : T(-__builtin_inf());
     }
     T m = T(-__builtin_inf());
 #pragma unroll
-    for (int k = 0; k < VPT; ++k) m = MODE == kLogSoftmax ? max_num(m, v[k]) : max_gt(m, v[k]);  // the padding never wins
+    for (int k = 0; k < VPT; ++k) m = max_skip_nan(m, v[k]);  // the padding never wins
     if (lds_steps > 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    for (int k = 0; k < lds_steps; ++k)
-        if (tid < n_lds - k * THREADS) m = MODE == kLogSoftmax ? max_num(m, lrow[k * THREADS]) : max_gt(m, lrow[k * THREADS]);
-    if (MODE == kLogSoftmax)
-        m = block_reduce<T, MaxNumOp, WAVES>(m, MaxNumOp{}, red, phase);
-    else
-        m = block_reduce<T, MaxGtOp, WAVES>(m, MaxGtOp{}, red, phase);
+    for (int k = 0; k < lds_full; ++k) m = max_skip_nan(m, lrow[k * THREADS]);
+    for (int k = lds_full; k < lds_steps; ++k)
+        if (tid < n - (VPT + k) * THREADS) m = max_skip_nan(m, lrow[k * THREADS]);
+    m = block_reduce<T, MaxSkipNanOp, WAVES>(m, MaxSkipNanOp{}, red, phase);
     // The -inf padding adds exp(-inf - m) = +0 for a finite or +inf maximum and NaN for a -inf one, where the sum of
-    // the real elements is NaN already, so the sum over the registers needs no bounds test.
+    // the real elements is NaN already, so the sum over the registers needs no bounds test. The gradient keeps
+    // e = exp(x - m) in place of x: its output is e / sum.
     T s = T(0);
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
-        s += t_exp<T>(v[k] - m);
+        const T e = t_exp<T>(v[k] - m);
+        s += e;
+        if (MODE == kLossBackward || MODE == kSoftmax) v[k] = e;
         if (kPinOrder) __builtin_amdgcn_sched_barrier(0);
     }
-    for (int k = 0; k < lds_steps; ++k)
-        if (tid < n_lds - k * THREADS) s += t_exp<T>(lrow[k * THREADS] - m);
+    auto lds_sum = [&](int k) __attribute__((always_inline)) {
+        const T e = t_exp<T>(lrow[k * THREADS] - m);
+        s += e;
+        if (MODE == kLossBackward || MODE == kSoftmax) lrow[k * THREADS] = e;
+    };
+    for (int k = 0; k < lds_full; ++k) lds_sum(k);
+    for (int k = lds_full; k < lds_steps; ++k)
+        if (tid < n - (VPT + k) * THREADS) lds_sum(k);
     s = block_reduce<T, SumOp, WAVES>(s, SumOp{}, red, phase);
-    if (MODE == kLogSoftmax) {
-        const T lse = t_log<T>(s);
-        T *yr = out + i * cols - lead;
-#pragma unroll
-        for (int k = 0; k < VPT; ++k) {
-            T *pk = uniform_ptr(yr + k * THREADS);
-            if (tid < n - k * THREADS && (k > 0 || tid >= lead)) __builtin_nontemporal_store((v[k] - m) - lse, pk + tid);
-            if (kPinOrder) __builtin_amdgcn_sched_barrier(0);
-        }
-        for (int k = 0; k < lds_steps; ++k)
-            if (tid < n_lds - k * THREADS) __builtin_nontemporal_store((lrow[k * THREADS] - m) - lse, yr + (VPT + k) * THREADS + tid);
-    } else if (MODE == kLossForward) {
+    if (MODE == kLossForward) {
         if (tid == 0) out[i] = (m + t_log<T>(s)) - x[i * cols + t];
-    } else {
-        const T lse = m + t_log<T>(s), g = dloss[i];
-        T *dr = out + i * cols - lead;
-        const int tt = (int)t + lead;  // the target's slot
-#pragma unroll
-        for (int k = 0; k < VPT; ++k) {
-            T *pk = uniform_ptr(dr + k * THREADS);
-            if (tid < n - k * THREADS && (k > 0 || tid >= lead))
-                __builtin_nontemporal_store(g * (t_exp<T>(v[k] - lse) - (tid == tt - k * THREADS ? T(1) : T(0))), pk + tid);
-            if (kPinOrder) __builtin_amdgcn_sched_barrier(0);
-        }
-        for (int k = 0; k < lds_steps; ++k)
-            if (tid < n_lds - k * THREADS)
-                __builtin_nontemporal_store(g * (t_exp<T>(lrow[k * THREADS] - lse) - (tid == tt - (VPT + k) * THREADS ? T(1) : T(0))),
-                                            dr + (VPT + k) * THREADS + tid);
+        return;
     }
+    // Outputs: step 0 is stored under the lane's own predicate (an offset before the row must not reach memory), every
+    // other step through its bounded resource. Values computed from empty slots are dropped by the bound.
+    T *yr = out + i * cols - lead;
+    // The bounds of the output steps equal those of the input steps; recomputing them from an opaque copy of `n` costs one
+    // scalar instruction per step, where keeping 32 of them alive across the kernel spills scalar registers.
+    int n_out = n;
+    asm volatile("" : "+s"(n_out));
+    const T lse = t_log<T>(s);                                     // log-softmax: (x - m) - ln(sum)
+    const T inv_s = T(1) / s, g = MODE == kLossBackward ? dloss[i] : T(0);  // gradient: g (e / sum - onehot)
+    const int tt = (int)t + lead;                                  // the target's slot
+    auto result = [&](T val, int slot0_of_step) __attribute__((always_inline)) {
+        if (MODE == kLogSoftmax) return (val - m) - lse;
+        if (MODE == kSoftmax) return val * inv_s;  // one correctly rounded 1 / sum per row, as the 128-bit row kernel
+        return g * (val * inv_s - (tid == tt - slot0_of_step ? T(1) : T(0)));
+    };
+    if (lead_ok) span_store(result(v[0], 0), span_of(out + i * cols, (int)cols * kElt), (tid - lead) * kElt);
+#pragma unroll
+    for (int k = 1; k < VPT; ++k) {
+        span_store(result(v[k], k * THREADS), step_span(yr, k, n_out), off);
+        if (kPinOrder) __builtin_amdgcn_sched_barrier(0);
+    }
+    for (int k = 0; k < lds_steps; ++k) span_store(result(lrow[k * THREADS], (VPT + k) * THREADS), step_span(yr, VPT + k, n_out), off);
 }
 
 // Cross-entropy loss of long fp32 rows in one streaming pass. The loss needs only the row's log-sum-exp and one
@@ -360,7 +412,7 @@ bool launch_resident(const T *x, const int64_t *target, const T *dloss, int64_t 
 #define FTH_HYBRID(VPT)                                                                                                         \
     if (need <= (VPT)) {                                                                                                       \
         const int lds_steps = (int)(steps - (VPT));                                                                            \
-        resident_rows_kernel<T, VPT, 1024, MODE, 8><<<dim3((unsigned)rows), dim3(1024), (size_t)lds_steps * 4096, st>>>(       \
+        resident_rows_kernel<T, VPT, 1024, MODE, 8, true><<<dim3((unsigned)rows), dim3(1024), (size_t)lds_steps * 4096, st>>>(       \
             x, target, dloss, cols, out, bad_index, lds_steps);                                                                \
         return true;                                                                                                           \
     }
@@ -374,7 +426,7 @@ bool launch_resident(const T *x, const int64_t *target, const T *dloss, int64_t 
 #define FTH_RESIDENT(THREADS, VPT)                                                                                                  \
     if (slots <= (int64_t)(THREADS) * (VPT)) {                                                                                     \
         if constexpr ((VPT) <= kMaxVpt)                                                                                            \
-            resident_rows_kernel<T, VPT, THREADS, MODE, 1><<<dim3((unsigned)rows), dim3(THREADS), 0, st>>>(x, target, dloss, cols, \
+            resident_rows_kernel<T, VPT, THREADS, MODE, 1, false><<<dim3((unsigned)rows), dim3(THREADS), 0, st>>>(x, target, dloss, cols, \
                                                                                                             out, bad_index, 0);    \
         return true;                                                                                                               \
     }
@@ -463,6 +515,15 @@ int32_t cross_entropy_entry(bool backward, const T *logits, const int64_t *targe
 }
 
 }  // namespace
+
+namespace fth {
+bool softmax_resident_rows(const float *x, float *y, int64_t rows, int64_t cols, hipStream_t st) {
+    return launch_resident<float, kSoftmax>(x, nullptr, nullptr, rows, cols, y, nullptr, st);
+}
+bool softmax_resident_rows(const double *x, double *y, int64_t rows, int64_t cols, hipStream_t st) {
+    return launch_resident<double, kSoftmax>(x, nullptr, nullptr, rows, cols, y, nullptr, st);
+}
+}  // namespace fth
 
 extern "C" {
 

@@ -81,22 +81,7 @@ template <typename T> struct Vec128;
 template <> struct Vec128<float> { using type = float4; static constexpr int n = 4; };
 template <> struct Vec128<double> { using type = double2; static constexpr int n = 2; };
 
-// exp(x) = 2^(x * log2 e) on the hardware exp2 unit. The product x * log2 e is carried in two
-// pieces (t + r, with the rounding error of the multiply recovered by an FMA and the low bits of
-// log2 e added), and 2^r is folded back as 1 + r ln 2, so the result stays within about 1.5 ULP
-// instead of the |x| * 2^-24 relative error of a bare exp2(x * log2e). -inf maps to exactly 0 and
-// NaN propagates, which the softmax special cases rely on. Results below 2^-126 flush to zero.
-__device__ __forceinline__ float dev_exp(float x) {
-    const float kL2eHi = 1.44269502162933349609375f;  // float(log2 e)
-    const float kL2eLo = 1.925963033500011e-8f;       // log2 e - float(log2 e)
-    const float kLn2 = 0.693147182464599609375f;
-    const float t = x * kL2eHi;
-    float r = __builtin_fmaf(x, kL2eHi, -t);
-    r = __builtin_fmaf(x, kL2eLo, r);
-    r = (x == -__builtin_inff()) ? 0.0f : r;
-    const float e = __builtin_amdgcn_exp2f(t);
-    return __builtin_fmaf(e * r, kLn2, e);
-}
+__device__ __forceinline__ float dev_exp(float x) { return fth::exp_hw(x); }
 __device__ __forceinline__ double dev_exp(double x) { return exp(x); }
 __device__ __forceinline__ float dev_sqrt(float x) { return sqrtf(x); }
 __device__ __forceinline__ double dev_sqrt(double x) { return sqrt(x); }
@@ -994,7 +979,10 @@ int32_t launch_softmax(const T *x, T *y, int64_t rows, int64_t cols, fth_stream 
 #undef L
     } else {
         FTH_ARG(rows <= kMaxGrid, "softmax: too many rows for one launch");
-        softmax_stream_kernel<T><<<dim3((unsigned)rows), dim3(kBlock), 0, st>>>(x, y, rows, cols);
+        // odd lengths, unaligned rows and rows beyond 8192 vectors (a vocabulary): still one read and one write while the
+        // row fits a workgroup's registers and LDS; only beyond that the three-sweep kernel
+        if (!fth::softmax_resident_rows(x, y, rows, cols, st))
+            softmax_stream_kernel<T><<<dim3((unsigned)rows), dim3(kBlock), 0, st>>>(x, y, rows, cols);
     }
     FTH_CHECK_LAUNCH("softmax");
     return FTH_OK;

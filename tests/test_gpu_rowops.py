@@ -12,7 +12,8 @@ from frankentorch_amd.device import DeviceBuffer
 pytestmark = pytest.mark.gpu
 
 # register-resident one-wave rows, four-wave rows, streaming rows, ragged / unaligned lengths
-SHAPES = [(1, 1), (3, 7), (64, 256), (33, 768), (5, 1024), (16, 4100), (9, 4096), (8, 16384), (3, 20000), (4, 50257), (7, 513)]
+SHAPES = [(1, 1), (3, 7), (64, 256), (33, 768), (5, 1024), (16, 4100), (9, 4096), (8, 16384), (3, 20000), (4, 50257), (7, 513),
+          (2, 40000), (2, 65536), (2, 65541)]  # beyond 8192 vectors: the register-and-LDS resident rows, then the sweeping kernel
 
 
 def _inputs(rows, cols, dtype, seed=11):
@@ -119,6 +120,32 @@ def test_softmax_special_values(hip, oracle, vectors):
     bits = dzo.to_host().ravel().view(np.uint32)
     for i, v in b["bits"]["f32_softmax_fast_bits"].items():
         assert bits[int(i)] == int(v, 16)
+
+
+@pytest.mark.parametrize("cols", [5, 1023, 50257, 40000])
+def test_softmax_ragged_and_long_rows_special_values(hip, oracle, cols):
+    """Rows that are no multiple of a 128-bit vector, or longer than 8192 vectors, take the resident-row kernel: the same
+    special cases as the short rows (an infinity or a NaN poisons its row only, -inf elements weigh nothing), and every
+    finite row sums to one."""
+    x = synth.normal(77, "x", (7, cols)) * np.float32(3.0)
+    x[0, cols // 2] = np.inf
+    x[1, cols - 1] = np.nan
+    x[2] = -np.inf
+    x[3, 0] = -np.inf
+    x[3, cols - 1] = -np.inf
+    x[4] = 5.0
+    dx, dy = DeviceBuffer.from_host(x), DeviceBuffer(x.shape)
+    hip.softmax_lastdim(dx, dy, 7, cols)
+    y, ref = dy.to_host(), oracle.softmax(x, 1)
+    assert np.array_equal(np.isnan(y), np.isnan(ref))
+    assert np.all(np.isnan(y[0])) and np.all(np.isnan(y[1])) and np.all(np.isnan(y[2]))
+    assert y[3, 0] == 0.0 and y[3, cols - 1] == 0.0
+    fin = [3, 4, 5, 6]
+    assert rel_err(y[fin], ref[fin]) <= TOL_ROW_F32
+    assert np.max(np.abs(y[fin].astype(np.float64).sum(axis=1) - 1.0)) <= 1e-5
+    assert np.all(y[4] == y[4, 0])
+    hip.softmax_lastdim(dx, dy, 7, cols)
+    assert np.array_equal(y.view(np.uint32), dy.to_host().view(np.uint32))
 
 
 def test_gelu_special_values_and_dense_accuracy(hip, oracle):
