@@ -1153,26 +1153,41 @@ struct StreamWorkspace {
 // A block that a larger request outgrows is retired, never handed back to the shared pool: kernels
 // queued on the stream may still be using it, the pool serves every stream and thread (so "ordered
 // on the same stream" would not protect the next owner), and a captured HIP graph keeps the address
-// it was recorded with for as long as its executable lives. Requests up to 512 MiB grow
-// geometrically, so the retired blocks of a stream add up to less than its current one.
+// it was recorded with for as long as its executable lives. Requests up to 4 GiB grow geometrically,
+// so the retired blocks of a (stream, slot) add up to less than its current one; only a single
+// request beyond 4 GiB (a transposed operand of more than 2^30 floats) retires its predecessor without
+// that bound. The totals are reported by fth_device_workspace_info.
+struct WorkspaceTable {
+    std::mutex mu;
+    std::map<std::pair<hipStream_t, int>, StreamWorkspace> table;
+    std::vector<void *> retired;
+    uint64_t live_bytes = 0, retired_bytes = 0;
+};
+WorkspaceTable &workspace_table() {
+    static WorkspaceTable *t = new WorkspaceTable();  // never destroyed: streams outlive static destructors
+    return *t;
+}
 int32_t get_workspace(hipStream_t st, size_t partial_bytes, void **partials, int slot = 0) {
-    static std::mutex mu;
-    static std::map<std::pair<hipStream_t, int>, StreamWorkspace> *table = new std::map<std::pair<hipStream_t, int>, StreamWorkspace>();
-    static std::vector<void *> *retired = new std::vector<void *>();
-    std::lock_guard<std::mutex> lock(mu);
-    StreamWorkspace &w = (*table)[std::make_pair(st, slot)];
+    WorkspaceTable &t = workspace_table();
+    std::lock_guard<std::mutex> lock(t.mu);
+    StreamWorkspace &w = t.table[std::make_pair(st, slot)];
     if (w.partial_bytes < partial_bytes) {
         size_t want = partial_bytes;
-        if (w.partial_bytes && want < 2 * w.partial_bytes && w.partial_bytes <= ((size_t)1 << 29)) want = 2 * w.partial_bytes;
+        if (w.partial_bytes && want < 2 * w.partial_bytes && w.partial_bytes <= ((size_t)1 << 31)) want = 2 * w.partial_bytes;
         void *fresh = nullptr;
         if (int32_t rc = fth::pool_alloc(&fresh, want)) {
             if (want == partial_bytes) return rc;
             want = partial_bytes;  // the doubled block did not fit: take exactly what is needed
             if (int32_t rc2 = fth::pool_alloc(&fresh, want)) return rc2;
         }
-        if (w.partials) retired->push_back(w.partials);
+        if (w.partials) {
+            t.retired.push_back(w.partials);
+            t.retired_bytes += w.partial_bytes;
+            t.live_bytes -= w.partial_bytes;
+        }
         w.partials = fresh;
         w.partial_bytes = want;
+        t.live_bytes += want;
     }
     *partials = w.partials;
     return FTH_OK;
@@ -1474,6 +1489,14 @@ template <typename T> int32_t launch_trans_a(GemmArgs<T> &p, const fth_gemm_desc
 }  // namespace
 
 extern "C" {
+
+int32_t fth_device_workspace_info(uint64_t *live_bytes, uint64_t *retired_bytes) {
+    WorkspaceTable &t = workspace_table();
+    std::lock_guard<std::mutex> lock(t.mu);
+    if (live_bytes) *live_bytes = t.live_bytes;
+    if (retired_bytes) *retired_bytes = t.retired_bytes;
+    return FTH_OK;
+}
 
 int32_t fth_dev_gemm_f32(const fth_gemm_desc *d, float alpha, const float *a, const float *b, float *c,
                          const float *bias, const float *residual, fth_stream s) {

@@ -292,6 +292,13 @@ def memory_info():
     return f.value, tot.value
 
 
+def gemm_workspace_info():
+    """(live, retired) bytes of the GEMM unit's split-tile / transposed-operand workspaces."""
+    live, ret = C.c_uint64(), C.c_uint64()
+    check(_lib.load().fth_device_workspace_info(C.byref(live), C.byref(ret)))
+    return live.value, ret.value
+
+
 def permute_0213(src, dst, d0, d1, d2, d3, stream=None):
     check(getattr(_lib.load(), "fth_dev_permute_0213_" + _sfx(src))(_ptr(src), _ptr(dst), d0, d1, d2, d3, stream))
 

@@ -126,6 +126,11 @@ int32_t fth_memcpy_d2d(void *dst_dev, const void *src_dev, size_t bytes);
 int32_t fth_memset_zero(void *dst_dev, size_t bytes);
 /* Free and total device memory in bytes as the driver reports them (hipMemGetInfo). */
 int32_t fth_device_memory_info(uint64_t *free_bytes, uint64_t *total_bytes);
+/* Device memory the GEMM unit holds for split-tile accumulators and transposed operands: `live_bytes` in the blocks in
+ * use (one per stream and purpose, grown geometrically), `retired_bytes` in outgrown blocks that are kept because
+ * queued kernels or a captured graph may still address them (less than `live_bytes` while no single request exceeds
+ * 4 GiB). Either pointer may be NULL. The reference's CPU kernels keep no such state. */
+int32_t fth_device_workspace_info(uint64_t *live_bytes, uint64_t *retired_bytes);
 
 typedef void *fth_stream; /* a hipStream_t; NULL selects the library's own ordered stream */
 typedef void *fth_event;  /* a hipEvent_t */

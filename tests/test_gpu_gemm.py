@@ -89,6 +89,27 @@ def test_gemm_with_a_stored_k_by_m(hip, oracle, m, n, k, dtype):
     assert rel_err(dc3.to_host()[2], oracle.gemm(np.ascontiguousarray(at3[2].T), b)) <= tol
 
 
+def test_gemm_workspace_growth_is_bounded(hip, oracle):
+    """Ragged [k, m] operands go through a transposed copy in a workspace that only grows; an outgrown block is retired
+    (queued kernels or a captured graph may still address it), and because blocks grow geometrically what has been retired
+    stays below what is live. fth_gemm_workspace_info reports both."""
+    live0, ret0 = hip.gemm_workspace_info()
+    for m, k in ((33, 77), (130, 301), (515, 1201), (1030, 4803), (2055, 9607)):
+        n = 24
+        at = synth.uniform(9, "wa", (k, m), -1, 1)
+        b = synth.uniform(9, "wb", (k, n), -1, 1)
+        da, db, dc = DeviceBuffer.from_host(at), DeviceBuffer.from_host(b), DeviceBuffer((m, n))
+        hip.gemm(hip.gemm_desc(m, n, k, trans_a=True), da, db, dc)
+        assert rel_err(dc.to_host(), oracle.gemm(np.ascontiguousarray(at.T), b)) <= TOL_GEMM_F32
+        live, ret = hip.gemm_workspace_info()
+        assert live >= m * k * 4
+        assert ret - ret0 < live, (m, k, live, ret)
+    assert live >= live0 and ret >= ret0
+    again = hip.gemm_workspace_info()
+    hip.gemm(hip.gemm_desc(m, n, k, trans_a=True), da, db, dc)  # a request that fits allocates and retires nothing
+    assert hip.gemm_workspace_info() == again
+
+
 def test_direct_to_lds_kernels_with_row_pitch_and_batches(hip, oracle):
     """Sub-blocks of larger buffers (pitch > row, 16-byte aligned offsets) and a batched problem whose
     tiles straddle workgroup ranges, through the direct kernels."""
