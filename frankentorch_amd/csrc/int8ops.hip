@@ -126,29 +126,43 @@ __device__ __forceinline__ const int8_t *uniform_ptr(const int8_t *ptr) {
 }
 
 constexpr int kBK = 64;     // bytes of K per stage
-constexpr int kStages = 4;  // ring of LDS stages: three loads in flight under one stage of MFMAs
 constexpr int kGroup = 8;   // tiles are walked in kGroup x kGroup squares, one square at a time per XCD
+
+// Calls f(integral_constant<int, 0>{}) ... f(integral_constant<int, N - 1>{}).
+template <int N, int I = 0, typename F> __device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(f);
+    }
+}
 
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
     // s_waitcnt with only the vector-memory counter set: low four bits [3:0], high two bits [15:14]
     __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
-// TW x TW MFMA tiles (32 x 32 each) per wavefront, 2 x 2 wavefronts: a 64 TW x 64 TW output tile per workgroup.
-// TW = 2 (128 x 128, two workgroups per compute unit) suits problems with few tiles; TW = 4 (256 x 256, one workgroup,
-// 256 accumulator registers per lane) halves both the L2 -> LDS traffic and the LDS reads per MFMA. The integer MFMA
+// TWM x TWN MFMA tiles (32 x 32 each) per wavefront, WM x WN wavefronts: a 32 TWM WM x 32 TWN WN output tile per workgroup.
+// (2, 2, 2, 2): 128 x 128, two workgroups per compute unit, for problems with few tiles. (4, 4, 2, 2): 256 x 256 on four
+// wavefronts, one per SIMD, 256 accumulator registers per lane: half the L2 -> LDS traffic and half the LDS reads per MFMA.
+// (4, 2, 2, 4): the same 256 x 256 tile on eight wavefronts of 128 x 64, two per SIMD, so that one wavefront's barrier and
+// load waits are covered by the other's MFMAs (three fragment reads per four MFMAs instead of two). The integer MFMA
 // retires 65 536 operations in 32 cycles, so an LDS-fed loop is bound by fragment reads: measured on this chip with no
-// global traffic at all, one 128-bit read per MFMA (TW = 2) sustains half of the matrix peak, one per two MFMAs (TW = 4)
-// four fifths.
-template <int TW>
-__global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8Args p) {
-    constexpr int BM = 64 * TW, BN = 64 * TW;
+// global traffic at all, one 128-bit read per MFMA sustains half of the matrix peak, one per two MFMAs four fifths.
+// NS: LDS stages in the ring; NS - 1 stages of loads are in flight under one stage of MFMAs (a ring of five, which takes all
+// 160 KiB of the LDS, measured the same as four: 0.372 against 0.374 of the int8 peak at 8192 x 4096 x 4096).
+template <int TWM, int TWN, int WM, int WN, int NS>
+__global__ __launch_bounds__(WM *WN * 64, TWM * TWN * 16 <= 128 ? 2 : 1) void i8_gemm_kernel(const I8Args p) {
+    constexpr int kStages = NS;
+    // (second bound: wavefronts per SIMD the register allocation must allow -- two while the accumulators take at most 128 registers)
+    constexpr int NW = WM * WN, NT = NW * 64;
+    constexpr int BM = 32 * TWM * WM, BN = 32 * TWN * WN;
     constexpr int A_BYTES = BM * kBK, STAGE = (BM + BN) * kBK;
-    constexpr int LD = BM / 64;        // load instructions per operand per wavefront per stage (16 rows each)
-    constexpr int LPS = 2 * LD;        // load instructions per stage per wavefront
+    constexpr int LDA = BM / 16 / NW, LDB = BN / 16 / NW;  // load instructions per operand per wavefront per stage (16 rows each)
+    constexpr int LPS = LDA + LDB;                         // load instructions per stage per wavefront
+    static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "a wavefront loads whole 16-row pieces of each operand");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];  // [kStages][A | B]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;  // 2 x 2 wavefronts
+    const int wm = wave / WN, wn = wave % WN;
     // Workgroup ids go round-robin over the 8 XCDs. Each XCD takes a contiguous run of the tile sequence, and the
     // sequence walks kGroup x kGroup squares of tiles, so the workgroups resident on one XCD at a time share a few
     // row panels of A and of B through that XCD's L2.
@@ -178,33 +192,38 @@ __global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8A
     // checks that this fits 32 bits). Rows past the end repeat the last row; their results are not stored.
     const int64_t a_row0 = m0 < p.m ? m0 : p.m - 1, b_row0 = n0 < p.n ? n0 : p.n - 1;
     const int8_t *a_base = uniform_ptr(p.a + a_row0 * p.k), *b_base = uniform_ptr(p.b + b_row0 * p.k);
-    unsigned a_off[LD], b_off[LD];
+    unsigned a_off[LDA], b_off[LDB];
 #pragma unroll
-    for (int i = 0; i < LD; ++i) {
-        const int r = wave * (16 * LD) + i * 16 + lrow;  // row inside the tile
-        const int q = lslot ^ ((r >> 2) & 3);            // the logical slot that lives at physical slot lslot
-        int64_t ar = m0 + r, br = n0 + r;
+    for (int i = 0; i < LDA; ++i) {
+        const int r = wave * (16 * LDA) + i * 16 + lrow;  // row inside the tile
+        const int q = lslot ^ ((r >> 2) & 3);             // the logical slot that lives at physical slot lslot
+        int64_t ar = m0 + r;
         ar = ar < p.m ? ar : p.m - 1;
-        br = br < p.n ? br : p.n - 1;
         a_off[i] = (unsigned)((ar - a_row0) * p.k) + (unsigned)q * 16u;
+    }
+#pragma unroll
+    for (int i = 0; i < LDB; ++i) {
+        const int r = wave * (16 * LDB) + i * 16 + lrow;
+        const int q = lslot ^ ((r >> 2) & 3);
+        int64_t br = n0 + r;
+        br = br < p.n ? br : p.n - 1;
         b_off[i] = (unsigned)((br - b_row0) * p.k) + (unsigned)q * 16u;
     }
     const int num_kt = (int)(p.k / kBK);
     auto issue = [&](int kt) __attribute__((always_inline)) {
-        const unsigned base = lds0 + (unsigned)(kt % kStages) * STAGE + wave_u * (LD * 1024u);
+        const unsigned base = lds0 + (unsigned)(kt % kStages) * STAGE;
         const int8_t *ak = a_base + (int64_t)kt * kBK, *bk = b_base + (int64_t)kt * kBK;  // scalar arithmetic
 #pragma unroll
-        for (int i = 0; i < LD; ++i) {
-            load_to_lds_16(ak, a_off[i], base + i * 1024u);
-            load_to_lds_16(bk, b_off[i], base + A_BYTES + i * 1024u);
-        }
+        for (int i = 0; i < LDA; ++i) load_to_lds_16(ak, a_off[i], base + wave_u * (LDA * 1024u) + i * 1024u);
+#pragma unroll
+        for (int i = 0; i < LDB; ++i) load_to_lds_16(bk, b_off[i], base + A_BYTES + wave_u * (LDB * 1024u) + i * 1024u);
     };
 
-    V16i acc[TW][TW];
+    V16i acc[TWM][TWN];
 #pragma unroll
-    for (int i = 0; i < TW; ++i)
+    for (int i = 0; i < TWM; ++i)
 #pragma unroll
-        for (int j = 0; j < TW; ++j)
+        for (int j = 0; j < TWN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
@@ -221,30 +240,30 @@ __global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8A
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
         const unsigned slot = ((unsigned)(ks * 2 + kg) ^ swz) << 4;
-        fa[ks] = (unsigned)(wm * (32 * TW) + frow) * kBK + slot;
-        fb[ks] = (unsigned)A_BYTES + (unsigned)(wn * (32 * TW) + frow) * kBK + slot;
+        fa[ks] = (unsigned)(wm * (32 * TWM) + frow) * kBK + slot;
+        fb[ks] = (unsigned)A_BYTES + (unsigned)(wn * (32 * TWN) + frow) * kBK + slot;
     }
-    V4i af[2][TW], bf[2][TW];  // fragment registers of the two 32-byte K steps of a stage
+    V4i af[2][TWM], bf[2][TWN];  // fragment registers of the two 32-byte K steps of a stage
     auto fetch = [&](auto stage_c, int ks) __attribute__((always_inline)) {
         constexpr int stage = decltype(stage_c)::value;
         const unsigned char *base = smem + stage * STAGE;
 #pragma unroll
-        for (int i = 0; i < TW; ++i) {
-            af[ks][i] = *reinterpret_cast<const V4i *>(base + fa[ks] + i * 32 * kBK);
-            bf[ks][i] = *reinterpret_cast<const V4i *>(base + fb[ks] + i * 32 * kBK);
-        }
+        for (int i = 0; i < TWM; ++i) af[ks][i] = *reinterpret_cast<const V4i *>(base + fa[ks] + i * 32 * kBK);
+#pragma unroll
+        for (int j = 0; j < TWN; ++j) bf[ks][j] = *reinterpret_cast<const V4i *>(base + fb[ks] + j * 32 * kBK);
     };
     auto mma = [&](int ks) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < TW; ++i)
+        for (int i = 0; i < TWM; ++i)
 #pragma unroll
-            for (int j = 0; j < TW; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks][i], bf[ks][j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < TWN; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks][i], bf[ks][j], acc[i][j], 0, 0, 0);
     };
     // Stage s has landed for everybody once each wavefront has waited for its own loads of s and passed a barrier.
     auto land = [&](int s_) __attribute__((always_inline)) {
         // loads of the stages after s_ stay in flight: LPS instructions each, at most kStages - 2 stages
         const int younger = num_kt - 1 - s_;
         if (younger >= kStages - 2) wait_vmcnt<(kStages - 2) * LPS>();
+        else if (kStages > 4 && younger == 2) wait_vmcnt<2 * LPS>();
         else if (younger == 1) wait_vmcnt<LPS>();
         else wait_vmcnt<0>();
         __syncthreads();
@@ -260,36 +279,24 @@ __global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8A
     auto step = [&](int kt, auto stage_c) __attribute__((always_inline)) {
         constexpr int stage = decltype(stage_c)::value;
         fetch(stage_c, 1);
-        __builtin_amdgcn_sched_barrier(0);
         mma(0);
-        __builtin_amdgcn_sched_barrier(0);
         land(kt + 1);  // also: every wavefront has finished reading stage kt, whose buffer takes stage kt + kStages
         if (kt + kStages < num_kt) issue(kt + kStages);
         fetch(std::integral_constant<int, (stage + 1) % kStages>{}, 0);
-        __builtin_amdgcn_sched_barrier(0);
         mma(1);
-        __builtin_amdgcn_sched_barrier(0);
     };
-    static_assert(kStages == 4, "the main loop is unrolled over four stages");
+    static_assert(kStages == 4 || kStages == 5, "the wait counts above cover rings of four and five stages");
     int kt = 0;
-    for (; kt + kStages < num_kt; kt += kStages) {
-        step(kt + 0, std::integral_constant<int, 0>{});
-        step(kt + 1, std::integral_constant<int, 1>{});
-        step(kt + 2, std::integral_constant<int, 2>{});
-        step(kt + 3, std::integral_constant<int, 3>{});
-    }
-    // one to four stages are left (kt is a multiple of four): all but the last as steps, then the last one's second half
+    for (; kt + kStages < num_kt; kt += kStages)
+        static_for<kStages>([&](auto S) __attribute__((always_inline)) { step(kt + decltype(S)::value, S); });
+    // one to kStages stages are left (kt is a multiple of kStages): all but the last as steps, then the last one's second half
     const int left = num_kt - kt;
-    if (left > 1) step(kt + 0, std::integral_constant<int, 0>{});
-    if (left > 2) step(kt + 1, std::integral_constant<int, 1>{});
-    if (left > 3) step(kt + 2, std::integral_constant<int, 2>{});
-    switch (left) {
-        case 1: fetch(std::integral_constant<int, 0>{}, 1); break;
-        case 2: fetch(std::integral_constant<int, 1>{}, 1); break;
-        case 3: fetch(std::integral_constant<int, 2>{}, 1); break;
-        default: fetch(std::integral_constant<int, 3>{}, 1); break;
-    }
-    __builtin_amdgcn_sched_barrier(0);
+    static_for<kStages - 1>([&](auto S) __attribute__((always_inline)) {
+        if (left > decltype(S)::value + 1) step(kt + decltype(S)::value, S);
+    });
+    static_for<kStages>([&](auto S) __attribute__((always_inline)) {
+        if (left == decltype(S)::value + 1) fetch(S, 1);
+    });
     mma(0);
     mma(1);
 
@@ -298,25 +305,26 @@ __global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8A
     // MFMA tile row.
     __syncthreads();
     float *row_scale = reinterpret_cast<float *>(smem);
-    for (int t = tid; t < BM; t += 256) row_scale[t] = (m0 + t < p.m) ? p.a_scales[m0 + t] : 0.0f;
+    for (int t = tid; t < BM; t += NT) row_scale[t] = (m0 + t < p.m) ? p.a_scales[m0 + t] : 0.0f;
     __syncthreads();
     const bool interior = m0 + BM <= p.m && n0 + BN <= p.n;  // no bounds tests on the common path
     const int64_t ldc = p.n;
     if (interior && p.vec_store) {
         // Interior tiles leave through LDS so that the output goes out in whole rows: in the accumulator a lane holds ONE
         // column, and storing from there writes 128-byte pieces; staged, a wavefront instruction writes 1 KiB of
-        // consecutive columns per row with 128-bit stores. One slab per MFMA tile row i: the 32 rows of both wavefront
-        // rows, 64 x BN floats.
+        // consecutive columns per row with 128-bit stores. One slab per MFMA tile row i: the 32 rows of each wavefront
+        // row, 32 WM x BN floats.
         float *stage = reinterpret_cast<float *>(smem) + BM;  // behind the row scales
         constexpr int V4 = BN / 4;                            // 128-bit vectors per output row
-        constexpr int PASSES = 64 * V4 / 256;
+        constexpr int PASSES = 32 * WM * V4 / NT;
+        static_assert(32 * WM * V4 % NT == 0, "a slab is a whole number of passes");
 #pragma unroll
-        for (int i = 0; i < TW; ++i) {
-            const int lrow0 = wm * (32 * TW) + i * 32 + 4 * kg;  // tile row of accumulator element 0
-            if (i > 0) __syncthreads();                          // the previous slab has been read
+        for (int i = 0; i < TWM; ++i) {
+            const int lrow0 = wm * (32 * TWM) + i * 32 + 4 * kg;  // tile row of accumulator element 0
+            if (i > 0) __syncthreads();                           // the previous slab has been read
 #pragma unroll
-            for (int j = 0; j < TW; ++j) {
-                const int lcol = wn * (32 * TW) + j * 32 + frow;
+            for (int j = 0; j < TWN; ++j) {
+                const int lcol = wn * (32 * TWN) + j * 32 + frow;
                 const float ws = p.b_scales[n0 + lcol];
                 const float bv = p.bias ? p.bias[n0 + lcol] : 0.0f;
 #pragma unroll
@@ -330,9 +338,9 @@ __global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8A
             __syncthreads();
 #pragma unroll
             for (int ps = 0; ps < PASSES; ++ps) {
-                const int f = ps * 256 + tid, srow = f / V4, c4 = f % V4;
+                const int f = ps * NT + tid, srow = f / V4, c4 = f % V4;
                 const float4 v = *reinterpret_cast<const float4 *>(stage + srow * BN + 4 * c4);
-                float *dst = p.c + (m0 + (srow >> 5) * (32 * TW) + i * 32 + (srow & 31)) * ldc + n0 + 4 * c4;
+                float *dst = p.c + (m0 + (srow >> 5) * (32 * TWM) + i * 32 + (srow & 31)) * ldc + n0 + 4 * c4;
                 typedef float nat_f4 __attribute__((ext_vector_type(4)));
                 nat_f4 nv = {v.x, v.y, v.z, v.w};
                 __builtin_nontemporal_store(nv, reinterpret_cast<nat_f4 *>(dst));
@@ -341,14 +349,14 @@ __global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8A
         return;
     }
 #pragma unroll
-    for (int i = 0; i < TW; ++i) {
-        const int lrow0 = wm * (32 * TW) + i * 32 + 4 * kg;  // tile row of accumulator element 0
+    for (int i = 0; i < TWM; ++i) {
+        const int lrow0 = wm * (32 * TWM) + i * 32 + 4 * kg;  // tile row of accumulator element 0
         float as_[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) as_[r] = row_scale[lrow0 + 8 * (r >> 2) + (r & 3)];
 #pragma unroll
-        for (int j = 0; j < TW; ++j) {
-            const int64_t col = n0 + wn * (32 * TW) + j * 32 + frow;
+        for (int j = 0; j < TWN; ++j) {
+            const int64_t col = n0 + wn * (32 * TWN) + j * 32 + frow;
             if (!interior && col >= p.n) continue;
             const float ws = p.b_scales[col];
             const float bv = p.bias ? p.bias[col] : 0.0f;
@@ -366,17 +374,18 @@ __global__ __launch_bounds__(256, TW == 2 ? 2 : 1) void i8_gemm_kernel(const I8A
     }
 }
 
-template <int TW> int32_t launch_i8_gemm(I8Args &p, hipStream_t st) {
-    constexpr int BM = 64 * TW;
-    constexpr size_t smem = (size_t)kStages * 2 * BM * kBK;  // 64 KiB (two workgroups per compute unit) or 128 KiB (one)
+template <int TWM, int TWN, int WM, int WN, int NS = 4> int32_t launch_i8_gemm(I8Args &p, hipStream_t st) {
+    constexpr int BM = 32 * TWM * WM, BN = 32 * TWN * WN;
+    constexpr size_t smem = (size_t)NS * (BM + BN) * kBK;  // 64 KiB (two workgroups per compute unit), 128 or 160 KiB (one)
     p.tiles_m = (int)fth::ceil_div(p.m, BM);
-    p.tiles_n = (int)fth::ceil_div(p.n, BM);
+    p.tiles_n = (int)fth::ceil_div(p.n, BN);
     static bool attr_set = false;
     if (!attr_set) {
-        FTH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(i8_gemm_kernel<TW>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        FTH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(i8_gemm_kernel<TWM, TWN, WM, WN, NS>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem));
         attr_set = true;
     }
-    i8_gemm_kernel<TW><<<dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(256), smem, st>>>(p);
+    i8_gemm_kernel<TWM, TWN, WM, WN, NS><<<dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(WM * WN * 64), smem, st>>>(p);
     FTH_CHECK_LAUNCH("i8_gemm");
     return FTH_OK;
 }
@@ -446,11 +455,15 @@ int32_t fth_dev_linear_int8_prequantized_f32(const int8_t *x_i8, const float *a_
         // and compute unit in this access pattern) is what bounds the 128 x 128 loop. The choice depends on the shape only.
         const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
         static const int forced = [] {
-            const char *e = std::getenv("FT_HIP_I8_TILE");  // tuning knob: 128 or 256; anything else = automatic
+            const char *e = std::getenv("FT_HIP_I8_TILE");  // tuning knob: 128, 256 (four wavefronts) or 512 (256 x 256 on eight); else automatic
             return e ? std::atoi(e) : 0;
         }();
-        const bool big = forced == 256 || (forced != 128 && tiles256 >= cus && k >= 2048);
-        if (int32_t rc = big ? launch_i8_gemm<4>(p, st) : launch_i8_gemm<2>(p, st)) return rc;
+        const bool big = forced == 256 || forced == 512 || (forced != 128 && tiles256 >= cus && k >= 2048);
+        int32_t rc;
+        if (!big) rc = launch_i8_gemm<2, 2, 2, 2>(p, st);
+        else if (forced == 256) rc = launch_i8_gemm<4, 4, 2, 2>(p, st);  // four wavefronts of 128 x 128 (kept for comparison)
+        else rc = launch_i8_gemm<4, 2, 2, 4>(p, st);                     // eight wavefronts of 128 x 64, two per SIMD
+        if (rc) return rc;
     } else {
         int64_t total;
         FTH_ARG(!__builtin_mul_overflow(m, n, &total) && fth::ceil_div(total, 256) <= 2147483647LL, "linear_int8: output too large for one launch");

@@ -75,6 +75,35 @@ def test_log_softmax_golden_bits_and_specials(hip, oracle, vectors):
     assert rel_err(got[fin], ref[fin]) <= TOL_ROW_F32
 
 
+@pytest.mark.parametrize("cols", [1, 63, 64, 1000, 1025, 24577, 50257])
+@pytest.mark.parametrize("in_off,out_off", [(1, 1), (3, 2), (0, 63), (5, 0)])
+def test_resident_rows_at_odd_element_offsets(hip, oracle, cols, in_off, out_off):
+    """Rows that start anywhere (operands at odd element offsets inside larger buffers, input and output aligned differently):
+    log-softmax, softmax and the loss gradient write exactly their rows -- the elements in front of the first row, between
+    the output's end and the buffer's end, stay as they were -- and match the checker."""
+    rows = 5
+    x = synth.normal(31, "x", (rows, cols)) * np.float32(2.5)
+    pad = 70
+    xin = np.full(rows * cols + 2 * pad, 7.0, np.float32)
+    xin[in_off:in_off + rows * cols] = x.ravel()
+    dxin = DeviceBuffer.from_host(xin)
+    guard = np.float32(-123.25)
+
+    def run(fn, ref):
+        dout = DeviceBuffer.from_host(np.full(rows * cols + 2 * pad, guard, np.float32))
+        fn(dxin.view(in_off), dout.view(out_off))
+        got = dout.to_host()
+        assert np.all(got[:out_off] == guard) and np.all(got[out_off + rows * cols:] == guard)
+        assert rel_err(got[out_off:out_off + rows * cols].reshape(rows, cols), ref) <= TOL_ROW_F32
+
+    run(lambda a, b: hip.log_softmax_strided(a, b, rows, cols, 1), oracle.log_softmax(x, 1))
+    run(lambda a, b: hip.softmax_lastdim(a, b, rows, cols), oracle.softmax(x, 1))
+    target = _targets(31, rows, cols)
+    dloss = synth.normal(31, "dloss", (rows,))
+    dt, dg = DeviceBuffer.from_host(target), DeviceBuffer.from_host(dloss)
+    run(lambda a, b: hip.cross_entropy_backward(a, dt, dg, rows, cols, b), oracle.cross_entropy_backward(x, target, dloss))
+
+
 def test_log_softmax_empty_is_a_no_op(hip):
     d = DeviceBuffer((4,))
     hip.log_softmax_strided(d, d, 0, 4, 1)
