@@ -113,12 +113,24 @@ __device__ __forceinline__ float f4_get(const float4 &v, int e) { return e == 0 
 // past seq_k are clamped to the last row (their scores are masked, their weights are zero).
 // MASK: an additive mask row is read for every (query, key) score, mask[bh * mask_bh_stride + qi * seq_k + key]
 // (sdpa_forward_masked_f64, crates/ft-kernel-cpu/src/lib.rs:4661-4741): score * scale + mask, then the same softmax.
-template <int D, int NW, bool PAIR, int BC, bool DIRECT, bool MASK, int MINW = 2>
+// KSPLIT (causal balancing for launches that are resident all at once; needs PAIR, four wavefronts, 64-key tiles, the direct
+// layout and no mask): the block owns 64 queries per pass and its wavefronts are (query half, key half) -- wavefront w takes
+// queries 32 (w % 2) .. and the 32-key sub-tile w / 2 of every tile -- so with the (long, short) pairing every wavefront of
+// every block does the same number of sub-tiles and no wavefront is left alone on its SIMD at the end (a lone wavefront's
+// score -> softmax -> output chain keeps the matrix unit about 0.6 busy). The two key halves of a query wavefront are merged
+// through LDS after the tile loop, in fixed order. K is single-buffered here (the next K tile is requested behind a barrier
+// that follows the score MFMAs and lands under the softmax and the output MFMAs), V double-buffered: 48 KiB per block,
+// three blocks per compute unit.
+template <int D, int NW, bool PAIR, int BC, bool DIRECT, bool MASK, int MINW = 2, bool KSPLIT = false>
 __global__ __launch_bounds__(64 * NW, MINW) void sdpa_mfma_kernel(const SdpaArgs p) {
     constexpr int kBC = BC;
     constexpr int KS = BC / 32;        // 32-key sub-tiles per tile
+    constexpr int KSW = KSPLIT ? 1 : KS;  // sub-tiles a wavefront multiplies per tile
     constexpr int NTH = 64 * NW;
-    constexpr int BQ = 32 * NW;
+    constexpr int QWV = KSPLIT ? NW / 2 : NW;  // wavefronts along the queries
+    constexpr int BQ = 32 * QWV;
+    constexpr int KBUFS = KSPLIT ? 1 : 2;
+    static_assert(!KSPLIT || (PAIR && NW == 4 && BC == 64 && DIRECT && !MASK), "key split: see the conditions above");
     constexpr int NDT = D / 32;        // 32-wide d-tiles of the output
     constexpr int KP = DIRECT ? D : D + 4;  // K tile row pitch (padded: odd number of 16-byte vectors)
     constexpr int VP = DIRECT ? D : D + 8;  // V tile row pitch (padded: rows j and j+4 land 32 banks apart)
@@ -130,12 +142,14 @@ __global__ __launch_bounds__(64 * NW, MINW) void sdpa_mfma_kernel(const SdpaArgs
     using VV = typename VecN<NDT>::type;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    float *Ks = reinterpret_cast<float *>(smem_raw);  // [2][kBC][KP]
-    float *Vs = Ks + 2 * KT;                          // [2][kBC][VP]
+    float *Ks = reinterpret_cast<float *>(smem_raw);  // [KBUFS][kBC][KP]
+    float *Vs = Ks + KBUFS * KT;                      // [2][kBC][VP]
 
     const fth_sdpa_desc &d = p.d;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lq = lane & 31, half = lane >> 5;
+    const int qw = KSPLIT ? (wave & (QWV - 1)) : wave;  // which 32 queries of the block
+    const int ksp = KSPLIT ? wave / QWV : 0;             // which 32-key half of each tile
 
     // ---- which (bh, unit): a unit is a query block, or a (heavy, light) pair of them ----
     const int units = PAIR ? (p.q_blocks + 1) / 2 : p.q_blocks;
@@ -174,7 +188,7 @@ __global__ __launch_bounds__(64 * NW, MINW) void sdpa_mfma_kernel(const SdpaArgs
         const int qb = pass == 0 ? qb_first : unit;
         // Row indices inside one head fit 32 bits (the launcher checks seq_q, seq_k < 2^31).
         const int q_blk0 = qb * BQ;
-        const int q_wave0 = q_blk0 + wave * 32;
+        const int q_wave0 = q_blk0 + qw * 32;
         const int qi = q_wave0 + lq;  // this lane's query
         const int seq_q_i = (int)d.seq_q;
         const bool q_live = qi < seq_q_i;
@@ -222,17 +236,19 @@ __global__ __launch_bounds__(64 * NW, MINW) void sdpa_mfma_kernel(const SdpaArgs
                 v_off[ci] = (unsigned)trow * (unsigned)d.v_row_stride * 4u + 16u * (unsigned)slot;
             }
         }
-        auto issue_tile = [&](int kt, int buf) __attribute__((always_inline)) {
+        // (WANT_K / WANT_V: the key-split variant requests the two tiles at different points of a step)
+        auto issue_part = [&](int kt, int buf, auto want_k, auto want_v) __attribute__((always_inline)) {
+            constexpr bool WANT_K = decltype(want_k)::value, WANT_V = decltype(want_v)::value;
             if constexpr (DIRECT) {
                 const int row_t0 = kt * kBC;
                 const float *kb = K + (int64_t)row_t0 * d.k_row_stride, *vb = Vg + (int64_t)row_t0 * d.v_row_stride;  // uniform
-                const unsigned kdst = lds0 + (unsigned)(buf * KT * 4) + wave_u * (CPW * 1024u);
-                const unsigned vdst = lds0 + (unsigned)((2 * KT + buf * VT) * 4) + wave_u * (CPW * 1024u);
+                const unsigned kdst = lds0 + (unsigned)((KBUFS == 2 ? buf : 0) * KT * 4) + wave_u * (CPW * 1024u);
+                const unsigned vdst = lds0 + (unsigned)((KBUFS * KT + buf * VT) * 4) + wave_u * (CPW * 1024u);
                 if (row_t0 + kBC <= seq_k_i) {
 #pragma unroll
                     for (int ci = 0; ci < CPW; ++ci) {
-                        load_to_lds_16(kb, k_off[ci], kdst + ci * 1024u);
-                        load_to_lds_16(vb, v_off[ci], vdst + ci * 1024u);
+                        if constexpr (WANT_K) load_to_lds_16(kb, k_off[ci], kdst + ci * 1024u);
+                        if constexpr (WANT_V) load_to_lds_16(vb, v_off[ci], vdst + ci * 1024u);
                     }
                 } else {  // the last, partial tile: rows past the end re-read the last row (their scores are masked)
 #pragma unroll
@@ -241,12 +257,15 @@ __global__ __launch_bounds__(64 * NW, MINW) void sdpa_mfma_kernel(const SdpaArgs
                         const int slot = lane % VPR;
                         const int kq = (slot & ~15) | ((slot ^ trow) & 15);
                         const int crow = row_t0 + trow < seq_k_i ? trow : seq_k_i - 1 - row_t0;
-                        load_to_lds_16(kb, (unsigned)crow * (unsigned)d.k_row_stride * 4u + 16u * (unsigned)kq, kdst + ci * 1024u);
-                        load_to_lds_16(vb, (unsigned)crow * (unsigned)d.v_row_stride * 4u + 16u * (unsigned)slot, vdst + ci * 1024u);
+                        if constexpr (WANT_K)
+                            load_to_lds_16(kb, (unsigned)crow * (unsigned)d.k_row_stride * 4u + 16u * (unsigned)kq, kdst + ci * 1024u);
+                        if constexpr (WANT_V)
+                            load_to_lds_16(vb, (unsigned)crow * (unsigned)d.v_row_stride * 4u + 16u * (unsigned)slot, vdst + ci * 1024u);
                     }
                 }
             }
         };
+        auto issue_tile = [&](int kt, int buf) __attribute__((always_inline)) { issue_part(kt, buf, std::true_type{}, std::true_type{}); };
         auto load_tile = [&](int kt) {
             if constexpr (DIRECT) return;
 #pragma unroll
@@ -295,17 +314,20 @@ __global__ __launch_bounds__(64 * NW, MINW) void sdpa_mfma_kernel(const SdpaArgs
         const float *kfrag[DIRECT ? 8 : 1];
         if constexpr (DIRECT) {
 #pragma unroll
-            for (int u = 0; u < 8; ++u) kfrag[u] = Ks + lq * KP + 4 * (((2 * u) ^ lx) & 15);
+            for (int u = 0; u < 8; ++u) kfrag[u] = Ks + (lq + 32 * ksp) * KP + 4 * (((2 * u) ^ lx) & 15);
         }
         // One tile of the loop; the LDS buffer index is a compile-time constant (the loop below alternates two copies),
         // so every LDS address of a tile is a per-lane base plus an immediate.
         auto tile_step = [&](const int kt, auto buf_c) __attribute__((always_inline)) {
             constexpr int buf = decltype(buf_c)::value;
-            const int key0 = kt * kBC;
+            const int key0 = kt * kBC + 32 * ksp;  // first key of this wavefront's part of the tile
             // The other buffer was released by the barrier that ended the previous tile.
-            if (kt + 1 < num_kt) issue_tile(kt + 1, buf ^ 1);
+            if (kt + 1 < num_kt) {
+                if constexpr (KSPLIT) issue_part(kt + 1, buf ^ 1, std::false_type{}, std::true_type{});
+                else issue_tile(kt + 1, buf ^ 1);
+            }
             // A wavefront whose every query precedes this tile's first key has nothing to add.
-            const bool wave_active = !d.causal || key0 <= wave_last_q;
+            const bool wave_active = (!d.causal || key0 <= wave_last_q) && key0 < seq_k_i;
             // ---- the tile's mask values, requested before the score MFMAs that hide their latency:
             //      lane (query qi) element r of sub-tile j is key key0 + 32 j + 8 (r / 4) + 4 half + r % 4 ----
             Acc16 mk[MASK ? KS : 1];
@@ -334,19 +356,19 @@ __global__ __launch_bounds__(64 * NW, MINW) void sdpa_mfma_kernel(const SdpaArgs
                 }
             }
             // ---- S^T = K_tile . Q^T, one 32-key sub-tile per accumulator ----
-            Acc16 s[KS];
+            Acc16 s[KSW];
             if (wave_active) {
 #pragma unroll
-                for (int j = 0; j < KS; ++j)
+                for (int j = 0; j < KSW; ++j)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) s[j][r] = 0.f;
                 const float *kp = Ks + buf * KT + lq * KP + 4 * half;  // staged layout
 #pragma unroll
                 for (int t = 0; t < D / 8; ++t) {
 #pragma unroll
-                    for (int j = 0; j < KS; ++j) {
+                    for (int j = 0; j < KSW; ++j) {
                         // direct layout: vector 2t + half of row lq sits in slot (2t + half) ^ (lq & 15) = 2t ^ lx
-                        const float4 kv = DIRECT ? *reinterpret_cast<const float4 *>(kfrag[t & 7] + buf * KT + j * 32 * KP + 4 * ((2 * t) & 16))
+                        const float4 kv = DIRECT ? *reinterpret_cast<const float4 *>(kfrag[t & 7] + (KBUFS == 2 ? buf : 0) * KT + j * 32 * KP + 4 * ((2 * t) & 16))
                                                  : *reinterpret_cast<const float4 *>(kp + j * 32 * KP + 8 * t);
                         s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.x, qr[t].x, s[j], 0, 0, 0);
                         s[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.y, qr[t].y, s[j], 0, 0, 0);
@@ -360,11 +382,18 @@ __global__ __launch_bounds__(64 * NW, MINW) void sdpa_mfma_kernel(const SdpaArgs
             // temporaries cannot be handed the registers the score accumulator is about to claim
             // (which makes the compiler wait for every load in flight before the first MFMA).
             if (kt + 1 < num_kt) load_tile(kt + 1);
+            if constexpr (KSPLIT) {
+                // every wavefront has read the one K buffer: the next K tile may land in it (under the softmax and the
+                // output MFMAs; the step's closing wait covers it)
+                __syncthreads();
+                if (kt + 1 < num_kt) issue_part(kt + 1, 0, std::true_type{}, std::false_type{});
+            }
             if (wave_active) {
                 // ---- scale, mask, online softmax (lane-local query) ----
-                const bool need_mask = (d.causal && key0 + kBC - 1 > q_wave0) || (key0 + kBC > seq_k_i);
+                constexpr int kMine = 32 * KSW;  // keys of the tile this wavefront scores
+                const bool need_mask = (d.causal && key0 + kMine - 1 > q_wave0) || (key0 + kMine > seq_k_i);
                 float mt = -__builtin_inff(), m_new, alpha, psum = 0.f;
-                const float *vp = Vs + buf * VT + (4 * half) * VP + NDT * lq;
+                const float *vp = Vs + buf * VT + (4 * half + 32 * ksp) * VP + NDT * lq;
                 if constexpr (!MASK) {
                     // Positive scale (the launcher sends unmasked calls with any other scale to the generic
                     // kernel): the row max is taken on the raw scores (scaling by a positive constant keeps
@@ -372,7 +401,7 @@ __global__ __launch_bounds__(64 * NW, MINW) void sdpa_mfma_kernel(const SdpaArgs
                     // the running max m kept in those log2 units.
                     if (need_mask) {  // wavefront-uniform; selects, no per-element branches
 #pragma unroll
-                        for (int j = 0; j < KS; ++j)
+                        for (int j = 0; j < KSW; ++j)
 #pragma unroll
                             for (int r = 0; r < 16; ++r) {
                                 const int key = key0 + 32 * j + 8 * (r >> 2) + 4 * half + (r & 3);
@@ -381,7 +410,7 @@ __global__ __launch_bounds__(64 * NW, MINW) void sdpa_mfma_kernel(const SdpaArgs
                             }
                     }
 #pragma unroll
-                    for (int j = 0; j < KS; ++j)
+                    for (int j = 0; j < KSW; ++j)
 #pragma unroll
                         for (int r = 0; r < 16; ++r) mt = fmaxf(mt, s[j][r]);
                     // fp32 MFMAs and vector instructions share issue cycles, so the bookkeeping is kept off the common
@@ -404,7 +433,7 @@ __global__ __launch_bounds__(64 * NW, MINW) void sdpa_mfma_kernel(const SdpaArgs
                     const float neg_m = -m_run;
                     // ---- O^T += V_tile^T . P^T with the exponentials in the same instruction stream ----
 #pragma unroll
-                    for (int j = 0; j < KS; ++j)
+                    for (int j = 0; j < KSW; ++j)
 #pragma unroll
                         for (int r = 0; r < 16; ++r) {
                             const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][r], c2, neg_m));
@@ -477,6 +506,34 @@ __global__ __launch_bounds__(64 * NW, MINW) void sdpa_mfma_kernel(const SdpaArgs
             tile_step(kt, std::integral_constant<int, 0>{});
             if (kt + 1 < num_kt) tile_step(kt + 1, std::integral_constant<int, 1>{});
         }
+        if constexpr (KSPLIT) {
+            // ---- merge the two key halves of each query wavefront (fixed order: half 0, then half 1) ----
+            // The tile buffers are free (the loop ends on a barrier). State of key half 1: the accumulators, the reference
+            // m (per query, the same in both lane halves) and the per-lane partial row sum, all relative to m.
+            float *mg = reinterpret_cast<float *>(smem_raw) + qw * ((NDT * 16 + 2) * 64) + lane;
+            if (ksp == 1) {
+#pragma unroll
+                for (int e = 0; e < NDT; ++e)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) mg[(e * 16 + r) * 64] = o[e][r];
+                mg[(NDT * 16) * 64] = m_run;
+                mg[(NDT * 16 + 1) * 64] = l_run;
+            }
+            __syncthreads();
+            if (ksp == 0) {
+                const float m1 = mg[(NDT * 16) * 64], l1 = mg[(NDT * 16 + 1) * 64];
+                const float m = fmaxf(m_run, m1);
+                // a half that saw no key of a query (m = -inf, sums 0) weighs nothing; both empty only when there is no key at all
+                const float a0 = (m_run == -__builtin_inff()) ? 0.f : __builtin_amdgcn_exp2f(m_run - m);
+                const float a1 = (m1 == -__builtin_inff()) ? 0.f : __builtin_amdgcn_exp2f(m1 - m);
+#pragma unroll
+                for (int e = 0; e < NDT; ++e)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) o[e][r] = o[e][r] * a0 + mg[(e * 16 + r) * 64] * a1;
+                l_run = l_run * a0 + l1 * a1;
+            }
+            __syncthreads();  // the merge area is tile memory again in the next pass
+        }
         {  // the two halves of the wavefront hold partial row sums of the same queries
             float llo, lhi;
             both_halves(l_run, llo, lhi);
@@ -484,7 +541,7 @@ __global__ __launch_bounds__(64 * NW, MINW) void sdpa_mfma_kernel(const SdpaArgs
         }
 
         // ---- normalise and store: lane owns query qi, d = NDT * rho + e ----
-        if (q_live) {
+        if (q_live && ksp == 0) {
             float *orow = O + (int64_t)qi * d.o_row_stride;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
@@ -820,18 +877,21 @@ template <int D> int32_t launch_mfma_f64(SdpaArgs &a, hipStream_t st) {
     return FTH_OK;
 }
 
-template <int D, int NW, bool PAIR, bool MASK, bool OCC3 = false> int32_t launch_mfma_cfg(SdpaArgs &a, hipStream_t st) {
-    // 64-key tiles where two workgroups still fit a CU; 32-key tiles (and a register budget for three) where three should
-    constexpr int BC = OCC3 ? 32 : (D <= 64 && (NW == 4 || D <= 32)) ? 64 : 32;
+template <int D, int NW, bool PAIR, bool MASK, bool OCC3 = false, bool KSPLIT = false> int32_t launch_mfma_cfg(SdpaArgs &a, hipStream_t st) {
+    // 64-key tiles where two workgroups still fit a CU; 32-key tiles (and a register budget for three) where three should;
+    // the key-split variant: 64-key tiles, K single-buffered, three per CU
+    constexpr int BC = KSPLIT ? 64 : OCC3 ? 32 : (D <= 64 && (NW == 4 || D <= 32)) ? 64 : 32;
     constexpr bool DIRECT = D >= 64 && FTH_SDPA_DIRECT;
-    constexpr size_t smem = DIRECT ? (size_t)2 * BC * 2 * D * sizeof(float) : (size_t)2 * BC * ((D + 4) + (D + 8)) * sizeof(float);
-    auto kern = sdpa_mfma_kernel<D, NW, PAIR, BC, DIRECT, MASK, OCC3 ? 3 : 2>;
+    constexpr size_t smem = KSPLIT   ? (size_t)3 * BC * D * sizeof(float)
+                            : DIRECT ? (size_t)2 * BC * 2 * D * sizeof(float)
+                                     : (size_t)2 * BC * ((D + 4) + (D + 8)) * sizeof(float);
+    auto kern = sdpa_mfma_kernel<D, NW, PAIR, BC, DIRECT, MASK, OCC3 ? 3 : 2, KSPLIT>;
     static bool attr_set = false;
     if (!attr_set) {
         FTH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    a.q_blocks = (int)fth::ceil_div(a.d.seq_q, 32 * NW);
+    a.q_blocks = (int)fth::ceil_div(a.d.seq_q, KSPLIT ? 16 * NW : 32 * NW);
     const int64_t units = PAIR ? (a.q_blocks + 1) / 2 : a.q_blocks;
     const int64_t grid = a.d.num_bh * units;
     FTH_ARG(grid <= 2147483647LL, "sdpa: grid too large");
@@ -1000,7 +1060,7 @@ template <int D> int32_t launch_mfma(SdpaArgs &a, hipStream_t st) {
     const int64_t wg128 = a.d.num_bh * fth::ceil_div(a.d.seq_q, 128);
     bool wide = D >= 128 || 2 * wg128 >= (int64_t)cus;  // D = 128 staging does not fit 2-wavefront blocks
     static const int forced = [] {
-        const char *e = std::getenv("FT_HIP_SDPA_CFG");  // tuning knob: bit 0 = 4 wavefronts, bit 1 = pairing, bit 2 = 32-key tiles at head size 64; -1 = auto
+        const char *e = std::getenv("FT_HIP_SDPA_CFG");  // tuning knob: bit 0 = 4 wavefronts, bit 1 = pairing, bit 2 = 32-key tiles at head size 64, bit 3 = key-split pairs at head size 64; -1 = auto
         return e ? std::atoi(e) : -1;
     }();
     if (forced >= 0) {
@@ -1012,6 +1072,13 @@ template <int D> int32_t launch_mfma(SdpaArgs &a, hipStream_t st) {
         // fit a compute unit (two of the 64-key ones do): everything is resident at once and the order of
         // fth::snake_order balances the compute units, which heaviest-first issue on two slots cannot (GPT-2's 96 heads
         // x 8 query blocks: the heaviest block alone is 8 of the 6.75 work units per slot).
+        if constexpr (FTH_SDPA_DIRECT) {
+            // More than two and at most three 128-query units per compute unit (GPT-2's 96 heads x S1024: exactly three): the
+            // key-split pairs, every wavefront of every block the same length and all resident at once. Measured there: 126.8 ->
+            // 119.2 us (0.647 -> 0.688 of the fp32 MFMA peak) against the unpaired blocks in the back-and-forth order.
+            const bool split = forced >= 0 ? (forced & 8) != 0 : (wg128 > 2 * (int64_t)cus && wg128 <= 3 * (int64_t)cus);
+            if (split && a.d.causal != 0 && !a.mask) return launch_mfma_cfg<D, 4, true, false, true, true>(a, st);
+        }
         const bool three = forced >= 0 ? (forced & 4) != 0 : (a.d.causal != 0 && wg128 > 2 * (int64_t)cus && wg128 <= 4 * (int64_t)cus);
         if (!a.mask && !pair && wide && three) return launch_mfma_cfg<D, 4, false, false, true>(a, st);
     }
@@ -1057,12 +1124,13 @@ int32_t sdpa_entry(const fth_sdpa_desc *d, double scale, const T *q, const T *k,
         // the unmasked MFMA kernels take the row maximum on the raw scores, which needs a positive scale
         if (strides_ok && d->d_k == d->d_v && d->seq_k > 0 && (masked || scale > T(0))) {
             // Too few 32-query blocks to give every compute unit one: the key-split kernel (one launch, no LDS staging)
-            static const bool small_off = [] {
-                const char *e = std::getenv("FT_HIP_SDPA_SMALL");  // tuning knob: 0 disables the small-problem kernel
-                return e && std::atoi(e) == 0;
+            static const int small_knob = [] {
+                const char *e = std::getenv("FT_HIP_SDPA_SMALL");  // tuning knob: 0 disables the small-problem kernel, 2 forces it
+                return e ? std::atoi(e) : 1;
             }();
+            const bool small_off = small_knob == 0;
             const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
-            if (!masked && !small_off && d->num_bh * fth::ceil_div(d->seq_q, 32) <= cus && d->seq_k <= 4096) {
+            if (!masked && !small_off && (small_knob == 2 || d->num_bh * fth::ceil_div(d->seq_q, 32) <= cus) && d->seq_k <= 4096) {
                 if (d->d_k == 64) return launch_small_sdpa<64>(a, st);  // (128: the merge buffers would exceed 64 KiB of LDS)
                 if (d->d_k == 32) return launch_small_sdpa<32>(a, st);
             }

@@ -127,10 +127,12 @@ def test_config4_full_size_sampled_heads_determinism_and_checksum(hip, oracle):
     assert np.array_equal(out[:, 0], v[:, 0])
 
 
-@pytest.mark.parametrize("bh,seq", [(96, 1024), (64, 1152), (32, 4096)])
+@pytest.mark.parametrize("bh,seq", [(96, 1024), (64, 1152), (70, 1000), (130, 520), (32, 4096)])
 def test_fully_resident_causal_launch_sampled_heads(hip, oracle, bh, seq):
-    """Causal, head size 64, between two and four query blocks per compute unit: every workgroup of the launch is
-    resident at once and the query blocks are handed out in the back-and-forth order (32-key tiles). Sampled
+    """Causal, head size 64, between two and four 128-query units per compute unit: every workgroup of the launch is
+    resident at once. Up to three per unit take the key-split pairs (a long and a short 64-query block per workgroup, each
+    wavefront one key half of every tile, merged through LDS; sequences that are no multiple of 64 and an odd number of
+    blocks among the cases), beyond that the query blocks are handed out in the back-and-forth order (32-key tiles). Sampled
     (batch, head) slices against the oracle, the first row, and bitwise equality of two runs."""
     D = 64
     s = 1.0 / math.sqrt(D)
