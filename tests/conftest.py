@@ -42,7 +42,7 @@ def hip():
 
 
 def rel_err(got, ref):
-    """max|got - ref| / max|ref|, the tolerance form BASELINE.json states."""
+    """max|got - ref| / max|ref|, the tolerance form of the metric definition."""
     got = np.asarray(got, dtype=np.float64)
     ref = np.asarray(ref, dtype=np.float64)
     denom = np.max(np.abs(ref)) if ref.size else 1.0
@@ -51,7 +51,7 @@ def rel_err(got, ref):
     return float(np.max(np.abs(got - ref)) / denom) if ref.size else 0.0
 
 
-# Tolerances of BASELINE.json: fp32 row ops, fp32 GEMM / attention, fp64.
+# Tolerances of the metric definition: fp32 row ops, fp32 GEMM / attention, fp64.
 TOL_ROW_F32 = 1e-5
 TOL_GEMM_F32 = 2e-5
 TOL_F64 = 1e-12
