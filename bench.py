@@ -467,6 +467,8 @@ def bench_backward(device, synth, steps, with_cpu):
          lambda: O.cross_entropy_forward(sample, tgt[:64])),
         ("cross_entropy_backward", 2 * nel + rows * 12, lambda: device.cross_entropy_backward(lg, dtgt, dloss, rows, vocab, lo),
          lambda: O.cross_entropy_backward(sample, tgt[:64], np.ones(64, np.float32))),
+        # softmax over the vocabulary: rows that are no multiple of a 128-bit vector and far beyond 8192 vectors
+        ("softmax_vocab", 2 * nel, lambda: device.softmax_lastdim(lg, lo, rows, vocab), lambda: O.softmax(sample, 1)),
     ):
         ms = timed(fn, max(5, steps // 5))
         gbs = nbytes / (ms * 1e-3) / 1e9
