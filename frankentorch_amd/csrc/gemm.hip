@@ -70,6 +70,10 @@ constexpr int kGroupM = 8;
 #define FTH_F32_MINW 2
 #endif
 
+// Internal epilogue bit (not part of fth_gemm_desc.epilogue): also emit the maximum of every output row over each 32-column
+// piece of the tile (GemmArgs::rowmax). fp32 direct kernel for whole tiles, the fix-up kernel for split ones.
+constexpr int kEpiRowMax = 64;
+
 template <typename T> struct Mfma;
 template <> struct Mfma<float> {
     static constexpr int MT = 32;   // output tile edge
@@ -134,6 +138,9 @@ template <typename T> struct GemmArgs {
     int64_t total_iters;     // batch * tiles_per_batch * ktiles
     T *partials;             // [grid][2][BM * BN] accumulator slots of split tiles
     int grid;                // workgroups of the main kernel (the fix-up kernel needs it too)
+    // Row maxima by column group (kEpiRowMax): [column groups][m], group g = columns [32 g, 32 g + 32), one MFMA tile wide.
+    // NaN = "not known, look at the stored values" (a group with a NaN in it).
+    T *rowmax = nullptr;
 };
 
 // Tile number -> (tile_m, tile_n): groups of kGroupM tile-rows, column-major inside a group.
@@ -464,6 +471,44 @@ template <typename T> __device__ __forceinline__ void load_to_lds_16(const T *ba
                  : "memory", "m0");
 }
 
+// ---- row maxima of an accumulator tile (kEpiRowMax) ----
+// In the 32 x 32 accumulator a lane holds 16 rows of ONE column, so the maximum of a row over the tile's columns is a
+// reduction over the 32 lanes of a wavefront half. It is done as a transposing butterfly: at each step a lane keeps one
+// half of its values and hands the other half to a partner lane, so 8 + 4 + 2 + 1 exchanges (instead of 16 x 4) leave
+// every lane with the maximum, over its 16-lane row, of ONE accumulator row; one exchange with lane ^ 16 completes the 32
+// columns. The partners are lane +- 4 and lane ^ 8 first (data-parallel-primitive row rotations, whose bank mask does the
+// keep / hand-over selection for free), then lane ^ 1 and lane ^ 2 (quad permutations, selection by v_cndmask).
+// The maximum is the NaN-propagating one (v_maximum3_f32): a group with a NaN in it comes out as NaN, which is exactly the
+// "not known, look at the stored values" marker the consumer expects, and +-inf are ordinary values.
+template <int CTRL, int BANKS> __device__ __forceinline__ float dpp_take(float old, float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, x), CTRL, 0xF, BANKS, false));
+}
+__device__ __forceinline__ float nan_max(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+// v[0 .. 16): this lane's 16 accumulator values (element r = row M::acc_row(r, lane)). Returns in every lane the maximum
+// over the 32 lanes of its wavefront half of element rowmax_elem_of_lane(lane).
+__device__ __forceinline__ float rowmax_fold(float (&v)[16], int lane) {
+    constexpr int kRor4 = 0x124, kRor8 = 0x128, kXor1 = 0xB1, kXor2 = 0x4E;  // row_ror:4, row_ror:8, quad_perm [1,0,3,2], [2,3,0,1]
+#pragma unroll
+    for (int k = 0; k < 8; ++k)  // banks 0, 2 (lane bit 2 clear) keep elements 0..7, banks 1, 3 keep 8..15
+        v[k] = nan_max(dpp_take<kRor4, 0x5>(v[k + 8], v[k]), dpp_take<kRor4, 0xA>(v[k], v[k + 8]));
+#pragma unroll
+    for (int k = 0; k < 4; ++k)  // banks 0, 1 (lane bit 3 clear) keep the lower four of those
+        v[k] = nan_max(dpp_take<kRor8, 0x3>(v[k + 4], v[k]), dpp_take<kRor8, 0xC>(v[k], v[k + 4]));
+    const bool up1 = (lane & 1) != 0, up2 = (lane & 2) != 0;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const float keep = up1 ? v[k + 2] : v[k], send = up1 ? v[k] : v[k + 2];
+        v[k] = nan_max(keep, dpp_take<kXor1, 0xF>(send, send));
+    }
+    const float keep = up2 ? v[1] : v[0], send = up2 ? v[0] : v[1];
+    const float m = nan_max(keep, dpp_take<kXor2, 0xF>(send, send));
+    // lane ^ 16 within 32 lanes: and 0x1F, or 0, xor 16
+    return nan_max(m, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, m), (16 << 10) | 0x1F)));
+}
+__device__ __forceinline__ int rowmax_elem_of_lane(int lane) {
+    return ((lane & 4) << 1) | ((lane & 8) >> 1) | ((lane & 1) << 1) | ((lane & 2) >> 1);
+}
+
 // EPI >= 0: the epilogue flags are this compile-time mask and alpha is 1 (straight-line output code);
 // EPI < 0: flags and alpha are read from the arguments.
 // TRANS_A: A is stored [k, m] (its tile is kept [k][m] in LDS and read element-wise, like a [k,n] B).
@@ -515,7 +560,8 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
 #pragma unroll
     for (int kc = 0; kc < NCH; ++kc) roff[kc] = ((kc * KG + lane / MT) ^ swz(lrow)) * EPV;
 
-    const int epi = EPI >= 0 ? EPI : p.epilogue;
+    constexpr bool ROWMAX = EPI >= 0 && (EPI & kEpiRowMax) != 0 && std::is_same<T, float>::value;
+    const int epi = EPI >= 0 ? (EPI & ~kEpiRowMax) : p.epilogue;
     const bool has_bias = (epi & FTH_EPI_BIAS) != 0;
     const bool has_gelu = (epi & FTH_EPI_GELU) != 0;
     const bool has_gelu_tanh = (epi & FTH_EPI_GELU_TANH) != 0;
@@ -710,6 +756,14 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
         if (has_res) v = v + rv;
         return v;
     };
+    // One 32 x 32 piece of a whole tile has been written: the maximum of each of its rows, one value per row from the
+    // lanes that hold it after the fold.
+    auto rowmax_emit = [&](float (&v)[16], int i, int j, int64_t m0_, int64_t n0_) __attribute__((always_inline)) {
+        const float mine = rowmax_fold(v, lane);
+        const int64_t row = m0_ + wm0 + i * MT + M::acc_row(rowmax_elem_of_lane(lane), lane);
+        const int64_t group = (n0_ + wn0 + j * MT) / MT;
+        if (lrow < 16 && row < p.m) p.rowmax[group * p.m + row] = mine;
+    };
     auto out_store = [&](auto S, auto &src, bool full, int64_t m0_, int64_t n0_, int64_t batch_, T *slot_) __attribute__((always_inline)) {
         constexpr int sidx = decltype(S)::value;
         if (full) {
@@ -718,6 +772,14 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
             for (int u = 0; u < TILES_PP; ++u) {
                 const int t = sidx * TILES_PP + u, i = t / TN, j = t % TN;
                 const int64_t col = n0_ + wn0 + j * MT + lrow;
+                float seen[ROWMAX ? 16 : 1];  // the values written, -inf where this lane wrote none
+                if constexpr (ROWMAX) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) seen[r] = -__builtin_inff();
+                }
+                auto note = [&](int r, T val) __attribute__((always_inline)) {
+                    if constexpr (ROWMAX) seen[r] = (float)val;
+                };
                 if (interior) {
                     const int64_t tile_off = batch_ * p.stride_c + (m0_ + wm0 + i * MT) * p.ldc + (n0_ + wn0 + j * MT);
                     T *cb = p.c + tile_off;
@@ -726,7 +788,9 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
                     for (int r = 0; r < M::ACC; ++r) {
                         const int64_t row_off = (int64_t)M::acc_row(r, 0) * p.ldc;
                         const T rv = !has_res ? T(0) : DEFER ? res[u][r] : (p.residual + tile_off + row_off)[lane_off];
-                        (cb + row_off)[lane_off] = finish(src[i][j][r], bv, rv);
+                        const T val = finish(src[i][j][r], bv, rv);
+                        (cb + row_off)[lane_off] = val;
+                        note(r, val);
                     }
                 } else if (col < p.n) {
                     T *C = p.c + batch_ * p.stride_c;
@@ -736,10 +800,13 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
                         const int64_t row = m0_ + wm0 + i * MT + M::acc_row(r, lane);
                         if (row < p.m) {
                             const T rv = !has_res ? T(0) : DEFER ? res[u][r] : p.residual[batch_ * p.stride_c + row * p.ldc + col];
-                            C[row * p.ldc + col] = finish(src[i][j][r], bv, rv);
+                            const T val = finish(src[i][j][r], bv, rv);
+                            C[row * p.ldc + col] = val;
+                            note(r, val);
                         }
                     }
                 }
+                if constexpr (ROWMAX) rowmax_emit(seen, i, j, m0_, n0_);
             }
         } else {
 #pragma unroll
@@ -943,6 +1010,14 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemm_fixup_kernel(const GemmArg
     tile_of_id(tile - batch * p.tiles_per_batch, p.tiles_m, p.tiles_n, tile_m, tile_n);
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
     T *C = p.c + batch * p.stride_c;
+    // Row maxima (GemmArgs::rowmax) of a split tile: this workgroup's share is exactly one 32 x 32 piece (all 16 values a
+    // lane holds of it), in the main kernel's lane layout, so the same fold applies.
+    constexpr bool ROWMAX = std::is_same<T, float>::value && PV == M::ACC && M::ACC == 16;
+    float seen[ROWMAX ? 16 : 1];
+    if constexpr (ROWMAX) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) seen[r] = -__builtin_inff();
+    }
     const bool has_bias = (p.epilogue & FTH_EPI_BIAS) != 0;
     const bool has_gelu = (p.epilogue & FTH_EPI_GELU) != 0;
     const bool has_gelu_tanh = (p.epilogue & FTH_EPI_GELU_TANH) != 0;
@@ -961,6 +1036,16 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemm_fixup_kernel(const GemmArg
             if (has_gelu_tanh) v = M::gelu_tanh(v);
             if (has_res) v = v + p.residual[batch * p.stride_c + row * p.ldc + col];
             C[row * p.ldc + col] = v;
+            if constexpr (ROWMAX) seen[u] = (float)v;
+        }
+    }
+    if constexpr (ROWMAX) {
+        if (p.rowmax != nullptr) {  // uniform: every lane takes part in the fold
+            const int j = (int)blockIdx.y % TN, i = (int)blockIdx.y / TN;
+            const float mine = rowmax_fold(seen, lane);
+            const int64_t row = m0 + wm0 + i * MT + M::acc_row(rowmax_elem_of_lane(lane), lane);
+            const int64_t group = (n0 + wn0 + j * MT) / MT;
+            if (lrow < 16 && row < p.m) p.rowmax[group * p.m + row] = (T)mine;
         }
     }
 }
@@ -1454,6 +1539,34 @@ int32_t gemm_entry(const fth_gemm_desc *d, T alpha, const T *a, const T *b, T *c
     return vecb ? launch_shape<T, false, false, true>(p, d->batch, st) : launch_shape<T, false, false, false>(p, d->batch, st);
 }
 
+// C = A . B^T (A [m, k], B [n, k], both row-major and contiguous) on 128 x 128 tiles with the row maxima of every 32-column
+// group as a by-product (GemmArgs::rowmax). Returns false, with nothing launched, where the direct-to-LDS kernel or the
+// large tiles do not apply.
+bool launch_nt_rowmax(int64_t m, int64_t n, int64_t k, const float *a, const float *b, float *c, float *rowmax, hipStream_t st, int32_t *rc) {
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    const int64_t lim = ((int64_t)1 << 32) / (128 * (int64_t)sizeof(float)) - 128;
+    const int cus = fth::compute_units() > 0 ? fth::compute_units() : 256;
+    const int64_t big_tiles = fth::ceil_div(m, 128) * fth::ceil_div(n, 128);
+    static const bool direct_off = [] {
+        const char *e = std::getenv("FT_HIP_GEMM_DIRECT");
+        return e && std::atoi(e) == 0;
+    }();
+    if (direct_off || m <= 0 || n <= 0 || k <= 0 || k % 32 != 0 || !al(a) || !al(b) || k > lim || n > lim || big_tiles < cus || forced_tile() > 0)
+        return false;
+    GemmArgs<float> p;
+    p.a = a; p.b = b; p.c = c; p.bias = nullptr; p.residual = nullptr;
+    p.m = m; p.n = n; p.k = k;
+    p.lda = k; p.ldb = k; p.ldc = n;
+    p.stride_a = m * k; p.stride_b = n * k; p.stride_c = m * n;
+    p.alpha = 1.f;
+    p.use_alpha = 0;
+    p.epilogue = 0;
+    p.tiles_m = p.tiles_n = 0;
+    p.rowmax = rowmax;
+    *rc = launch_direct_epi<float, 128, 128, 2, 2, 2, false, true, kEpiRowMax>(p, 1, st);
+    return true;
+}
+
 template <typename T> int32_t launch_trans_a(GemmArgs<T> &p, const fth_gemm_desc *d, hipStream_t st) {
     constexpr int EPV = Mfma<T>::EPV;
     constexpr int64_t DBK = 128 / (int64_t)sizeof(T);
@@ -1488,7 +1601,48 @@ template <typename T> int32_t launch_trans_a(GemmArgs<T> &p, const fth_gemm_desc
 
 }  // namespace
 
+namespace fth {
+int64_t gemm_rowmax_groups(int64_t n) { return fth::ceil_div(n, 128) * 4; }
+bool gemm_f32_nt_rowmax(int64_t m, int64_t n, int64_t k, const float *a, const float *b, float *c, float *rowmax, hipStream_t st,
+                        int32_t *rc) {
+    return launch_nt_rowmax(m, n, k, a, b, c, rowmax, st, rc);
+}
+}  // namespace fth
+
 extern "C" {
+
+int64_t fth_dev_linear_argmax_workspace_floats(int64_t rows, int64_t out_features) {
+    if (rows <= 0 || out_features <= 0) return 0;
+    return rows * fth::gemm_rowmax_groups(out_features);
+}
+
+int32_t fth_dev_linear_argmax_f32(const float *x, const float *w, int64_t rows, int64_t out_features, int64_t in_features,
+                                  float *logits, float *argmax, float *workspace, int64_t workspace_floats, fth_stream s) {
+    FTH_REQUIRE_DEVICE();
+    FTH_ARG(rows >= 0 && out_features >= 0 && in_features >= 0, "linear_argmax: negative extent");
+    if (rows == 0) return FTH_OK;
+    FTH_ARG(out_features > 0, "linear_argmax: argmax over an empty dimension");
+    FTH_ARG(x && w && logits && argmax, "linear_argmax: NULL operand");
+    hipStream_t st = fth::resolve_stream(s);
+    static const bool fused_off = [] {
+        const char *e = std::getenv("FT_HIP_LINEAR_ARGMAX_FUSED");  // tuning knob: 0 = always the two separate kernels
+        return e && std::atoi(e) == 0;
+    }();
+    if (!fused_off && workspace && workspace_floats >= fth_dev_linear_argmax_workspace_floats(rows, out_features)) {
+        int32_t rc = FTH_OK;
+        if (fth::gemm_f32_nt_rowmax(rows, out_features, in_features, x, w, logits, workspace, st, &rc)) {
+            if (rc) return rc;
+            return fth::argmax_from_group_max(logits, rows, out_features, workspace, fth::gemm_rowmax_groups(out_features), argmax, st);
+        }
+    }
+    fth_gemm_desc gd{};
+    gd.m = rows; gd.n = out_features; gd.k = in_features; gd.batch = 1;
+    gd.lda = in_features; gd.ldb = in_features; gd.ldc = out_features;
+    gd.trans_b = 1;
+    gd.epilogue = FTH_EPI_NONE;
+    if (int32_t rc = fth_dev_gemm_f32(&gd, 1.f, x, w, logits, nullptr, nullptr, s)) return rc;
+    return fth_dev_argmax_f32(logits, rows, out_features, 1, argmax, s);
+}
 
 int32_t fth_device_workspace_info(uint64_t *live_bytes, uint64_t *retired_bytes) {
     WorkspaceTable &t = workspace_table();

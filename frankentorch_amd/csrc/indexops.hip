@@ -197,6 +197,90 @@ __global__ __launch_bounds__(kBlock) void argmax_lastdim_kernel(const T *__restr
     }
 }
 
+// ---- argmax from the row maxima of column groups ----------------------------------------------
+// gmax[g * rows + row] is the maximum of row `row` over columns [32 g, 32 g + 32), written by the product that made the
+// logits, or NaN where that is not known (the group holds a NaN). A row's
+// argmax is then the first element equal to the largest group maximum, in the first group that attains it -- found by
+// reading that one group -- after the unknown groups have been scanned element by element with the rule of
+// argmax_lastdim_kernel (first strict maximum; the first NaN wins), whose answer this reproduces bit for bit: a known group
+// holds no NaN, its maximum is an element of it, and ties go to the earlier column either way. A workgroup takes 32
+// consecutive rows (their group maxima are one 128-byte segment) and deals the groups, in column order, to 32 slices whose
+// candidates are merged in that order.
+constexpr int kGroupCols = 32;
+constexpr int kGroupRows = 32;    // rows per workgroup: one per lane of a half wavefront
+constexpr int kGroupSlices = 32;  // column slices per workgroup (1024 threads)
+__global__ __launch_bounds__(kGroupRows * kGroupSlices) void argmax_group_kernel(const float *__restrict__ logits, int64_t rows, int64_t cols,
+                                                                                  const float *__restrict__ gmax, int groups,
+                                                                                  float *__restrict__ out) {
+    __shared__ float s_val[kGroupSlices][kGroupRows];
+    __shared__ int64_t s_idx[kGroupSlices][kGroupRows], s_nan[kGroupSlices][kGroupRows];
+    __shared__ int s_grp[kGroupSlices][kGroupRows];
+    const int lr = threadIdx.x % kGroupRows, slice = threadIdx.x / kGroupRows;
+    const int64_t row = (int64_t)blockIdx.x * kGroupRows + lr;
+    const bool live = row < rows;
+    const int per = (groups + kGroupSlices - 1) / kGroupSlices;
+    const int g0 = slice * per, g1 = g0 + per < groups ? g0 + per : groups;
+    float val = -__builtin_inff();
+    int64_t idx = 0, nan_idx = kNoNan;
+    int grp = -1;  // >= 0: idx is only the group's first column, the element is still to be found
+    const float *xr = logits + (live ? row : 0) * cols;
+    if (live) {
+        constexpr int kBatch = 8;  // group maxima fetched together: the loop is bound by memory latency, not by its arithmetic
+        for (int gb = g0; gb < g1; gb += kBatch) {
+            float mv[kBatch];
+#pragma unroll
+            for (int q = 0; q < kBatch; ++q) mv[q] = gb + q < g1 ? gmax[(int64_t)(gb + q) * rows + row] : -__builtin_inff();
+#pragma unroll
+            for (int q = 0; q < kBatch; ++q) {
+                const float m = mv[q];
+                const int g = gb + q;
+                if (m != m) {
+                    const int64_t c0 = (int64_t)g * kGroupCols, c1 = c0 + kGroupCols < cols ? c0 + kGroupCols : cols;
+                    for (int64_t c = c0; c < c1; ++c) {
+                        const float v = xr[c];
+                        if (v != v) {
+                            if (c < nan_idx) nan_idx = c;
+                        } else if (v > val) {
+                            val = v;
+                            idx = c;
+                            grp = -1;
+                        }
+                    }
+                } else if (m > val) {
+                    val = m;
+                    idx = (int64_t)g * kGroupCols;
+                    grp = g;
+                }
+            }
+        }
+    }
+    s_val[slice][lr] = val;
+    s_idx[slice][lr] = idx;
+    s_nan[slice][lr] = nan_idx;
+    s_grp[slice][lr] = grp;
+    __syncthreads();
+    if (slice != 0 || !live) return;
+    for (int sl = 1; sl < kGroupSlices; ++sl) {  // column order: a later slice wins only with a strictly larger value
+        if (s_val[sl][lr] > val) {
+            val = s_val[sl][lr];
+            idx = s_idx[sl][lr];
+            grp = s_grp[sl][lr];
+        }
+        if (s_nan[sl][lr] < nan_idx) nan_idx = s_nan[sl][lr];
+    }
+    if (nan_idx != kNoNan) {
+        idx = nan_idx;
+    } else if (grp >= 0) {
+        const int64_t c0 = (int64_t)grp * kGroupCols, c1 = c0 + kGroupCols < cols ? c0 + kGroupCols : cols;
+        for (int64_t c = c0; c < c1; ++c)
+            if (xr[c] == val) {
+                idx = c;
+                break;
+            }
+    }
+    out[row] = (float)idx;
+}
+
 // Strided argmax over [outer, reduce, inner], inner > 1: one thread per output, coalesced on inner.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void argmax_strided_kernel(const T *__restrict__ x, int64_t outer, int64_t reduce,
@@ -402,6 +486,21 @@ int32_t launch_transpose(const T *src, T *dst, int64_t batch, int64_t rows, int6
 }
 
 }  // namespace
+
+namespace fth {
+int32_t argmax_from_group_max(const float *logits, int64_t rows, int64_t cols, const float *rowmax, int64_t groups, float *out,
+                              hipStream_t st) {
+    FTH_REQUIRE_DEVICE();
+    if (rows <= 0) return FTH_OK;
+    FTH_ARG(logits && rowmax && out && cols > 0 && groups == fth::gemm_rowmax_groups(cols),
+            "argmax_from_group_max: the groups do not cover the columns");
+    FTH_ARG(fth::ceil_div(rows, kGroupRows) <= kMaxGrid && groups <= 2147483647LL, "argmax_from_group_max: too many rows for one launch");
+    argmax_group_kernel<<<dim3((unsigned)fth::ceil_div(rows, kGroupRows)), dim3(kGroupRows * kGroupSlices), 0, st>>>(logits, rows, cols, rowmax,
+                                                                                                                   (int)groups, out);
+    FTH_CHECK_LAUNCH("argmax_from_group_max");
+    return FTH_OK;
+}
+}  // namespace fth
 
 extern "C" {
 

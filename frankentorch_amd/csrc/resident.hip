@@ -332,9 +332,9 @@ struct fth_gpt2 {
     Stack stack;
     int64_t vocab = 0, max_pos = 0;
     float *wte = nullptr, *wpe = nullptr, *lnf_w = nullptr, *lnf_b = nullptr;
-    float *x0 = nullptr, *hidden = nullptr, *logits = nullptr;
+    float *x0 = nullptr, *hidden = nullptr, *logits = nullptr, *group_max = nullptr;
     int64_t *bad = nullptr;
-    int64_t tokens_cap = 0, logits_cap = 0;
+    int64_t tokens_cap = 0, logits_cap = 0, group_max_cap = 0;
 };
 
 extern "C" {
@@ -859,6 +859,13 @@ int32_t fth_gpt2_forward_dev(fth_gpt2 *g, const double *ids_dev, int64_t batch, 
         }
         logits = g->logits;
     }
+    if (argmax_dev && T > g->group_max_cap) {  // row maxima per column group of the logits, for the fused argmax
+        void *p = nullptr;
+        if (int32_t rc = fth::pool_alloc(&p, (size_t)fth_dev_linear_argmax_workspace_floats(T, g->vocab) * sizeof(float))) return rc;
+        st.owned.push_back(p);
+        g->group_max = static_cast<float *>(p);
+        g->group_max_cap = T;
+    }
     int32_t rc;
     if ((rc = fth_dev_embedding_add_f32(g->wte, g->vocab, g->wpe, g->max_pos, ids_dev, T, seq, d, g->x0, g->bad, s))) return rc;
     const float *x = nullptr;
@@ -866,10 +873,14 @@ int32_t fth_gpt2_forward_dev(fth_gpt2 *g, const double *ids_dev, int64_t batch, 
     if ((rc = fth_dev_layer_norm_f32(x, g->lnf_w, g->lnf_b, g->hidden, T, d, st.eps, s))) return rc;
     if (logits) {
         // Tied head: the [vocab, d_model] embedding table is exactly the [out, in] weight layout.
-        fth_gemm_desc gd = linear_desc(T, g->vocab, d, FTH_EPI_NONE);
-        if ((rc = fth_dev_gemm_f32(&gd, 1.f, g->hidden, g->wte, logits, nullptr, nullptr, s))) return rc;
-        if (argmax_dev)
-            if ((rc = fth_dev_argmax_f32(logits, T, g->vocab, 1, argmax_dev, s))) return rc;
+        if (argmax_dev) {
+            if ((rc = fth_dev_linear_argmax_f32(g->hidden, g->wte, T, g->vocab, d, logits, argmax_dev, g->group_max,
+                                                fth_dev_linear_argmax_workspace_floats(g->group_max_cap, g->vocab), s)))
+                return rc;
+        } else {
+            fth_gemm_desc gd = linear_desc(T, g->vocab, d, FTH_EPI_NONE);
+            if ((rc = fth_dev_gemm_f32(&gd, 1.f, g->hidden, g->wte, logits, nullptr, nullptr, s))) return rc;
+        }
     }
     return FTH_OK;
 }

@@ -273,6 +273,18 @@ def argmax(x, outer, reduce, inner, out, stream=None):
     check(getattr(_lib.load(), "fth_dev_argmax_" + _sfx(x))(_ptr(x), outer, reduce, inner, _ptr(out), stream))
 
 
+def linear_argmax_workspace_floats(rows, out_features) -> int:
+    return int(_lib.load().fth_dev_linear_argmax_workspace_floats(rows, out_features))
+
+
+def linear_argmax(x, w, rows, out_features, in_features, logits, out, workspace=None, stream=None):
+    """logits = x . w^T and out = argmax over the last dim of the logits (fp32); workspace: a float32 DeviceBuffer of
+    linear_argmax_workspace_floats(rows, out_features) elements, or None for the two separate kernels."""
+    n = 0 if workspace is None else workspace.size
+    check(_lib.load().fth_dev_linear_argmax_f32(_ptr(x), _ptr(w), rows, out_features, in_features, _ptr(logits), _ptr(out),
+                                                _ptr(workspace), n, stream))
+
+
 def copy(x, y, n, stream=None):
     check(getattr(_lib.load(), "fth_dev_copy_" + _sfx(x))(_ptr(x), _ptr(y), n, stream))
 

@@ -234,6 +234,17 @@ int32_t fth_dev_embedding_add_f32(const float *wte, int64_t vocab, const float *
  * (crates/ft-kernel-cpu/src/lib.rs:39443-39550; f64 :18653). */
 int32_t fth_dev_argmax_f32(const float *x, int64_t outer, int64_t reduce, int64_t inner, float *out, fth_stream s);
 int32_t fth_dev_argmax_f64(const double *x, int64_t outer, int64_t reduce, int64_t inner, double *out, fth_stream s);
+/* logits = x . w^T (x [rows, in_features], w [out_features, in_features], both contiguous) and argmax[r] = the argmax of
+ * row r of those logits, by the rule above, in one pass over the logits: the linear product of a greedy decoding step
+ * (Linear::forward without bias, crates/ft-nn/src/lib.rs:2965-3010, then argmax_dim :39443). With a workspace of
+ * fth_dev_linear_argmax_workspace_floats(rows, out_features) floats (device memory, contents ignored and overwritten) the
+ * product's epilogue records the maximum of each row over every 32-column group and the argmax kernel reads those and a
+ * few 32-column pieces of the logits instead of every row again; with workspace NULL or smaller, or for shapes the
+ * large-tile product kernel does not take, fth_dev_gemm_f32 and fth_dev_argmax_f32 run one after the other. The indices
+ * are the same either way, bit for bit those fth_dev_argmax_f32 gives on the logits written here. */
+int64_t fth_dev_linear_argmax_workspace_floats(int64_t rows, int64_t out_features);
+int32_t fth_dev_linear_argmax_f32(const float *x, const float *w, int64_t rows, int64_t out_features, int64_t in_features,
+                                  float *logits, float *argmax, float *workspace, int64_t workspace_floats, fth_stream s);
 
 /* Head split / merge: dst[((b*H+h)*S+s)*hd+c] = src[((b*S+s)*H+h)*hd+c] and its inverse
  * (TensorTape::permute_slice, perm [0,2,1,3], crates/ft-autograd/src/lib.rs:10733-10882). */

@@ -125,3 +125,106 @@ def test_embedding_add_and_permute(hip, oracle):
         back = DeviceBuffer(shape)
         hip.permute_0213(dy, back, shape[0], shape[2], shape[1], shape[3])
         assert np.array_equal(back.to_host(), x)  # split then merge is the identity
+
+
+def _linear_argmax_case(rows, n, k, seed):
+    """Integer-valued operands (every logit is exact and ties abound) with rows that drive the special values through the
+    product: NaN from inf * 0, +-inf from inf * w and from overflow, an all -inf row, an all-zero row."""
+    rng = np.random.default_rng(seed)
+    x = rng.integers(-1, 2, size=(rows, k)).astype(np.float32)
+    w = rng.integers(-1, 2, size=(n, k)).astype(np.float32)
+    w[:, 1] = rng.choice(np.array([-2, -1, 1, 2], np.float32), size=n)  # never zero
+    w[:, 3] = rng.integers(1, 4, size=n).astype(np.float32)              # positive
+    w[:, 4] = 1.0
+    late = n - n // 5
+    w[late, 4] = 0.0                                                     # the one zero of column 4
+    special = {}
+    r = rows // 7
+    x[r] = 0; x[r, 0] = np.inf; special["nan_from_inf_times_zero"] = r          # NaN wherever w[:, 0] == 0: the first wins
+    r = rows // 5
+    x[r] = 0; special["all_zero_row"] = r                                       # all ties: index 0
+    r = rows // 3
+    x[r] = 0; x[r, 1] = np.inf; special["inf_no_nan"] = r                       # +-inf only: the first +inf
+    r = rows // 2
+    x[r] = 0; x[r, 2] = 3e38; w[:, 2] = rng.integers(-3, 4, size=n)             # overflow to +-inf through finite operands
+    special["overflow"] = r
+    r = rows - 2
+    x[r] = 0; x[r, 3] = -np.inf; special["all_neg_inf"] = r                     # every logit -inf: index 0
+    r = rows - 1
+    x[r] = 0; x[r, 4] = np.inf; special["one_late_nan"] = r                     # +inf everywhere, one NaN late in the row
+    return x, w, special, late
+
+
+@pytest.mark.parametrize("rows,n,k", [(1500, 12901, 64), (1100, 16384, 32), (2100, 8200, 96)])
+def test_linear_argmax_fused_equals_gemm_then_argmax(hip, oracle, rows, n, k):
+    """The product that records group maxima in its epilogue and the argmax that reads them give, bit for bit, the indices
+    of the plain argmax kernel on the same logits, and the logits of the plain product; tiles the product splits over
+    several workgroups, ragged last tiles and rows of NaN / +-inf go through the element-by-element branch."""
+    x, w, special, late = _linear_argmax_case(rows, n, k, seed=rows + n)
+    dx, dw = DeviceBuffer.from_host(x), DeviceBuffer.from_host(w)
+    nws = hip.linear_argmax_workspace_floats(rows, n)
+    assert nws == rows * 4 * ((n + 127) // 128)
+    sentinel = np.full(nws, 12345.0, np.float32)
+    ws = DeviceBuffer.from_host(sentinel)
+    logits, idx = DeviceBuffer((rows, n), np.float32), DeviceBuffer((rows,), np.float32)
+    hip.linear_argmax(dx, dw, rows, n, k, logits, idx, workspace=ws)
+    got_logits, got = logits.to_host(), idx.to_host()
+    gm = ws.to_host().reshape(-1, rows)
+    assert not np.any(gm == 12345.0), "the product kernel with the row-maximum epilogue did not run"
+    # the recorded maxima are right wherever they claim to be known
+    known = ~np.isnan(gm)
+    assert known.mean() > 0.3 and (~known).sum() > 0
+    pad = np.full((rows, gm.shape[0] * 32), -np.inf, np.float32)
+    pad[:, :n] = np.where(np.isnan(got_logits), np.inf, got_logits)
+    true_gm = pad.reshape(rows, -1, 32).max(axis=2).T
+    assert np.array_equal(gm[known], true_gm[known])
+    # logits: the plain product's, bit for bit (both are exact here where finite)
+    plain = DeviceBuffer((rows, n), np.float32)
+    hip.gemm(hip.gemm_desc(rows, n, k, trans_b=True), dx, dw, plain)
+    assert np.array_equal(got_logits, plain.to_host(), equal_nan=True)
+    ordinary = np.ones(rows, bool)
+    ordinary[list(special.values())] = False
+    assert np.array_equal(got_logits[ordinary], (x[ordinary].astype(np.float64) @ w.T.astype(np.float64)).astype(np.float32))
+    # indices: the plain kernel's on the same logits, and the checker's
+    ref_idx = DeviceBuffer((rows,), np.float32)
+    hip.argmax(logits, rows, n, 1, ref_idx)
+    assert np.array_equal(got, ref_idx.to_host())
+    assert np.array_equal(got, oracle.argmax(got_logits, 1))
+    assert got[special["all_zero_row"]] == 0 and got[special["all_neg_inf"]] == 0 and got[special["one_late_nan"]] == late
+    assert got[special["nan_from_inf_times_zero"]] == np.flatnonzero(w[:, 0] == 0)[0]
+    assert got[special["inf_no_nan"]] == np.flatnonzero(w[:, 1] > 0)[0]
+    assert got[special["overflow"]] == np.flatnonzero(w[:, 2] >= 2)[0]  # 3e38 * 1 is finite, * 2 is +inf
+    # without a workspace: the two separate kernels, same answers
+    idx2, logits2 = DeviceBuffer((rows,), np.float32), DeviceBuffer((rows, n), np.float32)
+    hip.linear_argmax(dx, dw, rows, n, k, logits2, idx2)
+    assert np.array_equal(idx2.to_host(), got) and np.array_equal(logits2.to_host(), got_logits, equal_nan=True)
+
+
+def test_linear_argmax_random_logits_and_small_shapes(hip, oracle):
+    """Normal operands at the vocabulary width (no exact ties), and shapes the large-tile kernel does not take, which fall
+    back to the two kernels with the workspace left untouched."""
+    rows, n, k = 1024, 50257, 128
+    x = synth.normal(11, "la.x", (rows, k)).astype(np.float32)
+    w = synth.normal(12, "la.w", (n, k)).astype(np.float32)
+    dx, dw = DeviceBuffer.from_host(x), DeviceBuffer.from_host(w)
+    ws = DeviceBuffer((hip.linear_argmax_workspace_floats(rows, n),), np.float32)
+    logits, idx, ref_idx = DeviceBuffer((rows, n), np.float32), DeviceBuffer((rows,), np.float32), DeviceBuffer((rows,), np.float32)
+    hip.linear_argmax(dx, dw, rows, n, k, logits, idx, workspace=ws)
+    hip.argmax(logits, rows, n, 1, ref_idx)
+    got_logits = logits.to_host()
+    assert np.array_equal(idx.to_host(), ref_idx.to_host())
+    assert np.array_equal(idx.to_host(), oracle.argmax(got_logits, 1))
+    ref = x.astype(np.float64) @ w.T.astype(np.float64)
+    assert np.abs(got_logits - ref).max() / np.abs(ref).max() <= 2e-5
+    for rows, n, k in [(3, 700, 64), (300, 1000, 40), (1, 20000, 96)]:
+        x = synth.normal(13, "la.x2", (rows, k)).astype(np.float32)
+        w = synth.normal(14, "la.w2", (n, k)).astype(np.float32)
+        nws = hip.linear_argmax_workspace_floats(rows, n)
+        ws = DeviceBuffer.from_host(np.full(nws, 7.0, np.float32))
+        logits, idx = DeviceBuffer((rows, n), np.float32), DeviceBuffer((rows,), np.float32)
+        hip.linear_argmax(DeviceBuffer.from_host(x), DeviceBuffer.from_host(w), rows, n, k, logits, idx, workspace=ws)
+        assert np.all(ws.to_host() == 7.0)
+        got_logits = logits.to_host()
+        assert np.array_equal(idx.to_host(), oracle.argmax(got_logits, 1))
+        ref = x.astype(np.float64) @ w.T.astype(np.float64)
+        assert np.abs(got_logits - ref).max() / np.abs(ref).max() <= 2e-5
