@@ -714,6 +714,21 @@ def bench_gpt2(device, synth, steps):
         % (ms, T / (ms * 1e-3), tf, 100 * tf / FP32_MFMA_PEAK_TF))
     res = {"ms": round(ms, 3), "tokens/s": round(T / (ms * 1e-3), 1), "TFLOP/s": round(tf, 2), "frac": round(tf / FP32_MFMA_PEAK_TF, 4),
            "flop": flop, "workload": "GPT-2-small shape: 12L d768 h12 ffn3072 vocab50257 B8 S1024 fp32, logits + argmax"}
+    # The head alone, the two ways the library can run it: the product with row maxima recorded in its epilogue followed by the
+    # small finishing kernel (what the forward above uses), and the plain product followed by the argmax kernel over all logits.
+    hx = DeviceBuffer.from_host(synth.normal(4, "head.x", (T, d), 0.0, 1.0))
+    hw = DeviceBuffer.from_host(wte)
+    hws = DeviceBuffer((device.linear_argmax_workspace_floats(T, vocab),))
+    n_head = max(5, steps // 4)
+    head_ms = {}
+    for name, wsp in (("fused", hws), ("separate", None)):
+        head_ms[name] = event_time_ms(device, lambda: device.linear_argmax(hx, hw, T, vocab, d, dlog, dam, workspace=wsp), n_head, warm_s=0.2)
+    fn()  # dam again holds the forward's argmax
+    res["lm_head_argmax"] = {"fused_ms": round(head_ms["fused"], 3), "separate_ms": round(head_ms["separate"], 3),
+                             "workload": "logits [8192, 50257] = x [8192, 768] . wte^T and the row argmax, back to back"}
+    log("[gpt2] LM head + argmax alone: %.3f ms with the row maxima recorded in the product's epilogue, %.3f ms as two kernels"
+        % (head_ms["fused"], head_ms["separate"]))
+    del hx, hw, hws
     # Weight ingestion: the same weights as a safetensors checkpoint (Hugging Face names, Conv1D [in, out] matrices) in
     # host memory, loaded straight into resident buffers (pinned staging, transposes on the GPU).
     import json
