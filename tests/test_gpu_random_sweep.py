@@ -242,3 +242,39 @@ def test_small_problem_kernels_random_shapes(hip, seed):
         if epi & 4:
             r = r + res
         assert rel(c.to_host(), r) <= 2e-5 * max(1.0, math.sqrt(k) / 4)
+
+
+@pytest.mark.parametrize("seed", [81])
+def test_linear_argmax_random_shapes_equal_the_plain_argmax(hip, seed):
+    """Shapes on both sides of every condition of the one-pass path (tile count against the compute units, K a multiple of
+    32 or not, ragged last tiles, one row), small-integer operands so that equal logits are the rule, and a few rows that
+    carry inf / NaN through the product: the indices must be those of the plain argmax kernel on the logits written."""
+    rng = np.random.default_rng(seed)
+    for it in range(24):
+        big = it % 3 != 2
+        k = int(rng.choice([32, 64, 96, 160, 256])) if rng.random() < 0.8 else int(rng.integers(1, 200))
+        if big:
+            rows = int(rng.integers(300, 2600))
+            n_lo = 128 * -(-256 // -(-rows // 128))  # where a 256-compute-unit part has one 128 x 128 tile per unit
+            n = int(rng.integers(n_lo - 600, n_lo + 3000))
+        else:
+            rows, n = int(rng.integers(1, 300)), int(rng.integers(1, 3000))
+        print("linear_argmax", dict(rows=rows, n=n, k=k), flush=True)
+        x = rng.integers(-1, 2, size=(rows, k)).astype(np.float32)
+        w = rng.integers(-1, 2, size=(n, k)).astype(np.float32)
+        for r in rng.integers(0, rows, size=min(rows, 6)):
+            x[r, rng.integers(0, k)] = rng.choice(np.array([np.inf, -np.inf, np.nan, 3e38], np.float32))
+        nws = hip.linear_argmax_workspace_floats(rows, n)
+        ws = DeviceBuffer.from_host(np.full(nws, 4321.0, np.float32))
+        dx, dw = DeviceBuffer.from_host(x), DeviceBuffer.from_host(w)
+        logits, idx, ref_idx = DeviceBuffer((rows, n)), DeviceBuffer((rows,)), DeviceBuffer((rows,))
+        hip.linear_argmax(dx, dw, rows, n, k, logits, idx, workspace=ws)
+        hip.argmax(logits, rows, n, 1, ref_idx)
+        assert np.array_equal(idx.to_host(), ref_idx.to_host())
+        got = logits.to_host()
+        plain = DeviceBuffer((rows, n))
+        hip.gemm(hip.gemm_desc(rows, n, k, trans_b=True), dx, dw, plain)
+        assert np.array_equal(got, plain.to_host(), equal_nan=True)
+        took_one_pass = not np.all(ws.to_host() == 4321.0)
+        tiles = -(-rows // 128) * -(-n // 128)
+        assert took_one_pass == (tiles >= hip.device_info()["compute_units"] and k % 32 == 0), (tiles, k)
