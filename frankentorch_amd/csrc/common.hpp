@@ -36,10 +36,10 @@ bool softmax_resident_rows(const float *x, float *y, int64_t rows, int64_t cols,
 bool softmax_resident_rows(const double *x, double *y, int64_t rows, int64_t cols, hipStream_t st);
 
 // logits = x . w^T (x [m, k], w [n, k], contiguous) with, as a by-product of the product's epilogue, the maximum of every
-// row over each group of 32 columns: rowmax[group * m + row], gemm_rowmax_groups(n) groups, NaN where a group's maximum is
+// row over each group of 64 columns: rowmax[group * m + row], gemm_rowmax_groups(n) groups, NaN where a group's maximum is
 // not known (the group holds a NaN). Returns false, nothing launched, for shapes
 // the large-tile direct kernel does not take. argmax_from_group_max then finds each row's argmax (first strict maximum, the
-// first NaN wins: the rule of the argmax kernel, bit for bit) from those maxima and at most a few 32-column pieces of the
+// first NaN wins: the rule of the argmax kernel, bit for bit) from those maxima and at most a few 64-column pieces of the
 // stored logits, instead of reading every row again.
 int64_t gemm_rowmax_groups(int64_t n);
 bool gemm_f32_nt_rowmax(int64_t m, int64_t n, int64_t k, const float *a, const float *b, float *c, float *rowmax, hipStream_t st,

@@ -70,8 +70,8 @@ constexpr int kGroupM = 8;
 #define FTH_F32_MINW 2
 #endif
 
-// Internal epilogue bit (not part of fth_gemm_desc.epilogue): also emit the maximum of every output row over each 32-column
-// piece of the tile (GemmArgs::rowmax). fp32 direct kernel for whole tiles, the fix-up kernel for split ones.
+// Internal epilogue bit (not part of fth_gemm_desc.epilogue): also emit the maximum of every output row over each wavefront's
+// 64 columns of the tile (GemmArgs::rowmax). fp32 direct kernel for whole tiles, the fix-up kernel for split ones.
 constexpr int kEpiRowMax = 64;
 
 template <typename T> struct Mfma;
@@ -119,6 +119,27 @@ template <> struct Mfma<double> {
     }
 };
 
+// fp32 on v_mfma_f32_16x16x4_f32: accumulator element r of `lane` is row 4 (lane / 16) + r, column lane % 16. The same
+// multiply-add rate as the 32x32x2 form and the same operand traffic; measured on the products that keep a workgroup on
+// one long run of tiles it is the faster of the two (8192 x 50257 x 768: 4.71 -> 4.58 ms; 4096^3 with a [n, k] B: 0.925 ->
+// 0.936 of the matrix peak), on the short launches of the transformer block and on [k, m] A operands the slower one
+// (linear backward 0.597 -> 0.611 ms), so it is used where DirectMfma says and nowhere else.
+struct MfmaF32x16 : Mfma<float> {
+    static constexpr int MT = 16;
+    static constexpr int KG = 4;
+    static constexpr int ACC = 4;
+    using Acc = float __attribute__((ext_vector_type(4)));
+    __device__ __forceinline__ static Acc mma(float a, float b, Acc c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+    __device__ __forceinline__ static int acc_row(int r, int lane) { return 4 * (lane >> 4) + r; }
+};
+constexpr int kEpiRowMaxBit = 64;
+// The MFMA form of a direct-kernel instantiation: 16x16x4 for fp32 x . w^T on 128 x 128 tiles with no epilogue (with or
+// without the row maxima), 32x32x2 (fp32) / 16x16x4 (fp64) otherwise. A function of the instantiation alone, so a shape
+// always gets the same arithmetic.
+template <typename T, int BM, int BN, bool TRANS_A, bool TRANS_B, int EPI> struct DirectMfma { using type = Mfma<T>; };
+template <> struct DirectMfma<float, 128, 128, false, true, 0> { using type = MfmaF32x16; };
+template <> struct DirectMfma<float, 128, 128, false, true, kEpiRowMaxBit> { using type = MfmaF32x16; };
+
 template <typename T> struct GemmArgs {
     const T *a;
     const T *b;
@@ -139,7 +160,7 @@ template <typename T> struct GemmArgs {
     T *partials;             // [grid][2][BM * BN] accumulator slots of split tiles
     int grid;                // workgroups of the main kernel (the fix-up kernel needs it too)
     int order = 0;           // tile order inside a group of tile rows: 0 column-major, 1 row-major (tile_of_id)
-    // Row maxima by column group (kEpiRowMax): [column groups][m], group g = columns [32 g, 32 g + 32), one MFMA tile wide.
+    // Row maxima by column group (kEpiRowMax): [column groups][m], group g = columns [64 g, 64 g + 64), one wavefront's share of a tile.
     // NaN = "not known, look at the stored values" (a group with a NaN in it).
     T *rowmax = nullptr;
 };
@@ -483,50 +504,41 @@ template <typename T> __device__ __forceinline__ void load_to_lds_16(const T *ba
                  : "memory", "m0");
 }
 
-// ---- row maxima of an accumulator tile (kEpiRowMax) ----
-// In the 32 x 32 accumulator a lane holds 16 rows of ONE column, so the maximum of a row over the tile's columns is a
-// reduction over the 32 lanes of a wavefront half. It is done as a transposing butterfly: at each step a lane keeps one
-// half of its values and hands the other half to a partner lane, so 8 + 4 + 2 + 1 exchanges (instead of 16 x 4) leave
-// every lane with the maximum, over its 16-lane row, of ONE accumulator row; one exchange with lane ^ 16 completes the 32
-// columns. The partners are lane +- 4 and lane ^ 8 first (data-parallel-primitive row rotations, whose bank mask does the
-// keep / hand-over selection for free), then lane ^ 1 and lane ^ 2 (quad permutations, selection by v_cndmask).
+// ---- row maxima of a wavefront's share of a tile (kEpiRowMax, 16 x 16 accumulators) ----
+// A lane holds four consecutive rows of ONE column of each 16 x 16 accumulator, and a wavefront's 64 columns of a row block
+// are four accumulators side by side, so the four are combined in the lane first; what is left is a reduction over the 16
+// lanes of a DPP row (the lanes that share lane / 16, i.e. the same four rows). It is done as a transposing butterfly over
+// the quad -- a lane keeps two of its four rows and hands the other two to lane ^ 1, then one of two to lane ^ 2 -- followed
+// by two row rotations (by 4 and by 8 lanes) that combine the four quads: 3 + 2 exchanges instead of 4 x 4. Lane l ends up
+// with the maximum of row element rowmax_elem_of_lane(l) over the wavefront's 64 columns.
 // The maximum is the NaN-propagating one (v_maximum3_f32): a group with a NaN in it comes out as NaN, which is exactly the
 // "not known, look at the stored values" marker the consumer expects, and +-inf are ordinary values.
-template <int CTRL, int BANKS> __device__ __forceinline__ float dpp_take(float old, float x) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, x), CTRL, 0xF, BANKS, false));
+template <int CTRL> __device__ __forceinline__ float dpp_take(float x) {
+    const int xi = __builtin_bit_cast(int, x);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(xi, xi, CTRL, 0xF, 0xF, false));
 }
 __device__ __forceinline__ float nan_max(float a, float b) { return __builtin_elementwise_maximum(a, b); }
-// v[0 .. 16): this lane's 16 accumulator values (element r = row M::acc_row(r, lane)). Returns in every lane the maximum
-// over the 32 lanes of its wavefront half of element rowmax_elem_of_lane(lane).
-__device__ __forceinline__ float rowmax_fold(float (&v)[16], int lane) {
+__device__ __forceinline__ float rowmax_fold(float (&v)[4], int lane) {
     constexpr int kRor4 = 0x124, kRor8 = 0x128, kXor1 = 0xB1, kXor2 = 0x4E;  // row_ror:4, row_ror:8, quad_perm [1,0,3,2], [2,3,0,1]
-#pragma unroll
-    for (int k = 0; k < 8; ++k)  // banks 0, 2 (lane bit 2 clear) keep elements 0..7, banks 1, 3 keep 8..15
-        v[k] = nan_max(dpp_take<kRor4, 0x5>(v[k + 8], v[k]), dpp_take<kRor4, 0xA>(v[k], v[k + 8]));
-#pragma unroll
-    for (int k = 0; k < 4; ++k)  // banks 0, 1 (lane bit 3 clear) keep the lower four of those
-        v[k] = nan_max(dpp_take<kRor8, 0x3>(v[k + 4], v[k]), dpp_take<kRor8, 0xC>(v[k], v[k + 4]));
     const bool up1 = (lane & 1) != 0, up2 = (lane & 2) != 0;
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
         const float keep = up1 ? v[k + 2] : v[k], send = up1 ? v[k] : v[k + 2];
-        v[k] = nan_max(keep, dpp_take<kXor1, 0xF>(send, send));
+        v[k] = nan_max(keep, dpp_take<kXor1>(send));
     }
     const float keep = up2 ? v[1] : v[0], send = up2 ? v[0] : v[1];
-    const float m = nan_max(keep, dpp_take<kXor2, 0xF>(send, send));
-    // lane ^ 16 within 32 lanes: and 0x1F, or 0, xor 16
-    return nan_max(m, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, m), (16 << 10) | 0x1F)));
+    float m = nan_max(keep, dpp_take<kXor2>(send));
+    m = nan_max(m, dpp_take<kRor4>(m));
+    return nan_max(m, dpp_take<kRor8>(m));
 }
-__device__ __forceinline__ int rowmax_elem_of_lane(int lane) {
-    return ((lane & 4) << 1) | ((lane & 8) >> 1) | ((lane & 1) << 1) | ((lane & 2) >> 1);
-}
+__device__ __forceinline__ int rowmax_elem_of_lane(int lane) { return ((lane & 1) << 1) | ((lane >> 1) & 1); }
 
 // EPI >= 0: the epilogue flags are this compile-time mask and alpha is 1 (straight-line output code);
 // EPI < 0: flags and alpha are read from the arguments.
 // TRANS_A: A is stored [k, m] (its tile is kept [k][m] in LDS and read element-wise, like a [k,n] B).
 template <typename T, int BM, int BN, int WM, int WN, int MINW, bool TRANS_A, bool TRANS_B, int EPI>
 __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const GemmArgs<T> p) {
-    using M = Mfma<T>;
+    using M = typename DirectMfma<T, BM, BN, TRANS_A, TRANS_B, EPI>::type;
     using V = typename M::V;
     constexpr int MT = M::MT, KG = M::KG, EPV = M::EPV;
     constexpr int NW = WM * WN, NT = NW * kWave;
@@ -573,6 +585,7 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
     for (int kc = 0; kc < NCH; ++kc) roff[kc] = ((kc * KG + lane / MT) ^ swz(lrow)) * EPV;
 
     constexpr bool ROWMAX = EPI >= 0 && (EPI & kEpiRowMax) != 0 && std::is_same<T, float>::value;
+    static_assert(kEpiRowMax == kEpiRowMaxBit, "one bit, two names");
     const int epi = EPI >= 0 ? (EPI & ~kEpiRowMax) : p.epilogue;
     const bool has_bias = (epi & FTH_EPI_BIAS) != 0;
     const bool has_gelu = (epi & FTH_EPI_GELU) != 0;
@@ -768,29 +781,31 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
         if (has_res) v = v + rv;
         return v;
     };
-    // One 32 x 32 piece of a whole tile has been written: the maximum of each of its rows, one value per row from the
-    // lanes that hold it after the fold.
-    auto rowmax_emit = [&](float (&v)[16], int i, int j, int64_t m0_, int64_t n0_) __attribute__((always_inline)) {
+    // Row block i of a whole tile has been written (its TN accumulators side by side, combined in `v`): one maximum per row
+    // over this wavefront's 64 columns, from the lanes that hold it after the fold.
+    auto rowmax_emit = [&](float (&v)[4], int i, int64_t m0_, int64_t n0_) __attribute__((always_inline)) {
         const float mine = rowmax_fold(v, lane);
         const int64_t row = m0_ + wm0 + i * MT + M::acc_row(rowmax_elem_of_lane(lane), lane);
-        const int64_t group = (n0_ + wn0 + j * MT) / MT;
-        if (lrow < 16 && row < p.m) p.rowmax[group * p.m + row] = mine;
+        const int64_t group = (n0_ + wn0) / WTN;
+        if ((lane & 15) < 4 && row < p.m) p.rowmax[group * p.m + row] = mine;
     };
     auto out_store = [&](auto S, auto &src, bool full, int64_t m0_, int64_t n0_, int64_t batch_, T *slot_) __attribute__((always_inline)) {
         constexpr int sidx = decltype(S)::value;
         if (full) {
             const bool interior = is_interior(m0_, n0_);
+            // Row maxima: a share is one row block of the wavefront's part of the tile (its TN accumulators side by side).
+            static_assert(!ROWMAX || (M::ACC == 4 && TILES_PP == TN), "the row-maximum epilogue is written for 16 x 16 accumulators");
+            float seen[ROWMAX ? 4 : 1];  // per accumulator row: the largest value written, -inf where this lane wrote none
+            if constexpr (ROWMAX) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) seen[r] = -__builtin_inff();
+            }
 #pragma unroll
             for (int u = 0; u < TILES_PP; ++u) {
                 const int t = sidx * TILES_PP + u, i = t / TN, j = t % TN;
                 const int64_t col = n0_ + wn0 + j * MT + lrow;
-                float seen[ROWMAX ? 16 : 1];  // the values written, -inf where this lane wrote none
-                if constexpr (ROWMAX) {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) seen[r] = -__builtin_inff();
-                }
                 auto note = [&](int r, T val) __attribute__((always_inline)) {
-                    if constexpr (ROWMAX) seen[r] = (float)val;
+                    if constexpr (ROWMAX) seen[r] = nan_max(seen[r], (float)val);
                 };
                 if (interior) {
                     const int64_t tile_off = batch_ * p.stride_c + (m0_ + wm0 + i * MT) * p.ldc + (n0_ + wn0 + j * MT);
@@ -818,8 +833,8 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
                         }
                     }
                 }
-                if constexpr (ROWMAX) rowmax_emit(seen, i, j, m0_, n0_);
             }
+            if constexpr (ROWMAX) rowmax_emit(seen, sidx * TILES_PP / TN, m0_, n0_);
         } else {
 #pragma unroll
             for (int u = 0; u < TILES_PP; ++u) {
@@ -963,9 +978,8 @@ __global__ __launch_bounds__(WM *WN *kWave, MINW) void gemm_direct_kernel(const 
 // values each thread owned in the main kernel.
 constexpr int kFixupParts = 4;
 
-template <typename T, int BM, int BN, int WM, int WN>
+template <typename T, int BM, int BN, int WM, int WN, typename M>
 __global__ __launch_bounds__(WM *WN *kWave) void gemm_fixup_kernel(const GemmArgs<T> p) {
-    using M = Mfma<T>;
     using V = typename M::V;
     constexpr int MT = M::MT, EPV = M::EPV;
     constexpr int NT = WM * WN * kWave;
@@ -1022,13 +1036,14 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemm_fixup_kernel(const GemmArg
     tile_of_id(tile - batch * p.tiles_per_batch, p.tiles_m, p.tiles_n, tile_m, tile_n, p.order);
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
     T *C = p.c + batch * p.stride_c;
-    // Row maxima (GemmArgs::rowmax) of a split tile: this workgroup's share is exactly one 32 x 32 piece (all 16 values a
-    // lane holds of it), in the main kernel's lane layout, so the same fold applies.
-    constexpr bool ROWMAX = std::is_same<T, float>::value && PV == M::ACC && M::ACC == 16;
-    float seen[ROWMAX ? 16 : 1];
+    // Row maxima (GemmArgs::rowmax) of a split tile: with 16 x 16 accumulators this workgroup's share is exactly one row block
+    // of each wavefront's part of the tile (TN accumulators, 4 values a lane of each), in the main kernel's lane layout, so
+    // the same in-lane combination and fold apply.
+    constexpr bool ROWMAX = std::is_same<T, float>::value && M::ACC == 4 && PV == M::ACC * TN;
+    float seen[ROWMAX ? 4 : 1];
     if constexpr (ROWMAX) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) seen[r] = -__builtin_inff();
+        for (int r = 0; r < 4; ++r) seen[r] = -__builtin_inff();
     }
     const bool has_bias = (p.epilogue & FTH_EPI_BIAS) != 0;
     const bool has_gelu = (p.epilogue & FTH_EPI_GELU) != 0;
@@ -1048,16 +1063,16 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemm_fixup_kernel(const GemmArg
             if (has_gelu_tanh) v = M::gelu_tanh(v);
             if (has_res) v = v + p.residual[batch * p.stride_c + row * p.ldc + col];
             C[row * p.ldc + col] = v;
-            if constexpr (ROWMAX) seen[u] = (float)v;
+            if constexpr (ROWMAX) seen[r] = nan_max(seen[r], (float)v);
         }
     }
     if constexpr (ROWMAX) {
         if (p.rowmax != nullptr) {  // uniform: every lane takes part in the fold
-            const int j = (int)blockIdx.y % TN, i = (int)blockIdx.y / TN;
+            const int i = (int)blockIdx.y;  // the row block this share is
             const float mine = rowmax_fold(seen, lane);
             const int64_t row = m0 + wm0 + i * MT + M::acc_row(rowmax_elem_of_lane(lane), lane);
-            const int64_t group = (n0 + wn0 + j * MT) / MT;
-            if (lrow < 16 && row < p.m) p.rowmax[group * p.m + row] = (T)mine;
+            const int64_t group = (n0 + wn0) / WTN;
+            if ((lane & 15) < 4 && row < p.m) p.rowmax[group * p.m + row] = (T)mine;
         }
     }
 }
@@ -1294,7 +1309,7 @@ constexpr int kMinItersPerBlock = 4;  // never cut the iteration space finer tha
 
 // Launches a persistent main kernel over the stream-K schedule, then the fix-up kernel if any
 // tile is split. `blocks_per_cu` caches the kernel's occupancy (one static per kernel).
-template <typename T, int BM, int BN, int WM, int WN, typename Kern>
+template <typename T, int BM, int BN, int WM, int WN, typename MM, typename Kern>
 int32_t launch_persistent(Kern kern, size_t smem, int BK, int &blocks_per_cu, GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     constexpr int NT = WM * WN * kWave;
     if (blocks_per_cu == 0) {  // benign race: both calls are idempotent
@@ -1348,7 +1363,7 @@ int32_t launch_persistent(Kern kern, size_t smem, int BK, int &blocks_per_cu, Ge
     kern<<<dim3((unsigned)grid), dim3(NT), smem, st>>>(p);
     FTH_CHECK_LAUNCH("gemm");
     if (any_split) {
-        gemm_fixup_kernel<T, BM, BN, WM, WN><<<dim3((unsigned)(grid - 1), kFixupParts), dim3(NT), 0, st>>>(p);
+        gemm_fixup_kernel<T, BM, BN, WM, WN, MM><<<dim3((unsigned)(grid - 1), kFixupParts), dim3(NT), 0, st>>>(p);
         FTH_CHECK_LAUNCH("gemm_fixup");
     }
     return FTH_OK;
@@ -1359,7 +1374,7 @@ int32_t launch_config(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     constexpr int S = BK + Mfma<T>::EPV;
     constexpr size_t smem = (size_t)2 * (BM + BN) * S * sizeof(T);
     static int blocks_per_cu = 0;
-    return launch_persistent<T, BM, BN, WM, WN>(gemm_kernel<T, BM, BN, BK, WM, WN, MINW, TRANS_B, VEC, VECB>, smem, BK, blocks_per_cu, p,
+    return launch_persistent<T, BM, BN, WM, WN, Mfma<T>>(gemm_kernel<T, BM, BN, BK, WM, WN, MINW, TRANS_B, VEC, VECB>, smem, BK, blocks_per_cu, p,
                                                  batch, st);
 }
 
@@ -1368,7 +1383,8 @@ int32_t launch_direct_epi(GemmArgs<T> &p, int64_t batch, hipStream_t st) {
     constexpr int BK = 128 / (int)sizeof(T);
     constexpr size_t smem = (size_t)2 * (BM + BN) * BK * sizeof(T);
     static int blocks_per_cu = 0;
-    return launch_persistent<T, BM, BN, WM, WN>(gemm_direct_kernel<T, BM, BN, WM, WN, MINW, TRANS_A, TRANS_B, EPI>, smem, BK, blocks_per_cu, p,
+    return launch_persistent<T, BM, BN, WM, WN, typename DirectMfma<T, BM, BN, TRANS_A, TRANS_B, EPI>::type>(
+        gemm_direct_kernel<T, BM, BN, WM, WN, MINW, TRANS_A, TRANS_B, EPI>, smem, BK, blocks_per_cu, p,
                                                  batch, st);
 }
 
@@ -1558,7 +1574,7 @@ int32_t gemm_entry(const fth_gemm_desc *d, T alpha, const T *a, const T *b, T *c
     return vecb ? launch_shape<T, false, false, true>(p, d->batch, st) : launch_shape<T, false, false, false>(p, d->batch, st);
 }
 
-// C = A . B^T (A [m, k], B [n, k], both row-major and contiguous) on 128 x 128 tiles with the row maxima of every 32-column
+// C = A . B^T (A [m, k], B [n, k], both row-major and contiguous) on 128 x 128 tiles with the row maxima of every 64-column
 // group as a by-product (GemmArgs::rowmax). Returns false, with nothing launched, where the direct-to-LDS kernel or the
 // large tiles do not apply.
 bool launch_nt_rowmax(int64_t m, int64_t n, int64_t k, const float *a, const float *b, float *c, float *rowmax, hipStream_t st, int32_t *rc) {
@@ -1621,7 +1637,7 @@ template <typename T> int32_t launch_trans_a(GemmArgs<T> &p, const fth_gemm_desc
 }  // namespace
 
 namespace fth {
-int64_t gemm_rowmax_groups(int64_t n) { return fth::ceil_div(n, 128) * 4; }
+int64_t gemm_rowmax_groups(int64_t n) { return fth::ceil_div(n, 128) * 2; }
 bool gemm_f32_nt_rowmax(int64_t m, int64_t n, int64_t k, const float *a, const float *b, float *c, float *rowmax, hipStream_t st,
                         int32_t *rc) {
     return launch_nt_rowmax(m, n, k, a, b, c, rowmax, st, rc);

@@ -198,7 +198,7 @@ __global__ __launch_bounds__(kBlock) void argmax_lastdim_kernel(const T *__restr
 }
 
 // ---- argmax from the row maxima of column groups ----------------------------------------------
-// gmax[g * rows + row] is the maximum of row `row` over columns [32 g, 32 g + 32), written by the product that made the
+// gmax[g * rows + row] is the maximum of row `row` over columns [64 g, 64 g + 64), written by the product that made the
 // logits, or NaN where that is not known (the group holds a NaN). A row's
 // argmax is then the first element equal to the largest group maximum, in the first group that attains it -- found by
 // reading that one group -- after the unknown groups have been scanned element by element with the rule of
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(kBlock) void argmax_lastdim_kernel(const T *__restr
 // holds no NaN, its maximum is an element of it, and ties go to the earlier column either way. A workgroup takes 32
 // consecutive rows (their group maxima are one 128-byte segment) and deals the groups, in column order, to 32 slices whose
 // candidates are merged in that order.
-constexpr int kGroupCols = 32;
+constexpr int kGroupCols = 64;
 constexpr int kGroupRows = 32;    // rows per workgroup: one per lane of a half wavefront
 constexpr int kGroupSlices = 32;  // column slices per workgroup (1024 threads)
 __global__ __launch_bounds__(kGroupRows * kGroupSlices) void argmax_group_kernel(const float *__restrict__ logits, int64_t rows, int64_t cols,

@@ -238,8 +238,8 @@ int32_t fth_dev_argmax_f64(const double *x, int64_t outer, int64_t reduce, int64
  * row r of those logits, by the rule above, in one pass over the logits: the linear product of a greedy decoding step
  * (Linear::forward without bias, crates/ft-nn/src/lib.rs:2965-3010, then argmax_dim :39443). With a workspace of
  * fth_dev_linear_argmax_workspace_floats(rows, out_features) floats (device memory, contents ignored and overwritten) the
- * product's epilogue records the maximum of each row over every 32-column group and the argmax kernel reads those and a
- * few 32-column pieces of the logits instead of every row again; with workspace NULL or smaller, or for shapes the
+ * product's epilogue records the maximum of each row over every 64-column group and the argmax kernel reads those and a
+ * few 64-column pieces of the logits instead of every row again; with workspace NULL or smaller, or for shapes the
  * large-tile product kernel does not take, fth_dev_gemm_f32 and fth_dev_argmax_f32 run one after the other. The indices
  * are the same either way, bit for bit those fth_dev_argmax_f32 gives on the logits written here. */
 int64_t fth_dev_linear_argmax_workspace_floats(int64_t rows, int64_t out_features);
