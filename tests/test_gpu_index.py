@@ -155,7 +155,7 @@ def _linear_argmax_case(rows, n, k, seed):
     return x, w, special, late
 
 
-@pytest.mark.parametrize("rows,n,k", [(1500, 12901, 64), (1100, 16384, 32), (2100, 8200, 96)])
+@pytest.mark.parametrize("rows,n,k", [(1500, 12901, 64), (1100, 16384, 32), (2100, 8200, 96), (40, 40000, 64)])
 def test_linear_argmax_fused_equals_gemm_then_argmax(hip, oracle, rows, n, k):
     """The product that records group maxima in its epilogue and the argmax that reads them give, bit for bit, the indices
     of the plain argmax kernel on the same logits, and the logits of the plain product; tiles the product splits over
